@@ -1,0 +1,196 @@
+"""Oracle restatement of the layer math on the quantized-weight path (test infrastructure, see oracle/__init__.py).
+
+Weight-only numerics: BF16 activations, exactly dequantized weights, FP32 (or wider) accumulation, the rounding
+points of the reference kept.
+
+  dense_ref              x.float() @ W_deq.T, one rounding to BF16  (profiling/w3_bench.py:75 `y_exact`;
+                         hibana/kernels/w3.py:239-242 for W_deq)
+  nvfp4_dense_ref        bf16((x @ Wq^T)_fp32 * s2), Wq = e2m1 * e4m3 exact in BF16
+                         (tests/nemotron_reference.py:236-254; tests/gpu/test_bolt_kernels.py:29-32)
+  fc1_order              hibana/kernels/w3_moe.py:88-92
+  expert_plan            hibana/kernels/csrc/w3_gemm.cu:710-782: ascending distinct local experts, CSR starts, pair
+                         indices of each expert in ascending order (a stable sort by expert)
+  routed_experts_ref     hibana/kernels/w3_moe.py:193-214 with an identity `quant` (weight-only): h1 = bf16(fc1 x),
+                         h = bf16(silu(gate) * up) or bf16(relu(h1)^2) with an FP32 square, y = fc2 h in FP32 per pair
+  combine_ref            hibana/kernels/csrc/w3_gemm.cu:1196-1213: v = fma(w_k, y_k, v) over the row's slots in
+                         selection order, skipping ids outside the local range, one rounding to BF16
+  combine_shared_ref     hibana/kernels/flashnext_fused.py:530-571: bf16(bf16(routed) + sigmoid(x . g) * shared)
+  route_softmax_topk     hibana/model/flashnext/moe.py:141-144 (== flashnext_fused.py:278-319): softmax, top-k
+                         descending, renormalized
+  route_sigmoid_topk     hibana/model/nemotron/moe.py:1-12, tests/nemotron_reference.py:550-565: top-k of
+                         sigmoid + bias (ties to the lower id), weights from the plain sigmoid, renormalized, scaled
+  latent_moe_ref         tests/nemotron_reference.py:568-593 (ReLU^2 latent experts, BF16 linears, FP32 accumulate)
+  silu_and_mul           hibana/kernels/ops.py:86-92
+
+Pinned by (tests/test_oracle_layers.py): special cases that reduce to textbook routines (one token, one expert, weight
+one == two dense products; all weights zero == zero; a permutation of slots with equal weights), brute-force
+per-pair Python loops on tiny shapes written from the formula in w3_moe.py:205-213, torch.topk/softmax for the
+routing, and sortedness/CSR invariants for the plan.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+
+def bf16(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.bfloat16)
+
+
+def dense_ref(x: torch.Tensor, w_deq, wide: bool = True) -> torch.Tensor:
+    """x BF16 [M, K], w_deq float32 [N, K] -> BF16 [M, N]; accumulation in FP64 (`wide`) or FP32."""
+    w = torch.as_tensor(w_deq)
+    if wide:
+        return bf16((x.double() @ w.double().T).float())
+    return bf16(x.float() @ w.float().T)
+
+
+def nvfp4_dense_ref(x: torch.Tensor, w_unscaled, scale2: float, relu2: bool = False) -> torch.Tensor:
+    """x BF16 [M, K], w_unscaled float32 [N, K] = e2m1 * e4m3 (no global scale) -> BF16 [M, N]."""
+    w = torch.as_tensor(w_unscaled)
+    y = bf16(((x.double() @ w.double().T).float() * np.float32(scale2)))
+    if relu2:
+        y = bf16(torch.relu(y.float()).square())
+    return y
+
+
+def fc1_order(inter: int) -> np.ndarray:
+    out = np.empty(2 * inter, dtype=np.int64)
+    for b in range(inter // 16):
+        out[32 * b:32 * b + 16] = 16 * b + np.arange(16)
+        out[32 * b + 16:32 * b + 32] = inter + 16 * b + np.arange(16)
+    return out
+
+
+def expert_plan(ids: np.ndarray, e_lo: int, e_n: int):
+    """ids int [M, k] -> (experts ascending local ids [D], starts [D+1], order [sum counts] pair indices q = r*k + slot).
+    Pairs whose id is outside [e_lo, e_lo + e_n) are dropped."""
+    flat = np.asarray(ids).reshape(-1).astype(np.int64) - e_lo
+    valid = (flat >= 0) & (flat < e_n)
+    experts = np.unique(flat[valid])
+    starts = [0]
+    order = []
+    for e in experts:
+        q = np.nonzero(flat == e)[0]  # ascending
+        order.extend(q.tolist())
+        starts.append(len(order))
+    return experts, np.asarray(starts, dtype=np.int64), np.asarray(order, dtype=np.int64)
+
+
+def silu_and_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:
+    half = gate_up.shape[-1] // 2
+    if pairs:
+        blocks = gate_up.unflatten(-1, (half // pairs, 2, pairs))
+        return (torch.nn.functional.silu(blocks[..., 0, :]) * blocks[..., 1, :]).flatten(-2)
+    return torch.nn.functional.silu(gate_up[..., :half]) * gate_up[..., half:]
+
+
+def expert_pairs_ref(x: torch.Tensor, rows: np.ndarray, w13, w2, gated: bool) -> torch.Tensor:
+    """One expert on the token rows `rows` of x: w13 float32 [N1, K] with rows in checkpoint order ([up; gate] when
+    gated, up alone otherwise), w2 float32 [H, I] -> FP32 [len(rows), H]."""
+    w13, w2 = torch.as_tensor(w13).double(), torch.as_tensor(w2).double()
+    h1 = bf16((x[torch.as_tensor(rows)].double() @ w13.T).float()).float()
+    if gated:
+        inter = w13.shape[0] // 2
+        h = bf16(torch.nn.functional.silu(h1[:, inter:]) * h1[:, :inter])
+    else:
+        h = bf16(torch.relu(h1).square())
+    return (h.double() @ w2.T).float()
+
+
+def routed_experts_ref(x: torch.Tensor, ids: np.ndarray, get_expert, gated: bool, e_lo: int = 0, e_n: int = 512):
+    """FP32 pair outputs [M*k, H] (rows of dropped pairs are zero). get_expert(local id) -> (w13 [N1, K] float32 in
+    checkpoint row order, w2 [H, I] float32)."""
+    ids = np.asarray(ids)
+    m, k = ids.shape
+    experts, starts, order = expert_plan(ids, e_lo, e_n)
+    pairs = None
+    for d, e in enumerate(experts):
+        q = order[starts[d]:starts[d + 1]]
+        w13, w2 = get_expert(int(e))
+        y = expert_pairs_ref(x, q // k, w13, w2, gated)
+        if pairs is None:
+            pairs = torch.zeros(m * k, y.shape[1], dtype=torch.float32)
+        pairs[torch.as_tensor(q)] = y
+    return pairs
+
+
+def combine_ref(pairs: torch.Tensor, ids: np.ndarray, weights: torch.Tensor, e_lo: int = 0, e_n: int = 512) -> torch.Tensor:
+    """BF16 [M, H]: the FMA chain over the slots in selection order (an FP32 FMA is one rounding of the exact
+    a*b + c, reproduced here in FP64: the product of two FP32 values is exact there)."""
+    ids = np.asarray(ids)
+    m, k = ids.shape
+    v = torch.zeros(m, pairs.shape[1], dtype=torch.float32)
+    w = weights.float()
+    for slot in range(k):
+        local = ids[:, slot] - e_lo
+        keep = torch.as_tensor((local >= 0) & (local < e_n))
+        y = pairs.view(m, k, -1)[:, slot]
+        nxt = (v.double() + w[:, slot, None].double() * y.double()).float()
+        v = torch.where(keep[:, None], nxt, v)
+    return bf16(v)
+
+
+def combine_shared_ref(routed: torch.Tensor, shared: torch.Tensor, x: torch.Tensor = None, gate_vec: torch.Tensor = None):
+    """bf16(routed + g * shared) with g = sigmoid(x . gate_vec) in FP32, or 1 when no gate vector is given."""
+    r, s = routed.float(), shared.float()
+    if gate_vec is None:
+        return bf16(r + s)
+    g = torch.sigmoid((x.double() @ gate_vec.double()).float())[:, None]
+    return bf16(r + g * s)
+
+
+def moe_layer_ref(x, ids, weights, get_expert, gated: bool, shared=None, gate_vec=None, e_lo: int = 0, e_n: int = 512):
+    """The gated-MoE layer of hibana/model/flashnext/moe.py:177-192 on 3-bit experts: routed sum, plus the shared
+    expert (w13, w2 in checkpoint row order) rounded to BF16 on its own, combined as combine_shared_ref."""
+    pairs = routed_experts_ref(x, ids, get_expert, gated, e_lo, e_n)
+    if pairs is None:
+        width = shared[1].shape[0] if shared is not None else x.shape[1]
+        pairs = torch.zeros(np.asarray(ids).size, width)
+    routed = combine_ref(pairs, ids, weights, e_lo, e_n)
+    if shared is None:
+        return routed
+    s = bf16(expert_pairs_ref(x, np.arange(x.shape[0]), shared[0], shared[1], gated))
+    return combine_shared_ref(routed, s, x, gate_vec)
+
+
+def route_softmax_topk(logits: torch.Tensor, k: int):
+    probs = torch.softmax(logits.float(), dim=-1)
+    w, ids = torch.topk(probs, k, dim=-1)
+    return ids.to(torch.int32), (w / w.sum(-1, keepdim=True)).contiguous()
+
+
+def route_sigmoid_topk(logits: torch.Tensor, bias: torch.Tensor, k: int, scaling: float = 1.0):
+    s = torch.sigmoid(logits.float())
+    choice = s + bias.float()
+    # ties to the lower id: a stable descending sort
+    ids = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :k]
+    w = s.gather(1, ids)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20) * scaling
+    return ids.to(torch.int32), w.contiguous()
+
+
+def latent_experts_ref(lat: torch.Tensor, ids: np.ndarray, weights: torch.Tensor, get_expert):
+    """The routed part of the latent MoE: lat BF16 [M, L]; get_expert(e) -> (up_unscaled [I, L] float32, up_s2,
+    down_unscaled [L, I] float32, down_s2). Returns the FP32 accumulator [M, L]:
+    h = bf16(relu(bf16((lat up^T) s2))^2); acc[tok] += ((h down^T) s2) * w, experts in ascending id order."""
+    ids = np.asarray(ids)
+    m, k = ids.shape
+    acc = torch.zeros(m, lat.shape[1], dtype=torch.float32)
+    w = weights.float()
+    for e in np.unique(ids):
+        tok, slot = np.nonzero(ids == e)
+        up, up_s, down, down_s = get_expert(int(e))
+        t = torch.as_tensor(tok)
+        h = nvfp4_dense_ref(lat[t], up, up_s, relu2=True)
+        y = (h.double() @ torch.as_tensor(down).double().T).float() * np.float32(down_s)
+        acc.index_add_(0, t, y * w[t, torch.as_tensor(slot), None])
+    return acc
+
+
+def latent_moe_ref(x, fc1, fc2, ids, weights, get_expert):
+    """x BF16 [M, H], fc1 BF16 [L, H], fc2 BF16 [H, L] -> BF16 [M, H]:
+    lat = bf16(x fc1^T); out = bf16(bf16(acc) fc2^T)."""
+    lat = bf16((x.double() @ fc1.double().T).float())
+    acc = latent_experts_ref(lat, ids, weights, get_expert)
+    return bf16((bf16(acc).double() @ fc2.double().T).float())

@@ -1,0 +1,146 @@
+"""The oracle's layer math against special cases, brute force and library routines (CPU)."""
+import numpy as np
+import torch
+
+from oracle import layers as L
+
+
+def _experts(e, inter, hidden, gated, seed):
+    g = torch.Generator().manual_seed(seed)
+    n1 = 2 * inter if gated else inter
+    w13 = torch.randn(e, n1, hidden, generator=g) * 0.05
+    w2 = torch.randn(e, hidden, inter, generator=g) * 0.05
+    return lambda i: (w13[i].numpy(), w2[i].numpy()), w13, w2
+
+
+def test_fc1_order_pairs_up_and_gate_rows():
+    """tests/unit/test_w3_moe_pack.py:27-31 of the reference."""
+    order = L.fc1_order(128)
+    assert sorted(order.tolist()) == list(range(256))
+    blocks = order.reshape(-1, 32)
+    assert np.array_equal(blocks[:, 16:], blocks[:, :16] + 128)
+
+
+def test_plan_is_a_stable_sort_with_csr_starts():
+    g = np.random.default_rng(0)
+    ids = g.integers(0, 20, (37, 6))
+    ids[3, 2] = 512
+    experts, starts, order = L.expert_plan(ids, 4, 10)
+    flat = ids.reshape(-1) - 4
+    key = np.where((flat >= 0) & (flat < 10), flat, 512)
+    want = np.argsort(key, kind="stable")[:np.count_nonzero(key < 512)]
+    assert np.array_equal(order, want)
+    assert experts.tolist() == sorted(set(key[key < 512].tolist()))
+    for d, e in enumerate(experts):
+        assert (key[order[starts[d]:starts[d + 1]]] == e).all()
+    assert starts[0] == 0 and starts[-1] == len(order)
+
+
+def test_one_token_one_expert_reduces_to_two_dense_products():
+    get, w13, w2 = _experts(3, 64, 128, True, 1)
+    x = torch.randn(1, 128, generator=torch.Generator().manual_seed(2)).bfloat16()
+    out = L.moe_layer_ref(x, np.array([[2]]), torch.ones(1, 1), get, True)
+    h1 = (x.float() @ w13[2].T).bfloat16().float()
+    h = (torch.nn.functional.silu(h1[:, 64:]) * h1[:, :64]).bfloat16()
+    want = (h.float() @ w2[2].T).bfloat16()
+    assert torch.allclose(out.float(), want.float(), rtol=2 ** -7, atol=1e-6)
+    relu_get, r13, r2 = _experts(3, 64, 128, False, 4)
+    out = L.moe_layer_ref(x, np.array([[1]]), torch.ones(1, 1), relu_get, False)
+    h = torch.relu((x.float() @ r13[1].T).bfloat16().float()).square().bfloat16()
+    assert torch.allclose(out.float(), (h.float() @ r2[1].T).bfloat16().float(), rtol=2 ** -7, atol=1e-6)
+
+
+def test_matches_a_per_pair_loop_written_from_the_reference_formula():
+    """hibana/kernels/w3_moe.py:205-213 with an identity activation rounding, one (row, slot) at a time."""
+    import torch.nn.functional as F
+    for gated in (True, False):
+        get, w13, w2 = _experts(6, 32, 128, gated, 5)
+        gen = torch.Generator().manual_seed(6)
+        m, k, inter = 7, 3, 32
+        x = torch.randn(m, 128, generator=gen).bfloat16()
+        ids = torch.stack([torch.randperm(6, generator=gen)[:k] for _ in range(m)]).numpy()
+        ids[2, 1] = 512  # an unfilled slot
+        weights = torch.softmax(torch.randn(m, k, generator=gen), -1)
+        out = torch.zeros(m, 128)
+        for r in range(m):
+            for s in range(k):
+                e = int(ids[r, s])
+                if e >= 6:
+                    continue
+                h1 = (x[r:r + 1].float() @ w13[e].T).to(torch.bfloat16).float()
+                h = (F.silu(h1[:, inter:]) * h1[:, :inter] if gated else torch.relu(h1).square()).to(torch.bfloat16)
+                out[r] += float(weights[r, s]) * (h.float() @ w2[e].T)[0]
+        got = L.moe_layer_ref(x, ids, weights, get, gated, e_n=6)
+        assert torch.allclose(got.float(), out.bfloat16().float(), rtol=2 ** -6, atol=1e-5)
+
+
+def test_zero_weights_dropped_rows_and_slot_permutation():
+    get, _, _ = _experts(4, 32, 128, True, 7)
+    gen = torch.Generator().manual_seed(8)
+    x = torch.randn(3, 128, generator=gen).bfloat16()
+    ids = np.array([[0, 1], [2, 3], [512, 512]])
+    assert not L.moe_layer_ref(x, ids, torch.zeros(3, 2), get, True, e_n=4).any()
+    w = torch.full((3, 2), 0.5)
+    a = L.moe_layer_ref(x, ids, w, get, True, e_n=4)
+    b = L.moe_layer_ref(x, ids[:, ::-1].copy(), w, get, True, e_n=4)
+    assert not a[2].any() and torch.allclose(a.float(), b.float(), rtol=2 ** -7, atol=1e-6)
+    # expert-parallel halves add up to the whole (tests/gpu/test_w3_moe.py:84-105 of the reference)
+    lo = L.moe_layer_ref(x, ids, w, get, True, e_lo=0, e_n=2)
+    hi = L.moe_layer_ref(x, ids, w, lambda e: get(e + 2), True, e_lo=2, e_n=2)
+    assert torch.allclose(lo.float() + hi.float(), a.float(), rtol=2 ** -6, atol=1e-5)
+
+
+def test_shared_expert_and_gate():
+    get, w13, w2 = _experts(4, 32, 128, True, 9)
+    gen = torch.Generator().manual_seed(10)
+    x = torch.randn(5, 128, generator=gen).bfloat16()
+    ids = np.stack([np.array([0, 1]) for _ in range(5)])
+    w = torch.full((5, 2), 0.5)
+    routed = L.moe_layer_ref(x, ids, w, get, True, e_n=4)
+    shared = L.moe_layer_ref(x, np.full((5, 1), 3), torch.ones(5, 1), get, True, e_n=4)
+    both = L.moe_layer_ref(x, ids, w, get, True, shared=get(3), e_n=4)
+    assert torch.equal(both, (routed.float() + shared.float()).bfloat16())
+    gate = torch.randn(128, generator=gen) * 0.1
+    gated = L.moe_layer_ref(x, ids, w, get, True, shared=get(3), gate_vec=gate, e_n=4)
+    g = torch.sigmoid(x.float() @ gate)[:, None]
+    assert torch.allclose(gated.float(), (routed.float() + g * shared.float()).bfloat16().float(), rtol=2 ** -7, atol=1e-6)
+
+
+def test_routing_against_torch():
+    gen = torch.Generator().manual_seed(11)
+    logits = torch.randn(9, 64, generator=gen)
+    ids, w = L.route_softmax_topk(logits, 5)
+    sel = logits.gather(1, ids.long())
+    assert torch.allclose(w, torch.softmax(sel, -1), atol=1e-6)  # renormalized softmax == softmax over the selection
+    assert (sel[:, :-1] >= sel[:, 1:]).all()
+    bias = torch.randn(64, generator=gen) * 0.1
+    ids2, w2 = L.route_sigmoid_topk(logits, bias, 6, 2.5)
+    want = torch.topk(torch.sigmoid(logits) + bias, 6).indices
+    assert torch.equal(ids2.long().sort(-1).values, want.sort(-1).values)
+    assert torch.allclose(w2.sum(-1), torch.full((9,), 2.5), atol=1e-5)
+    tie = torch.zeros(1, 8)
+    assert L.route_sigmoid_topk(tie, torch.zeros(8), 3)[0].tolist() == [[0, 1, 2]]
+
+
+def test_latent_moe_single_expert_special_case():
+    gen = torch.Generator().manual_seed(12)
+    x = torch.randn(4, 64, generator=gen).bfloat16()
+    fc1 = (torch.randn(32, 64, generator=gen) * 0.1).bfloat16()
+    fc2 = (torch.randn(64, 32, generator=gen) * 0.1).bfloat16()
+    up = torch.randint(-6, 7, (48, 32), generator=gen).float() * 0.5
+    down = torch.randint(-6, 7, (32, 48), generator=gen).float() * 0.5
+    got = L.latent_moe_ref(x, fc1, fc2, np.zeros((4, 1), np.int64), torch.full((4, 1), 0.75), lambda e: (up.numpy(), 0.01, down.numpy(), 0.02))
+    lat = (x.float() @ fc1.float().T).bfloat16()
+    h = torch.relu(((lat.float() @ up.T) * 0.01).bfloat16().float()).square().bfloat16()
+    acc = (h.float() @ down.T) * 0.02 * 0.75
+    want = (acc.bfloat16().float() @ fc2.float().T).bfloat16()
+    assert torch.allclose(got.float(), want.float(), rtol=2 ** -6, atol=1e-6)
+
+
+def test_silu_and_mul_layouts():
+    gen = torch.Generator().manual_seed(13)
+    gu = torch.randn(3, 256, generator=gen)
+    plain = L.silu_and_mul(gu)
+    assert torch.allclose(plain, torch.nn.functional.silu(gu[:, :128]) * gu[:, 128:])
+    order = torch.arange(256).view(2, 2, 64).transpose(0, 1).reshape(-1)  # pair_order(256, 64)
+    assert torch.allclose(L.silu_and_mul(gu[:, order], pairs=64), plain)
