@@ -1,0 +1,81 @@
+"""ctypes binding of libhibana_hip.so (the C ABI declared in include/hibana_hip.h)."""
+from __future__ import annotations
+
+import ctypes as C
+from functools import lru_cache
+from pathlib import Path
+
+import torch
+
+LIBRARY = Path(__file__).resolve().parent / "libhibana_hip.so"
+
+HB_OK, HB_EINVAL, HB_ENULL, HB_EWORKSPACE, HB_ELAUNCH = 0, -1, -2, -3, -4
+
+
+class HbW3Experts(C.Structure):
+    _fields_ = [("fc1", C.c_void_p), ("fc1_rows", C.c_void_p), ("fc2", C.c_void_p), ("fc2_rows", C.c_void_p),
+                ("fc1_lut", C.c_int64), ("fc2_lut", C.c_int64), ("experts", C.c_int), ("base", C.c_int),
+                ("hidden", C.c_int), ("inter", C.c_int), ("hidden_out", C.c_int), ("gated", C.c_int)]
+
+
+_P, _I, _L, _Z, _F = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
+_EX = C.POINTER(HbW3Experts)
+# name -> (restype, argtypes): every symbol include/hibana_hip.h declares
+SIGNATURES = {
+    "hb_version": (_I, []),
+    "hb_error_string": (C.c_char_p, [_I]),
+    "hb_tune": (_I, [C.c_char_p, _I]),
+    "hb_w3_tiled_bytes": (_Z, [_L, _I]),
+    "hb_w3_repack": (_I, [_P, _P, _L, _I, _I, _P, _P]),
+    "hb_w3_pack_codes": (_I, [_P, _P, _L, _I, _I, _P, _P, _P]),
+    "hb_w3_unpack": (_I, [_P, _L, _I, _P, _P, _P]),
+    "hb_w3_unpack_planes": (_I, [_P, _P, _L, _I, _I, _P, _P, _P]),
+    "hb_w3_dequant": (_I, [_P, _P, _L, _L, _I, _P, _P]),
+    "hb_w3_gemm": (_I, [_P, _I, _P, _P, _L, _I, _I, _P, _P]),
+    "hb_w3_moe_workspace_bytes": (_Z, [_I, _I, _EX, _I]),
+    "hb_w3_moe": (_I, [_EX, _P, _P, _P, _I, _I, _I, _P, _P, _Z, _P]),
+    "hb_w3_moe_layer": (_I, [_EX, _EX, _P, _P, _P, _P, _I, _I, _P, _P, _Z, _P]),
+    "hb_moe_combine_pairs": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P]),
+    "hb_route_softmax_topk": (_I, [_P, _I, _I, _I, _P, _P, _P]),
+    "hb_nvfp4_tiled_bytes": (_Z, [_L, _I]),
+    "hb_nvfp4_repack": (_I, [_P, _P, _I, _L, _I, _P, _P]),
+    "hb_nvfp4_dequant": (_I, [_P, _F, _L, _I, _P, _P]),
+    "hb_nvfp4_gemm": (_I, [_P, _I, _P, _F, _I, _I, _I, _P, _P]),
+}
+
+
+@lru_cache(maxsize=1)
+def lib() -> C.CDLL:
+    """The loaded library; raises if it has not been built (python -m hibana_amd.build)."""
+    if not LIBRARY.exists():
+        raise RuntimeError(f"{LIBRARY} is missing: build it with `python -m hibana_amd.build` (hipcc, gfx950); there is no fallback path")
+    handle = C.CDLL(str(LIBRARY))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(handle, name)
+        fn.restype, fn.argtypes = restype, argtypes
+    return handle
+
+
+def check(code: int, what: str) -> None:
+    """Map a status code to the reference's error behaviour: ValueError for calls the kernels do not take,
+    RuntimeError for the rest."""
+    if code == HB_OK:
+        return
+    text = lib().hb_error_string(code).decode()
+    if code == HB_EINVAL:
+        raise ValueError(f"{what}: {text}")
+    raise RuntimeError(f"{what}: {text}")
+
+
+def ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def need_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("hibana_amd kernels run on the GPU only: got a CPU tensor (there is no CPU fallback)")

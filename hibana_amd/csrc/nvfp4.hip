@@ -1,0 +1,309 @@
+// NVFP4 (E2M1 codes, E4M3 scale per 16 weights, FP32 global scale) weight-only kernels for gfx950.
+//
+// Tile layout: blocks of 64 output rows x 128 k, NVFP4_BLOCK_BYTES each, [rows/64][K/128]:
+//   bytes    0..4095  codes: four 128-bit loads per lane, load nt of lane l at (nt * 64 + l) * 16. Lane l = 16 q + r owns,
+//                     for the 16-row tile nt, the weights  row 64 nb + 16 nt + r,  k = 128 c + 16 b + 4 q + i
+//                     (b = 0..7 the 16-blocks of the chunk, i = 0..3): dword b / 2 of the load, its low half for even b,
+//                     high half for odd b, nibble i. That is the B operand of v_mfma_f32_16x16x16_bf16, one MFMA per
+//                     16-block, so the block scale multiplies the MFMA's FP32 result.
+//   bytes 4096..4607  scales: 32 B per row-in-tile r at 4096 + 32 r: byte 8 nt + b is the E4M3 scale of row
+//                     64 nb + 16 nt + r, block 8 c + b.
+// Codes expand with v_cvt_scalef32_pk_bf16_fp4 (two weights per instruction, exact).
+#include "common.hpp"
+
+namespace hb {
+
+constexpr int NVFP4_BLOCK_BYTES = 4608;
+constexpr int NVFP4_SCALE_OFFSET = 4096;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+
+__host__ __device__ inline int64_t swizzled_scale_offset(int64_t r, int c, int groups_pad) {
+  return (r / 128) * 128 * groups_pad + (c / 4) * 512 + (r % 32) * 16 + ((r / 32) % 4) * 4 + c % 4;
+}
+
+// One thread per (block, tile, lane): the lane's four code dwords of one 16-row tile.
+__global__ __launch_bounds__(256) void nvfp4_repack_codes_kernel(const uint8_t* __restrict__ weight, int64_t blocks, int chunks,
+                                                                 uint8_t* __restrict__ tiled) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= blocks * 256) return;
+  const int64_t blk = id >> 8;
+  const int nt = (int)(id >> 6) & 3, lane = (int)(id & 63), q = lane >> 4, r = lane & 15;
+  const int64_t nb = blk / chunks;
+  const int c = (int)(blk % chunks);
+  const int64_t n = nb * 64 + nt * 16 + r;
+  const uint8_t* src = weight + n * (chunks * 64) + c * 64;  // 64 bytes per chunk per row
+  uint32_t d[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    // blocks 2e and 2e+1: bytes at k/2 = 8 b + 2 q, two bytes each (four nibbles)
+    const uint32_t lo = src[16 * e + 2 * q] | ((uint32_t)src[16 * e + 2 * q + 1] << 8);
+    const uint32_t hi = src[16 * e + 8 + 2 * q] | ((uint32_t)src[16 * e + 8 + 2 * q + 1] << 8);
+    d[e] = lo | (hi << 16);
+  }
+  *reinterpret_cast<u32x4_t*>(tiled + blk * NVFP4_BLOCK_BYTES + (nt * 64 + lane) * 16) = u32x4_t{d[0], d[1], d[2], d[3]};
+}
+
+// One thread per scale byte.
+__global__ __launch_bounds__(256) void nvfp4_repack_scales_kernel(const uint8_t* __restrict__ scales, int swizzled, int64_t blocks,
+                                                                  int chunks, uint8_t* __restrict__ tiled) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= blocks * 512) return;
+  const int64_t blk = id >> 9;
+  const int within = (int)(id & 511), r = within >> 5, nt = (within >> 3) & 3, b = within & 7;
+  const int64_t nb = blk / chunks;
+  const int c = (int)(blk % chunks);
+  const int64_t n = nb * 64 + nt * 16 + r;
+  const int groups = chunks * 8, g = 8 * c + b;
+  const uint8_t v = swizzled ? scales[swizzled_scale_offset(n, g, (groups + 3) / 4 * 4)] : scales[n * groups + g];
+  tiled[blk * NVFP4_BLOCK_BYTES + NVFP4_SCALE_OFFSET + 32 * r + 8 * nt + b] = v;
+}
+
+__device__ __forceinline__ float e2m1_to_f32(uint32_t code) {
+  const uint32_t a = code & 7u;
+  const float mag = a < 4u ? 0.5f * (float)a : a == 4u ? 2.0f : a == 5u ? 3.0f : a == 6u ? 4.0f : 6.0f;
+  return (code & 8u) ? -mag : mag;
+}
+
+// One thread per (block, tile, lane): 32 dequantized weights, e2m1 * float(scale) then * global (two roundings).
+__global__ __launch_bounds__(256) void nvfp4_dequant_kernel(const uint8_t* __restrict__ tiled, float global_scale, int64_t blocks, int chunks,
+                                                            float* __restrict__ out) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= blocks * 256) return;
+  const int64_t blk = id >> 8;
+  const int nt = (int)(id >> 6) & 3, lane = (int)(id & 63), q = lane >> 4, r = lane & 15;
+  const int64_t nb = blk / chunks;
+  const int c = (int)(blk % chunks);
+  const int k = chunks * 128;
+  const uint8_t* base = tiled + blk * NVFP4_BLOCK_BYTES;
+  const int64_t n = nb * 64 + nt * 16 + r;
+  const u32x4_t d = *reinterpret_cast<const u32x4_t*>(base + (nt * 64 + lane) * 16);
+  const uint32_t dw[4] = {d.x, d.y, d.z, d.w};
+  for (int b = 0; b < 8; b++) {
+    const float s = e4m3_to_f32(base[NVFP4_SCALE_OFFSET + 32 * r + 8 * nt + b]);
+    const uint32_t half = (dw[b >> 1] >> (16 * (b & 1))) & 0xffffu;
+    float* o = out + n * k + c * 128 + 16 * b + 4 * q;
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = __fmul_rn(__fmul_rn(e2m1_to_f32((half >> (4 * i)) & 15u), s), global_scale);
+  }
+}
+
+struct Nvfp4Params {
+  const uint8_t* w;
+  int n_blocks, chunks;
+  const uint16_t* a;
+  int64_t a_stride;
+  int m;
+  uint16_t* out;
+  int64_t out_stride;
+  float global_scale;
+  int relu2;
+  int ks, nbw;
+};
+
+struct Fp4Chunk {  // the weight side of a chunk: prefetched one chunk ahead
+  u32x4_t w0, w1, w2, w3, s0, s1;
+};
+
+struct Fp4Rows {  // the activation side: read from L2 when the chunk is computed
+  u32x2_t a0, a1, a2, a3, a4, a5, a6, a7;
+};
+
+__device__ __forceinline__ void load_fp4_chunk(Fp4Chunk& ch, const uint8_t* blk, int lane, int r16) {
+  const u32x4_t* b = reinterpret_cast<const u32x4_t*>(blk);
+  ch.w0 = __builtin_nontemporal_load(b + lane);
+  ch.w1 = __builtin_nontemporal_load(b + 64 + lane);
+  ch.w2 = __builtin_nontemporal_load(b + 128 + lane);
+  ch.w3 = __builtin_nontemporal_load(b + 192 + lane);
+  ch.s0 = __builtin_nontemporal_load(b + 256 + 2 * r16);
+  ch.s1 = __builtin_nontemporal_load(b + 257 + 2 * r16);
+}
+
+__device__ __forceinline__ void load_fp4_rows(Fp4Rows& ch, const uint16_t* arow) {
+  ch.a0 = *reinterpret_cast<const u32x2_t*>(arow);
+  ch.a1 = *reinterpret_cast<const u32x2_t*>(arow + 16);
+  ch.a2 = *reinterpret_cast<const u32x2_t*>(arow + 32);
+  ch.a3 = *reinterpret_cast<const u32x2_t*>(arow + 48);
+  ch.a4 = *reinterpret_cast<const u32x2_t*>(arow + 64);
+  ch.a5 = *reinterpret_cast<const u32x2_t*>(arow + 80);
+  ch.a6 = *reinterpret_cast<const u32x2_t*>(arow + 96);
+  ch.a7 = *reinterpret_cast<const u32x2_t*>(arow + 112);
+}
+
+// One 16-block: two conversions, one MFMA, the block scale folded into the accumulator.
+#define HB_FP4_BLOCK(codes, BYTE0, a_frag, scale_dword, SBYTE, acc)                                                                   \
+  {                                                                                                                                   \
+    u32x2_t packed;                                                                                                                   \
+    packed.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, 1.0f, BYTE0));                           \
+    packed.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, 1.0f, BYTE0 + 1));                       \
+    const f32x4_t part = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf16x4_t_s, a_frag), __builtin_bit_cast(bf16x4_t_s, packed), \
+                                                                   f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);                           \
+    const float s = __builtin_amdgcn_cvt_f32_fp8(scale_dword, SBYTE);                                                                 \
+    acc.x = fmaf(part.x, s, acc.x);                                                                                                   \
+    acc.y = fmaf(part.y, s, acc.y);                                                                                                   \
+    acc.z = fmaf(part.z, s, acc.z);                                                                                                   \
+    acc.w = fmaf(part.w, s, acc.w);                                                                                                   \
+  }
+
+typedef __attribute__((ext_vector_type(4))) short bf16x4_t_s;  // the 16x16x16 builtin takes its BF16 operands as 4 x i16
+
+__device__ __forceinline__ void fp4_tile(const u32x4_t& w, uint32_t sc_lo, uint32_t sc_hi, const Fp4Rows& ch, f32x4_t& acc) {
+  HB_FP4_BLOCK(w.x, 0, ch.a0, sc_lo, 0, acc)
+  HB_FP4_BLOCK(w.x, 2, ch.a1, sc_lo, 1, acc)
+  HB_FP4_BLOCK(w.y, 0, ch.a2, sc_lo, 2, acc)
+  HB_FP4_BLOCK(w.y, 2, ch.a3, sc_lo, 3, acc)
+  HB_FP4_BLOCK(w.z, 0, ch.a4, sc_hi, 0, acc)
+  HB_FP4_BLOCK(w.z, 2, ch.a5, sc_hi, 1, acc)
+  HB_FP4_BLOCK(w.w, 0, ch.a6, sc_hi, 2, acc)
+  HB_FP4_BLOCK(w.w, 2, ch.a7, sc_hi, 3, acc)
+}
+
+__device__ __forceinline__ void fp4_chunk(const Fp4Chunk& ch, const uint16_t* arow, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
+                                          f32x4_t& acc3) {
+  Fp4Rows rows;
+  load_fp4_rows(rows, arow);
+  fp4_tile(ch.w0, ch.s0.x, ch.s0.y, rows, acc0);
+  fp4_tile(ch.w1, ch.s0.z, ch.s0.w, rows, acc1);
+  fp4_tile(ch.w2, ch.s1.x, ch.s1.y, rows, acc2);
+  fp4_tile(ch.w3, ch.s1.z, ch.s1.w, rows, acc3);
+}
+
+__device__ __forceinline__ void nvfp4_emit(const Nvfp4Params& p, int nb, int p0, int rows, int t, int r, int q, int r16, float v) {
+  const int i = 4 * q + r;
+  if (i >= rows) return;
+  float y = round_bf16(v * p.global_scale);
+  if (p.relu2) {
+    y = fmaxf(y, 0.f);
+    y = y * y;
+  }
+  p.out[(int64_t)(p0 + i) * p.out_stride + nb * 64 + 16 * t + r16] = f32_to_bf16_bits(y);
+}
+
+// Dense y = x Wq^T: one wavefront per (64-row block, K range, slot of 16 activation rows), as the W3 stream.
+__global__ __launch_bounds__(1024) void nvfp4_stream_kernel(Nvfp4Params p) {
+  extern __shared__ float partial[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int ks = wave % p.ks, nbi = wave / p.ks;
+  const int nb = blockIdx.x * p.nbw + nbi;
+  const int p0 = blockIdx.y * 16, rows = min(16, p.m - p0);
+  const bool active = nb < p.n_blocks;
+  f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
+  if (active) {
+    const int c0 = (int)((int64_t)ks * p.chunks / p.ks), c1 = (int)((int64_t)(ks + 1) * p.chunks / p.ks);
+    const int64_t arow = p0 + min(r16, rows - 1);
+    const uint16_t* aptr = p.a + arow * p.a_stride + 4 * q + (int64_t)c0 * 128;
+    const uint8_t* blk = p.w + ((int64_t)nb * p.chunks + c0) * NVFP4_BLOCK_BYTES;
+    if (c0 < c1) {
+      Fp4Chunk even, odd;
+      load_fp4_chunk(even, blk, lane, r16);
+      int left = c1 - c0 - 1;
+      while (left >= 2) {
+        load_fp4_chunk(odd, blk + NVFP4_BLOCK_BYTES, lane, r16);
+        fp4_chunk(even, aptr, acc0, acc1, acc2, acc3);
+        blk += 2 * NVFP4_BLOCK_BYTES;
+        load_fp4_chunk(even, blk, lane, r16);
+        fp4_chunk(odd, aptr + 128, acc0, acc1, acc2, acc3);
+        aptr += 256;
+        left -= 2;
+      }
+      if (left == 1) {
+        load_fp4_chunk(odd, blk + NVFP4_BLOCK_BYTES, lane, r16);
+        fp4_chunk(even, aptr, acc0, acc1, acc2, acc3);
+        fp4_chunk(odd, aptr + 128, acc0, acc1, acc2, acc3);
+      } else {
+        fp4_chunk(even, aptr, acc0, acc1, acc2, acc3);
+      }
+    }
+  }
+  const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
+  if (p.ks == 1) {
+    if (!active) return;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      nvfp4_emit(p, nb, p0, rows, t, 0, q, r16, all[t].x);
+      nvfp4_emit(p, nb, p0, rows, t, 1, q, r16, all[t].y);
+      nvfp4_emit(p, nb, p0, rows, t, 2, q, r16, all[t].z);
+      nvfp4_emit(p, nb, p0, rows, t, 3, q, r16, all[t].w);
+    }
+    return;
+  }
+  float* mine = partial + (int64_t)wave * 1024;
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    mine[(t * 4 + 0) * 64 + lane] = all[t].x;
+    mine[(t * 4 + 1) * 64 + lane] = all[t].y;
+    mine[(t * 4 + 2) * 64 + lane] = all[t].z;
+    mine[(t * 4 + 3) * 64 + lane] = all[t].w;
+  }
+  __syncthreads();
+  if (!active) return;
+  const float* first = partial + (int64_t)nbi * p.ks * 1024;
+  for (int idx = ks; idx < 16; idx += p.ks) {
+    const int t = idx >> 2, r = idx & 3;
+    float v = 0.f;
+    for (int s = 0; s < p.ks; s++) v += first[s * 1024 + (t * 4 + r) * 64 + lane];
+    nvfp4_emit(p, nb, p0, rows, t, r, q, r16, v);
+  }
+}
+
+static inline unsigned grid_for(int64_t threads) { return (unsigned)((threads + 255) / 256); }
+
+}  // namespace hb
+
+using namespace hb;
+
+extern "C" size_t hb_nvfp4_tiled_bytes(int64_t rows, int k) {
+  if (rows <= 0 || k <= 0 || rows % 64 || k % 128) return 0;
+  return (size_t)(rows / 64) * (size_t)(k / 128) * NVFP4_BLOCK_BYTES;
+}
+
+extern "C" int hb_nvfp4_repack(const uint8_t* weight, const uint8_t* scales, int swizzled, int64_t rows, int k, void* tiled, void* stream) {
+  if (!weight || !scales || !tiled) return HB_ENULL;
+  if (rows <= 0 || k <= 0 || rows % 64 || k % 128) return HB_EINVAL;
+  const int chunks = k / 128;
+  const int64_t blocks = rows / 64 * chunks;
+  hipLaunchKernelGGL(nvfp4_repack_codes_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), weight, blocks, chunks,
+                     static_cast<uint8_t*>(tiled));
+  hipLaunchKernelGGL(nvfp4_repack_scales_kernel, dim3(grid_for(blocks * 512)), dim3(256), 0, as_stream(stream), scales, swizzled, blocks, chunks,
+                     static_cast<uint8_t*>(tiled));
+  return launch_status();
+}
+
+extern "C" int hb_nvfp4_dequant(const void* tiled, float global_scale, int64_t rows, int k, float* out, void* stream) {
+  if (!tiled || !out) return HB_ENULL;
+  if (rows <= 0 || k <= 0 || rows % 64 || k % 128) return HB_EINVAL;
+  const int chunks = k / 128;
+  const int64_t blocks = rows / 64 * chunks;
+  hipLaunchKernelGGL(nvfp4_dequant_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), static_cast<const uint8_t*>(tiled),
+                     global_scale, blocks, chunks, out);
+  return launch_status();
+}
+
+extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y, void* stream) {
+  if (!x || !tiled || !y) return HB_ENULL;
+  if (m <= 0 || n <= 0 || k <= 0 || n % 64 || k % 128) return HB_EINVAL;
+  Nvfp4Params p{};
+  p.w = static_cast<const uint8_t*>(tiled);
+  p.n_blocks = n / 64;
+  p.chunks = k / 128;
+  p.a = static_cast<const uint16_t*>(x);
+  p.a_stride = k;
+  p.m = m;
+  p.out = static_cast<uint16_t*>(y);
+  p.out_stride = n;
+  p.global_scale = global_scale;
+  p.relu2 = relu2;
+  const int64_t slots = (m + 15) / 16;
+  if (slots > 65535) return HB_EINVAL;
+  int ks = 1;
+  while (ks < 16 && (int64_t)p.n_blocks * slots * ks < 2048 && p.chunks / (2 * ks) >= 2) ks *= 2;
+  int nbw = ks >= 4 ? 1 : 4 / ks;
+  while (nbw > 1 && p.n_blocks % nbw) nbw /= 2;
+  p.ks = ks;
+  p.nbw = nbw;
+  const dim3 grid((unsigned)((p.n_blocks + nbw - 1) / nbw), (unsigned)slots);
+  const int waves = ks * nbw;
+  hipLaunchKernelGGL(nvfp4_stream_kernel, grid, dim3(64 * waves), ks > 1 ? (size_t)waves * 4096 : 0, as_stream(stream), p);
+  return launch_status();
+}

@@ -1,0 +1,244 @@
+// W3 format kernels: reference layout <-> tile layout, codes <-> planes, bit-exact dequantization.
+// These run at load time or in tests; the streaming GEMMs are in w3_stream.hip.
+#include "common.hpp"
+#include "w3_layout.hpp"
+
+namespace hb {
+
+// One thread per (block, lane): builds the lane's twelve code dwords from the reference planes.
+__global__ __launch_bounds__(256) void w3_repack_codes_kernel(const uint32_t* __restrict__ planes, int64_t blocks, int chunks,
+                                                              int bits, uint8_t* __restrict__ tiled) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= blocks * 64) return;
+  const int64_t blk = id >> 6;
+  const int lane = (int)(id & 63), q = lane >> 4, r = lane & 15;
+  const int64_t nb = blk / chunks;
+  const int c = (int)(blk % chunks);
+  uint32_t d[12];
+#pragma unroll
+  for (int i = 0; i < 12; i++) d[i] = 0;
+  for (int nt = 0; nt < 4; nt++) {
+    const int64_t n = nb * 64 + nt * 16 + r;
+    for (int j = 0; j < 4; j++)
+      for (int i = 0; i < 8; i++) {
+        const int k = c * 128 + j * 32 + q * 8 + i;
+        for (int b = 0; b < bits; b++) {
+          int64_t word;
+          int pos, dw, dpos;
+          w3_ref_bit_slot(n, k, b, bits, chunks, &word, &pos);
+          const uint32_t bit = (planes[word] >> pos) & 1u;
+          w3_bit_slot(nt, j, i, b, &dw, &dpos);
+          d[dw] |= bit << dpos;
+        }
+      }
+  }
+  uint8_t* base = tiled + blk * W3_BLOCK_BYTES;
+#pragma unroll
+  for (int i = 0; i < 12; i++) *reinterpret_cast<uint32_t*>(base + w3_dword_offset(lane, i)) = d[i];
+}
+
+// One thread per scale byte of the tile layout.
+__global__ __launch_bounds__(256) void w3_repack_scales_kernel(const uint8_t* __restrict__ scales, int64_t blocks, int chunks,
+                                                               uint8_t* __restrict__ tiled) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= blocks * 256) return;
+  const int64_t blk = id >> 8;
+  const int within = (int)(id & 255), r = within >> 4, nt = (within >> 2) & 3, j = within & 3;
+  const int64_t nb = blk / chunks;
+  const int c = (int)(blk % chunks);
+  const int64_t n = nb * 64 + nt * 16 + r;
+  tiled[blk * W3_BLOCK_BYTES + w3_scale_offset(nt, r, j)] = scales[w3_ref_scale_slot(n, 4 * c + j, chunks)];
+}
+
+// One thread per plane word of the reference layout.
+__global__ __launch_bounds__(256) void w3_pack_planes_kernel(const uint8_t* __restrict__ codes, int64_t rows, int k, int bits,
+                                                             uint32_t* __restrict__ planes) {
+  const int chunks = k >> 7;
+  const int64_t total = (rows >> 5) * chunks * bits * 128;
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= total) return;
+  const int e = (int)(id & 3), lane = (int)((id >> 2) & 31);
+  int64_t rest = id >> 7;
+  const int i = (int)(rest % bits);
+  rest /= bits;
+  const int kc = (int)(rest % chunks);
+  const int64_t nb = rest / chunks;
+  const int w = 4 * i + e, nt = w / bits, b = w % bits, g = lane >> 2, t = lane & 3;
+  const int64_t n = nb * 32 + nt * 8 + g;
+  uint32_t word = 0;
+  for (int s = 0; s < 8; s++)
+    for (int j = 0; j < 4; j++) {
+      const int kk = kc * 128 + s * 16 + t * 4 + j;
+      const uint32_t bit = (codes[n * k + kk] >> b) & 1u;
+      word |= bit << ((4 * j + b + 16 * (s >> 2) + (s & 3)) & 31);
+    }
+  planes[id] = word;
+}
+
+__global__ __launch_bounds__(256) void w3_pack_scales_kernel(const uint8_t* __restrict__ scale_bytes, int64_t rows, int k,
+                                                             uint8_t* __restrict__ scales) {
+  const int groups = k >> 5, chunks = k >> 7;
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= rows * groups) return;
+  const int64_t n = id / groups;
+  const int grp = (int)(id % groups);
+  scales[w3_ref_scale_slot(n, grp, chunks)] = scale_bytes[id];
+}
+
+// One thread per (block, tile, lane): the lane's 32 codes of one 16-row tile.
+__global__ __launch_bounds__(256) void w3_unpack_kernel(const uint8_t* __restrict__ tiled, int64_t blocks, int chunks,
+                                                        uint8_t* __restrict__ codes, uint8_t* __restrict__ scale_bytes) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= blocks * 256) return;
+  const int64_t blk = id >> 8;
+  const int nt = (int)(id >> 6) & 3, lane = (int)(id & 63), q = lane >> 4, r = lane & 15;
+  const int64_t nb = blk / chunks;
+  const int c = (int)(blk % chunks);
+  const int k = chunks * 128;
+  const uint8_t* base = tiled + blk * W3_BLOCK_BYTES;
+  const int64_t n = nb * 64 + nt * 16 + r;
+  if (codes) {
+    const uint32_t q0 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt));
+    const uint32_t q1 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 1));
+    const uint32_t q2 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 2));
+    uint32_t sel[8];
+    w3_selectors(q0, q1, q2, sel);
+    for (int j = 0; j < 4; j++) {
+      uint8_t* out = codes + n * k + c * 128 + j * 32 + q * 8;
+      *reinterpret_cast<uint32_t*>(out) = sel[2 * j];
+      *reinterpret_cast<uint32_t*>(out + 4) = sel[2 * j + 1];
+    }
+  }
+  if (scale_bytes && q == 0) {
+    for (int j = 0; j < 4; j++) scale_bytes[n * (k >> 5) + 4 * c + j] = base[w3_scale_offset(nt, r, j)];
+  }
+}
+
+// One thread per (row, 128-chunk) of the reference layout.
+__global__ __launch_bounds__(256) void w3_unpack_planes_kernel(const uint32_t* __restrict__ planes, const uint8_t* __restrict__ scales,
+                                                               int64_t rows, int k, int bits, uint8_t* __restrict__ codes,
+                                                               uint8_t* __restrict__ scale_bytes) {
+  const int chunks = k >> 7;
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= rows * chunks) return;
+  const int64_t n = id / chunks;
+  const int kc = (int)(id % chunks);
+  if (codes) {
+    for (int kk = kc * 128; kk < kc * 128 + 128; kk++) {
+      uint32_t code = 0;
+      for (int b = 0; b < bits; b++) {
+        int64_t word;
+        int pos;
+        w3_ref_bit_slot(n, kk, b, bits, chunks, &word, &pos);
+        code |= ((planes[word] >> pos) & 1u) << b;
+      }
+      codes[n * k + kk] = (uint8_t)code;
+    }
+  }
+  if (scale_bytes)
+    for (int j = 0; j < 4; j++) scale_bytes[n * (k >> 5) + 4 * kc + j] = scales[w3_ref_scale_slot(n, 4 * kc + j, chunks)];
+}
+
+// One thread per (block, tile, lane): 32 dequantized weights. Two FP32 products, each rounded:
+// effective = float(scale byte) * row_scale[row]; weight = level * effective.
+__global__ __launch_bounds__(256) void w3_dequant_kernel(const uint8_t* __restrict__ tiled, const float* __restrict__ row_scale,
+                                                         uint64_t lut, int64_t blocks, int chunks, float* __restrict__ out) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= blocks * 256) return;
+  const int64_t blk = id >> 8;
+  const int nt = (int)(id >> 6) & 3, lane = (int)(id & 63), q = lane >> 4, r = lane & 15;
+  const int64_t nb = blk / chunks;
+  const int c = (int)(blk % chunks);
+  const int k = chunks * 128;
+  const uint8_t* base = tiled + blk * W3_BLOCK_BYTES;
+  const int64_t n = nb * 64 + nt * 16 + r;
+  float level[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) level[i] = e4m3_to_f32((uint32_t)(lut >> (8 * i)) & 0xffu);
+  const uint32_t q0 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt));
+  const uint32_t q1 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 1));
+  const uint32_t q2 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 2));
+  uint32_t sel[8];
+  w3_selectors(q0, q1, q2, sel);
+  const float row = row_scale[n];
+  for (int j = 0; j < 4; j++) {
+    const float eff = __fmul_rn(e4m3_to_f32(base[w3_scale_offset(nt, r, j)]), row);
+    float* o = out + n * k + c * 128 + j * 32 + q * 8;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const uint32_t code = (sel[2 * j + (i >> 2)] >> (8 * (i & 3))) & 7u;
+      float lv = level[0];
+#pragma unroll
+      for (int t = 1; t < 8; t++) lv = code == (uint32_t)t ? level[t] : lv;
+      o[i] = __fmul_rn(lv, eff);
+    }
+  }
+}
+
+static inline unsigned grid_for(int64_t threads) { return (unsigned)((threads + 255) / 256); }
+
+}  // namespace hb
+
+using namespace hb;
+
+extern "C" size_t hb_w3_tiled_bytes(int64_t rows, int k) {
+  if (rows <= 0 || k <= 0 || rows % W3_BLOCK_ROWS || k % W3_CHUNK) return 0;
+  return (size_t)(rows / W3_BLOCK_ROWS) * (size_t)(k / W3_CHUNK) * W3_BLOCK_BYTES;
+}
+
+static int check_shape(int64_t rows, int k, int bits) {
+  if (rows <= 0 || k <= 0 || rows % W3_BLOCK_ROWS || k % W3_CHUNK || (bits != 2 && bits != 3)) return HB_EINVAL;
+  if ((rows / W3_BLOCK_ROWS) * (int64_t)(k / W3_CHUNK) * 256 > (int64_t)0x7fffffff * 256) return HB_EINVAL;
+  return HB_OK;
+}
+
+extern "C" int hb_w3_repack(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, void* tiled, void* stream) {
+  if (!planes || !scales || !tiled) return HB_ENULL;
+  if (int e = check_shape(rows, k, bits)) return e;
+  const int chunks = k / W3_CHUNK;
+  const int64_t blocks = rows / W3_BLOCK_ROWS * chunks;
+  hipLaunchKernelGGL(w3_repack_codes_kernel, dim3(grid_for(blocks * 64)), dim3(256), 0, as_stream(stream), planes, blocks, chunks, bits,
+                     static_cast<uint8_t*>(tiled));
+  hipLaunchKernelGGL(w3_repack_scales_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), scales, blocks, chunks,
+                     static_cast<uint8_t*>(tiled));
+  return launch_status();
+}
+
+extern "C" int hb_w3_pack_codes(const uint8_t* codes, const uint8_t* scale_bytes, int64_t rows, int k, int bits, uint32_t* planes,
+                                uint8_t* scales, void* stream) {
+  if (!codes || !scale_bytes || !planes || !scales) return HB_ENULL;
+  if (int e = check_shape(rows, k, bits)) return e;
+  const int64_t words = rows / 32 * (k / 128) * bits * 128;
+  hipLaunchKernelGGL(w3_pack_planes_kernel, dim3(grid_for(words)), dim3(256), 0, as_stream(stream), codes, rows, k, bits, planes);
+  hipLaunchKernelGGL(w3_pack_scales_kernel, dim3(grid_for(rows * (k / 32))), dim3(256), 0, as_stream(stream), scale_bytes, rows, k, scales);
+  return launch_status();
+}
+
+extern "C" int hb_w3_unpack(const void* tiled, int64_t rows, int k, uint8_t* codes, uint8_t* scale_bytes, void* stream) {
+  if (!tiled) return HB_ENULL;
+  if (int e = check_shape(rows, k, 3)) return e;
+  const int chunks = k / W3_CHUNK;
+  const int64_t blocks = rows / W3_BLOCK_ROWS * chunks;
+  hipLaunchKernelGGL(w3_unpack_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), static_cast<const uint8_t*>(tiled),
+                     blocks, chunks, codes, scale_bytes);
+  return launch_status();
+}
+
+extern "C" int hb_w3_unpack_planes(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, uint8_t* codes,
+                                   uint8_t* scale_bytes, void* stream) {
+  if (!planes || !scales) return HB_ENULL;
+  if (int e = check_shape(rows, k, bits)) return e;
+  hipLaunchKernelGGL(w3_unpack_planes_kernel, dim3(grid_for(rows * (k / 128))), dim3(256), 0, as_stream(stream), planes, scales, rows, k,
+                     bits, codes, scale_bytes);
+  return launch_status();
+}
+
+extern "C" int hb_w3_dequant(const void* tiled, const float* row_scale, int64_t lut, int64_t rows, int k, float* out, void* stream) {
+  if (!tiled || !row_scale || !out) return HB_ENULL;
+  if (int e = check_shape(rows, k, 3)) return e;
+  const int chunks = k / W3_CHUNK;
+  const int64_t blocks = rows / W3_BLOCK_ROWS * chunks;
+  hipLaunchKernelGGL(w3_dequant_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), static_cast<const uint8_t*>(tiled),
+                     row_scale, (uint64_t)lut, blocks, chunks, out);
+  return launch_status();
+}

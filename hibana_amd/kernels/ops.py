@@ -1,0 +1,78 @@
+"""Kernel entry points of the quantized linear / MoE path (hibana/kernels/ops.py:50-92 of the reference, plus the
+routing and combine ops of hibana/kernels/flashnext_fused.py that sit either side of the experts)."""
+from __future__ import annotations
+
+import torch
+
+from hibana_amd import _lib
+from hibana_amd.kernels import w3
+
+
+def w3_decode(lin, m: int, rows: int | None = None) -> bool:
+    """True when this call runs the 3-bit decode copy instead of the NVFP4 weights: at most `rows` rows (None:
+    w3.MAX_ROWS) (hibana/kernels/ops.py:50-53)."""
+    return lin.w3 is not None and m <= (rows or w3.MAX_ROWS) and w3.enabled()
+
+
+def nvfp4_linear(x: torch.Tensor, lin, prequantized=None, relu2: bool = False) -> torch.Tensor:
+    """BF16 x [M, K] -> BF16 [M, N] on NVFP4 weights, weight-only: bf16((x Wq^T)_fp32 * global scale); the 3-bit copy
+    serves the call when one is attached and enabled (hibana/kernels/ops.py:56-83)."""
+    if prequantized is not None:
+        raise ValueError("nvfp4_linear: NVFP4 activations are not taken by the weight-only kernels")
+    if x.dtype == torch.bfloat16 and w3_decode(lin, x.shape[0]) and not relu2:
+        return w3.w3_linear(x, lin.w3)
+    if x.dtype != torch.bfloat16 or x.ndim != 2 or x.shape[1] != lin.in_features:
+        raise ValueError("nvfp4_linear: x must be BF16 [M, in_features]")
+    _lib.need_gpu(x)
+    lin.tile()
+    m = x.shape[0]
+    y = torch.empty((m, lin.out_features), dtype=torch.bfloat16, device=x.device)
+    if m:
+        _lib.check(_lib.lib().hb_nvfp4_gemm(_lib.ptr(x.contiguous()), m, _lib.ptr(lin.tiled), lin.global_scale, lin.out_features,
+                                            lin.in_features, int(relu2), _lib.ptr(y), _lib.stream()), "nvfp4_linear")
+    return y
+
+
+def silu_and_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:
+    """silu(gate) * up of [..., gate | up], or (`pairs`) of gate and up alternating in blocks of `pairs` columns
+    (hibana/kernels/ops.py:86-92)."""
+    half = gate_up.shape[-1] // 2
+    if pairs:
+        blocks = gate_up.unflatten(-1, (half // pairs, 2, pairs))
+        return (torch.nn.functional.silu(blocks[..., 0, :]) * blocks[..., 1, :]).flatten(-2)
+    return torch.nn.functional.silu(gate_up[..., :half]) * gate_up[..., half:]
+
+
+def route_topk(logits: torch.Tensor, k: int):
+    """[M, E] FP32 logits -> (int32 ids [M, k], FP32 renormalized softmax weights [M, k]), largest first
+    (hibana/kernels/flashnext_fused.py:308-319, without the padded-slot table)."""
+    _lib.need_gpu(logits)
+    m, e = logits.shape
+    logits = logits.float().contiguous()
+    ids = torch.empty((m, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((m, k), dtype=torch.float32, device=logits.device)
+    if m:
+        _lib.check(_lib.lib().hb_route_softmax_topk(_lib.ptr(logits), m, e, k, _lib.ptr(ids), _lib.ptr(w), _lib.stream()), "route_topk")
+    return ids, w
+
+
+def moe_combine_pairs(y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None, x: torch.Tensor | None,
+                      gate_w: torch.Tensor | None, e_lo: int = 0, e_n: int = 512) -> torch.Tensor:
+    """bf16(bf16(sum_k w_k y_k over this rank's pairs, in slot order) + sigmoid(x . gate_w) * shared) from the unsummed
+    pair outputs y [m * topk, H] (FP32 or BF16) (hibana/kernels/flashnext_fused.py:556-571). `shared` None: the
+    routed sum alone; `gate_w` None: the shared output is added ungated."""
+    _lib.need_gpu(y, ids, weights)
+    m, topk = ids.shape
+    h = y.shape[1]
+    out = torch.empty((m, h), dtype=torch.bfloat16, device=y.device)
+    if m == 0:
+        return out
+    if y.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("moe_combine_pairs: pairs must be FP32 or BF16")
+    sh = None if shared is None else shared.to(torch.bfloat16).contiguous()
+    xx = None if x is None else x.to(torch.bfloat16).contiguous()
+    gw = None if gate_w is None else gate_w.float().contiguous()
+    _lib.check(_lib.lib().hb_moe_combine_pairs(_lib.ptr(y.contiguous()), int(y.dtype == torch.bfloat16), _lib.ptr(ids.to(torch.int32).contiguous()),
+                                               _lib.ptr(weights.float().contiguous()), _lib.ptr(sh), _lib.ptr(xx), _lib.ptr(gw), e_lo, e_n, m, topk, h,
+                                               _lib.ptr(out), _lib.stream()), "moe_combine_pairs")
+    return out

@@ -1,0 +1,286 @@
+"""Three-bit decode weights on MI355X: the reference's W3 format and op surface (hibana/kernels/w3.py), served by
+hand-written gfx950 kernels through the C ABI.
+
+Format (unchanged, it is what checkpoints hold; hibana/kernels/w3.py:75-91 of the reference): per weight a 3-bit
+code into an eight-level E4M3 codebook (2-bit with a four-level one), per 32 weights along K an E4M3 scale, per output
+row an FP32 multiplier; `planes` / `scales` in the reference's fragment order. At load time `tile()` repacks them into
+the 64-row x 128-k block layout the kernels stream (csrc/w3_layout.hpp); the fragment-order tensors can then be
+dropped (`release=True`).
+
+Arithmetic: weight-only. Activations stay BF16 (the reference re-quantizes them to E4M3 per 32-group,
+hibana/kernels/w3.py:25-28); weights are expanded exactly to BF16 in registers, products accumulate in FP32, the group
+scale multiplies each 32-group's FP32 partial sum, the row scale the total.
+
+Every function here that touches packed data runs on the GPU and raises on CPU tensors: there is no fallback path.
+"""
+from __future__ import annotations
+
+import os
+import struct
+from dataclasses import dataclass, replace
+
+import torch
+
+from hibana_amd import _lib
+
+MAX_ROWS = 128
+NARROW_ROWS = 64
+GROUP = 32
+CHUNK = 128
+FP8_MAX = 448.0
+CODEBOOKS = {
+    "uniform": (-3.5, -2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 3.5),
+    "lloyd": (-3.5, -2.25, -1.25, -0.40625, 0.40625, 1.25, 2.25, 3.5),
+    "lloyd2": (-1.5, -0.4375, 0.4375, 1.5),
+    "zero8": (-3.5, -2.5, -1.5, -0.625, 0.0, 0.875, 2.0, 3.5),
+}
+FIT_SCALES = tuple(0.55 + 0.05 * i for i in range(10))
+DEFAULT_CODEBOOK = "lloyd"
+
+_ENABLED: bool | None = None
+
+
+def enabled() -> bool:
+    """HIBANA_W3_DECODE: serve calls of at most MAX_ROWS rows from the 3-bit copies (hibana/kernels/w3.py:48-51)."""
+    if _ENABLED is not None:
+        return _ENABLED
+    return os.environ.get("HIBANA_W3_DECODE", "0").strip().lower() in ("1", "true", "yes", "on")
+
+
+def set_enabled(value: bool | None) -> None:
+    """Override HIBANA_W3_DECODE for this process (None: read the environment again)."""
+    global _ENABLED
+    _ENABLED = value
+
+
+@dataclass
+class W3Weight:
+    planes: torch.Tensor | None  # [N/32, K/128, bits, 32, 4] uint32, the reference's fragment order (None once released)
+    scales: torch.Tensor | None  # [N/32, K/128, 4, 32] uint8 E4M3
+    row_scale: torch.Tensor  # [N] float32
+    out_features: int
+    in_features: int
+    codebook: tuple[float, ...]
+    lut: int  # the codebook as eight E4M3 bytes, entry i in byte i
+    tiled: torch.Tensor | None = None  # uint8, the kernels' block layout (built by tile())
+
+    @property
+    def bytes(self) -> int:
+        n, k = self.out_features, self.in_features
+        return n * k * self.bits // 8 + n * k // GROUP + n * 4
+
+    @property
+    def bits(self) -> int:
+        return 2 if len(self.codebook) == 4 else 3
+
+
+def lut_of(codebook: tuple[float, ...]) -> int:
+    raw = torch.tensor(codebook, dtype=torch.float32).to(torch.float8_e4m3fn).view(torch.uint8).tolist()
+    return struct.unpack("<q", bytes(raw + [0] * (8 - len(raw))))[0]
+
+
+def _codebook(codebook) -> tuple[float, ...]:
+    name = DEFAULT_CODEBOOK if codebook is None else codebook
+    levels = CODEBOOKS[name] if isinstance(name, str) else tuple(float(v) for v in name)
+    if len(levels) not in (4, 8) or any(b < a for a, b in zip(levels, levels[1:])):
+        raise ValueError("a codebook is eight (or, two-bit, four) ascending levels")
+    if torch.tensor(levels).to(torch.float8_e4m3fn).float().tolist() != list(levels):
+        raise ValueError("codebook levels must be exactly representable in E4M3")
+    return levels
+
+
+def tile(w3: W3Weight, release: bool = False) -> W3Weight:
+    """Build the kernels' block layout from the fragment-order tensors (once). `release` drops the latter."""
+    if w3.tiled is None:
+        if w3.planes is None:
+            raise ValueError("W3Weight holds neither planes nor a tiled copy")
+        _lib.need_gpu(w3.planes, w3.scales)
+        n, k = w3.out_features, w3.in_features
+        size = _lib.lib().hb_w3_tiled_bytes(n, k)
+        if size == 0:
+            raise ValueError("W3 kernels need N a multiple of 64 and K a multiple of 128")
+        tiled = torch.empty(size, dtype=torch.uint8, device=w3.planes.device)
+        planes, scales = w3.planes.contiguous(), w3.scales.contiguous()
+        _lib.check(_lib.lib().hb_w3_repack(_lib.ptr(planes), _lib.ptr(scales), n, k, w3.bits, _lib.ptr(tiled), _lib.stream()), "w3 repack")
+        w3.tiled = tiled
+    if release:
+        w3.planes = w3.scales = None
+    return w3
+
+
+def pack_codes(q: torch.Tensor, scale_fp8: torch.Tensor, row_scale: torch.Tensor, codebook=None,
+               rows_per_chunk: int = 4096) -> W3Weight:
+    """Pack calibrated codes and their exact scales without quantizing again (hibana/kernels/w3.py:198-214)."""
+    n, k = q.shape
+    if n % 128 or k % CHUNK or rows_per_chunk < 128 or rows_per_chunk % 128:
+        raise ValueError("N, K and rows_per_chunk must be multiples of 128")
+    levels = _codebook(codebook)
+    if q.dtype not in (torch.uint8, torch.int32, torch.int64) or bool(((q < 0) | (q >= len(levels))).any()):
+        raise ValueError(f"codes must be integers between zero and {len(levels) - 1}")
+    if scale_fp8.shape != (n, k // GROUP) or scale_fp8.dtype != torch.float8_e4m3fn or row_scale.shape != (n,):
+        raise ValueError("calibrated scales do not match the weight shape")
+    sf = scale_fp8.float()
+    if not bool(torch.isfinite(sf).all()) or not bool(torch.isfinite(row_scale).all()) or bool((row_scale <= 0).any()) or bool((sf < 0).any()):
+        raise ValueError("calibrated scales must be finite and nonnegative, with positive row scales")
+    _lib.need_gpu(q, scale_fp8, row_scale)
+    bits = 2 if len(levels) == 4 else 3
+    dev = q.device
+    codes8 = q.to(torch.uint8).contiguous()
+    raw = scale_fp8.contiguous().view(torch.uint8)
+    planes = torch.empty((n // 32, k // CHUNK, bits, 32, 4), dtype=torch.uint32, device=dev)
+    scales = torch.empty((n // 32, k // CHUNK, 4, 32), dtype=torch.uint8, device=dev)
+    _lib.check(_lib.lib().hb_w3_pack_codes(_lib.ptr(codes8), _lib.ptr(raw), n, k, bits, _lib.ptr(planes), _lib.ptr(scales), _lib.stream()),
+               "w3 pack_codes")
+    return W3Weight(planes, scales, row_scale.float().contiguous(), n, k, levels, lut_of(levels))
+
+
+def pack(weight: torch.Tensor, codebook=None, rows_per_chunk: int = 4096, fit_scales: bool = False) -> W3Weight:
+    """Nearest-level quantization of a [N, K] float matrix (N, K multiples of 128), hibana/kernels/w3.py:126-172:
+    group scale = amax / largest level (or, `fit_scales`, the best of FIT_SCALES times that), row scale = largest
+    group scale / 448, group scale stored as E4M3 of the ratio, code = the nearest level of w / effective scale."""
+    n, k = weight.shape
+    if k % CHUNK or n % 128:
+        raise ValueError("N and K must be multiples of 128")
+    levels = _codebook(codebook)
+    lv = torch.tensor(levels, device=weight.device)
+    mids = (lv[1:] + lv[:-1]) / 2
+    # divisors as tensors: torch divides by a Python scalar on the GPU through its reciprocal, which is off by an ulp
+    top = torch.tensor(max(abs(v) for v in levels), device=weight.device)
+    fp8_max = torch.tensor(FP8_MAX, device=weight.device)
+    parts = []
+    for r0 in range(0, n, rows_per_chunk):
+        g = weight[r0:r0 + rows_per_chunk].float().unflatten(1, (k // GROUP, GROUP))
+        scale = g.abs().amax(dim=-1) / top
+        if fit_scales:
+            best_err = best = None
+            for mult in FIT_SCALES:
+                cand = scale * mult
+                deq = lv[torch.bucketize(g / cand.clamp_min(1e-30).unsqueeze(-1), mids)] * cand.unsqueeze(-1)
+                err = (deq - g).square().sum(-1)
+                if best is None:
+                    best_err, best = err, cand
+                else:
+                    take = err < best_err
+                    best_err, best = torch.where(take, err, best_err), torch.where(take, cand, best)
+            scale = best
+        row = (scale.amax(dim=-1) / fp8_max).clamp_min(1e-12)
+        stored = (scale / row.unsqueeze(1)).clamp(0, FP8_MAX).to(torch.float8_e4m3fn)
+        eff = stored.float() * row.unsqueeze(1)
+        q = torch.bucketize((g / eff.clamp_min(1e-30).unsqueeze(-1)).flatten(1), mids)
+        parts.append((q.to(torch.uint8), stored, row))
+    q = torch.cat([p[0] for p in parts])
+    stored = torch.cat([p[1] for p in parts])
+    row = torch.cat([p[2] for p in parts])
+    return pack_codes(q, stored, row, levels)
+
+
+def _unpack(w3: W3Weight, want_codes: bool, want_scales: bool):
+    n, k = w3.out_features, w3.in_features
+    src = w3.tiled if w3.tiled is not None else w3.planes
+    _lib.need_gpu(src)
+    dev = src.device
+    codes8 = torch.empty((n, k), dtype=torch.uint8, device=dev) if want_codes else None
+    raw = torch.empty((n, k // GROUP), dtype=torch.uint8, device=dev) if want_scales else None
+    if w3.tiled is not None:
+        _lib.check(_lib.lib().hb_w3_unpack(_lib.ptr(w3.tiled), n, k, _lib.ptr(codes8), _lib.ptr(raw), _lib.stream()), "w3 unpack")
+    else:
+        _lib.check(_lib.lib().hb_w3_unpack_planes(_lib.ptr(w3.planes.contiguous()), _lib.ptr(w3.scales.contiguous()), n, k, w3.bits,
+                                                  _lib.ptr(codes8), _lib.ptr(raw), _lib.stream()), "w3 unpack")
+    return codes8, raw
+
+
+def codes(w3: W3Weight) -> torch.Tensor:
+    """The codes of a packed matrix, [N, K] int64 (hibana/kernels/w3.py:217-229)."""
+    return _unpack(w3, True, False)[0].long()
+
+
+def scale_bytes(w3: W3Weight) -> torch.Tensor:
+    """The stored E4M3 group scales in matrix order, float8_e4m3fn [N, K/32]."""
+    return _unpack(w3, False, True)[1].view(torch.float8_e4m3fn)
+
+
+def group_scales(w3: W3Weight) -> torch.Tensor:
+    """Effective per-group scales, [N, K/32] float32 (hibana/kernels/w3.py:232-236)."""
+    return scale_bytes(w3).float() * w3.row_scale[:, None]
+
+
+def dequantize(w3: W3Weight) -> torch.Tensor:
+    """FP32 [N, K]: level[code] * (scale * row_scale), the reference's bits (hibana/kernels/w3.py:239-242)."""
+    tile(w3)
+    n, k = w3.out_features, w3.in_features
+    out = torch.empty((n, k), dtype=torch.float32, device=w3.tiled.device)
+    _lib.check(_lib.lib().hb_w3_dequant(_lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut, n, k, _lib.ptr(out), _lib.stream()), "w3 dequantize")
+    return out
+
+
+def pair_order(rows: int, block: int) -> torch.Tensor:
+    """Row order that interleaves [gate; up] in blocks of `block` rows (hibana/weights/modelopt.py:84-86)."""
+    half = torch.arange(rows // 2).unflatten(0, (rows // 2 // block, block))
+    return torch.stack((half, half + rows // 2), dim=1).reshape(-1)
+
+
+def interleave_rows(weight: W3Weight, block: int) -> W3Weight:
+    """`weight`'s rows in pair_order (an MLP's gate|up interleaved in blocks of `block`, a multiple of 32): planes and
+    scales move in whole 32-row tiles (hibana/kernels/w3.py:94-102). The tiled copy, if any, is rebuilt on demand."""
+    if weight.planes is None:
+        raise ValueError("interleave_rows needs the fragment-order tensors (they were released)")
+    tiles = pair_order(weight.out_features // 32, block // 32).to(weight.planes.device)
+    rows = pair_order(weight.out_features, block).to(weight.row_scale.device)
+    planes = weight.planes.view(torch.int32)[tiles].view(torch.uint32)
+    return replace(weight, planes=planes.contiguous(), scales=weight.scales[tiles].contiguous(),
+                   row_scale=weight.row_scale[rows].contiguous(), tiled=None)
+
+
+def quant_groups(x: torch.Tensor):
+    raise NotImplementedError("E4M3 activation quantization is not part of the weight-only kernels (activations stay BF16)")
+
+
+quant_rows = quant_groups
+
+
+def w3_linear(x: torch.Tensor, w3: W3Weight, x_scale: torch.Tensor | None = None, splits: int | None = None) -> torch.Tensor:
+    """y = x @ W^T for x [M, K] BF16, M <= MAX_ROWS; returns BF16 [M, N] (hibana/kernels/w3.py:340-365).
+    `splits` is accepted for signature compatibility; the K split is chosen by the library."""
+    m, k = x.shape
+    if m > MAX_ROWS or k != w3.in_features:
+        raise ValueError("w3_linear: unsupported call")
+    if x.dtype != torch.bfloat16:
+        raise ValueError("w3_linear: the weight-only kernels take BF16 activations")
+    _lib.need_gpu(x)
+    tile(w3)
+    x = x.contiguous()
+    y = torch.empty((m, w3.out_features), dtype=torch.bfloat16, device=x.device)
+    if m == 0:
+        return y
+    _lib.check(_lib.lib().hb_w3_gemm(_lib.ptr(x), m, _lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut, w3.out_features, k,
+                                     _lib.ptr(y), _lib.stream()), "w3_linear")
+    return y
+
+
+def attach(linears, codebook=DEFAULT_CODEBOOK) -> tuple[int, int]:
+    """Nearest-level 3-bit copies for (name, linear) pairs that have none; returns (matrices packed, bytes)
+    (hibana/kernels/w3.py:370-378)."""
+    count = total = 0
+    for _, lin in linears:
+        if getattr(lin, "w3", None) is None:
+            lin.w3 = tile(pack(lin.dequantize(), codebook))
+            total += lin.w3.bytes
+            count += 1
+    return count, total
+
+
+def attach_model(model, log=print, codebook=DEFAULT_CODEBOOK) -> dict:
+    """Pack 3-bit decode copies for every projection `model.linears()` lists (hibana/kernels/w3.py:381-404, without
+    the calibrated-checkpoint branch)."""
+    count, total = attach(list(model.linears()), codebook)
+    torch.cuda.synchronize()
+    model.w3_identity = "nearest:" + str(codebook)
+    log(f"  w3: packed {count} matrices, {total / 2**30:.2f} GiB of 3-bit decode weights (codebook {codebook})")
+    return {"matrices": count, "bytes": total}
+
+
+def attach_draft(draft, log=print, codebook=DEFAULT_CODEBOOK) -> dict:
+    count, total = attach(draft.fp8_weights.items(), codebook)
+    torch.cuda.synchronize()
+    log(f"  w3: packed {count} draft matrices, {total / 2**30:.2f} GiB")
+    return {"matrices": count, "bytes": total}

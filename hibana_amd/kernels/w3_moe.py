@@ -1,0 +1,187 @@
+"""Three-bit routed experts on MI355X behind the reference's `w3_moe` surface (hibana/kernels/w3_moe.py).
+
+A layer's experts are stacked W3 matrices: fc1 [E, N1, H] (gated: N1 = 2 I with rows in `fc1_order`, every 32-row
+block sixteen up rows then their sixteen gate rows; ReLU^2: N1 = I) and fc2 [E, H, I]. `w3_moe` is the routed sum in
+selection order; `moe_layer` adds the shared expert and the sigmoid-gated combine of the reference's MoeLayer
+(hibana/model/flashnext/moe.py:177-192) in the same chain of launches.
+
+The call is: one planning workgroup (expert-sorted pair list, slots of up to 16 rows), the fc1 stream (epilogue
+h = bf16(silu(bf16 gate) * bf16 up) or bf16(relu(bf16 up)^2)), the fc2 stream (FP32 per pair), the combine. Weight-only:
+x and h stay BF16. Deterministic (no floating-point atomics), graph-capturable, any number of rows.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import torch
+
+from hibana_amd import _lib
+from hibana_amd.kernels import w3
+
+EXPERTS = 512
+ORDER_IN_KERNEL = 640  # kept for the reference's callers; the planner here orders any number of pairs on the device
+WIDE_ROWS = 1024
+
+
+@dataclass
+class W3Experts:
+    planes13: torch.Tensor | None  # [E, N1/32, H/128, 3, 32, 4] uint32, fc1 rows in fc1_order
+    scales13: torch.Tensor | None  # [E, N1/32, H/128, 4, 32] uint8 E4M3
+    row13: torch.Tensor            # [E, N1] float32
+    planes2: torch.Tensor | None   # [E, H/32, I/128, 3, 32, 4]
+    scales2: torch.Tensor | None
+    row2: torch.Tensor             # [E, H]
+    codebook: tuple[float, ...]
+    lut: int
+    fc2_codebook: tuple[float, ...]
+    fc2_lut: int
+    base: int = 0
+    tiled13: torch.Tensor | None = None  # the kernels' block layout of the stacked fc1 / fc2 (built by tile())
+    tiled2: torch.Tensor | None = None
+    shape13: tuple[int, int] | None = None  # (N1, H), (H_out, I): kept when the fragment-order tensors are released
+    shape2: tuple[int, int] | None = None
+
+    def __post_init__(self):
+        if self.shape13 is None:
+            self.shape13 = (self.planes13.shape[1] * 32, self.planes13.shape[2] * w3.CHUNK)
+            self.shape2 = (self.planes2.shape[1] * 32, self.planes2.shape[2] * w3.CHUNK)
+
+    @property
+    def experts(self) -> int:
+        return self.row13.shape[0]
+
+    @property
+    def bytes(self) -> int:
+        (n1, h), (h2, i) = self.shape13, self.shape2
+        return self.experts * (n1 * h * 3 // 8 + n1 * h // 32 + n1 * 4 + h2 * i * 3 // 8 + h2 * i // 32 + h2 * 4)
+
+    def matrix(self, e: int, fc1: bool) -> w3.W3Weight:
+        """Expert e's fc1 (rows in fc1_order) or fc2 as a W3Weight (views, no copy)."""
+        p, s, r = (self.planes13, self.scales13, self.row13) if fc1 else (self.planes2, self.scales2, self.row2)
+        n, k = self.shape13 if fc1 else self.shape2
+        book = (self.codebook, self.lut) if fc1 else (self.fc2_codebook, self.fc2_lut)
+        tiled = self.tiled13 if fc1 else self.tiled2
+        part = None if tiled is None else tiled.view(self.experts, -1)[e]
+        return w3.W3Weight(None if p is None else p[e], None if s is None else s[e], r[e], n, k, *book, tiled=part)
+
+    def stacked(self, fc1: bool) -> w3.W3Weight:
+        """All experts' fc1 or fc2 as one W3Weight of E * N rows (the checkpoint entry)."""
+        p, s, r = (self.planes13, self.scales13, self.row13) if fc1 else (self.planes2, self.scales2, self.row2)
+        n, k = self.shape13 if fc1 else self.shape2
+        book = (self.codebook, self.lut) if fc1 else (self.fc2_codebook, self.fc2_lut)
+        e = self.experts
+        return w3.W3Weight(None if p is None else p.reshape(e * n // 32, *p.shape[2:]), None if s is None else s.reshape(e * n // 32, *s.shape[2:]),
+                           r.reshape(-1), e * n, k, *book, tiled=self.tiled13 if fc1 else self.tiled2)
+
+    @classmethod
+    def from_stacked(cls, fc1: w3.W3Weight, fc2: w3.W3Weight, experts: int, base: int = 0) -> "W3Experts":
+        def split(m):
+            return (m.planes.reshape(experts, -1, *m.planes.shape[1:]), m.scales.reshape(experts, -1, *m.scales.shape[1:]),
+                    m.row_scale.reshape(experts, -1))
+        return cls(*split(fc1), *split(fc2), fc1.codebook, fc1.lut, fc2.codebook, fc2.lut, base)
+
+
+def gated(experts: W3Experts) -> bool:
+    """Gated-SiLU experts (fc1 = [up; gate], 2 I rows) or ReLU^2 ones (fc1 = up, I rows)."""
+    return experts.shape13[0] == 2 * experts.shape2[1]
+
+
+def fc1_order(inter: int, device=None) -> torch.Tensor:
+    """Row permutation of w13 = [up; gate] (2 * inter rows): block b of 32 rows is up 16b..16b+15, then gate
+    16b..16b+15 (hibana/kernels/w3_moe.py:88-92)."""
+    cols = torch.arange(inter, device=device).unflatten(0, (inter // 16, 16))
+    return torch.stack((cols, cols + inter), dim=1).reshape(-1)
+
+
+def tile(experts: W3Experts, release: bool = False) -> W3Experts:
+    """Build the kernels' block layout of both stacks (once); `release` drops the fragment-order tensors."""
+    for fc1 in (True, False):
+        if (experts.tiled13 if fc1 else experts.tiled2) is None:
+            stacked = w3.tile(experts.stacked(fc1))
+            if fc1:
+                experts.tiled13 = stacked.tiled
+            else:
+                experts.tiled2 = stacked.tiled
+    if release:
+        experts.planes13 = experts.scales13 = experts.planes2 = experts.scales2 = None
+    return experts
+
+
+def _struct(experts: W3Experts) -> _lib.HbW3Experts:
+    tile(experts)
+    (n1, h), (h2, i) = experts.shape13, experts.shape2
+    return _lib.HbW3Experts(_lib.ptr(experts.tiled13), _lib.ptr(experts.row13), _lib.ptr(experts.tiled2), _lib.ptr(experts.row2),
+                            experts.lut, experts.fc2_lut, experts.experts, experts.base, h, i, h2, int(gated(experts)))
+
+
+def _check_call(experts: W3Experts, x, ids, weights):
+    if x.dtype != torch.bfloat16 or x.ndim != 2 or x.shape[1] != experts.shape13[1]:
+        raise ValueError("w3_moe: x must be BF16 [M, hidden]")
+    if ids.ndim != 2 or ids.shape[0] != x.shape[0] or weights.shape != ids.shape:
+        raise ValueError("w3_moe: ids and weights must be [M, k]")
+    _lib.need_gpu(x, ids, weights)
+
+
+def w3_moe(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, pairs: bool = False,
+           pairs_bf16: bool = False) -> torch.Tensor:
+    """Routed experts for x [M, H] BF16 with the router's ids [M, k] and weights [M, k] -> BF16 [M, H_out], the
+    weighted sum in selection order (no shared expert). An id outside this object's range base .. base + E - 1 (another
+    rank's expert, or the "no expert" id 512) adds nothing. With `pairs`, the FP32 (`pairs_bf16`: BF16) output of each
+    (row, k) pair [M * k, H_out], unsummed; rows of skipped pairs are unspecified
+    (hibana/kernels/w3_moe.py:158-179)."""
+    _check_call(experts, x, ids, weights)
+    m, k = ids.shape
+    h_out = experts.shape2[0]
+    mode = 2 if pairs and pairs_bf16 else int(pairs)
+    shape = (m * k, h_out) if pairs else (m, h_out)
+    out = torch.empty(shape, dtype=torch.float32 if mode == 1 else torch.bfloat16, device=x.device)
+    if m == 0:
+        return out
+    st = _struct(experts)
+    need = _lib.lib().hb_w3_moe_workspace_bytes(m, k, C.byref(st), 0)
+    ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    ids32 = ids.to(torch.int32).contiguous()
+    wt = weights.float().contiguous()
+    _lib.check(_lib.lib().hb_w3_moe(C.byref(st), _lib.ptr(x.contiguous()), _lib.ptr(ids32), _lib.ptr(wt), m, k, mode, _lib.ptr(out),
+                                    _lib.ptr(ws), need, _lib.stream()), "w3_moe")
+    return out
+
+
+def moe_layer(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, shared: W3Experts | None = None,
+              gate_vec: torch.Tensor | None = None) -> torch.Tensor:
+    """The MoE layer on 3-bit weights in one chain of launches: routed sum + the shared expert (`shared`: a one-expert
+    W3Experts of the same geometry) combined as bf16(bf16(routed) + g * bf16(shared)), g = sigmoid(x . gate_vec) or 1
+    (hibana/model/flashnext/moe.py:177-192)."""
+    _check_call(experts, x, ids, weights)
+    m, k = ids.shape
+    out = torch.empty((m, experts.shape2[0]), dtype=torch.bfloat16, device=x.device)
+    if m == 0:
+        return out
+    st = _struct(experts)
+    sh = _struct(shared) if shared is not None else None
+    need = _lib.lib().hb_w3_moe_workspace_bytes(m, k, C.byref(st), int(shared is not None))
+    ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    ids32 = ids.to(torch.int32).contiguous()
+    wt = weights.float().contiguous()
+    gv = None if gate_vec is None else gate_vec.float().contiguous()
+    _lib.check(_lib.lib().hb_w3_moe_layer(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(x.contiguous()),
+                                          _lib.ptr(ids32), _lib.ptr(wt), m, k, _lib.ptr(out), _lib.ptr(ws), need, _lib.stream()), "moe_layer")
+    return out
+
+
+def unswizzle_batched(swizzled: torch.Tensor, rows: int, groups: int) -> torch.Tensor:
+    """[E, ...] block scales in the 128x4 interleave -> float8_e4m3fn [E, rows, groups] (hibana/kernels/w3_moe.py:97-102)."""
+    from hibana_amd.weights.modelopt import unswizzle_block_scales
+    e = swizzled.shape[0]
+    flat = swizzled.reshape(e, -1).view(torch.uint8)
+    return torch.stack([unswizzle_block_scales(flat[i], rows, groups) for i in range(e)]).view(torch.float8_e4m3fn)
+
+
+def nvfp4_dequant(packed: torch.Tensor, scales: torch.Tensor, scale2: torch.Tensor) -> torch.Tensor:
+    """NVFP4 experts (uint8 [E, R, K/2], float8_e4m3fn [E, R, K/16], FP32 [E]) -> float32 [E, R, K]
+    (hibana/kernels/w3_moe.py:105-110)."""
+    from hibana_amd.weights.modelopt import unpack_fp4
+    e, r, _ = packed.shape
+    w = unpack_fp4(packed.reshape(e * r, -1), scales.reshape(e * r, -1)).reshape(e, r, -1)
+    return w * scale2.float().reshape(e, 1, 1)

@@ -1,0 +1,165 @@
+/*
+ * hibana_hip.h - C ABI of the MI355X (gfx950) quantized-weight linear / MoE expert kernels.
+ *
+ * Plain pointers and sizes only. Every pointer is a DEVICE pointer unless its comment says "host". The caller owns
+ * every buffer, including scratch ("workspace"); the library allocates nothing. `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream). Every function enqueues work on `stream` and returns without synchronizing;
+ * kernels use no floating-point atomics, so results are bitwise repeatable and the calls are graph-capturable.
+ * Return value: HB_OK (0) or a negative HB_E* code; hb_error_string() names it.
+ *
+ * Citations "ref:" give the interface of the reference (sharar-project/hibana, paths relative to its tree) that the
+ * entry point replaces.
+ */
+#ifndef HIBANA_HIP_H
+#define HIBANA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  HB_OK = 0,
+  HB_EINVAL = -1,     /* a shape, alignment or flag the kernels do not take (the Python layer raises ValueError) */
+  HB_ENULL = -2,      /* a required pointer is NULL */
+  HB_EWORKSPACE = -3, /* workspace smaller than hb_*_workspace_bytes() says */
+  HB_ELAUNCH = -4     /* the HIP runtime refused a launch (hipGetLastError is left set for the caller) */
+};
+
+/* Library version (major * 1000 + minor). */
+int hb_version(void);
+const char* hb_error_string(int code);
+
+/* Tuning knobs for experiments ("w3_ksplit", "w3_nbw", "moe_fc1_ksplit", ...); value 0 restores the built-in choice.
+ * Returns HB_EINVAL for an unknown key. Not thread-safe against concurrent launches. */
+int hb_tune(const char* key, int value);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * W3 format: 3-bit (or 2-bit) codes into an 8-entry E4M3 codebook, one E4M3 scale per 32 weights along K, one FP32
+ * multiplier per output row.
+ *
+ * Reference layout (what checkpoints hold; ref: hibana/kernels/w3.py:75-91):
+ *   planes uint32 [rows/32, K/128, bits, 32, 4], scales uint8 [rows/32, K/128, 4, 32], row_scale float [rows].
+ * Tile layout (what the kernels stream; built once at load time): blocks of 64 rows x 128 k, 3328 bytes each,
+ *   [rows/64][K/128]{ 3 x 64 lanes x 16 B of codes, 16 x 16 B of scales }, see hibana_amd/csrc/w3_layout.hpp.
+ * `rows` may stack several matrices (experts) of the same K as long as each has a multiple of 64 rows.
+ * ---------------------------------------------------------------------------------------------------------------- */
+
+/* Bytes of the tile layout of a [rows, k] matrix; 0 if rows % 64 or k % 128. */
+size_t hb_w3_tiled_bytes(int64_t rows, int k);
+
+/* Reference layout -> tile layout (load-time repack). bits = 3 or 2 (2-bit codes are widened to 3 bits).
+ * ref: the layout contract of w3_gemm's operands, hibana/kernels/csrc/w3_gemm.cu:1299-1315; hook point
+ * hibana/weights/w3_checkpoint.py:115-139 (CalibratedWeights._load). */
+int hb_w3_repack(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, void* tiled, void* stream);
+
+/* codes uint8 [rows, k] + E4M3 scale bytes uint8 [rows, k/32] -> reference layout (planes, scales).
+ * ref: w3._pack_codes_rows, hibana/kernels/w3.py:175-195. */
+int hb_w3_pack_codes(const uint8_t* codes, const uint8_t* scale_bytes, int64_t rows, int k, int bits, uint32_t* planes,
+                     uint8_t* scales, void* stream);
+
+/* Tile layout -> codes uint8 [rows, k] and E4M3 scale bytes uint8 [rows, k/32] (either output may be NULL).
+ * ref: w3.codes / the byte part of w3.group_scales, hibana/kernels/w3.py:217-236. */
+int hb_w3_unpack(const void* tiled, int64_t rows, int k, uint8_t* codes, uint8_t* scale_bytes, void* stream);
+
+/* Reference layout -> codes / scale bytes, same outputs as hb_w3_unpack (the unpack of a checkpoint tensor as stored).
+ * ref: hibana/kernels/w3.py:217-236. */
+int hb_w3_unpack_planes(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, uint8_t* codes,
+                        uint8_t* scale_bytes, void* stream);
+
+/* Tile layout -> float32 [rows, k]: level[code] * (float(e4m3 scale) * row_scale[row]), both products rounded to
+ * FP32 in this order (bit-exact with the reference's unpack). `lut` = the codebook as 8 E4M3 bytes, entry i in byte i.
+ * ref: w3.dequantize, hibana/kernels/w3.py:239-242; lut: w3.lut_of, :105-107. */
+int hb_w3_dequant(const void* tiled, const float* row_scale, int64_t lut, int64_t rows, int k, float* out, void* stream);
+
+/* y[m, n] = bf16( row_scale[n] * sum_g scale[n, g] * sum_{k in g} x[m, k] * level[code[n, k]] ), FP32 accumulation,
+ * x BF16 [m, k] row-major with row stride k, y BF16 [m, n]. Any m >= 1 (the reference stops at 128 rows).
+ * n % 64 == 0, k % 128 == 0.
+ * ref: w3_gemm / w3_gemm_wide, hibana/kernels/csrc/w3_gemm.cu:1299-1331,1385-1413 (called by w3.w3_linear,
+ * hibana/kernels/w3.py:340-365), in its weight-only form (BF16 activations are not re-quantized to E4M3). */
+int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, void* y,
+               void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Routed experts on W3 weights (gated SiLU when fc1 has 2*inter rows per expert in the reference's fc1_order, ReLU^2
+ * when it has inter rows).
+ * ---------------------------------------------------------------------------------------------------------------- */
+typedef struct hb_w3_experts {
+  const void* fc1;        /* tile layout of the stacked fc1 [experts * n1, hidden], n1 = gated ? 2*inter : inter */
+  const float* fc1_rows;  /* [experts, n1] */
+  const void* fc2;        /* tile layout of the stacked fc2 [experts * hidden_out, inter] */
+  const float* fc2_rows;  /* [experts, hidden_out] */
+  int64_t fc1_lut, fc2_lut;
+  int experts;            /* experts held here (expert parallel: one rank's range) */
+  int base;               /* id of the first one */
+  int hidden, inter, hidden_out; /* fc1 in-features, intermediate size, fc2 out-features (== hidden for these models) */
+  int gated;
+} hb_w3_experts;
+
+enum { HB_MOE_SUM = 0, HB_MOE_PAIRS_F32 = 1, HB_MOE_PAIRS_BF16 = 2 };
+
+/* Workspace bytes for hb_w3_moe / hb_w3_moe_layer with up to m rows of top-k ids (shared: 1 if a shared expert rides
+ * along). */
+size_t hb_w3_moe_workspace_bytes(int m, int topk, const hb_w3_experts* routed, int shared);
+
+/* Routed sum: out[r] = bf16( fma-chain over the row's slots, in selection order, of weights[r, s] * y[r, s] ),
+ * y = fc2_e( act( bf16(fc1_e x_r) ) ) in FP32, h rounded to BF16. ids int32 [m, topk]; an id outside
+ * [base, base + experts) adds nothing. mode HB_MOE_SUM: out BF16 [m, hidden_out]; HB_MOE_PAIRS_F32 / _BF16: out is
+ * the unsummed pair outputs [m * topk, hidden_out] (rows of dropped pairs are left untouched).
+ * ref: w3_moe, hibana/kernels/csrc/w3_gemm.cu:1366-1382 (run<S> :1215-1292; Python hibana/kernels/w3_moe.py:158-179),
+ * weight-only form. */
+int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32_t* ids, const float* weights, int m, int topk,
+              int mode, void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The whole MoE layer on 3-bit weights: routed sum + shared expert (a one-expert hb_w3_experts, may be NULL) +
+ * combine: out = bf16( bf16(routed) + g * bf16(shared) ), g = sigmoid(x . gate_vec) or 1 when gate_vec is NULL
+ * (float32 [hidden]).
+ * ref: MoeLayer.__call__, hibana/model/flashnext/moe.py:177-192 (w3_moe with pairs + moe_combine_pairs,
+ * hibana/kernels/flashnext_fused.py:530-571). */
+int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                    const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* out = bf16( bf16(sum over the row's local slots of w * pairs) + g * shared ) from unsummed pair outputs (FP32 or,
+ * pairs_bf16 != 0, BF16) [m * topk, h]; shared BF16 [m, h] or NULL; gate_vec float32 [h] or NULL (then g = 1; x
+ * unused). ref: moe_combine_pairs, hibana/kernels/flashnext_fused.py:530-571; with shared == NULL it is
+ * combine_kernel, hibana/kernels/csrc/w3_gemm.cu:1196-1213. */
+int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int32_t* ids, const float* weights, const void* shared,
+                         const void* x, const float* gate_vec, int e_lo, int e_n, int m, int topk, int h, void* out,
+                         void* stream);
+
+/* Softmax top-k routing: logits float32 [m, e] -> ids int32 [m, k] (descending probability, ties to the lower id),
+ * weights float32 [m, k] renormalized over the selection.
+ * ref: route_topk, hibana/kernels/flashnext_fused.py:278-319 (plain form, no padded-slot table). */
+int hb_route_softmax_topk(const float* logits, int m, int e, int k, int32_t* ids, float* weights, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * NVFP4 format: E2M1 codes two per byte (element 2i in the low nibble), one E4M3 scale per 16 weights, one FP32
+ * global scale. ref: hibana/weights/modelopt.py:57-81,150-156.
+ * Tile layout: blocks of 64 rows x 128 k, 4608 bytes each: { 4 x 64 lanes x 16 B of codes, 64 rows x 8 scale bytes }.
+ * ---------------------------------------------------------------------------------------------------------------- */
+size_t hb_nvfp4_tiled_bytes(int64_t rows, int k);
+
+/* weight uint8 [rows, k/2] + block scales E4M3 uint8 [rows, k/16] (row-major, unswizzled) or, swizzled != 0, in the
+ * CUTLASS 128x4 interleave [rows_pad128, (k/16)_pad4] -> tile layout.
+ * ref: the operand layout of mm_fp4 at hibana/kernels/ops.py:74-82; swizzle hibana/weights/modelopt.py:130-147. */
+int hb_nvfp4_repack(const uint8_t* weight, const uint8_t* scales, int swizzled, int64_t rows, int k, void* tiled,
+                    void* stream);
+
+/* Tile layout -> float32 [rows, k]: e2m1 * float(e4m3 scale) * global_scale (two FP32 roundings in this order).
+ * ref: unpack_fp4 / Nvfp4Linear.dequantize, hibana/weights/modelopt.py:73-77,150-156. */
+int hb_nvfp4_dequant(const void* tiled, float global_scale, int64_t rows, int k, float* out, void* stream);
+
+/* y = bf16( (x Wq^T)_fp32 * global_scale ), Wq = e2m1 * e4m3 (exact in BF16); relu2 != 0 applies
+ * bf16(relu(y)^2) on top. x BF16 [m, k], y BF16 [m, n]; n % 64 == 0, k % 128 == 0.
+ * ref: ops.nvfp4_linear, hibana/kernels/ops.py:56-83 in its weight-only form, which the reference states as
+ * ggml_bf16.matmul(..., "NVFP4"), hibana/kernels/ggml_bf16.py:125-159. */
+int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y,
+                  void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIBANA_HIP_H */

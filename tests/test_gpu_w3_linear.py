@@ -1,0 +1,82 @@
+"""The dense W3 linear on the GPU against the oracle (weight-only: BF16 activations, exact weights, FP32 accumulate)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import layers, w3_format as ow3
+from tests.util import MAX_REL, NORM_REL, errors, random_w3, to_device_w3
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("m", [1, 2, 5, 16, 17, 33, 64, 128])
+@pytest.mark.parametrize("n,k,codebook", [(128, 256, "uniform"), (512, 1024, "lloyd"), (1024, 640, "zero8"), (256, 2688, "lloyd")])
+def test_w3_linear_matches_the_oracle(m, n, k, codebook):
+    from hibana_amd.kernels import w3
+    packed, *_ = random_w3(n, k, 7, codebook)
+    dev = to_device_w3(packed)
+    g = torch.Generator().manual_seed(100 + m)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    x[:, ::97] *= 30  # outlier channels
+    want = layers.dense_ref(x, ow3.dequantize(packed))
+    got = w3.w3_linear(x.cuda(), dev)
+    assert got.dtype == torch.bfloat16 and got.shape == (m, n)
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    again = w3.w3_linear(x.cuda(), dev)
+    assert torch.equal(again, got)  # bitwise repeatable
+
+
+def test_every_k_split_gives_close_results_and_the_unsplit_bits_repeat():
+    from hibana_amd import _lib
+    from hibana_amd.kernels import w3
+    packed, *_ = random_w3(256, 2048, 8)
+    dev = to_device_w3(packed)
+    x = torch.randn(16, 2048, generator=torch.Generator().manual_seed(1)).bfloat16()
+    want = layers.dense_ref(x, ow3.dequantize(packed))
+    try:
+        for ks, nbw in ((1, 1), (1, 4), (2, 2), (4, 1), (8, 1), (16, 1), (4, 4)):
+            _lib.lib().hb_tune(b"w3_ksplit", ks)
+            _lib.lib().hb_tune(b"w3_nbw", nbw)
+            got = w3.w3_linear(x.cuda(), dev)
+            mx, nr = errors(got, want)
+            assert mx < MAX_REL and nr < NORM_REL, (ks, nbw, mx, nr)
+    finally:
+        _lib.lib().hb_tune(b"w3_ksplit", 0)
+        _lib.lib().hb_tune(b"w3_nbw", 0)
+
+
+def test_full_size_decode_projection_against_the_dequantized_product():
+    """BASELINE config 0 (M = 1, K = N = 5120, uniform codebook, one scale draw per 128): the kernel against
+    x @ dequantize(W)^T in FP32 on the GPU; the dequantization itself is pinned bit-exact on the smaller shapes."""
+    from hibana_amd.kernels import w3
+    torch.manual_seed(0)
+    n = k = 5120
+    q = torch.randint(0, 8, (n, k), device="cuda", dtype=torch.uint8)
+    s = (torch.randn(n, k // 128, device="cuda").abs() * 0.02 + 1e-3).repeat_interleave(4, dim=1)
+    row = (s.amax(dim=1) / 448.0).clamp_min(1e-12)
+    stored = (s / row[:, None]).to(torch.float8_e4m3fn)
+    weight = w3.pack_codes(q, stored, row, "uniform")
+    assert weight.bytes == 10_670_080
+    x = torch.randn(1, k, device="cuda").bfloat16()
+    deq = w3.dequantize(weight)
+    levels = torch.tensor(weight.codebook, device="cuda")
+    assert torch.equal(deq, levels[q.long()] * (stored.float() * row[:, None]).repeat_interleave(32, dim=1))
+    want = (x.float() @ deq.T).bfloat16()
+    got = w3.w3_linear(x, weight)
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    # linearity in x: f(2x) == 2 f(x) exactly (a power of two commutes with every rounding)
+    assert torch.equal(w3.w3_linear(x * 2, weight), got * 2)
+
+
+def test_unsupported_calls_raise():
+    from hibana_amd.kernels import w3
+    packed, *_ = random_w3(128, 256, 9)
+    dev = to_device_w3(packed)
+    with pytest.raises(ValueError):
+        w3.w3_linear(torch.zeros(129, 256, dtype=torch.bfloat16, device="cuda"), dev)
+    with pytest.raises(ValueError):
+        w3.w3_linear(torch.zeros(4, 128, dtype=torch.bfloat16, device="cuda"), dev)
+    with pytest.raises(RuntimeError):
+        w3.w3_linear(torch.zeros(4, 256, dtype=torch.bfloat16), dev)
