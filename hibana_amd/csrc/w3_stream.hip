@@ -12,6 +12,8 @@
 // repeatable.
 #include <string.h>
 
+#include <vector>
+
 #include "common.hpp"
 #include "w3_layout.hpp"
 
@@ -487,6 +489,13 @@ __global__ __launch_bounds__(64) void route_softmax_topk_kernel(const float* __r
 }
 
 // ---------------------------------------------------------------------------------------------------- host side
+// Measurement hook: events the caller created, recorded around each kernel of the next routed-expert chain.
+static std::vector<hipEvent_t> g_events;
+static size_t g_event_next = 0;
+static inline void mark(hipStream_t stream) {
+  if (g_event_next < g_events.size()) (void)hipEventRecord(g_events[g_event_next++], stream);
+}
+
 struct Tuning {
   int w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0;
 };
@@ -617,8 +626,10 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   if (slots > 65535 || pairs > 0x3fffffff) return HB_EINVAL;
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * ex->experts + PLAN_WAVES + 1) * sizeof(int);
   if (plan_lds > 160 * 1024) return HB_EINVAL;
+  mark(stream);
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, ex->base, ex->experts, shared_rows,
                      ws.plan, ws.order);
+  mark(stream);
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
   const int64_t est = pairs < 2 * ex->experts ? (pairs + 1) / 2 + (shared_rows + 15) / 16 : slots;  // rough number of busy slots
   StreamParams p{};
@@ -653,6 +664,7 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   } else {
     launch_stream<EPI_FC1_RELU2>(p, slots, stream);
   }
+  mark(stream);
   p.w = static_cast<const uint8_t*>(ex->fc2);
   p.expert_bytes = (int64_t)hb_w3_tiled_bytes(ex->hidden_out, ex->inter);
   p.rows = ex->fc2_rows;
@@ -677,11 +689,13 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   if (g_tune.moe_fc2_nbw) p.nbw = g_tune.moe_fc2_nbw;
   if (p.ks * p.nbw > 16 || p.ks > p.chunks) return HB_EINVAL;
   launch_stream<EPI_FC2>(p, slots, stream);
+  mark(stream);
   return launch_status();
 }
 
 void launch_combine(const CombineParams& c, hipStream_t stream) {
   hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)c.m, (unsigned)((c.h + 1023) / 1024)), dim3(256), 0, stream, c);
+  mark(stream);
 }
 
 }  // namespace
@@ -785,6 +799,13 @@ extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, i
   hipLaunchKernelGGL(route_softmax_topk_kernel, dim3((unsigned)m), dim3(64), (size_t)e * sizeof(float), as_stream(stream), logits, e, k, ids,
                      weights);
   return launch_status();
+}
+
+extern "C" int hb_debug_events(void* const* events, int count) {
+  if (count < 0 || (count > 0 && !events)) return HB_EINVAL;
+  g_events.assign(reinterpret_cast<hipEvent_t const*>(events), reinterpret_cast<hipEvent_t const*>(events) + count);
+  g_event_next = 0;
+  return HB_OK;
 }
 
 extern "C" int hb_version(void) { return 1000; }

@@ -36,6 +36,12 @@ const char* hb_error_string(int code);
  * Returns HB_EINVAL for an unknown key. Not thread-safe against concurrent launches. */
 int hb_tune(const char* key, int value);
 
+/* Measurement hook (no counterpart in the reference): `events` are hipEvent_t handles the caller created; the next
+ * routed-expert call (hb_w3_moe / hb_w3_moe_layer) records them, in order, at the five boundaries of its chain:
+ * before the plan kernel, after it, after fc1, after fc2, after the combine. count = 0 switches the hook off.
+ * Not for captured graphs. */
+int hb_debug_events(void* const* events, int count);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * W3 format: 3-bit (or 2-bit) codes into an 8-entry E4M3 codebook, one E4M3 scale per 32 weights along K, one FP32
  * multiplier per output row.

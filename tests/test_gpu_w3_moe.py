@@ -1,0 +1,198 @@
+"""The routed-expert kernels on the GPU against the oracle's layer math (weight-only, identity activation rounding):
+one row to prefill-sized calls, fewer experts per row, unfilled slots, expert-parallel halves, pair outputs, the
+shared expert and the gated combine, ReLU^2 experts. Mirrors tests/gpu/test_w3_moe.py and test_w3_moe_nemotron.py
+of the reference."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import layers
+from tests.util import MAX_REL, NORM_REL, errors, oracle_expert_getter, random_experts
+
+pytestmark = pytest.mark.gpu
+
+E, H, I, TOPK = 16, 256, 128, 10
+
+
+@pytest.fixture(scope="module")
+def gated():
+    ex, per = random_experts(E, H, I, True, 5)
+    return ex, oracle_expert_getter(per, True, I)
+
+
+@pytest.fixture(scope="module")
+def relu2():
+    ex, per = random_experts(8, 256, 384, False, 6, codebook="lloyd", fc2_codebook="zero8")
+    return ex, oracle_expert_getter(per, False, 384)
+
+
+def _inputs(m, k, seed, experts=E):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, H, generator=g).bfloat16()
+    x[:, ::97] *= 30
+    ids = torch.stack([torch.randperm(experts, generator=g)[:k] for _ in range(m)]).to(torch.int32)
+    weights = torch.softmax(torch.randn(m, k, generator=g), -1)
+    return x, ids, weights
+
+
+def _check(ex, get, x, ids, weights, is_gated=True, e_lo=0, e_n=None):
+    from hibana_amd.kernels import w3_moe
+    e_n = ex.experts if e_n is None else e_n
+    want = layers.moe_layer_ref(x, ids.numpy(), weights, get, is_gated, e_lo=e_lo, e_n=e_n)
+    got = w3_moe.w3_moe(ex, x.cuda(), ids.cuda(), weights.cuda())
+    assert got.dtype == torch.bfloat16 and got.shape == want.shape
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    assert torch.equal(w3_moe.w3_moe(ex, x.cuda(), ids.cuda(), weights.cuda()), got)  # no atomics in the sums
+    return got
+
+
+@pytest.mark.parametrize("m", [1, 2, 5, 16, 32, 64, 200])
+def test_kernel_matches_oracle(gated, m):
+    _check(*gated, *_inputs(m, TOPK, m))
+
+
+@pytest.mark.parametrize("k", [1, 5, 9])
+@pytest.mark.parametrize("m", [1, 5, 64])
+def test_fewer_experts_per_row(gated, m, k):
+    _check(*gated, *_inputs(m, k, 100 * k + m))
+
+
+@pytest.mark.parametrize("m", [2, 5, 16, 17, 80])
+def test_ids_past_the_last_expert_add_nothing(gated, m):
+    ex, get = gated
+    from hibana_amd.kernels import w3_moe
+    g = torch.Generator().manual_seed(300 + m)
+    x = torch.randn(m, H, generator=g).bfloat16()
+    ids = torch.full((m, TOPK), w3_moe.EXPERTS, dtype=torch.int32)
+    weights = torch.zeros(m, TOPK)
+    others = [e for e in range(E) if e != 3]
+    for r in range(m):  # every row shares expert 3, with 1 to 9 unfilled slots
+        n = 1 + r % 9
+        ids[r, :n] = torch.tensor([3] + [others[i] for i in torch.randperm(len(others), generator=g)[:n - 1].tolist()], dtype=torch.int32)
+        weights[r, :n] = torch.softmax(torch.randn(n, generator=g), -1)
+    ids[-1], weights[-1] = w3_moe.EXPERTS, 0.0  # a padded row
+    got = _check(ex, get, x, ids, weights)
+    assert torch.isfinite(got.float()).all() and not got[-1].any()
+
+
+@pytest.mark.parametrize("k", [TOPK, 5])
+@pytest.mark.parametrize("m", [1, 5, 80])
+def test_expert_parallel_halves_sum_to_the_whole(gated, m, k):
+    from dataclasses import replace
+
+    from hibana_amd.kernels import w3_moe
+    ex, get = gated
+    x, ids, weights = _inputs(m, k, 100 + m + k)
+    half = E // 2
+
+    def part(lo):
+        return replace(ex, planes13=ex.planes13[lo:lo + half], scales13=ex.scales13[lo:lo + half], row13=ex.row13[lo:lo + half],
+                       planes2=ex.planes2[lo:lo + half], scales2=ex.scales2[lo:lo + half], row2=ex.row2[lo:lo + half], base=lo,
+                       tiled13=None, tiled2=None)
+
+    whole = w3_moe.w3_moe(ex, x.cuda(), ids.cuda(), weights.cuda()).float()
+    lo, hi = part(0), part(half)
+    parts = w3_moe.w3_moe(lo, x.cuda(), ids.cuda(), weights.cuda()).float() + w3_moe.w3_moe(hi, x.cuda(), ids.cuda(), weights.cuda()).float()
+    assert float((parts - whole).norm() / whole.norm()) < NORM_REL
+    _check(hi, lambda e: get(e + half), x, ids, weights, e_lo=half, e_n=half)
+    only = torch.full_like(ids, half)  # every pair on the second rank: the first rank's partial is zero
+    assert not w3_moe.w3_moe(lo, x.cuda(), only.cuda(), weights.cuda()).any()
+
+
+@pytest.mark.parametrize("m", [1, 5, 64, 200])
+def test_pairs_then_combine_gives_the_same_bits(gated, m):
+    """`w3_moe(..., pairs=True)` summed by `moe_combine_pairs` == the kernel's own combine; BF16 pairs are the FP32
+    pairs rounded once (tests/gpu/test_w3_moe.py:132-186 of the reference)."""
+    from hibana_amd.kernels import ops, w3_moe
+    ex, get = gated
+    x, ids, weights = _inputs(m, TOPK, 300 + m)
+    ids[::3, -1] = w3_moe.EXPERTS
+    xd, idd, wd = x.cuda(), ids.cuda(), weights.cuda()
+    summed = w3_moe.w3_moe(ex, xd, idd, wd)
+    pairs = w3_moe.w3_moe(ex, xd, idd, wd, pairs=True)
+    assert pairs.dtype == torch.float32 and pairs.shape == (m * TOPK, H)
+    assert torch.equal(ops.moe_combine_pairs(pairs, idd, wd, None, None, None, 0, E), summed)
+    want_pairs = layers.routed_experts_ref(x, ids.numpy(), get, True, 0, E)
+    local = (ids.reshape(-1) < E)
+    mx, nr = errors(pairs[local.cuda()], want_pairs[local])
+    assert mx < MAX_REL and nr < NORM_REL
+    half = w3_moe.w3_moe(ex, xd, idd, wd, pairs=True, pairs_bf16=True)
+    assert half.dtype == torch.bfloat16
+    assert torch.equal(half[local.cuda()], pairs[local.cuda()].bfloat16())
+    shared = torch.randn(m, H, generator=torch.Generator().manual_seed(1)).bfloat16()
+    gate = torch.randn(H, generator=torch.Generator().manual_seed(2)) * 0.02
+    fused = ops.moe_combine_pairs(pairs, idd, wd, shared.cuda(), xd, gate.cuda(), 0, E)
+    want = layers.combine_shared_ref(summed.cpu(), shared, x, gate)
+    assert errors(fused, want)[0] < 2 ** -7  # one BF16 rounding apart at most (the sigmoid's dot product order)
+    assert torch.equal(ops.moe_combine_pairs(half, idd, wd, shared.cuda(), xd, gate.cuda(), 0, E),
+                       ops.moe_combine_pairs(half.float(), idd, wd, shared.cuda(), xd, gate.cuda(), 0, E))
+
+
+@pytest.mark.parametrize("m", [1, 7, 32, 100])
+@pytest.mark.parametrize("with_gate", [False, True])
+def test_layer_with_shared_expert(gated, m, with_gate):
+    from hibana_amd.kernels import w3_moe
+    ex, get = gated
+    shared_ex, shared_per = random_experts(1, H, I, True, 77)
+    shared_get = oracle_expert_getter(shared_per, True, I)
+    x, ids, weights = _inputs(m, TOPK, 500 + m)
+    gate = torch.randn(H, generator=torch.Generator().manual_seed(3)) * 0.05 if with_gate else None
+    want = layers.moe_layer_ref(x, ids.numpy(), weights, get, True, shared=shared_get(0), gate_vec=gate, e_n=E)
+    got = w3_moe.moe_layer(ex, x.cuda(), ids.cuda(), weights.cuda(), shared=shared_ex, gate_vec=None if gate is None else gate.cuda())
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    assert torch.equal(w3_moe.moe_layer(ex, x.cuda(), ids.cuda(), weights.cuda(), shared=shared_ex, gate_vec=None if gate is None else gate.cuda()), got)
+    # the layer without a shared expert is the routed sum
+    assert torch.equal(w3_moe.moe_layer(ex, x.cuda(), ids.cuda(), weights.cuda()), w3_moe.w3_moe(ex, x.cuda(), ids.cuda(), weights.cuda()))
+
+
+@pytest.mark.parametrize("m", [1, 16, 150])
+def test_relu2_experts_with_their_own_fc2_codebook(relu2, m):
+    """The latent experts' geometry in small (fc1 = up alone, h = relu(up)^2, top 6 of 8, a zero level in fc2)."""
+    ex, get = relu2
+    from hibana_amd.kernels import w3_moe
+    assert not w3_moe.gated(ex)
+    g = torch.Generator().manual_seed(700 + m)
+    x = (torch.randn(m, 256, generator=g) * 0.5).bfloat16()
+    ids = torch.stack([torch.randperm(8, generator=g)[:6] for _ in range(m)]).to(torch.int32)
+    ids[0, 2] = ids[0, 1]  # a duplicate expert in one row is legal: two pairs on one expert
+    weights = torch.rand(m, 6, generator=g)
+    _check(ex, get, x, ids, weights, is_gated=False)
+
+
+def test_graph_replay_gives_the_eager_bits(gated):
+    from hibana_amd.kernels import w3_moe
+    ex, _ = gated
+    x, ids, weights = _inputs(32, TOPK, 900)
+    xd, idd, wd = x.cuda(), ids.cuda(), weights.cuda()
+    eager = w3_moe.w3_moe(ex, xd, idd, wd)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = w3_moe.w3_moe(ex, xd, idd, wd)
+    for _ in range(3):
+        captured.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager)
+
+
+def test_plan_orders_many_pairs_on_the_device(gated):
+    """2,000 rows x 10: 20,000 pairs sorted by the planning kernel itself, against the oracle."""
+    _check(*gated, *_inputs(2000, TOPK, 1234))
+
+
+def test_bad_calls_raise(gated):
+    from hibana_amd.kernels import w3_moe
+    ex, _ = gated
+    x, ids, weights = _inputs(4, TOPK, 1)
+    with pytest.raises(ValueError):
+        w3_moe.w3_moe(ex, x.cuda().float(), ids.cuda(), weights.cuda())
+    with pytest.raises(ValueError):
+        w3_moe.w3_moe(ex, x.cuda()[:, :128], ids.cuda(), weights.cuda())
+    with pytest.raises(ValueError):
+        w3_moe.w3_moe(ex, x.cuda(), ids.cuda()[:2], weights.cuda())
+    with pytest.raises(RuntimeError):
+        w3_moe.w3_moe(ex, x, ids, weights)
