@@ -45,17 +45,23 @@ struct StreamParams {
   int ks, nbw;            // wavefronts per workgroup = ks (K splits) * nbw (64-row blocks)
 };
 
-struct Chunk {
+struct Chunk {  // the weight side of one 64-row x 128-k block
   u32x4_t w0, w1, w2, sc;
+};
+
+struct Rows {  // the activation side: four MFMA A fragments (one per 32-group), read from L2
   u32x4_t a0, a1, a2, a3;
 };
 
-__device__ __forceinline__ void load_chunk(Chunk& ch, const uint8_t* blk, const uint16_t* arow, int lane, int r16) {
+__device__ __forceinline__ void load_chunk(Chunk& ch, const uint8_t* blk, int lane, int r16) {
   const u32x4_t* b = reinterpret_cast<const u32x4_t*>(blk);
   ch.w0 = __builtin_nontemporal_load(b + lane);
   ch.w1 = __builtin_nontemporal_load(b + 64 + lane);
   ch.w2 = __builtin_nontemporal_load(b + 128 + lane);
   ch.sc = __builtin_nontemporal_load(b + 192 + r16);
+}
+
+__device__ __forceinline__ void load_rows(Rows& ch, const uint16_t* arow) {
   ch.a0 = *reinterpret_cast<const u32x4_t*>(arow);
   ch.a1 = *reinterpret_cast<const u32x4_t*>(arow + 32);
   ch.a2 = *reinterpret_cast<const u32x4_t*>(arow + 64);
@@ -74,7 +80,7 @@ __device__ __forceinline__ bf16x8_t expand8(uint32_t sel_lo, uint32_t sel_hi, ui
 }
 
 // One 16-row tile of a chunk: its three code dwords, its four scale bytes, the four activation fragments.
-__device__ __forceinline__ void compute_tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const Chunk& ch, f32x4_t& acc,
+__device__ __forceinline__ void compute_tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const Rows& ch, f32x4_t& acc,
                                              uint32_t lut_lo, uint32_t lut_hi) {
   uint32_t sel[8];
   w3_selectors(q0, q1, q2, sel);
@@ -91,41 +97,47 @@ __device__ __forceinline__ void compute_tile(uint32_t q0, uint32_t q1, uint32_t 
   acc.w = fmaf(p3.w, s3, fmaf(p2.w, s2, fmaf(p1.w, s1, fmaf(p0.w, s0, acc.w))));
 }
 
-__device__ __forceinline__ void compute_chunk(const Chunk& ch, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, uint32_t lut_lo,
-                                              uint32_t lut_hi) {
-  compute_tile(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, ch, acc0, lut_lo, lut_hi);
-  compute_tile(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, ch, acc1, lut_lo, lut_hi);
-  compute_tile(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, ch, acc2, lut_lo, lut_hi);
-  compute_tile(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, ch, acc3, lut_lo, lut_hi);
+__device__ __forceinline__ void compute_chunk(const Chunk& ch, const Rows& rows, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3,
+                                              uint32_t lut_lo, uint32_t lut_hi) {
+  compute_tile(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, rows, acc0, lut_lo, lut_hi);
+  compute_tile(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, rows, acc1, lut_lo, lut_hi);
+  compute_tile(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, rows, acc2, lut_lo, lut_hi);
+  compute_tile(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, rows, acc3, lut_lo, lut_hi);
 }
 
-__device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
+// The epilogue's roundings use the hardware FP32 -> BF16 conversion (round to nearest even).
+__device__ __forceinline__ uint16_t bf16_of(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+__device__ __forceinline__ float through_bf16(float f) { return (float)(__bf16)f; }
+
+// silu with the fast exponential and division: the result is rounded to BF16 right after (8 significant bits).
+__device__ __forceinline__ float silu(float g) { return __fdividef(g, 1.0f + __expf(-g)); }
 
 // One output element (or, gated, one up/gate pair) of the 64-row block: row tile `t` (gated: pair index), accumulator
 // register r of lane (q, r16); v0 / v1 are the K-complete sums before the row scale.
 template <int EPI>
 __device__ __forceinline__ void emit(const StreamParams& p, const float* rs, int nb, int p0, int rows, int t, int r, int q, int r16,
                                      float v0, float v1) {
+  if (r >= rows) return;    // wave-uniform: this accumulator register holds no row of the slot in any lane
   const int i = 4 * q + r;  // activation row of the slot held by this accumulator register
   if (i >= rows) return;
   const int64_t pos = p0 + i;
   if (EPI == EPI_FC1_GATED) {
     const int n_up = nb * 64 + 32 * t + r16;
-    const float up = round_bf16(v0 * rs[n_up]);
-    const float gate = round_bf16(v1 * rs[n_up + 16]);
-    reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = f32_to_bf16_bits(silu(gate) * up);
+    const float up = through_bf16(v0 * rs[n_up]);
+    const float gate = through_bf16(v1 * rs[n_up + 16]);
+    reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = bf16_of(silu(gate) * up);
   } else {
     const int n = nb * 64 + 16 * t + r16;
     const float y = v0 * rs[n];
     if (EPI == EPI_FC1_RELU2) {
-      const float h = fmaxf(round_bf16(y), 0.f);
-      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = f32_to_bf16_bits(h * h);
+      const float h = fmaxf(through_bf16(y), 0.f);
+      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(h * h);
     } else if (EPI == EPI_DENSE) {
-      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = f32_to_bf16_bits(y);
+      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(y);
     } else {
       const int64_t pair = p.order[pos];
       if (p.out_bf16) {
-        reinterpret_cast<uint16_t*>(p.out)[pair * p.out_stride + n] = f32_to_bf16_bits(y);
+        reinterpret_cast<uint16_t*>(p.out)[pair * p.out_stride + n] = bf16_of(y);
       } else {
         reinterpret_cast<float*>(p.out)[pair * p.out_stride + n] = y;
       }
@@ -133,65 +145,55 @@ __device__ __forceinline__ void emit(const StreamParams& p, const float* rs, int
   }
 }
 
+// What a workgroup needs to know about its slot (up to 16 activation rows of one expert, or of the dense matrix).
+struct Slot {
+  int p0, rows;        // first row (sorted position) and number of rows
+  const uint8_t* w;    // the expert's tile-layout matrix
+  const float* rs;     // its row scales
+  uint32_t lut_lo, lut_hi;
+};
+
 template <int EPI>
-__global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
-  extern __shared__ float partial[];  // [wave][tile][register][lane], only when ks > 1
+__device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
+  Slot s;
+  int expert = 0;
+  if (EPI == EPI_DENSE) {
+    s.p0 = slot * ROWS_PER_SLOT;
+    s.rows = min(ROWS_PER_SLOT, p.m - s.p0);
+  } else {
+    expert = p.plan[PLAN_HEADER + 4 * slot];
+    s.p0 = p.plan[PLAN_HEADER + 4 * slot + 1];
+    s.rows = p.plan[PLAN_HEADER + 4 * slot + 2];
+  }
+  s.w = expert < 0 ? p.w_shared : p.w + (int64_t)expert * p.expert_bytes;
+  s.rs = expert < 0 ? p.rows_shared : p.rows + (int64_t)expert * p.expert_rows;
+  s.lut_lo = expert < 0 ? p.lut_lo_shared : p.lut_lo;
+  s.lut_hi = expert < 0 ? p.lut_hi_shared : p.lut_hi;
+  return s;
+}
+
+// The activation row this lane feeds to the MFMA A operand (row r16 of the slot, columns from 8 q). Lanes past the
+// slot's last row read that last row again: their MFMA output rows are never stored.
+template <int EPI>
+__device__ __forceinline__ const uint16_t* activation_row(const StreamParams& p, const Slot& s, int q, int r16) {
+  int64_t arow = s.p0 + min(r16, s.rows - 1);
+  if (EPI == EPI_FC1_GATED || EPI == EPI_FC1_RELU2) {
+    const int pair = p.order[arow];
+    arow = pair < p.pairs ? pair / p.topk : pair - p.pairs;
+  }
+  return p.a + arow * p.a_stride + 8 * q;
+}
+
+// The end of a 64-row block: K-complete sums straight from the registers (ks == 1), or the K split's partial sums
+// exchanged through LDS (`partial`: 4 KB per wavefront) and added in split order, then the epilogue. With ks > 1 every
+// wavefront of the workgroup must call it (one workgroup barrier).
+template <int EPI>
+__device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& sl, int nb, bool active, int ks, int nbi, float* partial,
+                                             const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2, const f32x4_t& acc3) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q = lane >> 4, r16 = lane & 15;
-  const int ks = wave % p.ks, nbi = wave / p.ks;
-  const int nb = blockIdx.x * p.nbw + nbi;
-  const int slot = blockIdx.y;
-  int expert = 0, p0, rows;
-  if (EPI == EPI_DENSE) {
-    p0 = slot * ROWS_PER_SLOT;
-    rows = min(ROWS_PER_SLOT, p.m - p0);
-  } else {
-    if (slot >= p.plan[0]) return;  // the whole workgroup leaves
-    expert = p.plan[PLAN_HEADER + 4 * slot];
-    p0 = p.plan[PLAN_HEADER + 4 * slot + 1];
-    rows = p.plan[PLAN_HEADER + 4 * slot + 2];
-  }
-  const bool active = nb < p.n_blocks;
-  const uint8_t* w = expert < 0 ? p.w_shared : p.w + (int64_t)expert * p.expert_bytes;
-  const float* rs = expert < 0 ? p.rows_shared : p.rows + (int64_t)expert * p.expert_rows;
-  const uint32_t lut_lo = expert < 0 ? p.lut_lo_shared : p.lut_lo, lut_hi = expert < 0 ? p.lut_hi_shared : p.lut_hi;
-
-  f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
-
-  if (active) {
-    const int c0 = (int)((int64_t)ks * p.chunks / p.ks), c1 = (int)((int64_t)(ks + 1) * p.chunks / p.ks);
-    // lanes past the slot's last row read that last row again: their MFMA output rows are never stored
-    int64_t arow = p0 + min(r16, rows - 1);
-    if (EPI == EPI_FC1_GATED || EPI == EPI_FC1_RELU2) {
-      const int pair = p.order[arow];
-      arow = pair < p.pairs ? pair / p.topk : pair - p.pairs;
-    }
-    const uint16_t* aptr = p.a + arow * p.a_stride + 8 * q + (int64_t)c0 * 128;
-    const uint8_t* blk = w + ((int64_t)nb * p.chunks + c0) * W3_BLOCK_BYTES;
-    if (c0 < c1) {
-      // two chunk buffers in ping-pong: the next block's loads are in flight while this one is expanded
-      Chunk even, odd;
-      load_chunk(even, blk, aptr, lane, r16);
-      int left = c1 - c0 - 1;  // chunks not yet requested
-      while (left >= 2) {
-        load_chunk(odd, blk + W3_BLOCK_BYTES, aptr + 128, lane, r16);
-        compute_chunk(even, acc0, acc1, acc2, acc3, lut_lo, lut_hi);
-        blk += 2 * W3_BLOCK_BYTES;
-        aptr += 256;
-        load_chunk(even, blk, aptr, lane, r16);
-        compute_chunk(odd, acc0, acc1, acc2, acc3, lut_lo, lut_hi);
-        left -= 2;
-      }
-      if (left == 1) {
-        load_chunk(odd, blk + W3_BLOCK_BYTES, aptr + 128, lane, r16);
-        compute_chunk(even, acc0, acc1, acc2, acc3, lut_lo, lut_hi);
-        compute_chunk(odd, acc0, acc1, acc2, acc3, lut_lo, lut_hi);
-      } else {
-        compute_chunk(even, acc0, acc1, acc2, acc3, lut_lo, lut_hi);
-      }
-    }
-  }
-
+  const int p0 = sl.p0, rows = sl.rows;
+  const float* rs = sl.rs;
   if (p.ks == 1) {
     if (!active) return;
     if (EPI == EPI_FC1_GATED) {
@@ -215,8 +217,6 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
     }
     return;
   }
-
-  // K split across the wavefronts of the workgroup: partials through LDS, summed in split order.
   float* mine = partial + (int64_t)wave * 1024;
   {
     const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
@@ -234,6 +234,7 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   if (EPI == EPI_FC1_GATED) {
     for (int idx = ks; idx < 8; idx += p.ks) {
       const int t = idx >> 2, r = idx & 3;
+      if (r >= rows) continue;
       float up = 0.f, gate = 0.f;
       for (int s = 0; s < p.ks; s++) {
         up += first[s * 1024 + ((2 * t) * 4 + r) * 64 + lane];
@@ -244,11 +245,59 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   } else {
     for (int idx = ks; idx < 16; idx += p.ks) {
       const int t = idx >> 2, r = idx & 3;
+      if (r >= rows) continue;
       float v = 0.f;
       for (int s = 0; s < p.ks; s++) v += first[s * 1024 + (t * 4 + r) * 64 + lane];
       emit<EPI>(p, rs, nb, p0, rows, t, r, q, r16, v, 0.f);
     }
   }
+}
+
+// General kernel, any K: one workgroup per (run of p.nbw 64-row blocks, slot), K split p.ks ways across its wavefronts.
+// Weights and activations of chunk i + 1 are requested together before chunk i is expanded (two register buffers).
+template <int EPI>
+__global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
+  extern __shared__ float partial[];
+  if (EPI != EPI_DENSE && (int)blockIdx.y >= p.plan[0]) return;  // a slot the plan did not fill: the whole workgroup leaves
+  const Slot sl = slot_of<EPI>(p, blockIdx.y);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int ks = wave % p.ks, nbi = wave / p.ks;
+  const int nb = blockIdx.x * p.nbw + nbi;
+  const bool active = nb < p.n_blocks;
+  f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
+  if (active) {
+    const int c0 = (int)((int64_t)ks * p.chunks / p.ks), c1 = (int)((int64_t)(ks + 1) * p.chunks / p.ks);
+    const uint8_t* blk = sl.w + ((int64_t)nb * p.chunks + c0) * W3_BLOCK_BYTES;
+    if (c0 < c1) {
+      Chunk we, wo;
+      Rows ae, ao;
+      load_chunk(we, blk, lane, r16);
+      const uint16_t* aptr = activation_row<EPI>(p, sl, q, r16) + (int64_t)c0 * 128;
+      load_rows(ae, aptr);
+      int left = c1 - c0 - 1;  // chunks not yet requested
+      while (left >= 2) {
+        load_chunk(wo, blk + W3_BLOCK_BYTES, lane, r16);
+        load_rows(ao, aptr + 128);
+        compute_chunk(we, ae, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+        blk += 2 * W3_BLOCK_BYTES;
+        aptr += 256;
+        load_chunk(we, blk, lane, r16);
+        load_rows(ae, aptr);
+        compute_chunk(wo, ao, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+        left -= 2;
+      }
+      if (left == 1) {
+        load_chunk(wo, blk + W3_BLOCK_BYTES, lane, r16);
+        load_rows(ao, aptr + 128);
+        compute_chunk(we, ae, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+        compute_chunk(wo, ao, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+      } else {
+        compute_chunk(we, ae, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+      }
+    }
+  }
+  finish_block<EPI>(p, sl, nb, active, ks, nbi, partial, acc0, acc1, acc2, acc3);
 }
 
 // ---------------------------------------------------------------------------------------------------- expert plan
@@ -262,29 +311,45 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
 constexpr int PLAN_THREADS = 1024;
 constexpr int PLAN_WAVES = PLAN_THREADS / 64;
 
-__device__ __forceinline__ int block_exclusive_scan(int v, int* scratch /* PLAN_WAVES + 1 ints */, int* total) {
+struct Scan3 {
+  int a, b, c;
+};
+
+// Exclusive scan of three integers per thread over the workgroup at once; `total` receives the three sums.
+__device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 3 * (PLAN_WAVES + 1) ints */, Scan3* total) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int inc = v;
+  Scan3 inc = v;
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) {
-    const int o = __shfl_up(inc, d);
-    if (lane >= d) inc += o;
+    const int oa = __shfl_up(inc.a, d), ob = __shfl_up(inc.b, d), oc = __shfl_up(inc.c, d);
+    if (lane >= d) {
+      inc.a += oa;
+      inc.b += ob;
+      inc.c += oc;
+    }
   }
   __syncthreads();  // scratch may still be read from a previous scan
-  if (lane == 63) scratch[wave] = inc;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int wv = 0; wv < PLAN_WAVES; wv++) {
-      const int c = scratch[wv];
-      scratch[wv] = run;
-      run += c;
-    }
-    scratch[PLAN_WAVES] = run;
+  if (lane == 63) {
+    scratch[wave] = inc.a;
+    scratch[PLAN_WAVES + 1 + wave] = inc.b;
+    scratch[2 * (PLAN_WAVES + 1) + wave] = inc.c;
   }
   __syncthreads();
-  *total = scratch[PLAN_WAVES];
-  return scratch[wave] + inc - v;
+  if (threadIdx.x < 3) {
+    int* row = scratch + threadIdx.x * (PLAN_WAVES + 1);
+    int run = 0;
+    for (int wv = 0; wv < PLAN_WAVES; wv++) {
+      const int c = row[wv];
+      row[wv] = run;
+      run += c;
+    }
+    row[PLAN_WAVES] = run;
+  }
+  __syncthreads();
+  total->a = scratch[PLAN_WAVES];
+  total->b = scratch[2 * PLAN_WAVES + 1];
+  total->c = scratch[3 * PLAN_WAVES + 2];
+  return Scan3{scratch[wave] + inc.a - v.a, scratch[PLAN_WAVES + 1 + wave] + inc.b - v.b, scratch[2 * (PLAN_WAVES + 1) + wave] + inc.c - v.c};
 }
 
 __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* __restrict__ ids, int pairs, int e_lo, int e_n,
@@ -292,7 +357,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* _
   extern __shared__ int lds[];
   int* seg_count = lds;                         // [PLAN_WAVES][e_n]: pairs of expert e in segment w, then running positions
   int* start = lds + PLAN_WAVES * e_n;          // [e_n]: first sorted position of expert e
-  int* scratch = start + e_n;                   // [PLAN_WAVES + 1]
+  int* scratch = start + e_n;                   // [3 * (PLAN_WAVES + 1)]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int i = threadIdx.x; i < PLAN_WAVES * e_n; i += PLAN_THREADS) seg_count[i] = 0;
   __syncthreads();
@@ -311,12 +376,11 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* _
     int count = 0;
     if (e < e_n)
       for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
-    int tot_count, tot_distinct, tot_slots;
-    const int my_start = kept + block_exclusive_scan(count, scratch, &tot_count);
     const int my_slots = (count + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
-    const int my_distinct = distinct + block_exclusive_scan(count > 0 ? 1 : 0, scratch, &tot_distinct);
-    const int my_slot = slots + block_exclusive_scan(my_slots, scratch, &tot_slots);
-    (void)my_distinct;
+    Scan3 tot;
+    const Scan3 at = block_exclusive_scan3(Scan3{count, count > 0 ? 1 : 0, my_slots}, scratch, &tot);
+    const int my_start = kept + at.a, my_slot = slots + at.c;
+    const int tot_count = tot.a, tot_distinct = tot.b, tot_slots = tot.c;
     if (e < e_n) {
       start[e] = my_start;
       for (int s = 0; s < my_slots; s++) {
@@ -401,6 +465,9 @@ struct CombineParams {
   uint16_t* out;
 };
 
+constexpr int COMBINE_SPAN = 512;  // columns per workgroup (two per thread)
+constexpr int COMBINE_MAX_TOPK = 32;
+
 __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
   __shared__ float red[4];
   const int r = blockIdx.x;
@@ -415,58 +482,95 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
     dot = (red[0] + red[1]) + (red[2] + red[3]);
     g = 1.0f / (1.0f + expf(-dot));
   }
-  for (int c = blockIdx.y * 1024 + threadIdx.x; c < min(p.h, (int)(blockIdx.y + 1) * 1024); c += 256) {
-    float v = 0.f;
-    for (int s = 0; s < p.topk; s++) {
+  const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
+  if (c >= p.h) return;
+  float v0 = 0.f, v1 = 0.f;
+  // every slot's pair is read (so the loads are all in flight together) and a dropped slot contributes fma(0, 0, v)
+  for (int s0 = 0; s0 < p.topk; s0 += 8) {
+    float y0[8], y1[8], w[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int s = min(s0 + j, p.topk - 1);
       const int e = p.ids[r * p.topk + s] - p.e_lo;
-      if (e < 0 || e >= p.e_n) continue;
+      const bool keep = s0 + j < p.topk && e >= 0 && e < p.e_n;
       const int64_t at = ((int64_t)r * p.topk + s) * p.h + c;
-      const float y = p.pairs_bf16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.pairs)[at]) : reinterpret_cast<const float*>(p.pairs)[at];
-      v = fmaf(p.weights[r * p.topk + s], y, v);
+      float a, b;
+      if (p.pairs_bf16) {
+        const uint32_t two = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.pairs) + at);
+        a = __uint_as_float(two << 16);
+        b = __uint_as_float(two & 0xffff0000u);
+      } else {
+        const float2 two = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.pairs) + at);
+        a = two.x;
+        b = two.y;
+      }
+      y0[j] = keep ? a : 0.f;
+      y1[j] = keep ? b : 0.f;
+      w[j] = keep ? p.weights[r * p.topk + s] : 0.f;
     }
-    float o = v;
-    if (p.shared) {
-      const int64_t at = (int64_t)r * p.shared_stride + c;
-      const float s = p.shared_f32 ? round_bf16(reinterpret_cast<const float*>(p.shared)[at]) : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.shared)[at]);
-      o = round_bf16(v) + g * s;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      v0 = fmaf(w[j], y0[j], v0);
+      v1 = fmaf(w[j], y1[j], v1);
     }
-    p.out[(int64_t)r * p.h + c] = f32_to_bf16_bits(o);
   }
+  if (p.shared) {
+    const int64_t at = (int64_t)r * p.shared_stride + c;
+    float s0, s1;
+    if (p.shared_f32) {
+      const float2 two = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.shared) + at);
+      s0 = round_bf16(two.x);
+      s1 = round_bf16(two.y);
+    } else {
+      const uint32_t two = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.shared) + at);
+      s0 = __uint_as_float(two << 16);
+      s1 = __uint_as_float(two & 0xffff0000u);
+    }
+    v0 = round_bf16(v0) + g * s0;
+    v1 = round_bf16(v1) + g * s1;
+  }
+  *reinterpret_cast<uint32_t*>(p.out + (int64_t)r * p.h + c) = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
 }
 
 // ---------------------------------------------------------------------------------------------------- routing
 // Softmax top-k (hibana/kernels/flashnext_fused.py:278-319 of the reference): one wavefront per row.
+constexpr int ROUTE_PER_LANE = 16;  // up to 1024 experts: lane l holds experts l, l + 64, ...
+
 __global__ __launch_bounds__(64) void route_softmax_topk_kernel(const float* __restrict__ logits, int e, int k, int32_t* __restrict__ ids,
                                                                 float* __restrict__ weights) {
-  extern __shared__ float prob[];
   const int r = blockIdx.x, lane = threadIdx.x;
   const float* row = logits + (int64_t)r * e;
+  float v[ROUTE_PER_LANE];
   float mx = -INFINITY;
-  for (int i = lane; i < e; i += 64) mx = fmaxf(mx, row[i]);
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; j++) {
+    const int i = lane + 64 * j;
+    v[j] = i < e ? row[i] : -INFINITY;
+    mx = fmaxf(mx, v[j]);
+  }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
   float sum = 0.f;
-  for (int i = lane; i < e; i += 64) {
-    const float pr = expf(row[i] - mx);
-    prob[i] = pr;
-    sum += pr;
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; j++) {
+    v[j] = lane + 64 * j < e ? expf(v[j] - mx) : -1.f;
+    sum += fmaxf(v[j], 0.f);
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d);
-  __syncthreads();
-  for (int i = lane; i < e; i += 64) prob[i] = prob[i] / sum;
-  __syncthreads();
-  float total = 0.f;
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; j++) v[j] = v[j] >= 0.f ? v[j] / sum : -1.f;
+  float total = 0.f, mine = 0.f;
+  int mine_id = 0;
   for (int s = 0; s < k; s++) {
     float best = -1.f;
     int at = 0x7fffffff;
-    for (int i = lane; i < e; i += 64) {
-      const float v = prob[i];
-      if (v > best) {
-        best = v;
-        at = i;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; j++)
+      if (v[j] > best) {  // ascending index within the lane: the first of equals stays
+        best = v[j];
+        at = lane + 64 * j;
       }
-    }
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
       const float ob = __shfl_xor(best, d);
@@ -476,16 +580,21 @@ __global__ __launch_bounds__(64) void route_softmax_topk_kernel(const float* __r
         at = oa;
       }
     }
-    if (lane == 0) {
-      ids[r * k + s] = at;
-      weights[r * k + s] = best;
-    }
     total += best;
-    __syncthreads();
-    if (lane == 0) prob[at] = -1.f;
-    __syncthreads();
+    if (lane == s) {
+      mine = best;
+      mine_id = at;
+    }
+    if ((at & 63) == lane) {
+#pragma unroll
+      for (int j = 0; j < ROUTE_PER_LANE; j++)
+        if (j == (at >> 6)) v[j] = -1.f;
+    }
   }
-  if (lane < k) weights[r * k + lane] = weights[r * k + lane] / total;
+  if (lane < k) {
+    ids[r * k + lane] = mine_id;
+    weights[r * k + lane] = mine / total;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------- host side
@@ -501,29 +610,36 @@ struct Tuning {
 };
 static Tuning g_tune;
 
-static int pow2_floor(int v) {
-  int p = 1;
-  while (2 * p <= v) p *= 2;
-  return p;
-}
-
-// Wavefronts per workgroup: K is split until a launch has about `want` wavefronts, keeping at least two chunks per
+// Wavefronts per workgroup: K is split until a launch has about `want` wavefronts, keeping at least four chunks per
 // wavefront; what is left of a 4-wavefront workgroup takes neighbouring 64-row blocks.
 static void pick_shape(int n_blocks, int chunks, int64_t slots, int want, int* ks, int* nbw) {
   int k = 1;
-  while (k < 16 && (int64_t)n_blocks * slots * k < want && chunks / (2 * k) >= 2) k *= 2;
+  while (k < 16 && (int64_t)n_blocks * slots * k < want && chunks / (2 * k) >= 4) k *= 2;
   int b = k >= 4 ? 1 : 4 / k;
   while (b > 1 && n_blocks % b) b /= 2;
   *ks = k;
   *nbw = b;
 }
 
+// Launch one W3 stream. `busy_slots` is the caller's estimate of the slots that will have rows (the grid covers
+// `slots`, the upper bound); K is split until the launch has a few thousand wavefronts.
+struct Launch {
+  int ks, nbw;  // 0: chosen here
+};
+
 template <int EPI>
-static void launch_stream(StreamParams& p, int64_t slots, hipStream_t stream) {
+static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Launch want, hipStream_t stream) {
+  pick_shape(p.n_blocks, p.chunks, busy_slots, 8192, &p.ks, &p.nbw);
+  if (want.ks) {
+    p.ks = want.ks;
+    if (!want.nbw) p.nbw = 1;
+  }
+  if (want.nbw) p.nbw = want.nbw;
+  if (p.ks * p.nbw > 16 || p.ks > p.chunks) return HB_EINVAL;
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
-  const size_t lds = p.ks > 1 ? (size_t)waves * 4096 : 0;
-  hipLaunchKernelGGL(w3_stream_kernel<EPI>, grid, dim3(64 * waves), lds, stream, p);
+  hipLaunchKernelGGL(w3_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
+  return HB_OK;
 }
 
 }  // namespace hb
@@ -564,11 +680,7 @@ extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* 
   p.out_stride = n;
   const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
   if (slots > 65535) return HB_EINVAL;
-  pick_shape(p.n_blocks, p.chunks, slots, 2048, &p.ks, &p.nbw);
-  if (g_tune.w3_ksplit) p.ks = g_tune.w3_ksplit;
-  if (g_tune.w3_nbw) p.nbw = g_tune.w3_nbw;
-  if (p.ks * p.nbw > 16 || p.ks > p.chunks) return HB_EINVAL;
-  launch_stream<EPI_DENSE>(p, slots, as_stream(stream));
+  if (int e = launch_stream<EPI_DENSE>(p, slots, slots, Launch{g_tune.w3_ksplit, g_tune.w3_nbw}, as_stream(stream))) return e;
   return launch_status();
 }
 
@@ -624,8 +736,8 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   const int shared_rows = shared ? m : 0;
   const int64_t slots = max_slots(pairs, ex->experts, shared_rows);
   if (slots > 65535 || pairs > 0x3fffffff) return HB_EINVAL;
-  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * ex->experts + PLAN_WAVES + 1) * sizeof(int);
-  if (plan_lds > 160 * 1024) return HB_EINVAL;
+  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * ex->experts + 3 * (PLAN_WAVES + 1)) * sizeof(int);
+  if (plan_lds > 64 * 1024) return HB_EINVAL;
   mark(stream);
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, ex->base, ex->experts, shared_rows,
                      ws.plan, ws.order);
@@ -655,46 +767,36 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   p.pairs = (int)pairs;
   p.out = ws.h;
   p.out_stride = ex->inter;
-  pick_shape(p.n_blocks, p.chunks, est, 4096, &p.ks, &p.nbw);
-  if (g_tune.moe_fc1_ksplit) p.ks = g_tune.moe_fc1_ksplit;
-  if (g_tune.moe_fc1_nbw) p.nbw = g_tune.moe_fc1_nbw;
-  if (p.ks * p.nbw > 16 || p.ks > p.chunks) return HB_EINVAL;
-  if (ex->gated) {
-    launch_stream<EPI_FC1_GATED>(p, slots, stream);
-  } else {
-    launch_stream<EPI_FC1_RELU2>(p, slots, stream);
-  }
-  mark(stream);
-  p.w = static_cast<const uint8_t*>(ex->fc2);
-  p.expert_bytes = (int64_t)hb_w3_tiled_bytes(ex->hidden_out, ex->inter);
-  p.rows = ex->fc2_rows;
-  p.expert_rows = ex->hidden_out;
-  p.lut_lo = (uint32_t)((uint64_t)ex->fc2_lut & 0xffffffffu);
-  p.lut_hi = (uint32_t)((uint64_t)ex->fc2_lut >> 32);
+  StreamParams f2 = p;
+  f2.w = static_cast<const uint8_t*>(ex->fc2);
+  f2.expert_bytes = (int64_t)hb_w3_tiled_bytes(ex->hidden_out, ex->inter);
+  f2.rows = ex->fc2_rows;
+  f2.expert_rows = ex->hidden_out;
+  f2.lut_lo = (uint32_t)((uint64_t)ex->fc2_lut & 0xffffffffu);
+  f2.lut_hi = (uint32_t)((uint64_t)ex->fc2_lut >> 32);
   if (shared) {
-    p.w_shared = static_cast<const uint8_t*>(shared->fc2);
-    p.rows_shared = shared->fc2_rows;
-    p.lut_lo_shared = (uint32_t)((uint64_t)shared->fc2_lut & 0xffffffffu);
-    p.lut_hi_shared = (uint32_t)((uint64_t)shared->fc2_lut >> 32);
+    f2.w_shared = static_cast<const uint8_t*>(shared->fc2);
+    f2.rows_shared = shared->fc2_rows;
+    f2.lut_lo_shared = (uint32_t)((uint64_t)shared->fc2_lut & 0xffffffffu);
+    f2.lut_hi_shared = (uint32_t)((uint64_t)shared->fc2_lut >> 32);
   }
-  p.n_blocks = ex->hidden_out / W3_BLOCK_ROWS;
-  p.chunks = ex->inter / W3_CHUNK;
-  p.a = ws.h;
-  p.a_stride = ex->inter;
-  p.out = out_pairs;
-  p.out_stride = ex->hidden_out;
-  p.out_bf16 = pairs_bf16;
-  pick_shape(p.n_blocks, p.chunks, est, 4096, &p.ks, &p.nbw);
-  if (g_tune.moe_fc2_ksplit) p.ks = g_tune.moe_fc2_ksplit;
-  if (g_tune.moe_fc2_nbw) p.nbw = g_tune.moe_fc2_nbw;
-  if (p.ks * p.nbw > 16 || p.ks > p.chunks) return HB_EINVAL;
-  launch_stream<EPI_FC2>(p, slots, stream);
+  f2.n_blocks = ex->hidden_out / W3_BLOCK_ROWS;
+  f2.chunks = ex->inter / W3_CHUNK;
+  f2.a = ws.h;
+  f2.a_stride = ex->inter;
+  f2.out = out_pairs;
+  f2.out_stride = ex->hidden_out;
+  f2.out_bf16 = pairs_bf16;
+  const Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
+  if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) return e;
+  mark(stream);
+  if (int e = launch_stream<EPI_FC2>(f2, slots, est, l2, stream)) return e;
   mark(stream);
   return launch_status();
 }
 
 void launch_combine(const CombineParams& c, hipStream_t stream) {
-  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)c.m, (unsigned)((c.h + 1023) / 1024)), dim3(256), 0, stream, c);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)c.m, (unsigned)((c.h + COMBINE_SPAN - 1) / COMBINE_SPAN)), dim3(256), 0, stream, c);
   mark(stream);
 }
 
@@ -772,7 +874,7 @@ extern "C" int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int
                                     void* stream) {
   if (!pairs || !ids || !weights || !out) return HB_ENULL;
   if (gate_vec && shared && !x) return HB_ENULL;
-  if (m <= 0 || topk <= 0 || h <= 0) return HB_EINVAL;
+  if (m <= 0 || topk <= 0 || h <= 0 || h % 2) return HB_EINVAL;
   CombineParams c{};
   c.pairs = pairs;
   c.pairs_bf16 = pairs_bf16;
@@ -795,9 +897,8 @@ extern "C" int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int
 
 extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, int32_t* ids, float* weights, void* stream) {
   if (!logits || !ids || !weights) return HB_ENULL;
-  if (m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || (size_t)e * 4 > 64 * 1024) return HB_EINVAL;
-  hipLaunchKernelGGL(route_softmax_topk_kernel, dim3((unsigned)m), dim3(64), (size_t)e * sizeof(float), as_stream(stream), logits, e, k, ids,
-                     weights);
+  if (m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE) return HB_EINVAL;
+  hipLaunchKernelGGL(route_softmax_topk_kernel, dim3((unsigned)m), dim3(64), 0, as_stream(stream), logits, e, k, ids, weights);
   return launch_status();
 }
 

@@ -35,9 +35,8 @@ def test_every_k_split_gives_close_results_and_the_unsplit_bits_repeat():
     x = torch.randn(16, 2048, generator=torch.Generator().manual_seed(1)).bfloat16()
     want = layers.dense_ref(x, ow3.dequantize(packed))
     try:
-        for ks, nbw in ((1, 1), (1, 4), (2, 2), (4, 1), (8, 1), (16, 1), (4, 4)):
-            _lib.lib().hb_tune(b"w3_ksplit", ks)
-            _lib.lib().hb_tune(b"w3_nbw", nbw)
+        for ks, nbw in ((1, 1), (1, 4), (2, 2), (4, 1), (8, 1), (16, 1), (4, 4), (0, 0)):
+            assert _lib.lib().hb_tune(b"w3_ksplit", ks) == 0 and _lib.lib().hb_tune(b"w3_nbw", nbw) == 0
             got = w3.w3_linear(x.cuda(), dev)
             mx, nr = errors(got, want)
             assert mx < MAX_REL and nr < NORM_REL, (ks, nbw, mx, nr)
