@@ -1,0 +1,104 @@
+"""CPU checks: the C ABI library loads and exports every symbol include/hibana_hip.h declares, argument validation
+that needs no GPU, and the host-side logic that mirrors the reference interface."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from hibana_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "hibana_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hb_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared()
+    assert len(names) >= 20
+    handle = C.CDLL(str(_lib.LIBRARY))
+    for name in names:
+        assert hasattr(handle, name), name
+    assert sorted(_lib.SIGNATURES) == names  # the Python binding covers the header, nothing more, nothing less
+
+
+def test_validation_without_a_gpu():
+    lib = _lib.lib()
+    assert lib.hb_version() >= 1000
+    assert lib.hb_error_string(0) == b"ok" and b"workspace" in lib.hb_error_string(_lib.HB_EWORKSPACE)
+    assert lib.hb_w3_tiled_bytes(1024, 2048) == 1024 * 2048 * 3 // 8 + 1024 * 2048 // 32
+    assert lib.hb_w3_tiled_bytes(96, 2048) == 0 and lib.hb_w3_tiled_bytes(128, 100) == 0
+    assert lib.hb_nvfp4_tiled_bytes(128, 256) == 128 * 256 // 2 + 128 * 256 // 16
+    assert lib.hb_nvfp4_tiled_bytes(128, 64) == 0
+    assert lib.hb_tune(b"no_such_knob", 1) == _lib.HB_EINVAL and lib.hb_tune(b"w3_ksplit", 3) == _lib.HB_EINVAL
+    assert lib.hb_tune(b"w3_ksplit", 4) == 0 and lib.hb_tune(b"w3_ksplit", 0) == 0
+    assert lib.hb_w3_repack(None, None, 128, 128, 3, None, None) == _lib.HB_ENULL
+    assert lib.hb_w3_gemm(None, 1, None, None, 0, 128, 128, None, None) == _lib.HB_ENULL
+    assert lib.hb_nvfp4_gemm(None, 1, None, 1.0, 128, 128, 0, None, None) == _lib.HB_ENULL
+    assert lib.hb_w3_moe_workspace_bytes(4, 2, None, 0) == 0
+    ex = _lib.HbW3Experts(1, 1, 1, 1, 0, 0, 8, 0, 256, 128, 256, 1)
+    need = lib.hb_w3_moe_workspace_bytes(32, 10, C.byref(ex), 1)
+    assert need >= (320 + 32) * (128 * 2 + 256 * 4)
+    bad = _lib.HbW3Experts(1, 1, 1, 1, 0, 0, 8, 0, 200, 128, 256, 1)  # hidden not a multiple of 128
+    assert lib.hb_w3_moe_workspace_bytes(32, 10, C.byref(bad), 1) == 0
+    assert lib.hb_w3_moe(C.byref(bad), None, None, None, 1, 1, 0, None, None, 0, None) == _lib.HB_EINVAL
+    with pytest.raises(ValueError):
+        _lib.check(_lib.HB_EINVAL, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.HB_ELAUNCH, "x")
+
+
+def test_host_logic_mirrors_the_reference_interface(monkeypatch):
+    from hibana_amd.kernels import ops, w3, w3_moe
+    from hibana_amd.weights import modelopt
+    from hibana_amd.weights.linear import Linear
+    from oracle import layers, nvfp4_format as onv, w3_format as ow3
+    assert w3.MAX_ROWS == 128 and w3.GROUP == 32 and w3.CHUNK == 128 and w3.DEFAULT_CODEBOOK == "lloyd"
+    assert w3.CODEBOOKS == ow3.CODEBOOKS and w3_moe.EXPERTS == 512 and w3_moe.ORDER_IN_KERNEL == 640 and w3_moe.WIDE_ROWS == 1024
+    for name, levels in w3.CODEBOOKS.items():
+        assert w3.lut_of(levels) == ow3.lut_of(levels), name
+    with pytest.raises(ValueError):
+        w3._codebook((-3.5, -2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 3.3))
+    with pytest.raises(ValueError):
+        w3._codebook((1.0, 0.5, 2.0, 3.0))
+    assert w3_moe.fc1_order(128).tolist() == layers.fc1_order(128).tolist()
+    assert w3.pair_order(512, 64).tolist() == ow3.pair_order(512, 64).tolist() == modelopt.pair_order(512, 64).tolist()
+    s = torch.arange(130 * 6, dtype=torch.float32).reshape(130, 6)
+    sw = modelopt.swizzle_block_scales(s)
+    assert sw.shape == (256, 8) and (sw.numpy() == onv.swizzle_block_scales(s.numpy())).all()
+    assert torch.equal(modelopt.unswizzle_block_scales(sw, 130, 6), s)
+    gu = torch.randn(3, 256)
+    assert torch.allclose(ops.silu_and_mul(gu), layers.silu_and_mul(gu)) and torch.allclose(ops.silu_and_mul(gu, 64), layers.silu_and_mul(gu, 64))
+    monkeypatch.delenv("HIBANA_W3_DECODE", raising=False)
+    assert not w3.enabled()
+    monkeypatch.setenv("HIBANA_W3_DECODE", "1")
+    assert w3.enabled()
+    lin = modelopt.Nvfp4Linear(torch.zeros(128, 64, dtype=torch.uint8), torch.zeros(128, 8).to(torch.float8_e4m3fn), torch.tensor(2.0),
+                               torch.tensor(4.0), 128, 128)
+    assert isinstance(lin, Linear) and lin.global_scale == 8.0 and lin.bytes == 128 * 64 + 128 * 8 and lin.w3 is None
+    assert not ops.w3_decode(lin, 4)
+    lin.w3 = object()
+    assert ops.w3_decode(lin, 4) and not ops.w3_decode(lin, 129) and not ops.w3_decode(lin, 4, rows=2)
+    # the ops have no CPU path: they raise rather than fall back
+    with pytest.raises(RuntimeError):
+        modelopt.unpack_fp4(torch.zeros(64, 64, dtype=torch.uint8), torch.zeros(64, 8, dtype=torch.uint8))
+    with pytest.raises(RuntimeError):
+        ops.route_topk(torch.zeros(2, 8), 2)
+    with pytest.raises(RuntimeError):
+        w3.pack_codes(torch.zeros(128, 128, dtype=torch.uint8), torch.zeros(128, 4).to(torch.float8_e4m3fn), torch.ones(128))
+    with pytest.raises(ValueError):
+        w3.pack_codes(torch.full((128, 128), 9, dtype=torch.uint8), torch.zeros(128, 4).to(torch.float8_e4m3fn), torch.ones(128))
+    with pytest.raises(NotImplementedError):
+        w3.quant_groups(torch.zeros(1, 32))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert run.returncode != 0 and "ONE GPU" in run.stderr
