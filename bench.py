@@ -15,7 +15,6 @@ from __future__ import annotations
 import argparse
 import ctypes as C
 import json
-import os
 import sys
 import time
 
@@ -53,53 +52,37 @@ class Hip:
         return ms.value
 
 
-def cpu_baseline(layer, x, ids, weights, budget_s: float = 20.0):
-    """The oracle's layer (dequantize the experts a call names + FP32 matmuls + combine) on this host's cores, on the
-    first `t` tokens of the batch, t grown until about `budget_s` of CPU work has been spent."""
+def cpu_baseline(layer, x, ids, weights, budget_s: float = 15.0):
+    """The CPU oracle's layer (oracle/c/w3_oracle.c: unpack the experts a call names from the checkpoint layout, FP32
+    matmuls, SiLU gate, combine, shared expert; OpenMP over rows) on this host's cores: whole 32-token layer calls,
+    repeated until about `budget_s` of CPU time is spent."""
     import numpy as np
     import torch
 
-    from oracle import layers
-    from oracle import w3_format as ow3
-    from hibana_amd.kernels import w3
+    from oracle import c_port
 
-    torch.set_num_threads(os.cpu_count() or 1)
     experts, shared = layer
-    inverse = np.argsort(layers.fc1_order(INTER))
 
-    def host(mat):  # the checkpoint-layout view of one matrix, as the oracle takes it
-        codes = w3.codes(mat).cpu().numpy()
-        raw = w3.scale_bytes(mat).view(torch.uint8).cpu().numpy()
-        return ow3.pack_codes(codes, raw, mat.row_scale.cpu().numpy(), mat.codebook)
+    def host(ex):
+        u32 = lambda t: t.view(torch.int32).cpu().numpy().view(np.uint32)  # noqa: E731
+        (n1, h), (_, i) = ex.shape13, ex.shape2
+        return c_port.HostExperts(u32(ex.planes13), ex.scales13.cpu().numpy(), ex.row13.cpu().numpy(), u32(ex.planes2), ex.scales2.cpu().numpy(),
+                                  ex.row2.cpu().numpy(), ex.codebook, ex.fc2_codebook, h, i, n1 == 2 * i)
 
-    fetched = {}
-
-    def fetch(e, src=experts):
-        key = (id(src), e)
-        if key not in fetched:
-            fetched[key] = (host(src.matrix(e, True)), host(src.matrix(e, False)))
-        return fetched[key]
-
-    spent, tokens, t = 0.0, 0, 1
-    xs, idn, wts = x.cpu(), ids.cpu().numpy(), weights.cpu()
-    sample = ""
-    while True:
-        rows = slice(0, t)
-        for e in np.unique(idn[rows]):
-            fetch(int(e))
-        sh = fetch(0, shared)
+    routed, sh = host(experts), host(shared)
+    xb = x.view(torch.int16).cpu().numpy().view(np.uint16)
+    idn, wn = ids.cpu().numpy(), weights.cpu().numpy()
+    out, distinct = c_port.moe_layer(routed, xb, idn, wn, sh)  # warm-up, and the result the GPU is compared with below
+    calls, spent = 0, 0.0
+    while spent < budget_s and calls < 50:
         t0 = time.perf_counter()
-        get = lambda e: (ow3.dequantize(fetch(e)[0])[inverse], ow3.dequantize(fetch(e)[1]))  # noqa: E731
-        shared_w = (ow3.dequantize(sh[0])[inverse], ow3.dequantize(sh[1]))
-        layers.moe_layer_ref(xs[rows], idn[rows], wts[rows], get, True, shared=shared_w, e_n=EXPERTS)
-        dt = time.perf_counter() - t0
-        spent += dt
-        tokens, last = t, dt
-        sample = f"first {t} of {M} tokens of one layer call ({len(np.unique(idn[rows]))} distinct experts + shared), oracle unpack + FP32 matmul"
-        if spent + 2.5 * dt > budget_s or t >= M:
-            break
-        t = min(M, 2 * t)
-    return {"value": tokens / last, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port", "sample": sample}
+        c_port.moe_layer(routed, xb, idn, wn, sh)
+        spent += time.perf_counter() - t0
+        calls += 1
+    info = {"value": M * calls / spent, "unit": "tokens/s", "cores": c_port.threads(), "kind": "port",
+            "sample": f"{calls} whole layer calls of {M} tokens on layer 0 ({distinct} distinct experts + shared): C/OpenMP oracle, "
+                      f"unpack from the checkpoint layout + FP32 matmul"}
+    return info, torch.from_numpy(out.view(np.int16).copy()).view(torch.bfloat16)
 
 
 def main() -> int:
@@ -125,8 +108,9 @@ def main() -> int:
     torch.cuda.set_device(dev)
     layers = []
     for i in range(args.layers):
-        layers.append((synthetic.w3_experts(EXPERTS, HIDDEN, INTER, True, 100 + i, dev),
-                       synthetic.w3_experts(1, HIDDEN, INTER, True, 900 + i, dev)))
+        keep = i == 0 and not args.no_cpu  # the CPU leg reads layer 0 in the checkpoint layout
+        layers.append((synthetic.w3_experts(EXPERTS, HIDDEN, INTER, True, 100 + i, dev, release=not keep),
+                       synthetic.w3_experts(1, HIDDEN, INTER, True, 900 + i, dev, release=not keep)))
     logits = [synthetic.zipf_logits(M, EXPERTS, ZIPF, 3000 + i, dev) for i in range(args.layers)]
     x = torch.randn(M, HIDDEN, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
     torch.cuda.synchronize()
@@ -178,7 +162,12 @@ def main() -> int:
     chain_gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     ids0, w0 = ops.route_topk(logits[0], TOPK)
-    cpu = None if args.no_cpu else cpu_baseline(layers[0], x, ids0, w0)
+    cpu, check = None, None
+    if not args.no_cpu:
+        cpu, want = cpu_baseline(layers[0], x, ids0, w0)
+        got = w3_moe.moe_layer(layers[0][0], x, ids0, w0, shared=layers[0][1]).float().cpu()
+        check = {"max_rel_vs_cpu_oracle": float((got - want.float()).abs().max() / want.float().abs().max()),
+                 "norm_rel_vs_cpu_oracle": float((got - want.float()).norm() / want.float().norm())}
     line = {
         "metric": "w3 MoE layer tokens/s at the verify batch (M=32), with achieved HBM GB/s",
         "value": M * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -192,6 +181,7 @@ def main() -> int:
         "layer_chain": {"algorithmic_bytes_per_step": step_bytes, "achieved_GBs": chain_gbs, "frac_of_hbm_peak": chain_gbs / HBM_PEAK_GBS,
                         "kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
         "cpu_baseline": cpu,
+        "parity": check,
     }
     print(json.dumps(line))
     return 0
