@@ -29,6 +29,7 @@ def w3_bytes(n: int, k: int) -> int:
 
 FC1_BYTES, FC2_BYTES = w3_bytes(2 * INTER, HIDDEN), w3_bytes(HIDDEN, INTER)
 EXPERT_BYTES = FC1_BYTES + FC2_BYTES  # 1 290 240
+FC1_TRAFFIC_RATIO = 1.018  # measured HBM bytes / algorithmic bytes of the fc1 launch (counter runs, see the roofline entry)
 
 
 class Hip:
@@ -92,6 +93,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--layers", type=int, default=6, help="distinct layers the steps cycle through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (a known-size "
+                    "reference for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no sharding, no collectives); run with --gpus 1", file=sys.stderr)
@@ -161,6 +164,11 @@ def main() -> int:
     step_bytes = mean([(distinct[i % args.layers] + 1) * EXPERT_BYTES + 2 * M * HIDDEN * 2 for i in range(args.steps)])
     chain_gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    if args.copy_mib:
+        src = torch.empty(args.copy_mib << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
     ids0, w0 = ops.route_topk(logits[0], TOPK)
     cpu, check = None, None
     if not args.no_cpu:
@@ -177,7 +185,10 @@ def main() -> int:
                                "top-10 Zipf(1.1) routing, SiLU-gated, codebook lloyd",
                    "layers_cycled": args.layers, "distinct_experts_per_step": mean(distinct), "timed_as": "one HIP-graph replay of all steps"},
         "roofline": {"bound": "hbm", "kernel": "w3_stream_kernel<fc1 gated>", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "launch_bytes": fc1_launch_bytes, "launch_ms": fc1_ms},
+                     "frac": achieved / HBM_PEAK_GBS,
+                     # HBM bytes a launch: the ratio of scaled FETCH_SIZE + WRITE_SIZE to the algorithmic bytes measured with
+                     # rocprofv3 --pmc on this workload (profiles/w3_moe_layer_config3_hbm_traffic.md), applied to this run's bytes
+                     "traffic": FC1_TRAFFIC_RATIO * fc1_launch_bytes, "launch_bytes": fc1_launch_bytes, "launch_ms": fc1_ms},
         "layer_chain": {"algorithmic_bytes_per_step": step_bytes, "achieved_GBs": chain_gbs, "frac_of_hbm_peak": chain_gbs / HBM_PEAK_GBS,
                         "kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
         "cpu_baseline": cpu,
