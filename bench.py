@@ -187,7 +187,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "kernel": "w3_stream_kernel<fc1 gated>", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      # HBM bytes a launch: the ratio of scaled FETCH_SIZE + WRITE_SIZE to the algorithmic bytes measured with
-                     # rocprofv3 --pmc on this workload (profiles/w3_moe_layer_config3_hbm_traffic.md), applied to this run's bytes
+                     # rocprofv3 --pmc on this workload (summary kept under profiles/), applied to this run's bytes
                      "traffic": FC1_TRAFFIC_RATIO * fc1_launch_bytes, "launch_bytes": fc1_launch_bytes, "launch_ms": fc1_ms},
         "layer_chain": {"algorithmic_bytes_per_step": step_bytes, "achieved_GBs": chain_gbs, "frac_of_hbm_peak": chain_gbs / HBM_PEAK_GBS,
                         "kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},

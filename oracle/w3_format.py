@@ -26,6 +26,10 @@ Pinned by (tests/test_oracle_w3.py):
   pack                 codes == bucketize(w / scale, mids), extremes used, error < 0.22, byte count
                        (test_w3_pack.py:34-54); 2-bit variant and fitted scales (:57-76)
   interleave_rows      interleave_rows(pack(w)) == pack(w[pair_order]) (tests/unit/test_mlp_pairs.py:27-34)
+
+PARITY UNPINNED: pack(fit_scales=True) picks, per group, the first of FIT_SCALES whose float32 squared error is strictly
+the least; the error sum's summation order differs between numpy and torch, so an exact tie could resolve differently
+from the reference. Only the reference's error bounds for the fitted variant are held (test_w3_pack.py:57-76).
 """
 from __future__ import annotations
 
