@@ -18,8 +18,15 @@ class HbW3Experts(C.Structure):
                 ("hidden", C.c_int), ("inter", C.c_int), ("hidden_out", C.c_int), ("gated", C.c_int)]
 
 
+class HbNvfp4Experts(C.Structure):
+    _fields_ = [("fc1", C.c_void_p), ("fc1_scale2", C.c_void_p), ("fc2", C.c_void_p), ("fc2_scale2", C.c_void_p),
+                ("experts", C.c_int), ("base", C.c_int), ("hidden", C.c_int), ("inter", C.c_int),
+                ("hidden_out", C.c_int), ("gated", C.c_int)]
+
+
 _P, _I, _L, _Z, _F = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 _EX = C.POINTER(HbW3Experts)
+_EX4 = C.POINTER(HbNvfp4Experts)
 # name -> (restype, argtypes): every symbol include/hibana_hip.h declares
 SIGNATURES = {
     "hb_version": (_I, []),
@@ -42,6 +49,8 @@ SIGNATURES = {
     "hb_nvfp4_repack": (_I, [_P, _P, _I, _L, _I, _P, _P]),
     "hb_nvfp4_dequant": (_I, [_P, _F, _L, _I, _P, _P]),
     "hb_nvfp4_gemm": (_I, [_P, _I, _P, _F, _I, _I, _I, _P, _P]),
+    "hb_nvfp4_moe_workspace_bytes": (_Z, [_I, _I, _EX4]),
+    "hb_nvfp4_moe": (_I, [_EX4, _P, _P, _P, _I, _I, _I, _P, _P, _Z, _P]),
 }
 
 

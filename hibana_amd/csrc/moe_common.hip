@@ -1,0 +1,402 @@
+// Kernels and host helpers shared by every routed-expert call: the expert plan, the combine, softmax top-k routing.
+#include <string.h>
+
+#include <vector>
+
+#include "stream_common.hpp"
+
+namespace hb {
+
+// ---------------------------------------------------------------------------------------------------- expert plan
+//
+// The expert-sorted pair list of a routed call (the reference's prep kernel, hibana/kernels/csrc/w3_gemm.cu:710-782):
+// distinct local experts in ascending id, each expert's pairs in ascending pair index (a stable sort), cut into slots
+// of at most 16 rows. One workgroup; any number of pairs. Integer atomics on LDS counters only (order-independent).
+//   plan[0] = slots, plan[1] = distinct experts, plan[2] = kept routed pairs,
+//   plan[16 + 4 s ..] = { local expert id (-1: the shared expert), first sorted position, rows, 0 }
+//   order[pos] = pair index (row * topk + slot; shared expert rows: pairs + row)
+constexpr int PLAN_THREADS = 1024;
+constexpr int PLAN_WAVES = PLAN_THREADS / 64;
+
+struct Scan3 {
+  int a, b, c;
+};
+
+// Exclusive scan of three integers per thread over the workgroup at once; `total` receives the three sums.
+__device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 3 * (PLAN_WAVES + 1) ints */, Scan3* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  Scan3 inc = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int oa = __shfl_up(inc.a, d), ob = __shfl_up(inc.b, d), oc = __shfl_up(inc.c, d);
+    if (lane >= d) {
+      inc.a += oa;
+      inc.b += ob;
+      inc.c += oc;
+    }
+  }
+  __syncthreads();  // scratch may still be read from a previous scan
+  if (lane == 63) {
+    scratch[wave] = inc.a;
+    scratch[PLAN_WAVES + 1 + wave] = inc.b;
+    scratch[2 * (PLAN_WAVES + 1) + wave] = inc.c;
+  }
+  __syncthreads();
+  if (threadIdx.x < 3) {
+    int* row = scratch + threadIdx.x * (PLAN_WAVES + 1);
+    int run = 0;
+    for (int wv = 0; wv < PLAN_WAVES; wv++) {
+      const int c = row[wv];
+      row[wv] = run;
+      run += c;
+    }
+    row[PLAN_WAVES] = run;
+  }
+  __syncthreads();
+  total->a = scratch[PLAN_WAVES];
+  total->b = scratch[2 * PLAN_WAVES + 1];
+  total->c = scratch[3 * PLAN_WAVES + 2];
+  return Scan3{scratch[wave] + inc.a - v.a, scratch[PLAN_WAVES + 1 + wave] + inc.b - v.b, scratch[2 * (PLAN_WAVES + 1) + wave] + inc.c - v.c};
+}
+
+__global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* __restrict__ ids, int pairs, int e_lo, int e_n,
+                                                                int shared_rows, int32_t* __restrict__ plan, int32_t* __restrict__ order) {
+  extern __shared__ int lds[];
+  int* seg_count = lds;                         // [PLAN_WAVES][e_n]: pairs of expert e in segment w, then running positions
+  int* start = lds + PLAN_WAVES * e_n;          // [e_n]: first sorted position of expert e
+  int* scratch = start + e_n;                   // [3 * (PLAN_WAVES + 1)]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < PLAN_WAVES * e_n; i += PLAN_THREADS) seg_count[i] = 0;
+  __syncthreads();
+  // segment w = pairs [w * seg, (w + 1) * seg), seg a multiple of 64
+  const int seg = ((pairs + PLAN_WAVES - 1) / PLAN_WAVES + 63) / 64 * 64;
+  const int lo = wave * seg, hi = min(pairs, lo + seg);
+  for (int i = lo + lane; i < hi; i += 64) {
+    const int e = ids[i] - e_lo;
+    if (e >= 0 && e < e_n) atomicAdd(&seg_count[wave * e_n + e], 1);
+  }
+  __syncthreads();
+  // per expert: total count, exclusive positions; slots of 16 rows
+  int kept = 0, distinct = 0, slots = 0;
+  for (int base = 0; base < e_n; base += PLAN_THREADS) {  // experts in ascending id, PLAN_THREADS at a time
+    const int e = base + threadIdx.x;
+    int count = 0;
+    if (e < e_n)
+      for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
+    const int my_slots = (count + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
+    Scan3 tot;
+    const Scan3 at = block_exclusive_scan3(Scan3{count, count > 0 ? 1 : 0, my_slots}, scratch, &tot);
+    const int my_start = kept + at.a, my_slot = slots + at.c;
+    const int tot_count = tot.a, tot_distinct = tot.b, tot_slots = tot.c;
+    if (e < e_n) {
+      start[e] = my_start;
+      for (int s = 0; s < my_slots; s++) {
+        int32_t* entry = plan + PLAN_HEADER + 4 * (my_slot + s);
+        entry[0] = e;
+        entry[1] = my_start + s * ROWS_PER_SLOT;
+        entry[2] = min(ROWS_PER_SLOT, count - s * ROWS_PER_SLOT);
+        entry[3] = 0;
+      }
+      // turn the per-segment counts into the first position of each segment's run
+      int run = my_start;
+      for (int wv = 0; wv < PLAN_WAVES; wv++) {
+        const int c = seg_count[wv * e_n + e];
+        seg_count[wv * e_n + e] = run;
+        run += c;
+      }
+    }
+    kept += tot_count;
+    distinct += tot_distinct;
+    slots += tot_slots;
+  }
+  __syncthreads();
+  // the shared expert's rows follow the routed pairs
+  const int shared_slots = (shared_rows + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
+  for (int s = threadIdx.x; s < shared_slots; s += PLAN_THREADS) {
+    int32_t* entry = plan + PLAN_HEADER + 4 * (slots + s);
+    entry[0] = -1;
+    entry[1] = kept + s * ROWS_PER_SLOT;
+    entry[2] = min(ROWS_PER_SLOT, shared_rows - s * ROWS_PER_SLOT);
+    entry[3] = 0;
+  }
+  for (int r = threadIdx.x; r < shared_rows; r += PLAN_THREADS) order[kept + r] = pairs + r;
+  if (threadIdx.x == 0) {
+    plan[0] = slots + shared_slots;
+    plan[1] = distinct;
+    plan[2] = kept;
+  }
+  // stable placement: each wavefront walks its segment 64 pairs at a time; a lane's position is its expert's running
+  // position in this segment plus the number of lower lanes of the tile with the same expert
+  for (int i0 = lo; i0 < hi; i0 += 64) {
+    const int i = i0 + lane;
+    int e = -1;
+    if (i < hi) {
+      e = ids[i] - e_lo;
+      if (e < 0 || e >= e_n) e = -1;
+    }
+    uint64_t same = __ballot(e >= 0);
+#pragma unroll
+    for (int b = 0; b < 20; b++) {
+      const uint64_t m = __ballot((e >> b) & 1);
+      same &= ((e >> b) & 1) ? m : ~m;
+    }
+    if (e >= 0) {
+      const uint64_t below = same & ((1ull << lane) - 1ull);
+      const int base = seg_count[wave * e_n + e];
+      order[base + __popcll(below)] = i;
+      const bool last = (same >> lane) == 1ull;  // the highest lane of this expert in the tile advances the counter
+      if (last) seg_count[wave * e_n + e] = base + __popcll(same);
+    }
+    // the read of `base` above and the update by `last` are in the same wavefront; LDS operations of one wavefront
+    // execute in program order, and the next tile's reads come after this write
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------- combine
+//
+// out[r, c] = bf16( bf16(sum over the row's local slots, in selection order, of fma(w, y)) + g * shared ), one
+// workgroup per (row, 1024-column span). The reference's combine (hibana/kernels/csrc/w3_gemm.cu:1196-1213) when no
+// shared expert is given; with one, its fused form (hibana/kernels/flashnext_fused.py:530-571).
+constexpr int COMBINE_SPAN = 512;  // columns per workgroup (two per thread)
+constexpr int COMBINE_MAX_TOPK = 32;
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  float g = 1.0f;
+  if (p.gate_vec && p.shared) {
+    float dot = 0.f;
+    for (int i = threadIdx.x; i < p.hx; i += 256) dot += bf16_bits_to_f32(p.x[(int64_t)r * p.hx + i]) * p.gate_vec[i];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) dot += __shfl_xor(dot, d);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = dot;
+    __syncthreads();
+    dot = (red[0] + red[1]) + (red[2] + red[3]);
+    g = 1.0f / (1.0f + expf(-dot));
+  }
+  const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
+  if (c >= p.h) return;
+  float v0 = 0.f, v1 = 0.f;
+  // every slot's pair is read (so the loads are all in flight together) and a dropped slot contributes fma(0, 0, v)
+  for (int s0 = 0; s0 < p.topk; s0 += 8) {
+    float y0[8], y1[8], w[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int s = min(s0 + j, p.topk - 1);
+      const int e = p.ids[r * p.topk + s] - p.e_lo;
+      const bool keep = s0 + j < p.topk && e >= 0 && e < p.e_n;
+      const int64_t at = ((int64_t)r * p.topk + s) * p.h + c;
+      float a, b;
+      if (p.pairs_bf16) {
+        const uint32_t two = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.pairs) + at);
+        a = __uint_as_float(two << 16);
+        b = __uint_as_float(two & 0xffff0000u);
+      } else {
+        const float2 two = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.pairs) + at);
+        a = two.x;
+        b = two.y;
+      }
+      y0[j] = keep ? a : 0.f;
+      y1[j] = keep ? b : 0.f;
+      w[j] = keep ? p.weights[r * p.topk + s] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      v0 = fmaf(w[j], y0[j], v0);
+      v1 = fmaf(w[j], y1[j], v1);
+    }
+  }
+  if (p.shared) {
+    const int64_t at = (int64_t)r * p.shared_stride + c;
+    float s0, s1;
+    if (p.shared_f32) {
+      const float2 two = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.shared) + at);
+      s0 = round_bf16(two.x);
+      s1 = round_bf16(two.y);
+    } else {
+      const uint32_t two = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.shared) + at);
+      s0 = __uint_as_float(two << 16);
+      s1 = __uint_as_float(two & 0xffff0000u);
+    }
+    v0 = round_bf16(v0) + g * s0;
+    v1 = round_bf16(v1) + g * s1;
+  }
+  *reinterpret_cast<uint32_t*>(p.out + (int64_t)r * p.h + c) = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
+}
+
+// ---------------------------------------------------------------------------------------------------- routing
+// Softmax top-k (hibana/kernels/flashnext_fused.py:278-319 of the reference): one wavefront per row.
+constexpr int ROUTE_PER_LANE = 16;  // up to 1024 experts: lane l holds experts l, l + 64, ...
+
+__global__ __launch_bounds__(64) void route_softmax_topk_kernel(const float* __restrict__ logits, int e, int k, int32_t* __restrict__ ids,
+                                                                float* __restrict__ weights) {
+  const int r = blockIdx.x, lane = threadIdx.x;
+  const float* row = logits + (int64_t)r * e;
+  float v[ROUTE_PER_LANE];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; j++) {
+    const int i = lane + 64 * j;
+    v[j] = i < e ? row[i] : -INFINITY;
+    mx = fmaxf(mx, v[j]);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; j++) {
+    v[j] = lane + 64 * j < e ? expf(v[j] - mx) : -1.f;
+    sum += fmaxf(v[j], 0.f);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d);
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; j++) v[j] = v[j] >= 0.f ? v[j] / sum : -1.f;
+  float total = 0.f, mine = 0.f;
+  int mine_id = 0;
+  for (int s = 0; s < k; s++) {
+    float best = -1.f;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; j++)
+      if (v[j] > best) {  // ascending index within the lane: the first of equals stays
+        best = v[j];
+        at = lane + 64 * j;
+      }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      const float ob = __shfl_xor(best, d);
+      const int oa = __shfl_xor(at, d);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    total += best;
+    if (lane == s) {
+      mine = best;
+      mine_id = at;
+    }
+    if ((at & 63) == lane) {
+#pragma unroll
+      for (int j = 0; j < ROUTE_PER_LANE; j++)
+        if (j == (at >> 6)) v[j] = -1.f;
+    }
+  }
+  if (lane < k) {
+    ids[r * k + lane] = mine_id;
+    weights[r * k + lane] = mine / total;
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------------------- host side
+static std::vector<hipEvent_t> g_events;
+static size_t g_event_next = 0;
+void moe_mark(hipStream_t stream) {
+  if (g_event_next < g_events.size()) (void)hipEventRecord(g_events[g_event_next++], stream);
+}
+
+void pick_shape(int n_blocks, int chunks, int64_t slots, int want, int* ks, int* nbw) {
+  int k = 1;
+  while (k < 16 && (int64_t)n_blocks * slots * k < want && chunks / (2 * k) >= 4) k *= 2;
+  int b = k >= 4 ? 1 : 4 / k;
+  while (b > 1 && n_blocks % b) b /= 2;
+  *ks = k;
+  *nbw = b;
+}
+
+int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows) {
+  const int64_t routed = pairs < pairs / ROWS_PER_SLOT + experts ? pairs : pairs / ROWS_PER_SLOT + experts;
+  return routed + (shared_rows + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
+}
+
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int hidden_out, int shared) {
+  const int64_t pairs = (int64_t)m * topk, rows = pairs + (shared ? m : 0);
+  MoeWorkspace w{};
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    void* ptr = base ? static_cast<char*>(base) + off : nullptr;
+    off += align256(bytes);
+    return ptr;
+  };
+  w.plan = static_cast<int32_t*>(take((PLAN_HEADER + 4 * moe_max_slots(pairs, experts, shared ? m : 0)) * sizeof(int32_t)));
+  w.order = static_cast<int32_t*>(take(rows * sizeof(int32_t)));
+  w.h = static_cast<uint16_t*>(take((size_t)rows * inter * sizeof(uint16_t)));
+  w.y = static_cast<float*>(take((size_t)rows * hidden_out * sizeof(float)));
+  w.bytes = off;
+  return w;
+}
+
+int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream) {
+  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
+  if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
+  moe_mark(stream);
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order);
+  moe_mark(stream);
+  return HB_OK;
+}
+
+void moe_launch_combine(const CombineParams& c, hipStream_t stream) {
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)c.m, (unsigned)((c.h + COMBINE_SPAN - 1) / COMBINE_SPAN)), dim3(256), 0, stream, c);
+  moe_mark(stream);
+}
+
+}  // namespace hb
+
+using namespace hb;
+
+extern "C" int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int32_t* ids, const float* weights, const void* shared,
+                                    const void* x, const float* gate_vec, int e_lo, int e_n, int m, int topk, int h, void* out,
+                                    void* stream) {
+  if (!pairs || !ids || !weights || !out) return HB_ENULL;
+  if (gate_vec && shared && !x) return HB_ENULL;
+  if (m <= 0 || topk <= 0 || h <= 0 || h % 2) return HB_EINVAL;
+  CombineParams c{};
+  c.pairs = pairs;
+  c.pairs_bf16 = pairs_bf16;
+  c.ids = ids;
+  c.weights = weights;
+  c.shared = shared;
+  c.shared_stride = h;
+  c.x = static_cast<const uint16_t*>(x);
+  c.gate_vec = gate_vec;
+  c.hx = h;
+  c.e_lo = e_lo;
+  c.e_n = e_n;
+  c.m = m;
+  c.topk = topk;
+  c.h = h;
+  c.out = static_cast<uint16_t*>(out);
+  moe_launch_combine(c, as_stream(stream));
+  return launch_status();
+}
+
+extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, int32_t* ids, float* weights, void* stream) {
+  if (!logits || !ids || !weights) return HB_ENULL;
+  if (m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE) return HB_EINVAL;
+  hipLaunchKernelGGL(route_softmax_topk_kernel, dim3((unsigned)m), dim3(64), 0, as_stream(stream), logits, e, k, ids, weights);
+  return launch_status();
+}
+
+extern "C" int hb_debug_events(void* const* events, int count) {
+  if (count < 0 || (count > 0 && !events)) return HB_EINVAL;
+  g_events.assign(reinterpret_cast<hipEvent_t const*>(events), reinterpret_cast<hipEvent_t const*>(events) + count);
+  g_event_next = 0;
+  return HB_OK;
+}
+
+extern "C" int hb_version(void) { return 1000; }
+
+extern "C" const char* hb_error_string(int code) {
+  switch (code) {
+    case HB_OK: return "ok";
+    case HB_EINVAL: return "unsupported shape, alignment or flag";
+    case HB_ENULL: return "a required pointer is null";
+    case HB_EWORKSPACE: return "workspace too small";
+    case HB_ELAUNCH: return "the HIP runtime refused a launch";
+    default: return "unknown error";
+  }
+}

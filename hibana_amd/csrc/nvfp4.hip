@@ -9,7 +9,7 @@
 //   bytes 4096..4607  scales: 32 B per row-in-tile r at 4096 + 32 r: byte 8 nt + b is the E4M3 scale of row
 //                     64 nb + 16 nt + r, block 8 c + b.
 // Codes expand with v_cvt_scalef32_pk_bf16_fp4 (two weights per instruction, exact).
-#include "common.hpp"
+#include "stream_common.hpp"
 
 namespace hb {
 
@@ -88,19 +88,6 @@ __global__ __launch_bounds__(256) void nvfp4_dequant_kernel(const uint8_t* __res
   }
 }
 
-struct Nvfp4Params {
-  const uint8_t* w;
-  int n_blocks, chunks;
-  const uint16_t* a;
-  int64_t a_stride;
-  int m;
-  uint16_t* out;
-  int64_t out_stride;
-  float global_scale;
-  int relu2;
-  int ks, nbw;
-};
-
 struct Fp4Chunk {  // the weight side of a chunk: prefetched one chunk ahead
   u32x4_t w0, w1, w2, w3, s0, s1;
 };
@@ -168,32 +155,23 @@ __device__ __forceinline__ void fp4_chunk(const Fp4Chunk& ch, const uint16_t* ar
   fp4_tile(ch.w3, ch.s1.z, ch.s1.w, rows, acc3);
 }
 
-__device__ __forceinline__ void nvfp4_emit(const Nvfp4Params& p, int nb, int p0, int rows, int t, int r, int q, int r16, float v) {
-  const int i = 4 * q + r;
-  if (i >= rows) return;
-  float y = round_bf16(v * p.global_scale);
-  if (p.relu2) {
-    y = fmaxf(y, 0.f);
-    y = y * y;
-  }
-  p.out[(int64_t)(p0 + i) * p.out_stride + nb * 64 + 16 * t + r16] = f32_to_bf16_bits(y);
-}
-
-// Dense y = x Wq^T: one wavefront per (64-row block, K range, slot of 16 activation rows), as the W3 stream.
-__global__ __launch_bounds__(1024) void nvfp4_stream_kernel(Nvfp4Params p) {
+// y = x Wq^T, dense or grouped by the expert plan: one wavefront per (64-row block, K range, slot of 16 activation rows),
+// the same launch shape, slot table, K-split exchange and epilogues as the W3 stream.
+template <int EPI>
+__global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
   extern __shared__ float partial[];
+  if (!epi_dense(EPI) && (int)blockIdx.y >= p.plan[0]) return;  // a slot the plan did not fill
+  const Slot sl = slot_of<EPI>(p, blockIdx.y);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q = lane >> 4, r16 = lane & 15;
   const int ks = wave % p.ks, nbi = wave / p.ks;
   const int nb = blockIdx.x * p.nbw + nbi;
-  const int p0 = blockIdx.y * 16, rows = min(16, p.m - p0);
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
   if (active) {
     const int c0 = (int)((int64_t)ks * p.chunks / p.ks), c1 = (int)((int64_t)(ks + 1) * p.chunks / p.ks);
-    const int64_t arow = p0 + min(r16, rows - 1);
-    const uint16_t* aptr = p.a + arow * p.a_stride + 4 * q + (int64_t)c0 * 128;
-    const uint8_t* blk = p.w + ((int64_t)nb * p.chunks + c0) * NVFP4_BLOCK_BYTES;
+    const uint16_t* aptr = activation_row<EPI>(p, sl, r16) + 4 * q + (int64_t)c0 * 128;
+    const uint8_t* blk = sl.w + ((int64_t)nb * p.chunks + c0) * NVFP4_BLOCK_BYTES;
     if (c0 < c1) {
       Fp4Chunk even, odd;
       load_fp4_chunk(even, blk, lane, r16);
@@ -216,35 +194,16 @@ __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(Nvfp4Params p) {
       }
     }
   }
-  const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
-  if (p.ks == 1) {
-    if (!active) return;
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      nvfp4_emit(p, nb, p0, rows, t, 0, q, r16, all[t].x);
-      nvfp4_emit(p, nb, p0, rows, t, 1, q, r16, all[t].y);
-      nvfp4_emit(p, nb, p0, rows, t, 2, q, r16, all[t].z);
-      nvfp4_emit(p, nb, p0, rows, t, 3, q, r16, all[t].w);
-    }
-    return;
-  }
-  float* mine = partial + (int64_t)wave * 1024;
-#pragma unroll
-  for (int t = 0; t < 4; t++) {
-    mine[(t * 4 + 0) * 64 + lane] = all[t].x;
-    mine[(t * 4 + 1) * 64 + lane] = all[t].y;
-    mine[(t * 4 + 2) * 64 + lane] = all[t].z;
-    mine[(t * 4 + 3) * 64 + lane] = all[t].w;
-  }
-  __syncthreads();
-  if (!active) return;
-  const float* first = partial + (int64_t)nbi * p.ks * 1024;
-  for (int idx = ks; idx < 16; idx += p.ks) {
-    const int t = idx >> 2, r = idx & 3;
-    float v = 0.f;
-    for (int s = 0; s < p.ks; s++) v += first[s * 1024 + (t * 4 + r) * 64 + lane];
-    nvfp4_emit(p, nb, p0, rows, t, r, q, r16, v);
-  }
+  finish_block<EPI, false>(p, sl, nb, active, ks, nbi, partial, acc0, acc1, acc2, acc3);
+}
+
+template <int EPI>
+static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipStream_t stream) {
+  pick_shape(p.n_blocks, p.chunks, busy_slots, 4096, &p.ks, &p.nbw);
+  const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
+  const int waves = p.ks * p.nbw;
+  hipLaunchKernelGGL(nvfp4_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
+  return HB_OK;
 }
 
 static inline unsigned grid_for(int64_t threads) { return (unsigned)((threads + 255) / 256); }
@@ -283,27 +242,105 @@ extern "C" int hb_nvfp4_dequant(const void* tiled, float global_scale, int64_t r
 extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y, void* stream) {
   if (!x || !tiled || !y) return HB_ENULL;
   if (m <= 0 || n <= 0 || k <= 0 || n % 64 || k % 128) return HB_EINVAL;
-  Nvfp4Params p{};
+  StreamParams p{};
   p.w = static_cast<const uint8_t*>(tiled);
+  p.scalar = global_scale;
   p.n_blocks = n / 64;
   p.chunks = k / 128;
   p.a = static_cast<const uint16_t*>(x);
   p.a_stride = k;
   p.m = m;
-  p.out = static_cast<uint16_t*>(y);
+  p.out = y;
   p.out_stride = n;
-  p.global_scale = global_scale;
-  p.relu2 = relu2;
-  const int64_t slots = (m + 15) / 16;
+  const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
   if (slots > 65535) return HB_EINVAL;
-  int ks = 1;
-  while (ks < 16 && (int64_t)p.n_blocks * slots * ks < 2048 && p.chunks / (2 * ks) >= 2) ks *= 2;
-  int nbw = ks >= 4 ? 1 : 4 / ks;
-  while (nbw > 1 && p.n_blocks % nbw) nbw /= 2;
-  p.ks = ks;
-  p.nbw = nbw;
-  const dim3 grid((unsigned)((p.n_blocks + nbw - 1) / nbw), (unsigned)slots);
-  const int waves = ks * nbw;
-  hipLaunchKernelGGL(nvfp4_stream_kernel, grid, dim3(64 * waves), ks > 1 ? (size_t)waves * 4096 : 0, as_stream(stream), p);
+  if (int e = relu2 ? launch_nvfp4<EPI_DENSE_RELU2>(p, slots, slots, as_stream(stream)) : launch_nvfp4<EPI_DENSE>(p, slots, slots, as_stream(stream)))
+    return e;
+  return launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------ routed experts
+namespace {
+
+int check_experts(const hb_nvfp4_experts* ex) {
+  if (!ex) return HB_ENULL;
+  if (!ex->fc1 || !ex->fc1_scale2 || !ex->fc2 || !ex->fc2_scale2) return HB_ENULL;
+  if (ex->experts <= 0 || ex->hidden <= 0 || ex->inter <= 0 || ex->hidden_out <= 0) return HB_EINVAL;
+  const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
+  if (ex->hidden % 128 || ex->inter % 128 || n1 % 64 || ex->hidden_out % 64) return HB_EINVAL;
+  return HB_OK;
+}
+
+// plan -> fc1 -> fc2: `out_pairs` receives fc2's per-pair outputs.
+int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, int m, int topk, const MoeWorkspace& ws, void* out_pairs,
+                int pairs_bf16, hipStream_t stream) {
+  const int64_t pairs = (int64_t)m * topk;
+  const int64_t slots = moe_max_slots(pairs, ex->experts, 0);
+  if (slots > 65535) return HB_EINVAL;
+  if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, 0, ws, stream)) return e;
+  const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
+  const int64_t est = pairs < 2 * ex->experts ? (pairs + 1) / 2 : slots;
+  StreamParams p{};
+  p.w = static_cast<const uint8_t*>(ex->fc1);
+  p.expert_bytes = (int64_t)hb_nvfp4_tiled_bytes(n1, ex->hidden);
+  p.scalars = ex->fc1_scale2;
+  p.n_blocks = n1 / 64;
+  p.chunks = ex->hidden / 128;
+  p.a = static_cast<const uint16_t*>(x);
+  p.a_stride = ex->hidden;
+  p.plan = ws.plan;
+  p.order = ws.order;
+  p.topk = topk;
+  p.pairs = (int)pairs;
+  p.out = ws.h;
+  p.out_stride = ex->inter;
+  StreamParams f2 = p;
+  f2.w = static_cast<const uint8_t*>(ex->fc2);
+  f2.expert_bytes = (int64_t)hb_nvfp4_tiled_bytes(ex->hidden_out, ex->inter);
+  f2.scalars = ex->fc2_scale2;
+  f2.n_blocks = ex->hidden_out / 64;
+  f2.chunks = ex->inter / 128;
+  f2.a = ws.h;
+  f2.a_stride = ex->inter;
+  f2.out = out_pairs;
+  f2.out_stride = ex->hidden_out;
+  f2.out_bf16 = pairs_bf16;
+  if (int e = ex->gated ? launch_nvfp4<EPI_FC1_GATED>(p, slots, est, stream) : launch_nvfp4<EPI_FC1_RELU2>(p, slots, est, stream)) return e;
+  moe_mark(stream);
+  if (int e = launch_nvfp4<EPI_FC2>(f2, slots, est, stream)) return e;
+  moe_mark(stream);
+  return launch_status();
+}
+
+}  // namespace
+
+extern "C" size_t hb_nvfp4_moe_workspace_bytes(int m, int topk, const hb_nvfp4_experts* routed) {
+  if (!routed || m <= 0 || topk <= 0 || check_experts(routed) != HB_OK) return 0;
+  return moe_carve(nullptr, m, topk, routed->experts, routed->inter, routed->hidden_out, 0).bytes;
+}
+
+extern "C" int hb_nvfp4_moe(const hb_nvfp4_experts* routed, const void* x, const int32_t* ids, const float* weights, int m, int topk, int mode,
+                            void* out, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int e = check_experts(routed)) return e;
+  if (!x || !ids || !weights || !out || !workspace) return HB_ENULL;
+  if (m <= 0 || topk <= 0 || mode < HB_MOE_SUM || mode > HB_MOE_PAIRS_BF16) return HB_EINVAL;
+  const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, 0);
+  if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
+  const bool sum = mode == HB_MOE_SUM;
+  void* pairs_out = sum ? static_cast<void*>(ws.y) : out;
+  if (int e = run_experts(routed, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16, as_stream(stream))) return e;
+  if (sum) {
+    CombineParams c{};
+    c.pairs = ws.y;
+    c.ids = ids;
+    c.weights = weights;
+    c.e_lo = routed->base;
+    c.e_n = routed->experts;
+    c.m = m;
+    c.topk = topk;
+    c.h = routed->hidden_out;
+    c.out = static_cast<uint16_t*>(out);
+    moe_launch_combine(c, as_stream(stream));
+  }
   return launch_status();
 }

@@ -1,0 +1,228 @@
+// Shared by the W3 and NVFP4 weight streams: launch parameters, the slot table of a routed call, the epilogues
+// (row / global scale, the reference's rounding points, SiLU gate or ReLU^2, pair outputs), the K-split exchange through
+// LDS, and the host-side helpers of a routed call (workspace, plan launch, combine launch).
+#pragma once
+
+#include "common.hpp"
+
+namespace hb {
+
+enum { EPI_DENSE = 0, EPI_FC1_GATED = 1, EPI_FC1_RELU2 = 2, EPI_FC2 = 3, EPI_DENSE_RELU2 = 4 };
+constexpr bool epi_dense(int epi) { return epi == EPI_DENSE || epi == EPI_DENSE_RELU2; }
+constexpr bool epi_gathers(int epi) { return epi == EPI_FC1_GATED || epi == EPI_FC1_RELU2; }  // activation rows found through `order`
+constexpr int ROWS_PER_SLOT = 16;
+constexpr int PLAN_HEADER = 16;  // plan[0] = slots, plan[1] = distinct experts, plan[2] = routed pairs kept
+
+struct StreamParams {
+  const uint8_t* w;       // tile layout, expert 0
+  int64_t expert_bytes;   // bytes between experts
+  const float* rows;      // row scales, expert 0
+  int64_t expert_rows;    // floats between experts
+  const uint8_t* w_shared;  // the shared expert (slot expert id < 0), or null
+  const float* rows_shared;
+  const float* scalars;   // formats with one FP32 scale per matrix: [experts], or null for `scalar`
+  float scalar, scalar_shared;
+  uint32_t lut_lo, lut_hi, lut_lo_shared, lut_hi_shared;
+  int n_blocks;           // 64-row blocks per expert matrix
+  int chunks;             // K / 128
+  const uint16_t* a;      // BF16 activations
+  int64_t a_stride;       // elements between rows
+  const int32_t* plan;    // grouped calls: slot table
+  const int32_t* order;   // grouped calls: sorted position -> pair index
+  int m;                  // dense calls: rows
+  int topk, pairs;        // grouped calls: pair q < pairs belongs to token q / topk, q >= pairs to token q - pairs
+  void* out;
+  int64_t out_stride;     // elements between output rows
+  int out_bf16;           // EPI_FC2: pair outputs in BF16 instead of FP32
+  int ks, nbw;            // wavefronts per workgroup = ks (K splits) * nbw (64-row blocks)
+};
+
+// The epilogue's roundings use the hardware FP32 -> BF16 conversion (round to nearest even).
+__device__ __forceinline__ uint16_t bf16_of(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+__device__ __forceinline__ float through_bf16(float f) { return (float)(__bf16)f; }
+
+// silu with the fast exponential and division: the result is rounded to BF16 right after (8 significant bits).
+__device__ __forceinline__ float silu(float g) { return __fdividef(g, 1.0f + __expf(-g)); }
+
+// What a workgroup needs to know about its slot (up to 16 activation rows of one expert, or of the dense matrix).
+struct Slot {
+  int p0, rows;        // first row (sorted position) and number of rows
+  const uint8_t* w;    // the expert's tile-layout matrix
+  const float* rs;     // its row scales (formats that have them)
+  float scalar;        // its FP32 scale (formats with one per matrix)
+  uint32_t lut_lo, lut_hi;
+};
+
+// One output element (or, gated, one up/gate pair) of the 64-row block: row tile `t` (gated: pair index), accumulator
+// register r of lane (q, r16); v0 / v1 are the K-complete sums before the FP32 scale (per output row with PER_ROW, else
+// one per matrix).
+template <int EPI, bool PER_ROW>
+__device__ __forceinline__ void emit(const StreamParams& p, const Slot& sl, int nb, int t, int r, int q, int r16, float v0, float v1) {
+  if (r >= sl.rows) return;  // wave-uniform: this accumulator register holds no row of the slot in any lane
+  const int i = 4 * q + r;   // activation row of the slot held by this accumulator register
+  if (i >= sl.rows) return;
+  const int64_t pos = sl.p0 + i;
+  if (EPI == EPI_FC1_GATED) {
+    const int n_up = nb * 64 + 32 * t + r16;
+    const float up = through_bf16(v0 * (PER_ROW ? sl.rs[n_up] : sl.scalar));
+    const float gate = through_bf16(v1 * (PER_ROW ? sl.rs[n_up + 16] : sl.scalar));
+    reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = bf16_of(silu(gate) * up);
+  } else {
+    const int n = nb * 64 + 16 * t + r16;
+    const float y = v0 * (PER_ROW ? sl.rs[n] : sl.scalar);
+    if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
+      const float h = fmaxf(through_bf16(y), 0.f);
+      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(h * h);
+    } else if (EPI == EPI_DENSE) {
+      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(y);
+    } else {
+      const int64_t pair = p.order[pos];
+      if (p.out_bf16) {
+        reinterpret_cast<uint16_t*>(p.out)[pair * p.out_stride + n] = bf16_of(y);
+      } else {
+        reinterpret_cast<float*>(p.out)[pair * p.out_stride + n] = y;
+      }
+    }
+  }
+}
+
+template <int EPI>
+__device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
+  Slot s;
+  int expert = 0;
+  if (epi_dense(EPI)) {
+    s.p0 = slot * ROWS_PER_SLOT;
+    s.rows = min(ROWS_PER_SLOT, p.m - s.p0);
+  } else {
+    expert = p.plan[PLAN_HEADER + 4 * slot];
+    s.p0 = p.plan[PLAN_HEADER + 4 * slot + 1];
+    s.rows = p.plan[PLAN_HEADER + 4 * slot + 2];
+  }
+  s.w = expert < 0 ? p.w_shared : p.w + (int64_t)expert * p.expert_bytes;
+  s.rs = expert < 0 ? p.rows_shared : p.rows + (int64_t)expert * p.expert_rows;
+  s.scalar = expert < 0 ? p.scalar_shared : p.scalars ? p.scalars[expert] : p.scalar;
+  s.lut_lo = expert < 0 ? p.lut_lo_shared : p.lut_lo;
+  s.lut_hi = expert < 0 ? p.lut_hi_shared : p.lut_hi;
+  return s;
+}
+
+// The activation row this lane feeds to the MFMA A operand (row r16 of the slot). Lanes past the slot's last row read
+// that last row again: their MFMA output rows are never stored.
+template <int EPI>
+__device__ __forceinline__ const uint16_t* activation_row(const StreamParams& p, const Slot& s, int r16) {
+  int64_t arow = s.p0 + min(r16, s.rows - 1);
+  if (epi_gathers(EPI)) {
+    const int pair = p.order[arow];
+    arow = pair < p.pairs ? pair / p.topk : pair - p.pairs;
+  }
+  return p.a + arow * p.a_stride;
+}
+
+// The end of a 64-row block: K-complete sums straight from the registers (ks == 1), or the K split's partial sums
+// exchanged through LDS (`partial`: 4 KB per wavefront) and added in split order, then the epilogue. With ks > 1 every
+// wavefront of the workgroup must call it (one workgroup barrier).
+template <int EPI, bool PER_ROW>
+__device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& sl, int nb, bool active, int ks, int nbi, float* partial,
+                                             const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2, const f32x4_t& acc3) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int rows = sl.rows;
+  if (p.ks == 1) {
+    if (!active) return;
+    if (EPI == EPI_FC1_GATED) {
+      emit<EPI, PER_ROW>(p, sl, nb, 0, 0, q, r16, acc0.x, acc1.x);
+      emit<EPI, PER_ROW>(p, sl, nb, 0, 1, q, r16, acc0.y, acc1.y);
+      emit<EPI, PER_ROW>(p, sl, nb, 0, 2, q, r16, acc0.z, acc1.z);
+      emit<EPI, PER_ROW>(p, sl, nb, 0, 3, q, r16, acc0.w, acc1.w);
+      emit<EPI, PER_ROW>(p, sl, nb, 1, 0, q, r16, acc2.x, acc3.x);
+      emit<EPI, PER_ROW>(p, sl, nb, 1, 1, q, r16, acc2.y, acc3.y);
+      emit<EPI, PER_ROW>(p, sl, nb, 1, 2, q, r16, acc2.z, acc3.z);
+      emit<EPI, PER_ROW>(p, sl, nb, 1, 3, q, r16, acc2.w, acc3.w);
+    } else {
+      const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        emit<EPI, PER_ROW>(p, sl, nb, t, 0, q, r16, all[t].x, 0.f);
+        emit<EPI, PER_ROW>(p, sl, nb, t, 1, q, r16, all[t].y, 0.f);
+        emit<EPI, PER_ROW>(p, sl, nb, t, 2, q, r16, all[t].z, 0.f);
+        emit<EPI, PER_ROW>(p, sl, nb, t, 3, q, r16, all[t].w, 0.f);
+      }
+    }
+    return;
+  }
+  float* mine = partial + (int64_t)wave * 1024;
+  {
+    const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      mine[(t * 4 + 0) * 64 + lane] = all[t].x;
+      mine[(t * 4 + 1) * 64 + lane] = all[t].y;
+      mine[(t * 4 + 2) * 64 + lane] = all[t].z;
+      mine[(t * 4 + 3) * 64 + lane] = all[t].w;
+    }
+  }
+  __syncthreads();
+  if (!active) return;
+  const float* first = partial + (int64_t)nbi * p.ks * 1024;
+  if (EPI == EPI_FC1_GATED) {
+    for (int idx = ks; idx < 8; idx += p.ks) {
+      const int t = idx >> 2, r = idx & 3;
+      if (r >= rows) continue;
+      float up = 0.f, gate = 0.f;
+      for (int s = 0; s < p.ks; s++) {
+        up += first[s * 1024 + ((2 * t) * 4 + r) * 64 + lane];
+        gate += first[s * 1024 + ((2 * t + 1) * 4 + r) * 64 + lane];
+      }
+      emit<EPI, PER_ROW>(p, sl, nb, t, r, q, r16, up, gate);
+    }
+  } else {
+    for (int idx = ks; idx < 16; idx += p.ks) {
+      const int t = idx >> 2, r = idx & 3;
+      if (r >= rows) continue;
+      float v = 0.f;
+      for (int s = 0; s < p.ks; s++) v += first[s * 1024 + (t * 4 + r) * 64 + lane];
+      emit<EPI, PER_ROW>(p, sl, nb, t, r, q, r16, v, 0.f);
+    }
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------------------- host side
+// Workspace of a routed call, carved from one caller-owned buffer.
+struct MoeWorkspace {
+  int32_t* plan;
+  int32_t* order;
+  uint16_t* h;   // [(pairs + shared rows), inter] BF16, in sorted order
+  float* y;      // [(pairs + shared rows), hidden_out] FP32 (or BF16 pairs), by pair index
+  size_t bytes;
+};
+
+int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows);
+MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int hidden_out, int shared);
+// Enqueue the plan kernel; HB_EINVAL if the expert count does not fit its LDS.
+int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream);
+
+struct CombineParams {
+  const void* pairs;      // [m * topk (+ m), h] FP32 or BF16
+  int pairs_bf16;
+  const int32_t* ids;
+  const float* weights;
+  const void* shared;     // BF16 [m, h], FP32 [m, h] (shared_f32) or null
+  int shared_f32;
+  int64_t shared_stride;
+  const uint16_t* x;      // BF16 [m, hx] for the gate
+  const float* gate_vec;  // [hx] or null
+  int hx;
+  int e_lo, e_n, m, topk, h;
+  uint16_t* out;
+};
+void moe_launch_combine(const CombineParams& c, hipStream_t stream);
+
+// Measurement hook: records the caller's next event (if any) on the stream.
+void moe_mark(hipStream_t stream);
+
+// Wavefronts per workgroup of a stream launch: K is split until the launch has about `want` wavefronts, keeping at
+// least four chunks per wavefront; what is left of a 4-wavefront workgroup takes neighbouring 64-row blocks.
+void pick_shape(int n_blocks, int chunks, int64_t slots, int want, int* ks, int* nbw);
+
+}  // namespace hb

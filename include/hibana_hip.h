@@ -165,6 +165,30 @@ int hb_nvfp4_dequant(const void* tiled, float global_scale, int64_t rows, int k,
 int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y,
                   void* stream);
 
+/* ------------------------------------------------------------------------------------------------------------------
+ * Routed experts on NVFP4 weights (ReLU^2 when fc1 has inter rows per expert, gated SiLU when it has 2*inter rows in
+ * the W3 path's fc1_order).
+ * ---------------------------------------------------------------------------------------------------------------- */
+typedef struct hb_nvfp4_experts {
+  const void* fc1;          /* tile layout of the stacked fc1 [experts * n1, hidden], n1 = gated ? 2*inter : inter */
+  const float* fc1_scale2;  /* [experts] FP32 scale of each fc1 matrix (the checkpoint's weight_scale_2) */
+  const void* fc2;          /* tile layout of the stacked fc2 [experts * hidden_out, inter] */
+  const float* fc2_scale2;  /* [experts]; a routed_scaling_factor is folded in here by the caller */
+  int experts, base;        /* experts held here and the id of the first one */
+  int hidden, inter, hidden_out;
+  int gated;
+} hb_nvfp4_experts;
+
+size_t hb_nvfp4_moe_workspace_bytes(int m, int topk, const hb_nvfp4_experts* routed);
+
+/* Routed sum on NVFP4 experts, same contract and modes as hb_w3_moe:
+ * h = bf16(act(bf16((x up_e^T)_fp32 * s2))), y = (h down_e^T)_fp32 * s2, out[r] = bf16(sum_s weights[r, s] * y[r, s]).
+ * ref: B12xExperts.__call__, hibana/kernels/b12x_moe.py:58-68 (caller NemotronMoe.routed,
+ * hibana/model/nemotron/moe.py:476-482) in the weight-only form stated by moe_mixer,
+ * tests/nemotron_reference.py:568-593. */
+int hb_nvfp4_moe(const hb_nvfp4_experts* routed, const void* x, const int32_t* ids, const float* weights, int m,
+                 int topk, int mode, void* out, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
