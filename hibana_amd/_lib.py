@@ -45,6 +45,7 @@ SIGNATURES = {
     "hb_w3_moe_layer": (_I, [_EX, _EX, _P, _P, _P, _P, _I, _I, _P, _P, _Z, _P]),
     "hb_moe_combine_pairs": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P]),
     "hb_route_softmax_topk": (_I, [_P, _I, _I, _I, _P, _P, _P]),
+    "hb_route_sigmoid_topk": (_I, [_P, _L, _P, _I, _I, _I, _I, _P, _I, _I, _P, _P, _P, _P]),
     "hb_nvfp4_tiled_bytes": (_Z, [_L, _I]),
     "hb_nvfp4_repack": (_I, [_P, _P, _I, _L, _I, _P, _P]),
     "hb_nvfp4_dequant": (_I, [_P, _F, _L, _I, _P, _P]),

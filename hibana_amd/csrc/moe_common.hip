@@ -225,70 +225,131 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------- routing
-// Softmax top-k (hibana/kernels/flashnext_fused.py:278-319 of the reference): one wavefront per row.
-constexpr int ROUTE_PER_LANE = 16;  // up to 1024 experts: lane l holds experts l, l + 64, ...
+// Top-k routing, one wavefront per row: softmax over all experts, top-k, renormalized
+// (hibana/kernels/flashnext_fused.py:278-319 of the reference), or sigmoid scores chosen by score + bias with the plain
+// scores as weights (hibana/model/nemotron/moe.py:57-121). Lane l holds experts l * per .. l * per + per - 1 in
+// registers as order-preserving 32-bit keys, so a selection round is a register scan, one wave-wide integer maximum
+// (DPP within rows of 16, four scalar reads across them) and a ballot: among equal scores the lowest lane, then the
+// lowest register, wins - the lowest expert id.
+constexpr int ROUTE_PER_LANE = 16;  // up to 1024 experts
 
-__global__ __launch_bounds__(64) void route_softmax_topk_kernel(const float* __restrict__ logits, int e, int k, int32_t* __restrict__ ids,
-                                                                float* __restrict__ weights) {
-  const int r = blockIdx.x, lane = threadIdx.x;
-  const float* row = logits + (int64_t)r * e;
-  float v[ROUTE_PER_LANE];
-  float mx = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < ROUTE_PER_LANE; j++) {
-    const int i = lane + 64 * j;
-    v[j] = i < e ? row[i] : -INFINITY;
-    mx = fmaxf(mx, v[j]);
-  }
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
-  float sum = 0.f;
-#pragma unroll
-  for (int j = 0; j < ROUTE_PER_LANE; j++) {
-    v[j] = lane + 64 * j < e ? expf(v[j] - mx) : -1.f;
-    sum += fmaxf(v[j], 0.f);
-  }
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d);
-#pragma unroll
-  for (int j = 0; j < ROUTE_PER_LANE; j++) v[j] = v[j] >= 0.f ? v[j] / sum : -1.f;
-  float total = 0.f, mine = 0.f;
-  int mine_id = 0;
-  for (int s = 0; s < k; s++) {
-    float best = -1.f;
-    int at = 0x7fffffff;
-#pragma unroll
-    for (int j = 0; j < ROUTE_PER_LANE; j++)
-      if (v[j] > best) {  // ascending index within the lane: the first of equals stays
-        best = v[j];
-        at = lane + 64 * j;
-      }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-      const float ob = __shfl_xor(best, d);
-      const int oa = __shfl_xor(at, d);
-      if (ob > best || (ob == best && oa < at)) {
-        best = ob;
-        at = oa;
-      }
-    }
-    total += best;
-    if (lane == s) {
-      mine = best;
-      mine_id = at;
-    }
-    if ((at & 63) == lane) {
-#pragma unroll
-      for (int j = 0; j < ROUTE_PER_LANE; j++)
-        if (j == (at >> 6)) v[j] = -1.f;
-    }
-  }
-  if (lane < k) {
-    ids[r * k + lane] = mine_id;
-    weights[r * k + lane] = mine / total;
-  }
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false));   // lane ^ 1
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false));   // lane ^ 2
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, false));  // mirror within 8
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x140, 0xF, 0xF, false));  // mirror within 16
+  const uint32_t a = __builtin_amdgcn_readlane((int)x, 0), b = __builtin_amdgcn_readlane((int)x, 16);
+  const uint32_t c = __builtin_amdgcn_readlane((int)x, 32), d = __builtin_amdgcn_readlane((int)x, 48);
+  return max(max(a, b), max(c, d));
 }
 
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+  return v;
+}
+
+// Key of a score: larger score <=> larger key, every real key above 0 (the key of an empty register).
+__device__ __forceinline__ uint32_t score_key(float v) {
+  const int32_t bits = __builtin_bit_cast(int32_t, v);
+  return (uint32_t)(bits ^ ((bits >> 31) & 0x7fffffff)) ^ 0x80000000u;
+}
+
+struct RouteParams {
+  const float* logits;   // [m, stride]: e logits a row (sigmoid: followed by `latent` FP32 columns)
+  int64_t stride;
+  const float* bias;     // sigmoid: [e] added to the scores for the choice only
+  const int32_t* slots;  // sigmoid: row r is real iff slots[r / steps] != 0 (null: every row)
+  int steps, repeat;
+  int e, k, per, latent;
+  int32_t* ids;
+  float* weights;
+  uint16_t* lat;         // sigmoid: BF16 [m, latent], the row's latent columns
+};
+
+template <bool SIGMOID>
+__global__ __launch_bounds__(64) void route_topk_kernel(RouteParams p) {
+  const int r = blockIdx.x, lane = threadIdx.x;
+  const int e = p.e, per = p.per, first = lane * per;
+  bool padded = false;
+  if (SIGMOID) {
+    const float* src = p.logits + (int64_t)r * p.stride + e;
+    for (int c = lane; c < p.latent; c += 64) p.lat[(int64_t)r * p.latent + c] = __builtin_bit_cast(uint16_t, (__bf16)src[c]);
+    padded = p.slots && p.slots[r / p.steps] == 0;
+  }
+  const float* row = p.logits + (int64_t)(padded ? 0 : r) * p.stride;  // a padded row repeats row 0's first choice
+  float val[ROUTE_PER_LANE];   // the weight an expert would get before renormalization
+  uint32_t key[ROUTE_PER_LANE];
+  if (SIGMOID) {
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; j++) {
+      const int i = first + j;
+      const bool real = j < per && i < e;
+      val[j] = real ? 1.0f / (1.0f + expf(-row[i])) : 0.f;
+      key[j] = real ? score_key(val[j] + p.bias[i]) : 0u;
+    }
+  } else {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; j++) {
+      const int i = first + j;
+      val[j] = j < per && i < e ? row[i] : -INFINITY;
+      mx = fmaxf(mx, val[j]);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; j++) {
+      val[j] = j < per && first + j < e ? expf(val[j] - mx) : 0.f;
+      sum += val[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; j++) {
+      val[j] = val[j] / sum;
+      key[j] = j < per && first + j < e ? score_key(val[j]) : 0u;
+    }
+  }
+  float total = 0.f, mine = 0.f;
+  int mine_id = 0;
+  for (int s = 0; s < p.k; s++) {
+    uint32_t best = 0;
+    int at = 0;
+    float bv = 0.f;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; j++)
+      if (key[j] > best) {  // ascending index within the lane: the first of equals stays
+        best = key[j];
+        at = j;
+        bv = val[j];
+      }
+    const uint32_t top = wave_max_u32(best);
+    const int winner = __builtin_ctzll(__ballot(best == top));
+    const int wj = __builtin_amdgcn_readlane(at, winner);
+    const float wv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv), winner));
+    total += wv;
+    if (lane == s) {
+      mine = wv;
+      mine_id = winner * per + wj;
+    }
+    if (lane == winner) {
+#pragma unroll
+      for (int j = 0; j < ROUTE_PER_LANE; j++)
+        if (j == wj) key[j] = 0u;
+    }
+  }
+  if (lane < p.k) {
+    int id = mine_id;
+    float w = SIGMOID ? mine / (total + 1e-20f) : mine / total;
+    if (padded) {
+      id = p.repeat ? __builtin_amdgcn_readfirstlane(mine_id) : e;
+      w = 0.f;
+    }
+    p.ids[(int64_t)r * p.k + lane] = id;
+    p.weights[(int64_t)r * p.k + lane] = w;
+  }
+}
 
 // ---------------------------------------------------------------------------------------------------- host side
 static std::vector<hipEvent_t> g_events;
@@ -377,7 +438,38 @@ extern "C" int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int
 extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, int32_t* ids, float* weights, void* stream) {
   if (!logits || !ids || !weights) return HB_ENULL;
   if (m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE) return HB_EINVAL;
-  hipLaunchKernelGGL(route_softmax_topk_kernel, dim3((unsigned)m), dim3(64), 0, as_stream(stream), logits, e, k, ids, weights);
+  RouteParams p{};
+  p.logits = logits;
+  p.stride = e;
+  p.e = e;
+  p.k = k;
+  p.per = (e + 63) / 64;
+  p.ids = ids;
+  p.weights = weights;
+  hipLaunchKernelGGL(route_topk_kernel<false>, dim3((unsigned)m), dim3(64), 0, as_stream(stream), p);
+  return launch_status();
+}
+
+extern "C" int hb_route_sigmoid_topk(const float* fused, int64_t stride, const float* bias, int m, int e, int k, int latent,
+                                     const int32_t* slots, int steps, int repeat, int32_t* ids, float* weights, void* lat, void* stream) {
+  if (!fused || !bias || !ids || !weights || (latent > 0 && !lat)) return HB_ENULL;
+  if (m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE || latent < 0 || stride < (int64_t)e + latent || steps <= 0)
+    return HB_EINVAL;
+  RouteParams p{};
+  p.logits = fused;
+  p.stride = stride;
+  p.bias = bias;
+  p.slots = slots;
+  p.steps = steps;
+  p.repeat = repeat;
+  p.e = e;
+  p.k = k;
+  p.per = (e + 63) / 64;
+  p.latent = latent;
+  p.ids = ids;
+  p.weights = weights;
+  p.lat = static_cast<uint16_t*>(lat);
+  hipLaunchKernelGGL(route_topk_kernel<true>, dim3((unsigned)m), dim3(64), 0, as_stream(stream), p);
   return launch_status();
 }
 

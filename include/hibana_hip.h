@@ -141,6 +141,16 @@ int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int32_t* ids, 
  * ref: route_topk, hibana/kernels/flashnext_fused.py:278-319 (plain form, no padded-slot table). */
 int hb_route_softmax_topk(const float* logits, int m, int e, int k, int32_t* ids, float* weights, void* stream);
 
+/* Sigmoid top-k routing of the latent MoE on the fused router|fc1_latent GEMM output: fused FP32 [m, stride], columns
+ * 0..e-1 the router logits, e..e+latent-1 the latent projection. s = 1 / (1 + exp(-logit)); ids = the k largest of
+ * s + bias[e] in descending order, equal scores to the lower id; weights = s[ids] / (sum of s[ids] + 1e-20) (no
+ * routed scaling factor); lat BF16 [m, latent] = the latent columns rounded (latent may be 0). slots (may be NULL):
+ * row r is real iff slots[r / steps] != 0; a padded row gets weight 0 and row 0's first choice (repeat != 0) or id e.
+ * ref: route_topk / _route_kernel, hibana/model/nemotron/moe.py:75-121. */
+int hb_route_sigmoid_topk(const float* fused, int64_t stride, const float* bias, int m, int e, int k, int latent,
+                          const int32_t* slots, int steps, int repeat, int32_t* ids, float* weights, void* lat,
+                          void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * NVFP4 format: E2M1 codes two per byte (element 2i in the low nibble), one E4M3 scale per 16 weights, one FP32
  * global scale. ref: hibana/weights/modelopt.py:57-81,150-156.

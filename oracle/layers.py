@@ -188,9 +188,13 @@ def latent_experts_ref(lat: torch.Tensor, ids: np.ndarray, weights: torch.Tensor
     return acc
 
 
-def latent_moe_ref(x, fc1, fc2, ids, weights, get_expert):
+def latent_moe_ref(x, fc1, fc2, ids, weights, get_expert, shared=None):
     """x BF16 [M, H], fc1 BF16 [L, H], fc2 BF16 [H, L] -> BF16 [M, H]:
-    lat = bf16(x fc1^T); out = bf16(bf16(acc) fc2^T)."""
+    lat = bf16(x fc1^T); out = bf16(shared + bf16(acc) fc2^T), `shared` the shared expert's BF16 output [M, H] (addmm: one
+    rounding of the FP32 sum) or None (hibana/model/nemotron/moe.py:508-517 of the reference)."""
     lat = bf16((x.double() @ fc1.double().T).float())
     acc = latent_experts_ref(lat, ids, weights, get_expert)
-    return bf16((bf16(acc).double() @ fc2.double().T).float())
+    y = bf16(acc).double() @ fc2.double().T
+    if shared is not None:
+        y = y + shared.double()
+    return bf16(y.float())
