@@ -119,31 +119,30 @@ def main() -> int:
     torch.cuda.synchronize()
 
     def step(i: int):
-        ids, wts = ops.route_topk(logits[i % args.layers], TOPK)
-        return w3_moe.moe_layer(layers[i % args.layers][0], x, ids, wts, shared=layers[i % args.layers][1])
+        return w3_moe.moe_layer_logits(layers[i % args.layers][0], x, logits[i % args.layers], TOPK, shared=layers[i % args.layers][1])
 
     distinct = [int(torch.unique(ops.route_topk(lg, TOPK)[0]).numel()) for lg in logits]
     for i in range(max(args.warmup, args.layers)):  # untimed: also builds every layer's tiled weights and warms the allocator
         step(i)
     torch.cuda.synchronize()
 
-    # live kernel timing: HIP events at the kernel boundaries of the chain, on the stream the kernels run on
+    # live kernel timing: each kernel of the chain is launched with its own (start, stop) HIP event pair, which the
+    # runtime stamps with that kernel's begin and end on the stream it runs on
     hip = Hip()
-    names = ["plan", "fc1", "fc2", "combine"]
+    names = ["route", "plan", "fc1", "fc2", "combine"]
     per_kernel = {n: [] for n in names}
-    fc1_gbs = []
     reps = 5
     for rep in range(reps):
         for i in range(args.layers):
-            evs = hip.events(5)
-            _lib.check(_lib.lib().hb_debug_events(evs, 5), "events")
+            evs = hip.events(2 * len(names))
+            _lib.check(_lib.lib().hb_debug_events(evs, len(evs)), "events")
             step(i)
             _lib.lib().hb_debug_events(None, 0)
-            ms = [hip.elapsed_ms(evs[j], evs[j + 1]) for j in range(4)]
+            torch.cuda.synchronize()
+            ms = [hip.elapsed_ms(evs[2 * j], evs[2 * j + 1]) for j in range(len(names))]
             if rep:  # the first sweep is untimed
                 for n, v in zip(names, ms):
                     per_kernel[n].append(v)
-                fc1_gbs.append((distinct[i] + 1) * FC1_BYTES / (ms[1] * 1e-3) / 1e9)
     mean = lambda v: sum(v) / len(v)  # noqa: E731
     fc1_ms = mean(per_kernel["fc1"])
     fc1_launch_bytes = mean([(d + 1) * FC1_BYTES for d in distinct])

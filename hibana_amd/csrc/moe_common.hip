@@ -7,6 +7,146 @@
 
 namespace hb {
 
+// ---------------------------------------------------------------------------------------------------- routing
+// Top-k routing, one wavefront per row: softmax over all experts, top-k, renormalized
+// (hibana/kernels/flashnext_fused.py:278-319 of the reference), or sigmoid scores chosen by score + bias with the plain
+// scores as weights (hibana/model/nemotron/moe.py:57-121). Lane l holds experts l * per .. l * per + per - 1 in
+// registers as order-preserving 32-bit keys, so a selection round is a register scan, one wave-wide integer maximum
+// (DPP within rows of 16, four scalar reads across them) and a ballot: among equal scores the lowest lane, then the
+// lowest register, wins - the lowest expert id.
+constexpr int ROUTE_PER_LANE = 16;  // up to 1024 experts (instantiated for 8 and 16 registers a lane)
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false));   // lane ^ 1
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false));   // lane ^ 2
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, false));  // mirror within 8
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x140, 0xF, 0xF, false));  // mirror within 16
+  const uint32_t a = __builtin_amdgcn_readlane((int)x, 0), b = __builtin_amdgcn_readlane((int)x, 16);
+  const uint32_t c = __builtin_amdgcn_readlane((int)x, 32), d = __builtin_amdgcn_readlane((int)x, 48);
+  return max(max(a, b), max(c, d));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+  return v;
+}
+
+// Key of a score: larger score <=> larger key, every real key above 0 (the key of an empty register).
+__device__ __forceinline__ uint32_t score_key(float v) {
+  const int32_t bits = __builtin_bit_cast(int32_t, v);
+  return (uint32_t)(bits ^ ((bits >> 31) & 0x7fffffff)) ^ 0x80000000u;
+}
+
+struct RouteParams {
+  const float* logits;   // [m, stride]: e logits a row (sigmoid: followed by `latent` FP32 columns)
+  int64_t stride;
+  const float* bias;     // sigmoid: [e] added to the scores for the choice only
+  const int32_t* slots;  // sigmoid: row r is real iff slots[r / steps] != 0 (null: every row)
+  int steps, repeat;
+  int e, k, per, latent;
+  int32_t* ids;
+  float* weights;
+  uint16_t* lat;         // sigmoid: BF16 [m, latent], the row's latent columns
+};
+
+template <bool SIGMOID, int PER>
+__device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane) {
+  const int e = p.e, per = p.per, first = lane * per;
+  bool padded = false;
+  if (SIGMOID) {
+    const float* src = p.logits + (int64_t)r * p.stride + e;
+    for (int c = lane; c < p.latent; c += 64) p.lat[(int64_t)r * p.latent + c] = __builtin_bit_cast(uint16_t, (__bf16)src[c]);
+    padded = p.slots && p.slots[r / p.steps] == 0;
+  }
+  const float* row = p.logits + (int64_t)(padded ? 0 : r) * p.stride;  // a padded row repeats row 0's first choice
+  float val[PER];   // the weight an expert would get before renormalization
+  uint32_t key[PER];
+  if (SIGMOID) {
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      const int i = first + j;
+      const bool real = j < per && i < e;
+      val[j] = real ? 1.0f / (1.0f + expf(-row[i])) : 0.f;
+      key[j] = real ? score_key(val[j] + p.bias[i]) : 0u;
+    }
+  } else {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      const int i = first + j;
+      val[j] = j < per && i < e ? row[i] : -INFINITY;
+      mx = fmaxf(mx, val[j]);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      val[j] = j < per && first + j < e ? expf(val[j] - mx) : 0.f;
+      sum += val[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      val[j] = val[j] / sum;
+      key[j] = j < per && first + j < e ? score_key(val[j]) : 0u;
+    }
+  }
+  float total = 0.f, mine = 0.f;
+  int mine_id = 0;
+  for (int s = 0; s < p.k; s++) {
+    uint32_t best = 0;
+    int at = 0;
+    float bv = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++)
+      if (key[j] > best) {  // ascending index within the lane: the first of equals stays
+        best = key[j];
+        at = j;
+        bv = val[j];
+      }
+    const uint32_t top = wave_max_u32(best);
+    const int winner = __builtin_ctzll(__ballot(best == top));
+    const int wj = __builtin_amdgcn_readlane(at, winner);
+    const float wv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv), winner));
+    total += wv;
+    if (lane == s) {
+      mine = wv;
+      mine_id = winner * per + wj;
+    }
+    if (lane == winner) {
+#pragma unroll
+      for (int j = 0; j < PER; j++)
+        if (j == wj) key[j] = 0u;
+    }
+  }
+  if (lane < p.k) {
+    int id = mine_id;
+    float w = SIGMOID ? mine / (total + 1e-20f) : mine / total;
+    if (padded) {
+      id = p.repeat ? __builtin_amdgcn_readfirstlane(mine_id) : e;
+      w = 0.f;
+    }
+    p.ids[(int64_t)r * p.k + lane] = id;
+    p.weights[(int64_t)r * p.k + lane] = w;
+  }
+}
+
+template <bool SIGMOID, int PER>
+__global__ __launch_bounds__(64) void route_topk_kernel(RouteParams p) {
+  route_row<SIGMOID, PER>(p, blockIdx.x, threadIdx.x);
+}
+
+template <bool SIGMOID>
+static void launch_route(const RouteParams& p, int m, hipStream_t stream) {
+  if (p.per <= 8) {
+    HB_LAUNCH((route_topk_kernel<SIGMOID, 8>), dim3((unsigned)m), dim3(64), 0, stream, p);
+  } else {
+    HB_LAUNCH((route_topk_kernel<SIGMOID, 16>), dim3((unsigned)m), dim3(64), 0, stream, p);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------- expert plan
 //
 // The expert-sorted pair list of a routed call (the reference's prep kernel, hibana/kernels/csrc/w3_gemm.cu:710-782):
@@ -17,6 +157,7 @@ namespace hb {
 //   order[pos] = pair index (row * topk + slot; shared expert rows: pairs + row)
 constexpr int PLAN_THREADS = 1024;
 constexpr int PLAN_WAVES = PLAN_THREADS / 64;
+constexpr int ROUTE_FUSED_ROWS = 16;  // up to this many rows the plan workgroup routes them itself (one a wavefront)
 
 struct Scan3 {
   int a, b, c;
@@ -59,9 +200,22 @@ __device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 
   return Scan3{scratch[wave] + inc.a - v.a, scratch[PLAN_WAVES + 1 + wave] + inc.b - v.b, scratch[2 * (PLAN_WAVES + 1) + wave] + inc.c - v.c};
 }
 
-__global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* __restrict__ ids, int pairs, int e_lo, int e_n,
-                                                                int shared_rows, int32_t* __restrict__ plan, int32_t* __restrict__ order) {
+// With `route.logits` set the workgroup first routes the route.m rows itself (softmax top-k, a row a wavefront at a
+// time) into route.ids / route.weights, which `ids` then names.
+__global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
+                                                                int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
+                                                                int route_rows) {
   extern __shared__ int lds[];
+  if (route.logits) {
+    for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
+      if (route.per <= 8) {
+        route_row<false, 8>(route, r, threadIdx.x & 63);
+      } else {
+        route_row<false, 16>(route, r, threadIdx.x & 63);
+      }
+    }
+    __syncthreads();
+  }
   int* seg_count = lds;                         // [PLAN_WAVES][e_n]: pairs of expert e in segment w, then running positions
   int* start = lds + PLAN_WAVES * e_n;          // [e_n]: first sorted position of expert e
   int* scratch = start + e_n;                   // [3 * (PLAN_WAVES + 1)]
@@ -224,138 +378,15 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
   *reinterpret_cast<uint32_t*>(p.out + (int64_t)r * p.h + c) = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
 }
 
-// ---------------------------------------------------------------------------------------------------- routing
-// Top-k routing, one wavefront per row: softmax over all experts, top-k, renormalized
-// (hibana/kernels/flashnext_fused.py:278-319 of the reference), or sigmoid scores chosen by score + bias with the plain
-// scores as weights (hibana/model/nemotron/moe.py:57-121). Lane l holds experts l * per .. l * per + per - 1 in
-// registers as order-preserving 32-bit keys, so a selection round is a register scan, one wave-wide integer maximum
-// (DPP within rows of 16, four scalar reads across them) and a ballot: among equal scores the lowest lane, then the
-// lowest register, wins - the lowest expert id.
-constexpr int ROUTE_PER_LANE = 16;  // up to 1024 experts
-
-__device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
-  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false));   // lane ^ 1
-  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false));   // lane ^ 2
-  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, false));  // mirror within 8
-  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x140, 0xF, 0xF, false));  // mirror within 16
-  const uint32_t a = __builtin_amdgcn_readlane((int)x, 0), b = __builtin_amdgcn_readlane((int)x, 16);
-  const uint32_t c = __builtin_amdgcn_readlane((int)x, 32), d = __builtin_amdgcn_readlane((int)x, 48);
-  return max(max(a, b), max(c, d));
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
-  return v;
-}
-
-// Key of a score: larger score <=> larger key, every real key above 0 (the key of an empty register).
-__device__ __forceinline__ uint32_t score_key(float v) {
-  const int32_t bits = __builtin_bit_cast(int32_t, v);
-  return (uint32_t)(bits ^ ((bits >> 31) & 0x7fffffff)) ^ 0x80000000u;
-}
-
-struct RouteParams {
-  const float* logits;   // [m, stride]: e logits a row (sigmoid: followed by `latent` FP32 columns)
-  int64_t stride;
-  const float* bias;     // sigmoid: [e] added to the scores for the choice only
-  const int32_t* slots;  // sigmoid: row r is real iff slots[r / steps] != 0 (null: every row)
-  int steps, repeat;
-  int e, k, per, latent;
-  int32_t* ids;
-  float* weights;
-  uint16_t* lat;         // sigmoid: BF16 [m, latent], the row's latent columns
-};
-
-template <bool SIGMOID>
-__global__ __launch_bounds__(64) void route_topk_kernel(RouteParams p) {
-  const int r = blockIdx.x, lane = threadIdx.x;
-  const int e = p.e, per = p.per, first = lane * per;
-  bool padded = false;
-  if (SIGMOID) {
-    const float* src = p.logits + (int64_t)r * p.stride + e;
-    for (int c = lane; c < p.latent; c += 64) p.lat[(int64_t)r * p.latent + c] = __builtin_bit_cast(uint16_t, (__bf16)src[c]);
-    padded = p.slots && p.slots[r / p.steps] == 0;
-  }
-  const float* row = p.logits + (int64_t)(padded ? 0 : r) * p.stride;  // a padded row repeats row 0's first choice
-  float val[ROUTE_PER_LANE];   // the weight an expert would get before renormalization
-  uint32_t key[ROUTE_PER_LANE];
-  if (SIGMOID) {
-#pragma unroll
-    for (int j = 0; j < ROUTE_PER_LANE; j++) {
-      const int i = first + j;
-      const bool real = j < per && i < e;
-      val[j] = real ? 1.0f / (1.0f + expf(-row[i])) : 0.f;
-      key[j] = real ? score_key(val[j] + p.bias[i]) : 0u;
-    }
-  } else {
-    float mx = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < ROUTE_PER_LANE; j++) {
-      const int i = first + j;
-      val[j] = j < per && i < e ? row[i] : -INFINITY;
-      mx = fmaxf(mx, val[j]);
-    }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
-    float sum = 0.f;
-#pragma unroll
-    for (int j = 0; j < ROUTE_PER_LANE; j++) {
-      val[j] = j < per && first + j < e ? expf(val[j] - mx) : 0.f;
-      sum += val[j];
-    }
-    sum = wave_sum(sum);
-#pragma unroll
-    for (int j = 0; j < ROUTE_PER_LANE; j++) {
-      val[j] = val[j] / sum;
-      key[j] = j < per && first + j < e ? score_key(val[j]) : 0u;
-    }
-  }
-  float total = 0.f, mine = 0.f;
-  int mine_id = 0;
-  for (int s = 0; s < p.k; s++) {
-    uint32_t best = 0;
-    int at = 0;
-    float bv = 0.f;
-#pragma unroll
-    for (int j = 0; j < ROUTE_PER_LANE; j++)
-      if (key[j] > best) {  // ascending index within the lane: the first of equals stays
-        best = key[j];
-        at = j;
-        bv = val[j];
-      }
-    const uint32_t top = wave_max_u32(best);
-    const int winner = __builtin_ctzll(__ballot(best == top));
-    const int wj = __builtin_amdgcn_readlane(at, winner);
-    const float wv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv), winner));
-    total += wv;
-    if (lane == s) {
-      mine = wv;
-      mine_id = winner * per + wj;
-    }
-    if (lane == winner) {
-#pragma unroll
-      for (int j = 0; j < ROUTE_PER_LANE; j++)
-        if (j == wj) key[j] = 0u;
-    }
-  }
-  if (lane < p.k) {
-    int id = mine_id;
-    float w = SIGMOID ? mine / (total + 1e-20f) : mine / total;
-    if (padded) {
-      id = p.repeat ? __builtin_amdgcn_readfirstlane(mine_id) : e;
-      w = 0.f;
-    }
-    p.ids[(int64_t)r * p.k + lane] = id;
-    p.weights[(int64_t)r * p.k + lane] = w;
-  }
-}
-
 // ---------------------------------------------------------------------------------------------------- host side
 static std::vector<hipEvent_t> g_events;
 static size_t g_event_next = 0;
-void moe_mark(hipStream_t stream) {
-  if (g_event_next < g_events.size()) (void)hipEventRecord(g_events[g_event_next++], stream);
+bool moe_next_events(hipEvent_t* start, hipEvent_t* stop) {
+  if (g_event_next + 1 >= g_events.size()) return false;
+  *start = g_events[g_event_next];
+  *stop = g_events[g_event_next + 1];
+  g_event_next += 2;
+  return true;
 }
 
 void pick_shape(int n_blocks, int chunks, int64_t slots, int want, int* ks, int* nbw) {
@@ -394,15 +425,36 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream) {
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
-  moe_mark(stream);
-  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order);
-  moe_mark(stream);
+  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0);
+  return HB_OK;
+}
+
+int moe_check_route(int m, int e, int k) { return m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE ? HB_EINVAL : HB_OK; }
+
+int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
+                          const MoeWorkspace& ws, hipStream_t stream) {
+  if (int err = moe_check_route(m, e, topk)) return err;
+  RouteParams rp{};
+  rp.logits = logits;
+  rp.stride = e;
+  rp.e = e;
+  rp.k = topk;
+  rp.per = (e + 63) / 64;
+  rp.ids = ids;
+  rp.weights = weights;
+  const int64_t pairs = (int64_t)m * topk;
+  if (m > ROUTE_FUSED_ROWS) {  // many rows: a wavefront a row over the whole device, then the plan
+    launch_route<false>(rp, m, stream);
+    return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream);
+  }
+  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
+  if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
+  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m);
   return HB_OK;
 }
 
 void moe_launch_combine(const CombineParams& c, hipStream_t stream) {
-  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)c.m, (unsigned)((c.h + COMBINE_SPAN - 1) / COMBINE_SPAN)), dim3(256), 0, stream, c);
-  moe_mark(stream);
+  HB_LAUNCH(moe_combine_kernel, dim3((unsigned)c.m, (unsigned)((c.h + COMBINE_SPAN - 1) / COMBINE_SPAN)), dim3(256), 0, stream, c);
 }
 
 }  // namespace hb
@@ -446,7 +498,7 @@ extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, i
   p.per = (e + 63) / 64;
   p.ids = ids;
   p.weights = weights;
-  hipLaunchKernelGGL(route_topk_kernel<false>, dim3((unsigned)m), dim3(64), 0, as_stream(stream), p);
+  launch_route<false>(p, m, as_stream(stream));
   return launch_status();
 }
 
@@ -469,7 +521,7 @@ extern "C" int hb_route_sigmoid_topk(const float* fused, int64_t stride, const f
   p.ids = ids;
   p.weights = weights;
   p.lat = static_cast<uint16_t*>(lat);
-  hipLaunchKernelGGL(route_topk_kernel<true>, dim3((unsigned)m), dim3(64), 0, as_stream(stream), p);
+  launch_route<true>(p, m, as_stream(stream));
   return launch_status();
 }
 

@@ -202,7 +202,7 @@ static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipS
   pick_shape(p.n_blocks, p.chunks, busy_slots, 4096, &p.ks, &p.nbw);
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
-  hipLaunchKernelGGL(nvfp4_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
+  HB_LAUNCH(nvfp4_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
   return HB_OK;
 }
 
@@ -306,9 +306,7 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
   f2.out_stride = ex->hidden_out;
   f2.out_bf16 = pairs_bf16;
   if (int e = ex->gated ? launch_nvfp4<EPI_FC1_GATED>(p, slots, est, stream) : launch_nvfp4<EPI_FC1_RELU2>(p, slots, est, stream)) return e;
-  moe_mark(stream);
   if (int e = launch_nvfp4<EPI_FC2>(f2, slots, est, stream)) return e;
-  moe_mark(stream);
   return launch_status();
 }
 

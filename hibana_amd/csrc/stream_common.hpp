@@ -3,6 +3,8 @@
 // LDS, and the host-side helpers of a routed call (workspace, plan launch, combine launch).
 #pragma once
 
+#include <hip/hip_ext.h>
+
 #include "common.hpp"
 
 namespace hb {
@@ -202,6 +204,11 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
 // Enqueue the plan kernel; HB_EINVAL if the expert count does not fit its LDS.
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream);
 
+// Softmax top-k routing of `m` rows of `e` logits into ids / weights [m, topk], then the plan of those ids: one launch
+// for up to a few dozen rows, two beyond.
+int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
+                          const MoeWorkspace& ws, hipStream_t stream);
+
 struct CombineParams {
   const void* pairs;      // [m * topk (+ m), h] FP32 or BF16
   int pairs_bf16;
@@ -218,8 +225,19 @@ struct CombineParams {
 };
 void moe_launch_combine(const CombineParams& c, hipStream_t stream);
 
-// Measurement hook: records the caller's next event (if any) on the stream.
-void moe_mark(hipStream_t stream);
+// Measurement hook: the caller's next (start, stop) event pair, if any is armed. A kernel launched through HB_LAUNCH
+// then carries the pair: the runtime stamps the two events with that kernel's own begin and end.
+bool moe_next_events(hipEvent_t* start, hipEvent_t* stop);
+
+#define HB_LAUNCH(kernel, grid, block, lds, stream, ...)                                            \
+  do {                                                                                              \
+    hipEvent_t hb_e0_, hb_e1_;                                                                      \
+    if (hb::moe_next_events(&hb_e0_, &hb_e1_)) {                                                    \
+      hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, hb_e0_, hb_e1_, 0, __VA_ARGS__);      \
+    } else {                                                                                        \
+      hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                            \
+    }                                                                                               \
+  } while (0)
 
 // Wavefronts per workgroup of a stream launch: K is split until the launch has about `want` wavefronts, keeping at
 // least four chunks per wavefront; what is left of a 4-wavefront workgroup takes neighbouring 64-row blocks.

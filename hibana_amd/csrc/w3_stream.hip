@@ -147,7 +147,7 @@ static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Lau
   if (p.ks * p.nbw > 16 || p.ks > p.chunks) return HB_EINVAL;
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
-  hipLaunchKernelGGL(w3_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
+  HB_LAUNCH(w3_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
   return HB_OK;
 }
 
@@ -207,13 +207,25 @@ int check_experts(const hb_w3_experts* ex) {
 
 // plan -> fc1 -> fc2 (-> combine): `out_pairs` receives fc2's per-pair outputs (the workspace's y unless the caller
 // wants the pairs themselves).
+struct Routing {  // set: the chain routes `logits` [m, e] itself into the caller's ids / weights
+  const float* logits;
+  int e;
+  int32_t* ids;
+  float* weights;
+};
+
 int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void* x, const int32_t* ids, int m, int topk,
-                const MoeWorkspace& ws, void* out_pairs, int pairs_bf16, hipStream_t stream) {
+                const MoeWorkspace& ws, void* out_pairs, int pairs_bf16, hipStream_t stream, const Routing* route = nullptr) {
   const int64_t pairs = (int64_t)m * topk;
   const int shared_rows = shared ? m : 0;
   const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows);
   if (slots > 65535) return HB_EINVAL;
-  if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, shared_rows, ws, stream)) return e;
+  if (route) {
+    if (int e = moe_launch_route_plan(route->logits, m, route->e, topk, route->ids, route->weights, ex->base, ex->experts, shared_rows, ws, stream))
+      return e;
+  } else if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, shared_rows, ws, stream)) {
+    return e;
+  }
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
   const int64_t est = pairs < 2 * ex->experts ? (pairs + 1) / 2 + (shared_rows + 15) / 16 : slots;  // rough number of busy slots
   StreamParams p{};
@@ -261,9 +273,7 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   f2.out_bf16 = pairs_bf16;
   const Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
   if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) return e;
-  moe_mark(stream);
   if (int e = launch_stream<EPI_FC2>(f2, slots, est, l2, stream)) return e;
-  moe_mark(stream);
   return launch_status();
 }
 
@@ -299,9 +309,9 @@ extern "C" int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32
   return launch_status();
 }
 
-extern "C" int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
-                               const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
-                               size_t workspace_bytes, void* stream) {
+static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x, const int32_t* ids,
+                     const float* weights, int m, int topk, void* out, void* workspace, size_t workspace_bytes, void* stream,
+                     const Routing* route) {
   if (int e = check_experts(routed)) return e;
   if (shared) {
     if (int e = check_experts(shared)) return e;
@@ -313,7 +323,7 @@ extern "C" int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts*
   if (m <= 0 || topk <= 0) return HB_EINVAL;
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, shared ? 1 : 0);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
-  if (int e = run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream))) return e;
+  if (int e = run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream), route)) return e;
   CombineParams c{};
   c.pairs = ws.y;
   c.ids = ids;
@@ -336,3 +346,16 @@ extern "C" int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts*
   return launch_status();
 }
 
+extern "C" int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                               const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, nullptr);
+}
+
+extern "C" int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                                      const float* logits, int experts_total, int m, int topk, int32_t* ids, float* weights, void* out,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  if (!logits) return HB_ENULL;
+  const Routing route{logits, experts_total, ids, weights};
+  return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, &route);
+}

@@ -170,6 +170,32 @@ def moe_layer(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: t
     return out
 
 
+def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, topk: int, shared: W3Experts | None = None,
+                     gate_vec: torch.Tensor | None = None, return_routing: bool = False):
+    """`moe_layer` from the router's FP32 logits [M, E_total]: softmax top-k routing (ops.route_topk's arithmetic) runs
+    in the same chain - inside the planning workgroup up to 16 rows, so that a decode step is four launches -
+    (hibana/model/flashnext/moe.py:122-144,177-192). With `return_routing`, also the ids and weights it used."""
+    if x.dtype != torch.bfloat16 or x.ndim != 2 or x.shape[1] != experts.shape13[1]:
+        raise ValueError("moe_layer_logits: x must be BF16 [M, hidden]")
+    if logits.ndim != 2 or logits.shape[0] != x.shape[0] or logits.dtype != torch.float32:
+        raise ValueError("moe_layer_logits: logits must be FP32 [M, experts]")
+    _lib.need_gpu(x, logits)
+    m, e_total = logits.shape
+    out = torch.empty((m, experts.shape2[0]), dtype=torch.bfloat16, device=x.device)
+    ids = torch.empty((m, topk), dtype=torch.int32, device=x.device)
+    wt = torch.empty((m, topk), dtype=torch.float32, device=x.device)
+    if m:
+        st = _struct(experts)
+        sh = _struct(shared) if shared is not None else None
+        need = _lib.lib().hb_w3_moe_workspace_bytes(m, topk, C.byref(st), int(shared is not None))
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+        gv = None if gate_vec is None else gate_vec.float().contiguous()
+        _lib.check(_lib.lib().hb_w3_moe_layer_logits(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(x.contiguous()),
+                                                     _lib.ptr(logits.contiguous()), e_total, m, topk, _lib.ptr(ids), _lib.ptr(wt), _lib.ptr(out),
+                                                     _lib.ptr(ws), need, _lib.stream()), "moe_layer_logits")
+    return (out, ids, wt) if return_routing else out
+
+
 def unswizzle_batched(swizzled: torch.Tensor, rows: int, groups: int) -> torch.Tensor:
     """[E, ...] block scales in the 128x4 interleave -> float8_e4m3fn [E, rows, groups] (hibana/kernels/w3_moe.py:97-102)."""
     from hibana_amd.weights.modelopt import unswizzle_block_scales

@@ -36,10 +36,11 @@ const char* hb_error_string(int code);
  * Returns HB_EINVAL for an unknown key. Not thread-safe against concurrent launches. */
 int hb_tune(const char* key, int value);
 
-/* Measurement hook (no counterpart in the reference): `events` are hipEvent_t handles the caller created; the next
- * routed-expert call (hb_w3_moe / hb_w3_moe_layer) records them, in order, at the five boundaries of its chain:
- * before the plan kernel, after it, after fc1, after fc2, after the combine. count = 0 switches the hook off.
- * Not for captured graphs. */
+/* Measurement hook (no counterpart in the reference): `events` are hipEvent_t handles the caller created, taken in
+ * (start, stop) pairs: each kernel the next calls launch carries the next pair, and the runtime stamps the two events
+ * with that kernel's own begin and end (hipEventElapsedTime(start, stop) is the kernel's duration). A routed call
+ * launches plan, fc1, fc2 and, when it sums, combine; hb_w3_moe_layer_logits launches the routing kernel first when it
+ * has more than 16 rows. count = 0 switches the hook off. Not for captured graphs. */
 int hb_debug_events(void* const* events, int count);
 
 /* ------------------------------------------------------------------------------------------------------------------
@@ -127,6 +128,14 @@ int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32_t* ids, co
 int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
                     const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
                     size_t workspace_bytes, void* stream);
+
+/* The same layer from the router's logits (float32 [m, experts_total]): softmax top-k routing as
+ * hb_route_softmax_topk, written to ids int32 [m, topk] and weights float32 [m, topk] (caller's buffers), then the
+ * chain of hb_w3_moe_layer. Up to 16 rows the routing runs inside the planning workgroup (one launch fewer).
+ * ref: MoeLayer.__call__ with its route step, hibana/model/flashnext/moe.py:122-144,177-192. */
+int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec,
+                           const void* x, const float* logits, int experts_total, int m, int topk, int32_t* ids,
+                           float* weights, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* out = bf16( bf16(sum over the row's local slots of w * pairs) + g * shared ) from unsummed pair outputs (FP32 or,
  * pairs_bf16 != 0, BF16) [m * topk, h]; shared BF16 [m, h] or NULL; gate_vec float32 [h] or NULL (then g = 1; x

@@ -147,6 +147,23 @@ def test_layer_with_shared_expert(gated, m, with_gate):
     assert torch.equal(w3_moe.moe_layer(ex, x.cuda(), ids.cuda(), weights.cuda()), w3_moe.w3_moe(ex, x.cuda(), ids.cuda(), weights.cuda()))
 
 
+@pytest.mark.parametrize("m", [1, 16, 17, 32, 200])
+def test_layer_from_logits_is_route_then_layer(gated, m):
+    """Routing inside the chain (in the planning workgroup up to 16 rows, its own launch beyond) gives the bits of
+    ops.route_topk followed by moe_layer."""
+    from hibana_amd.kernels import ops, w3_moe
+    ex, _ = gated
+    shared_ex, _ = random_experts(1, H, I, True, 78)
+    g = torch.Generator().manual_seed(m)
+    x = torch.randn(m, H, generator=g).bfloat16().cuda()
+    logits = (torch.randn(m, E, generator=g) * 2).cuda()
+    ids, wts = ops.route_topk(logits, TOPK)
+    want = w3_moe.moe_layer(ex, x, ids, wts, shared=shared_ex)
+    got, got_ids, got_w = w3_moe.moe_layer_logits(ex, x, logits, TOPK, shared=shared_ex, return_routing=True)
+    assert torch.equal(got_ids, ids) and torch.equal(got_w, wts) and torch.equal(got, want)
+    assert torch.equal(w3_moe.moe_layer_logits(ex, x, logits, TOPK), w3_moe.moe_layer(ex, x, ids, wts))
+
+
 @pytest.mark.parametrize("m", [1, 16, 150])
 def test_relu2_experts_with_their_own_fc2_codebook(relu2, m):
     """The latent experts' geometry in small (fc1 = up alone, h = relu(up)^2, top 6 of 8, a zero level in fc2)."""
