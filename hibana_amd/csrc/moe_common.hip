@@ -204,7 +204,7 @@ __device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 
 // time) into route.ids / route.weights, which `ids` then names.
 __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
                                                                 int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
-                                                                int route_rows) {
+                                                                int route_rows, int slot_rows) {
   extern __shared__ int lds[];
   if (route.logits) {
     for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
     int count = 0;
     if (e < e_n)
       for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
-    const int my_slots = (count + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
+    const int my_slots = (count + slot_rows - 1) / slot_rows;
     Scan3 tot;
     const Scan3 at = block_exclusive_scan3(Scan3{count, count > 0 ? 1 : 0, my_slots}, scratch, &tot);
     const int my_start = kept + at.a, my_slot = slots + at.c;
@@ -247,8 +247,8 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
       for (int s = 0; s < my_slots; s++) {
         int32_t* entry = plan + PLAN_HEADER + 4 * (my_slot + s);
         entry[0] = e;
-        entry[1] = my_start + s * ROWS_PER_SLOT;
-        entry[2] = min(ROWS_PER_SLOT, count - s * ROWS_PER_SLOT);
+        entry[1] = my_start + s * slot_rows;
+        entry[2] = min(slot_rows, count - s * slot_rows);
         entry[3] = 0;
       }
       // turn the per-segment counts into the first position of each segment's run
@@ -265,12 +265,12 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   }
   __syncthreads();
   // the shared expert's rows follow the routed pairs
-  const int shared_slots = (shared_rows + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
+  const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
   for (int s = threadIdx.x; s < shared_slots; s += PLAN_THREADS) {
     int32_t* entry = plan + PLAN_HEADER + 4 * (slots + s);
     entry[0] = -1;
-    entry[1] = kept + s * ROWS_PER_SLOT;
-    entry[2] = min(ROWS_PER_SLOT, shared_rows - s * ROWS_PER_SLOT);
+    entry[1] = kept + s * slot_rows;
+    entry[2] = min(slot_rows, shared_rows - s * slot_rows);
     entry[3] = 0;
   }
   for (int r = threadIdx.x; r < shared_rows; r += PLAN_THREADS) order[kept + r] = pairs + r;
@@ -398,9 +398,9 @@ void pick_shape(int n_blocks, int chunks, int64_t slots, int want, int* ks, int*
   *nbw = b;
 }
 
-int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows) {
-  const int64_t routed = pairs < pairs / ROWS_PER_SLOT + experts ? pairs : pairs / ROWS_PER_SLOT + experts;
-  return routed + (shared_rows + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
+int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows, int slot_rows) {
+  const int64_t routed = pairs < pairs / slot_rows + experts ? pairs : pairs / slot_rows + experts;
+  return routed + (shared_rows + slot_rows - 1) / slot_rows;
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -414,7 +414,7 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
     off += align256(bytes);
     return ptr;
   };
-  w.plan = static_cast<int32_t*>(take((PLAN_HEADER + 4 * moe_max_slots(pairs, experts, shared ? m : 0)) * sizeof(int32_t)));
+  w.plan = static_cast<int32_t*>(take((PLAN_HEADER + 4 * moe_max_slots(pairs, experts, shared ? m : 0, ROWS_PER_SLOT)) * sizeof(int32_t)));
   w.order = static_cast<int32_t*>(take(rows * sizeof(int32_t)));
   w.h = static_cast<uint16_t*>(take((size_t)rows * inter * sizeof(uint16_t)));
   w.y = static_cast<float*>(take((size_t)rows * hidden_out * sizeof(float)));
@@ -422,10 +422,10 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
   return w;
 }
 
-int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream) {
+int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream, int slot_rows) {
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
-  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0);
+  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0, slot_rows);
   return HB_OK;
 }
 
@@ -445,11 +445,11 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   const int64_t pairs = (int64_t)m * topk;
   if (m > ROUTE_FUSED_ROWS) {  // many rows: a wavefront a row over the whole device, then the plan
     launch_route<false>(rp, m, stream);
-    return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream);
+    return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, ROWS_PER_SLOT);
   }
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
-  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m);
+  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, ROWS_PER_SLOT);
   return HB_OK;
 }
 

@@ -9,6 +9,8 @@
 //   bytes 4096..4607  scales: 32 B per row-in-tile r at 4096 + 32 r: byte 8 nt + b is the E4M3 scale of row
 //                     64 nb + 16 nt + r, block 8 c + b.
 // Codes expand with v_cvt_scalef32_pk_bf16_fp4 (two weights per instruction, exact).
+#include <string.h>
+
 #include "stream_common.hpp"
 
 namespace hb {
@@ -206,6 +208,177 @@ static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipS
   return HB_OK;
 }
 
+// ------------------------------------------------------------------------------------- prefill: slots of 128 rows
+// When an expert has many rows (a prefill chunk: dozens of rows an expert) the grouped product is a dense contraction
+// and belongs on the MFMA pipe: one workgroup of four wavefronts takes a slot of up to 128 activation rows of one
+// expert and four neighbouring 64-row weight blocks (one a wavefront), all of K. Per 128-k chunk
+//   - the slot's activation tile (128 rows x 128 k BF16, 32 KB) is brought into LDS by LDS-direct loads
+//     (global_load_lds_dwordx4: no registers in between), double buffered, pieces XOR-swizzled within a row so that the
+//     A fragment reads of sixteen rows hit sixteen different bank groups;
+//   - each wavefront expands its block's codes ONCE to scaled BF16 (e2m1 * e4m3 is exact in BF16) and reuses the four B
+//     fragments for every 16-row tile of the slot: v_mfma_f32_16x16x32_bf16, accumulators for 8 x 4 tiles in registers.
+// The K order inside one MFMA follows the tile layout's ownership (lane q holds k = 4q..4q+3 of both 16-blocks of a
+// 32-step), which the A fragment mirrors with two 8-byte LDS reads.
+constexpr int TILE_ROWS = 128;
+constexpr int TILE_MT = TILE_ROWS / 16;
+constexpr int TILE_BUF = TILE_ROWS * 256;  // bytes of one activation buffer
+
+__device__ __forceinline__ uint32_t scaled_pair(uint32_t codes, int byte, float scale) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  f32x2_t w;
+  switch (byte) {  // the byte selector is an immediate of the instruction
+    case 0: w = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 0); break;
+    case 1: w = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 1); break;
+    case 2: w = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 2); break;
+    default: w = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 3); break;
+  }
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_v;
+  const bf16x2_v packed = {(__bf16)(w.x * scale), (__bf16)(w.y * scale)};
+  return __builtin_bit_cast(uint32_t, packed);
+}
+
+// The B fragment of k-step s (blocks 2s, 2s + 1) of one 16-row tile: its code dword and the two block scales.
+__device__ __forceinline__ bf16x8_t scaled_fragment(uint32_t codes, float s_even, float s_odd) {
+  u32x4_t packed;
+  packed.x = scaled_pair(codes, 0, s_even);
+  packed.y = scaled_pair(codes, 1, s_even);
+  packed.z = scaled_pair(codes, 2, s_odd);
+  packed.w = scaled_pair(codes, 3, s_odd);
+  return __builtin_bit_cast(bf16x8_t, packed);
+}
+
+template <int EPI>
+__device__ __forceinline__ void stage_tile(const StreamParams& p, const int32_t* rowtab, uint8_t* buf, int chunk, int tiles, int wave, int lane) {
+  // a wavefront brings rows wave * 32 .. + 31 in eight instructions of four rows each: lane l lands at byte 16 l of the
+  // instruction's kilobyte, i.e. row (l >> 4), slot (l & 15) of it, and therefore fetches piece slot ^ (row & 15)
+  const int sub = lane >> 4, slot = lane & 15;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const int row = wave * 32 + j * 4 + sub;
+    if (wave * 32 + j * 4 < tiles * 16) {  // wave-uniform: whole 16-row tiles past the slot's rows are never read
+      const uint16_t* src = p.a + (int64_t)rowtab[row] * p.a_stride + (int64_t)chunk * 128 + ((slot ^ (row & 15)) << 3);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
+                                       (__attribute__((address_space(3))) void*)(buf + (wave * 32 + j * 4) * 256), 16, 0, 0);
+    }
+  }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(256, 2) void nvfp4_tile_kernel(StreamParams p) {
+  extern __shared__ __align__(16) uint8_t tile_lds[];  // two activation buffers, then the row table
+  if ((int)blockIdx.y >= p.plan[0]) return;
+  const Slot sl = slot_of<EPI>(p, blockIdx.y);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int nb = blockIdx.x * 4 + wave;
+  const bool active = nb < p.n_blocks;
+  const int tiles = (sl.rows + 15) >> 4;
+  int32_t* rowtab = reinterpret_cast<int32_t*>(tile_lds + 2 * TILE_BUF);
+  if (threadIdx.x < TILE_ROWS) {  // the source row of each slot row (rows past the last repeat it)
+    int64_t arow = sl.p0 + min((int)threadIdx.x, sl.rows - 1);
+    if (epi_gathers(EPI)) {
+      const int pair = p.order[arow];
+      arow = pair < p.pairs ? pair / p.topk : pair - p.pairs;
+    }
+    rowtab[threadIdx.x] = (int)arow;
+  }
+  __syncthreads();
+  f32x4_t acc[TILE_MT][4];
+#pragma unroll
+  for (int t = 0; t < TILE_MT; t++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) acc[t][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const uint8_t* blk = sl.w + (int64_t)(active ? nb : 0) * p.chunks * NVFP4_BLOCK_BYTES;
+  Fp4Chunk cur, nxt;
+  load_fp4_chunk(cur, blk, lane, r16);
+  stage_tile<EPI>(p, rowtab, tile_lds, 0, tiles, wave, lane);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int c = 0; c < p.chunks; c++) {
+    uint8_t* buf = tile_lds + (c & 1) * TILE_BUF;
+    if (c + 1 < p.chunks) {
+      load_fp4_chunk(nxt, blk + (int64_t)(c + 1) * NVFP4_BLOCK_BYTES, lane, r16);
+      stage_tile<EPI>(p, rowtab, tile_lds + ((c + 1) & 1) * TILE_BUF, c + 1, tiles, wave, lane);
+    }
+    const u32x4_t w[4] = {cur.w0, cur.w1, cur.w2, cur.w3};
+    const uint32_t sc[8] = {cur.s0.x, cur.s0.y, cur.s0.z, cur.s0.w, cur.s1.x, cur.s1.y, cur.s1.z, cur.s1.w};  // tile nt: dwords 2nt, 2nt + 1
+#pragma unroll
+    for (int s = 0; s < 4; s++) {  // 32-k steps of the chunk: blocks 2s, 2s + 1
+      bf16x8_t b[4];
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++) {
+        const uint32_t sd = sc[2 * nt + (s >> 1)];
+        const float s_even = (s & 1) ? __builtin_amdgcn_cvt_f32_fp8(sd, 2) : __builtin_amdgcn_cvt_f32_fp8(sd, 0);
+        const float s_odd = (s & 1) ? __builtin_amdgcn_cvt_f32_fp8(sd, 3) : __builtin_amdgcn_cvt_f32_fp8(sd, 1);
+        b[nt] = scaled_fragment(w[nt][s], s_even, s_odd);
+      }
+      // lane (q, r16): row 16 t + r16, k = 32 s + 4 q .. + 3 (piece 4 s + q / 2, half q & 1) and the same 16 further
+      const int half = (q & 1) << 3;
+      const int slot_lo = ((4 * s + (q >> 1)) ^ r16) << 4, slot_hi = ((4 * s + 2 + (q >> 1)) ^ r16) << 4;
+#pragma unroll
+      for (int t = 0; t < TILE_MT; t++) {
+        if (t < tiles) {
+          const uint8_t* row = buf + (16 * t + r16) * 256 + half;
+          u32x4_t a;
+          const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(row + slot_lo), hi = *reinterpret_cast<const u32x2_t*>(row + slot_hi);
+          a.x = lo.x;
+          a.y = lo.y;
+          a.z = hi.x;
+          a.w = hi.y;
+          const bf16x8_t af = __builtin_bit_cast(bf16x8_t, a);
+#pragma unroll
+          for (int nt = 0; nt < 4; nt++) acc[t][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, b[nt], acc[t][nt], 0, 0, 0);
+        }
+      }
+    }
+    cur = nxt;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's LDS-direct loads have landed before it signals
+    __syncthreads();                                   // the next buffer is complete and this one is free to refill
+  }
+  if (!active) return;
+  // accumulator register r of lane (q, r16) of tile (t, nt): slot row 16 t + 4 q + r, weight row nb * 64 + 16 nt + r16
+#pragma unroll
+  for (int t = 0; t < TILE_MT; t++) {
+    if (t < tiles) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int i = 16 * t + 4 * q + r;
+        if (i < sl.rows) {
+          const int64_t pos = sl.p0 + i;
+          if (EPI == EPI_FC1_GATED) {
+#pragma unroll
+            for (int g = 0; g < 2; g++) {
+              const float up = through_bf16(acc[t][2 * g][r] * sl.scalar), gate = through_bf16(acc[t][2 * g + 1][r] * sl.scalar);
+              reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * g + r16] = bf16_of(silu(gate) * up);
+            }
+          } else {
+            const int64_t at = (EPI == EPI_FC2 ? (int64_t)p.order[pos] : pos) * p.out_stride + nb * 64 + r16;
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) {
+              const float y = acc[t][nt][r] * sl.scalar;
+              if (EPI == EPI_FC1_RELU2) {
+                const float h = fmaxf(through_bf16(y), 0.f);
+                reinterpret_cast<uint16_t*>(p.out)[at + 16 * nt] = bf16_of(h * h);
+              } else if (p.out_bf16) {
+                reinterpret_cast<uint16_t*>(p.out)[at + 16 * nt] = bf16_of(y);
+              } else {
+                reinterpret_cast<float*>(p.out)[at + 16 * nt] = y;
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int EPI>
+static int launch_nvfp4_tile(StreamParams& p, int64_t slots, hipStream_t stream) {
+  const dim3 grid((unsigned)((p.n_blocks + 3) / 4), (unsigned)slots);
+  HB_LAUNCH(nvfp4_tile_kernel<EPI>, grid, dim3(256), 2 * TILE_BUF + TILE_ROWS * sizeof(int32_t), stream, p);
+  return HB_OK;
+}
+
 static inline unsigned grid_for(int64_t threads) { return (unsigned)((threads + 255) / 256); }
 
 }  // namespace hb
@@ -262,6 +435,9 @@ extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float glob
 // ------------------------------------------------------------------------------------------------ routed experts
 namespace {
 
+constexpr int TILE_DENSE_ROWS = 24;  // average rows an expert from which the tile kernel serves the call
+int g_nvfp4_tile = 0;                // experiments: 1 forces the tile kernel, 2 the stream (hb_tune "nvfp4_tile")
+
 int check_experts(const hb_nvfp4_experts* ex) {
   if (!ex) return HB_ENULL;
   if (!ex->fc1 || !ex->fc1_scale2 || !ex->fc2 || !ex->fc2_scale2) return HB_ENULL;
@@ -275,9 +451,13 @@ int check_experts(const hb_nvfp4_experts* ex) {
 int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, int m, int topk, const MoeWorkspace& ws, void* out_pairs,
                 int pairs_bf16, hipStream_t stream) {
   const int64_t pairs = (int64_t)m * topk;
-  const int64_t slots = moe_max_slots(pairs, ex->experts, 0);
+  // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel; below that the
+  // 16-row slots of the weight stream
+  const bool dense = g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && pairs >= (int64_t)ex->experts * TILE_DENSE_ROWS);
+  const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
+  const int64_t slots = moe_max_slots(pairs, ex->experts, 0, slot_rows);
   if (slots > 65535) return HB_EINVAL;
-  if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, 0, ws, stream)) return e;
+  if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, 0, ws, stream, slot_rows)) return e;
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
   const int64_t est = pairs < 2 * ex->experts ? (pairs + 1) / 2 : slots;
   StreamParams p{};
@@ -305,12 +485,23 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
   f2.out = out_pairs;
   f2.out_stride = ex->hidden_out;
   f2.out_bf16 = pairs_bf16;
+  if (dense) {
+    if (int e = ex->gated ? launch_nvfp4_tile<EPI_FC1_GATED>(p, slots, stream) : launch_nvfp4_tile<EPI_FC1_RELU2>(p, slots, stream)) return e;
+    if (int e = launch_nvfp4_tile<EPI_FC2>(f2, slots, stream)) return e;
+    return launch_status();
+  }
   if (int e = ex->gated ? launch_nvfp4<EPI_FC1_GATED>(p, slots, est, stream) : launch_nvfp4<EPI_FC1_RELU2>(p, slots, est, stream)) return e;
   if (int e = launch_nvfp4<EPI_FC2>(f2, slots, est, stream)) return e;
   return launch_status();
 }
 
 }  // namespace
+
+int hb::nvfp4_tune(const char* key, int value) {
+  if (strcmp(key, "nvfp4_tile")) return HB_EINVAL;
+  g_nvfp4_tile = value;
+  return HB_OK;
+}
 
 extern "C" size_t hb_nvfp4_moe_workspace_bytes(int m, int topk, const hb_nvfp4_experts* routed) {
   if (!routed || m <= 0 || topk <= 0 || check_experts(routed) != HB_OK) return 0;

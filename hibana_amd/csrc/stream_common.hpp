@@ -199,10 +199,11 @@ struct MoeWorkspace {
   size_t bytes;
 };
 
-int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows);
+int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows, int slot_rows = ROWS_PER_SLOT);
 MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int hidden_out, int shared);
 // Enqueue the plan kernel; HB_EINVAL if the expert count does not fit its LDS.
-int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream);
+int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream,
+                    int slot_rows = ROWS_PER_SLOT);
 
 // Softmax top-k routing of `m` rows of `e` logits into ids / weights [m, topk], then the plan of those ids: one launch
 // for up to a few dozen rows, two beyond.
@@ -242,5 +243,8 @@ bool moe_next_events(hipEvent_t* start, hipEvent_t* stop);
 // Wavefronts per workgroup of a stream launch: K is split until the launch has about `want` wavefronts, keeping at
 // least four chunks per wavefront; what is left of a 4-wavefront workgroup takes neighbouring 64-row blocks.
 void pick_shape(int n_blocks, int chunks, int64_t slots, int want, int* ks, int* nbw);
+
+// hb_tune keys of the NVFP4 kernels ("nvfp4_tile": 1 forces the tile kernel, 2 the stream, 0 the built-in choice).
+int nvfp4_tune(const char* key, int value);
 
 }  // namespace hb

@@ -169,7 +169,7 @@ extern "C" int hb_tune(const char* key, int value) {
       *t.slot = value;
       return HB_OK;
     }
-  return HB_EINVAL;
+  return nvfp4_tune(key, value);
 }
 
 extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, void* y, void* stream) {
