@@ -86,6 +86,75 @@ def cpu_baseline(layer, x, ids, weights, budget_s: float = 15.0):
     return info, torch.from_numpy(out.view(np.int16).copy()).view(torch.bfloat16)
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def latent_prefill(args) -> int:
+    """BASELINE config 4 (not the headline line; `--config 4`): the NVFP4 latent-MoE layer on a prefill chunk of 2048
+    tokens - hidden 4096 projected to latent 1024, 512 ReLU^2 experts of intermediate 2688, top-22 by sigmoid scores.
+    A step is the whole block (fused router|fc1_latent GEMM, routing, plan, the two expert GEMMs on the MFMA tile kernel,
+    combine, fc2_latent GEMM); the roofline entry is the fc1 expert GEMM against the dense BF16 MFMA peak."""
+    import torch
+
+    from hibana_amd import _lib, synthetic
+    from hibana_amd.model import nemotron_moe
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tokens, hidden, latent, inter, experts, topk = 2048, 4096, 1024, 2688, 512, 22
+    g = torch.Generator(device=dev).manual_seed(5)
+    ex = synthetic.nvfp4_experts(experts, latent, inter, 11, dev)
+    router = torch.randn(experts, hidden, device=dev, generator=g) * (1.0 / hidden ** 0.5)  # logits ~ N(0, 1) for x ~ N(0, 1)
+    fc1 = torch.randn(latent, hidden, device=dev, generator=g) * 0.02
+    fc2 = (torch.randn(hidden, latent, device=dev, generator=g) * 0.02).bfloat16()
+    block = nemotron_moe.NemotronMoe(torch.cat([router, fc1]).bfloat16(), torch.zeros(experts, device=dev), fc2, ex, topk)
+    x = torch.randn(tokens, hidden, device=dev, generator=g).bfloat16()
+    for _ in range(max(args.warmup, 2)):
+        block(x)
+    torch.cuda.synchronize()
+    hip = Hip()
+    names = ["route", "plan", "fc1", "fc2", "combine"]
+    per_kernel = {n: [] for n in names}
+    for rep in range(4):
+        evs = hip.events(2 * len(names))
+        _lib.check(_lib.lib().hb_debug_events(evs, len(evs)), "events")
+        block(x)
+        _lib.lib().hb_debug_events(None, 0)
+        torch.cuda.synchronize()
+        if rep:
+            for j, n in enumerate(names):
+                per_kernel[n].append(hip.elapsed_ms(evs[2 * j], evs[2 * j + 1]))
+    mean = lambda v: sum(v) / len(v)  # noqa: E731
+    steps = max(1, args.steps // 10)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = [block(x) for _ in range(steps)]
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    del outs
+    gemm_flops = tokens * topk * 2 * inter * latent  # one expert GEMM (fc1 or fc2), useful flops
+    fc1_ms = mean(per_kernel["fc1"])
+    line = {
+        "metric": "NVFP4 latent-MoE layer tokens/s on a 2048-token prefill chunk, with achieved MFMA TFLOP/s",
+        "value": tokens * steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 4: NVFP4 latent-MoE layer, 2048 tokens, hidden 4096 -> latent 1024, 512 experts x inter 2688, "
+                               "ReLU^2, top-22 sigmoid routing of N(0,1) logits, no shared expert", "timed_as": "one HIP-graph replay of all steps"},
+        "roofline": {"bound": "mfma", "kernel": "nvfp4_tile_kernel<fc1 relu2>", "achieved": gemm_flops / (fc1_ms * 1e-3) / 1e12,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None, "launch_flops": gemm_flops, "launch_ms": fc1_ms},
+        "layer_chain": {"kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -93,6 +162,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--layers", type=int, default=6, help="distinct layers the steps cycle through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--config", type=int, default=3, choices=(3, 4), help="3: the headline w3 verify-batch layer; 4: the NVFP4 prefill layer")
     ap.add_argument("--copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (a known-size "
                     "reference for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
@@ -107,6 +177,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
         return 2
+    if args.config == 4:
+        return latent_prefill(args)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     layers = []

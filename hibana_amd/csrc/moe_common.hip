@@ -157,6 +157,7 @@ static void launch_route(const RouteParams& p, int m, hipStream_t stream) {
 //   order[pos] = pair index (row * topk + slot; shared expert rows: pairs + row)
 constexpr int PLAN_THREADS = 1024;
 constexpr int PLAN_WAVES = PLAN_THREADS / 64;
+constexpr int PLAN_BATCH = 8;  // tiles of 64 pairs whose ids a wavefront requests at once
 constexpr int ROUTE_FUSED_ROWS = 16;  // up to this many rows the plan workgroup routes them itself (one a wavefront)
 
 struct Scan3 {
@@ -225,9 +226,19 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   // segment w = pairs [w * seg, (w + 1) * seg), seg a multiple of 64
   const int seg = ((pairs + PLAN_WAVES - 1) / PLAN_WAVES + 63) / 64 * 64;
   const int lo = wave * seg, hi = min(pairs, lo + seg);
-  for (int i = lo + lane; i < hi; i += 64) {
-    const int e = ids[i] - e_lo;
-    if (e >= 0 && e < e_n) atomicAdd(&seg_count[wave * e_n + e], 1);
+  const int batch = seg > 64 ? PLAN_BATCH : 1;  // long segments: the ids of a batch of tiles are requested together
+  for (int i0 = lo + lane; i0 < hi; i0 += 64 * batch) {
+    if (batch == 1) {
+      const int e = ids[i0] - e_lo;
+      if (e >= 0 && e < e_n) atomicAdd(&seg_count[wave * e_n + e], 1);
+      continue;
+    }
+    int e[PLAN_BATCH];
+#pragma unroll
+    for (int j = 0; j < PLAN_BATCH; j++) e[j] = i0 + 64 * j < hi ? ids[i0 + 64 * j] - e_lo : -1;
+#pragma unroll
+    for (int j = 0; j < PLAN_BATCH; j++)
+      if (e[j] >= 0 && e[j] < e_n) atomicAdd(&seg_count[wave * e_n + e[j]], 1);
   }
   __syncthreads();
   // per expert: total count, exclusive positions; slots of 16 rows
@@ -281,25 +292,34 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   }
   // stable placement: each wavefront walks its segment 64 pairs at a time; a lane's position is its expert's running
   // position in this segment plus the number of lower lanes of the tile with the same expert
-  for (int i0 = lo; i0 < hi; i0 += 64) {
-    const int i = i0 + lane;
-    int e = -1;
-    if (i < hi) {
-      e = ids[i] - e_lo;
-      if (e < 0 || e >= e_n) e = -1;
-    }
-    uint64_t same = __ballot(e >= 0);
+  int id_bits = 1;
+  while ((1 << id_bits) < e_n) id_bits++;
+  for (int i0 = lo; i0 < hi; i0 += 64 * batch) {
+    int eb[PLAN_BATCH];
 #pragma unroll
-    for (int b = 0; b < 20; b++) {
-      const uint64_t m = __ballot((e >> b) & 1);
-      same &= ((e >> b) & 1) ? m : ~m;
+    for (int j = 0; j < PLAN_BATCH; j++) {
+      const int i = i0 + 64 * j + lane;
+      int e = j < batch && i < hi ? ids[i] - e_lo : -1;
+      if (e < 0 || e >= e_n) e = -1;
+      eb[j] = e;
     }
-    if (e >= 0) {
-      const uint64_t below = same & ((1ull << lane) - 1ull);
-      const int base = seg_count[wave * e_n + e];
-      order[base + __popcll(below)] = i;
-      const bool last = (same >> lane) == 1ull;  // the highest lane of this expert in the tile advances the counter
-      if (last) seg_count[wave * e_n + e] = base + __popcll(same);
+#pragma unroll
+    for (int j = 0; j < PLAN_BATCH; j++) {
+      if (j < batch && i0 + 64 * j < hi) {  // wave-uniform: some pair of the segment is in this tile
+        const int i = i0 + 64 * j + lane, e = eb[j];
+        uint64_t same = __ballot(e >= 0);
+        for (int b = 0; b < id_bits; b++) {
+          const uint64_t m = __ballot((e >> b) & 1);
+          same &= ((e >> b) & 1) ? m : ~m;
+        }
+        if (e >= 0) {
+          const uint64_t below = same & ((1ull << lane) - 1ull);
+          const int base = seg_count[wave * e_n + e];
+          order[base + __popcll(below)] = i;
+          const bool last = (same >> lane) == 1ull;  // the highest lane of this expert in the tile advances the counter
+          if (last) seg_count[wave * e_n + e] = base + __popcll(same);
+        }
+      }
     }
     // the read of `base` above and the update by `last` are in the same wavefront; LDS operations of one wavefront
     // execute in program order, and the next tile's reads come after this write

@@ -49,3 +49,22 @@ def zipf_logits(rows: int, experts: int, s: float, seed: int, device="cuda") -> 
     gumbel = -(-u.log()).log()
     jitter = 1e-6 * torch.rand(rows, experts, generator=g, dtype=torch.float64)
     return (logp[None, :] + gumbel + jitter).float().to(device)
+
+
+def nvfp4_experts(experts: int, hidden: int, inter: int, seed: int, device="cuda", global_scale: float = 1.0 / 448.0, routed_scaling: float = 1.0,
+                  keep: bool = False):
+    """`experts` random ReLU^2 NVFP4 experts (up [inter, hidden], down [hidden, inter]): E2M1 codes uniform over the 16
+    codes, one E4M3 scale per 16 drawn as |N(0, 1)| clipped to [2^-6, 448], every matrix's FP32 scale `global_scale`;
+    as a `B12xExperts`, block scales handed over in the 128x4 interleave as a checkpoint loader would."""
+    from hibana_amd.kernels import b12x_moe
+    from hibana_amd.weights.modelopt import swizzle_block_scales
+    g = torch.Generator(device=device).manual_seed(seed)
+
+    def stack(rows, k):
+        w = torch.randint(0, 256, (experts, rows, k // 2), dtype=torch.uint8, device=device, generator=g)
+        sc = torch.randn(experts, rows, k // 16, device=device, generator=g).abs().clamp(2.0 ** -6, 448.0).to(torch.float8_e4m3fn)
+        return w, torch.stack([swizzle_block_scales(sc[e]) for e in range(experts)]), torch.full((experts,), global_scale, device=device)
+
+    w1, s1, g1 = stack(inter, hidden)
+    w2, s2, g2 = stack(hidden, inter)
+    return b12x_moe.B12xExperts(w1, s1, g1, 1.0, w2, s2, g2, 1.0, routed_scaling=routed_scaling, release=not keep)
