@@ -452,7 +452,7 @@ int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int sh
 int moe_check_route(int m, int e, int k) { return m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE ? HB_EINVAL : HB_OK; }
 
 int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
-                          const MoeWorkspace& ws, hipStream_t stream) {
+                          const MoeWorkspace& ws, hipStream_t stream, int slot_rows) {
   if (int err = moe_check_route(m, e, topk)) return err;
   RouteParams rp{};
   rp.logits = logits;
@@ -465,11 +465,11 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   const int64_t pairs = (int64_t)m * topk;
   if (m > ROUTE_FUSED_ROWS) {  // many rows: a wavefront a row over the whole device, then the plan
     launch_route<false>(rp, m, stream);
-    return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, ROWS_PER_SLOT);
+    return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, slot_rows);
   }
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
-  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, ROWS_PER_SLOT);
+  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, slot_rows);
   return HB_OK;
 }
 

@@ -12,6 +12,7 @@
 #include <string.h>
 
 #include "stream_common.hpp"
+#include "tile_kernel.hpp"
 
 namespace hb {
 
@@ -208,21 +209,7 @@ static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipS
   return HB_OK;
 }
 
-// ------------------------------------------------------------------------------------- prefill: slots of 128 rows
-// When an expert has many rows (a prefill chunk: dozens of rows an expert) the grouped product is a dense contraction
-// and belongs on the MFMA pipe: one workgroup of four wavefronts takes a slot of up to 128 activation rows of one
-// expert and four neighbouring 64-row weight blocks (one a wavefront), all of K. Per 128-k chunk
-//   - the slot's activation tile (128 rows x 128 k BF16, 32 KB) is brought into LDS by LDS-direct loads
-//     (global_load_lds_dwordx4: no registers in between), double buffered, pieces XOR-swizzled within a row so that the
-//     A fragment reads of sixteen rows hit sixteen different bank groups;
-//   - each wavefront expands its block's codes ONCE to scaled BF16 (e2m1 * e4m3 is exact in BF16) and reuses the four B
-//     fragments for every 16-row tile of the slot: v_mfma_f32_16x16x32_bf16, accumulators for 8 x 4 tiles in registers.
-// The K order inside one MFMA follows the tile layout's ownership (lane q holds k = 4q..4q+3 of both 16-blocks of a
-// 32-step), which the A fragment mirrors with two 8-byte LDS reads.
-constexpr int TILE_ROWS = 128;
-constexpr int TILE_MT = TILE_ROWS / 16;
-constexpr int TILE_BUF = TILE_ROWS * 256;  // bytes of one activation buffer
-
+// ------------------------------------------------------------------------------ the prefill kernel's NVFP4 format
 __device__ __forceinline__ uint32_t scaled_pair(uint32_t codes, int byte, float scale) {
   typedef __attribute__((ext_vector_type(2))) float f32x2_t;
   f32x2_t w;
@@ -237,147 +224,30 @@ __device__ __forceinline__ uint32_t scaled_pair(uint32_t codes, int byte, float 
   return __builtin_bit_cast(uint32_t, packed);
 }
 
-// The B fragment of k-step s (blocks 2s, 2s + 1) of one 16-row tile: its code dword and the two block scales.
-__device__ __forceinline__ bf16x8_t scaled_fragment(uint32_t codes, float s_even, float s_odd) {
-  u32x4_t packed;
-  packed.x = scaled_pair(codes, 0, s_even);
-  packed.y = scaled_pair(codes, 1, s_even);
-  packed.z = scaled_pair(codes, 2, s_odd);
-  packed.w = scaled_pair(codes, 3, s_odd);
-  return __builtin_bit_cast(bf16x8_t, packed);
-}
+struct TileNvfp4 {
+  typedef Fp4Chunk Chunk;
+  static constexpr int BLOCK_BYTES = NVFP4_BLOCK_BYTES;
+  static constexpr bool SPLIT_A = true, PER_ROW = false;
+  static __device__ __forceinline__ void load(Chunk& ch, const uint8_t* blk, int lane, int r16) { load_fp4_chunk(ch, blk, lane, r16); }
+  // k-step s = blocks 2 s, 2 s + 1: dword s of the tile's codes (low half the even block), scale bytes 2 s, 2 s + 1 of
+  // the tile's eight
+  static __device__ __forceinline__ bf16x8_t fragment(const Chunk& ch, int nt, int s, const Slot&) {
+    const u32x4_t w = nt == 0 ? ch.w0 : nt == 1 ? ch.w1 : nt == 2 ? ch.w2 : ch.w3;
+    const u32x4_t sc4 = nt < 2 ? ch.s0 : ch.s1;
+    const uint32_t sd = (nt & 1) ? (s < 2 ? sc4.z : sc4.w) : (s < 2 ? sc4.x : sc4.y);
+    const float s_even = (s & 1) ? __builtin_amdgcn_cvt_f32_fp8(sd, 2) : __builtin_amdgcn_cvt_f32_fp8(sd, 0);
+    const float s_odd = (s & 1) ? __builtin_amdgcn_cvt_f32_fp8(sd, 3) : __builtin_amdgcn_cvt_f32_fp8(sd, 1);
+    const uint32_t codes = w[s];
+    u32x4_t packed;
+    packed.x = scaled_pair(codes, 0, s_even);
+    packed.y = scaled_pair(codes, 1, s_even);
+    packed.z = scaled_pair(codes, 2, s_odd);
+    packed.w = scaled_pair(codes, 3, s_odd);
+    return __builtin_bit_cast(bf16x8_t, packed);
+  }
+};
 
-template <int EPI>
-__device__ __forceinline__ void stage_tile(const StreamParams& p, const int32_t* rowtab, uint8_t* buf, int chunk, int tiles, int wave, int lane) {
-  // a wavefront brings rows wave * 32 .. + 31 in eight instructions of four rows each: lane l lands at byte 16 l of the
-  // instruction's kilobyte, i.e. row (l >> 4), slot (l & 15) of it, and therefore fetches piece slot ^ (row & 15)
-  const int sub = lane >> 4, slot = lane & 15;
-#pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const int row = wave * 32 + j * 4 + sub;
-    if (wave * 32 + j * 4 < tiles * 16) {  // wave-uniform: whole 16-row tiles past the slot's rows are never read
-      const uint16_t* src = p.a + (int64_t)rowtab[row] * p.a_stride + (int64_t)chunk * 128 + ((slot ^ (row & 15)) << 3);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
-                                       (__attribute__((address_space(3))) void*)(buf + (wave * 32 + j * 4) * 256), 16, 0, 0);
-    }
-  }
-}
-
-template <int EPI>
-__global__ __launch_bounds__(256, 2) void nvfp4_tile_kernel(StreamParams p) {
-  extern __shared__ __align__(16) uint8_t tile_lds[];  // two activation buffers, then the row table
-  if ((int)blockIdx.y >= p.plan[0]) return;
-  const Slot sl = slot_of<EPI>(p, blockIdx.y);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int q = lane >> 4, r16 = lane & 15;
-  const int nb = blockIdx.x * 4 + wave;
-  const bool active = nb < p.n_blocks;
-  const int tiles = (sl.rows + 15) >> 4;
-  int32_t* rowtab = reinterpret_cast<int32_t*>(tile_lds + 2 * TILE_BUF);
-  if (threadIdx.x < TILE_ROWS) {  // the source row of each slot row (rows past the last repeat it)
-    int64_t arow = sl.p0 + min((int)threadIdx.x, sl.rows - 1);
-    if (epi_gathers(EPI)) {
-      const int pair = p.order[arow];
-      arow = pair < p.pairs ? pair / p.topk : pair - p.pairs;
-    }
-    rowtab[threadIdx.x] = (int)arow;
-  }
-  __syncthreads();
-  f32x4_t acc[TILE_MT][4];
-#pragma unroll
-  for (int t = 0; t < TILE_MT; t++)
-#pragma unroll
-    for (int nt = 0; nt < 4; nt++) acc[t][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const uint8_t* blk = sl.w + (int64_t)(active ? nb : 0) * p.chunks * NVFP4_BLOCK_BYTES;
-  Fp4Chunk cur, nxt;
-  load_fp4_chunk(cur, blk, lane, r16);
-  stage_tile<EPI>(p, rowtab, tile_lds, 0, tiles, wave, lane);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  for (int c = 0; c < p.chunks; c++) {
-    uint8_t* buf = tile_lds + (c & 1) * TILE_BUF;
-    if (c + 1 < p.chunks) {
-      load_fp4_chunk(nxt, blk + (int64_t)(c + 1) * NVFP4_BLOCK_BYTES, lane, r16);
-      stage_tile<EPI>(p, rowtab, tile_lds + ((c + 1) & 1) * TILE_BUF, c + 1, tiles, wave, lane);
-    }
-    const u32x4_t w[4] = {cur.w0, cur.w1, cur.w2, cur.w3};
-    const uint32_t sc[8] = {cur.s0.x, cur.s0.y, cur.s0.z, cur.s0.w, cur.s1.x, cur.s1.y, cur.s1.z, cur.s1.w};  // tile nt: dwords 2nt, 2nt + 1
-#pragma unroll
-    for (int s = 0; s < 4; s++) {  // 32-k steps of the chunk: blocks 2s, 2s + 1
-      bf16x8_t b[4];
-#pragma unroll
-      for (int nt = 0; nt < 4; nt++) {
-        const uint32_t sd = sc[2 * nt + (s >> 1)];
-        const float s_even = (s & 1) ? __builtin_amdgcn_cvt_f32_fp8(sd, 2) : __builtin_amdgcn_cvt_f32_fp8(sd, 0);
-        const float s_odd = (s & 1) ? __builtin_amdgcn_cvt_f32_fp8(sd, 3) : __builtin_amdgcn_cvt_f32_fp8(sd, 1);
-        b[nt] = scaled_fragment(w[nt][s], s_even, s_odd);
-      }
-      // lane (q, r16): row 16 t + r16, k = 32 s + 4 q .. + 3 (piece 4 s + q / 2, half q & 1) and the same 16 further
-      const int half = (q & 1) << 3;
-      const int slot_lo = ((4 * s + (q >> 1)) ^ r16) << 4, slot_hi = ((4 * s + 2 + (q >> 1)) ^ r16) << 4;
-#pragma unroll
-      for (int t = 0; t < TILE_MT; t++) {
-        if (t < tiles) {
-          const uint8_t* row = buf + (16 * t + r16) * 256 + half;
-          u32x4_t a;
-          const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(row + slot_lo), hi = *reinterpret_cast<const u32x2_t*>(row + slot_hi);
-          a.x = lo.x;
-          a.y = lo.y;
-          a.z = hi.x;
-          a.w = hi.y;
-          const bf16x8_t af = __builtin_bit_cast(bf16x8_t, a);
-#pragma unroll
-          for (int nt = 0; nt < 4; nt++) acc[t][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, b[nt], acc[t][nt], 0, 0, 0);
-        }
-      }
-    }
-    cur = nxt;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's LDS-direct loads have landed before it signals
-    __syncthreads();                                   // the next buffer is complete and this one is free to refill
-  }
-  if (!active) return;
-  // accumulator register r of lane (q, r16) of tile (t, nt): slot row 16 t + 4 q + r, weight row nb * 64 + 16 nt + r16
-#pragma unroll
-  for (int t = 0; t < TILE_MT; t++) {
-    if (t < tiles) {
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int i = 16 * t + 4 * q + r;
-        if (i < sl.rows) {
-          const int64_t pos = sl.p0 + i;
-          if (EPI == EPI_FC1_GATED) {
-#pragma unroll
-            for (int g = 0; g < 2; g++) {
-              const float up = through_bf16(acc[t][2 * g][r] * sl.scalar), gate = through_bf16(acc[t][2 * g + 1][r] * sl.scalar);
-              reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * g + r16] = bf16_of(silu(gate) * up);
-            }
-          } else {
-            const int64_t at = (EPI == EPI_FC2 ? (int64_t)p.order[pos] : pos) * p.out_stride + nb * 64 + r16;
-#pragma unroll
-            for (int nt = 0; nt < 4; nt++) {
-              const float y = acc[t][nt][r] * sl.scalar;
-              if (EPI == EPI_FC1_RELU2) {
-                const float h = fmaxf(through_bf16(y), 0.f);
-                reinterpret_cast<uint16_t*>(p.out)[at + 16 * nt] = bf16_of(h * h);
-              } else if (p.out_bf16) {
-                reinterpret_cast<uint16_t*>(p.out)[at + 16 * nt] = bf16_of(y);
-              } else {
-                reinterpret_cast<float*>(p.out)[at + 16 * nt] = y;
-              }
-            }
-          }
-        }
-      }
-    }
-  }
-}
-
-template <int EPI>
-static int launch_nvfp4_tile(StreamParams& p, int64_t slots, hipStream_t stream) {
-  const dim3 grid((unsigned)((p.n_blocks + 3) / 4), (unsigned)slots);
-  HB_LAUNCH(nvfp4_tile_kernel<EPI>, grid, dim3(256), 2 * TILE_BUF + TILE_ROWS * sizeof(int32_t), stream, p);
-  return HB_OK;
-}
+static int g_nvfp4_tile = 0;  // experiments: 1 forces the tile kernel, 2 the stream (hb_tune "nvfp4_tile")
 
 static inline unsigned grid_for(int64_t threads) { return (unsigned)((threads + 255) / 256); }
 
@@ -425,6 +295,12 @@ extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float glob
   p.m = m;
   p.out = y;
   p.out_stride = n;
+  if (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && tile_serves_dense(m, p.n_blocks))) {
+    const int64_t tile_slots = (m + TILE_ROWS - 1) / TILE_ROWS;
+    if (int e = relu2 ? launch_tile<TileNvfp4, EPI_DENSE_RELU2>(p, tile_slots, as_stream(stream)) : launch_tile<TileNvfp4, EPI_DENSE>(p, tile_slots, as_stream(stream)))
+      return e;
+    return launch_status();
+  }
   const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
   if (slots > 65535) return HB_EINVAL;
   if (int e = relu2 ? launch_nvfp4<EPI_DENSE_RELU2>(p, slots, slots, as_stream(stream)) : launch_nvfp4<EPI_DENSE>(p, slots, slots, as_stream(stream)))
@@ -435,8 +311,6 @@ extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float glob
 // ------------------------------------------------------------------------------------------------ routed experts
 namespace {
 
-constexpr int TILE_DENSE_ROWS = 24;  // average rows an expert from which the tile kernel serves the call
-int g_nvfp4_tile = 0;                // experiments: 1 forces the tile kernel, 2 the stream (hb_tune "nvfp4_tile")
 
 int check_experts(const hb_nvfp4_experts* ex) {
   if (!ex) return HB_ENULL;
@@ -486,8 +360,8 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
   f2.out_stride = ex->hidden_out;
   f2.out_bf16 = pairs_bf16;
   if (dense) {
-    if (int e = ex->gated ? launch_nvfp4_tile<EPI_FC1_GATED>(p, slots, stream) : launch_nvfp4_tile<EPI_FC1_RELU2>(p, slots, stream)) return e;
-    if (int e = launch_nvfp4_tile<EPI_FC2>(f2, slots, stream)) return e;
+    if (int e = ex->gated ? launch_tile<TileNvfp4, EPI_FC1_GATED>(p, slots, stream) : launch_tile<TileNvfp4, EPI_FC1_RELU2>(p, slots, stream)) return e;
+    if (int e = launch_tile<TileNvfp4, EPI_FC2>(f2, slots, stream)) return e;
     return launch_status();
   }
   if (int e = ex->gated ? launch_nvfp4<EPI_FC1_GATED>(p, slots, est, stream) : launch_nvfp4<EPI_FC1_RELU2>(p, slots, est, stream)) return e;

@@ -32,6 +32,7 @@ struct StreamParams {
   const int32_t* plan;    // grouped calls: slot table
   const int32_t* order;   // grouped calls: sorted position -> pair index
   int m;                  // dense calls: rows
+  int slot_rows;          // dense calls: rows a slot (0: ROWS_PER_SLOT)
   int topk, pairs;        // grouped calls: pair q < pairs belongs to token q / topk, q >= pairs to token q - pairs
   void* out;
   int64_t out_stride;     // elements between output rows
@@ -93,8 +94,9 @@ __device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
   Slot s;
   int expert = 0;
   if (epi_dense(EPI)) {
-    s.p0 = slot * ROWS_PER_SLOT;
-    s.rows = min(ROWS_PER_SLOT, p.m - s.p0);
+    const int per = p.slot_rows ? p.slot_rows : ROWS_PER_SLOT;
+    s.p0 = slot * per;
+    s.rows = min(per, p.m - s.p0);
   } else {
     expert = p.plan[PLAN_HEADER + 4 * slot];
     s.p0 = p.plan[PLAN_HEADER + 4 * slot + 1];
@@ -208,7 +210,7 @@ int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int sh
 // Softmax top-k routing of `m` rows of `e` logits into ids / weights [m, topk], then the plan of those ids: one launch
 // for up to a few dozen rows, two beyond.
 int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
-                          const MoeWorkspace& ws, hipStream_t stream);
+                          const MoeWorkspace& ws, hipStream_t stream, int slot_rows = ROWS_PER_SLOT);
 
 struct CombineParams {
   const void* pairs;      // [m * topk (+ m), h] FP32 or BF16

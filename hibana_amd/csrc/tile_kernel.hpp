@@ -1,0 +1,170 @@
+// The prefill-size kernel of the routed experts and the dense linears, shared by the weight formats.
+//
+// When an expert (or a dense call) has many activation rows the product is a dense contraction and belongs on the MFMA
+// pipe: one workgroup of four wavefronts takes a slot of up to 128 activation rows and four neighbouring 64-row weight
+// blocks (one a wavefront), all of K. Per 128-k chunk
+//   - the slot's activation tile (128 rows x 128 k BF16, 32 KB) is brought into LDS by LDS-direct loads
+//     (global_load_lds_dwordx4: no registers in between), double buffered, the sixteen 16-byte pieces of a row
+//     XOR-swizzled by the row so that the A fragment reads of sixteen rows hit sixteen different bank groups;
+//   - each wavefront expands its block's codes ONCE to scaled BF16 (code value x block / group scale: exact in BF16 for
+//     both formats) and reuses the four B fragments for every 16-row tile of the slot: v_mfma_f32_16x16x32_bf16,
+//     accumulators for 8 x 4 tiles in registers; the FP32 matrix / row scale is applied in the epilogue.
+//
+// A format provides: Chunk (the registers of one 64-row x 128-k block), BLOCK_BYTES, load(), fragment() (the scaled B
+// operand of 16-row tile nt and 32-k step s), SPLIT_A (how the lane's eight k of a step lie: NVFP4's tile layout gives
+// lane q the k 4q..4q+3 of both 16-blocks of the step, so its A fragment is two 8-byte reads; W3's gives it 8q..8q+7),
+// and PER_ROW (FP32 scale per output row, else one per matrix).
+#pragma once
+
+#include "stream_common.hpp"
+
+namespace hb {
+
+constexpr int TILE_ROWS = 128;
+constexpr int TILE_MT = TILE_ROWS / 16;
+constexpr int TILE_BUF = TILE_ROWS * 256;  // bytes of one activation buffer
+constexpr int TILE_DENSE_ROWS = 24;        // average rows an expert from which the tile kernel serves a routed call
+typedef __attribute__((ext_vector_type(2))) uint32_t tile_u32x2_t;
+
+__device__ __forceinline__ void stage_tile(const StreamParams& p, const int32_t* rowtab, uint8_t* buf, int chunk, int tiles, int wave, int lane) {
+  // a wavefront brings rows wave * 32 .. + 31 in eight instructions of four rows each: lane l lands at byte 16 l of the
+  // instruction's kilobyte, i.e. row (l >> 4), slot (l & 15) of it, and therefore fetches piece slot ^ (row & 15)
+  const int sub = lane >> 4, slot = lane & 15;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const int row = wave * 32 + j * 4 + sub;
+    if (wave * 32 + j * 4 < tiles * 16) {  // wave-uniform: whole 16-row tiles past the slot's rows are never read
+      const uint16_t* src = p.a + (int64_t)rowtab[row] * p.a_stride + (int64_t)chunk * 128 + ((slot ^ (row & 15)) << 3);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
+                                       (__attribute__((address_space(3))) void*)(buf + (wave * 32 + j * 4) * 256), 16, 0, 0);
+    }
+  }
+}
+
+template <class Fmt, int EPI>
+__global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
+  extern __shared__ __align__(16) uint8_t tile_lds[];  // two activation buffers, then the row table
+  if (!epi_dense(EPI) && (int)blockIdx.y >= p.plan[0]) return;
+  const Slot sl = slot_of<EPI>(p, blockIdx.y);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int nb = blockIdx.x * 4 + wave;
+  const bool active = nb < p.n_blocks;
+  const int tiles = (sl.rows + 15) >> 4;
+  int32_t* rowtab = reinterpret_cast<int32_t*>(tile_lds + 2 * TILE_BUF);
+  if (threadIdx.x < TILE_ROWS) {  // the source row of each slot row (rows past the last repeat it)
+    int64_t arow = sl.p0 + min((int)threadIdx.x, sl.rows - 1);
+    if (epi_gathers(EPI)) {
+      const int pair = p.order[arow];
+      arow = pair < p.pairs ? pair / p.topk : pair - p.pairs;
+    }
+    rowtab[threadIdx.x] = (int)arow;
+  }
+  __syncthreads();
+  f32x4_t acc[TILE_MT][4];
+#pragma unroll
+  for (int t = 0; t < TILE_MT; t++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) acc[t][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const uint8_t* blk = sl.w + (int64_t)(active ? nb : 0) * p.chunks * Fmt::BLOCK_BYTES;
+  typename Fmt::Chunk cur, nxt;
+  Fmt::load(cur, blk, lane, r16);
+  stage_tile(p, rowtab, tile_lds, 0, tiles, wave, lane);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int c = 0; c < p.chunks; c++) {
+    uint8_t* buf = tile_lds + (c & 1) * TILE_BUF;
+    if (c + 1 < p.chunks) {
+      Fmt::load(nxt, blk + (int64_t)(c + 1) * Fmt::BLOCK_BYTES, lane, r16);
+      stage_tile(p, rowtab, tile_lds + ((c + 1) & 1) * TILE_BUF, c + 1, tiles, wave, lane);
+    }
+#pragma unroll
+    for (int s = 0; s < 4; s++) {  // 32-k steps of the chunk
+      bf16x8_t b[4];
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++) b[nt] = Fmt::fragment(cur, nt, s, sl);
+      // lane (q, r16) of tile t: row 16 t + r16; its eight k of the step as the format's tile layout owns them
+      const int half = (q & 1) << 3;
+      const int slot_lo = ((4 * s + (q >> 1)) ^ r16) << 4, slot_hi = ((4 * s + 2 + (q >> 1)) ^ r16) << 4;
+      const int slot_one = ((4 * s + q) ^ r16) << 4;
+#pragma unroll
+      for (int t = 0; t < TILE_MT; t++) {
+        if (t < tiles) {
+          const uint8_t* row = buf + (16 * t + r16) * 256;
+          u32x4_t a;
+          if (Fmt::SPLIT_A) {
+            const tile_u32x2_t lo = *reinterpret_cast<const tile_u32x2_t*>(row + half + slot_lo);
+            const tile_u32x2_t hi = *reinterpret_cast<const tile_u32x2_t*>(row + half + slot_hi);
+            a = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+          } else {
+            a = *reinterpret_cast<const u32x4_t*>(row + slot_one);
+          }
+          const bf16x8_t af = __builtin_bit_cast(bf16x8_t, a);
+#pragma unroll
+          for (int nt = 0; nt < 4; nt++) acc[t][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, b[nt], acc[t][nt], 0, 0, 0);
+        }
+      }
+    }
+    cur = nxt;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's LDS-direct loads have landed before it signals
+    __syncthreads();                                   // the next buffer is complete and this one is free to refill
+  }
+  if (!active) return;
+  // accumulator register r of lane (q, r16) of tile (t, nt): slot row 16 t + 4 q + r, weight row nb * 64 + 16 nt + r16
+  float scale[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++) scale[nt] = Fmt::PER_ROW ? sl.rs[nb * 64 + 16 * nt + r16] : sl.scalar;
+#pragma unroll
+  for (int t = 0; t < TILE_MT; t++) {
+    if (t < tiles) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int i = 16 * t + 4 * q + r;
+        if (i < sl.rows) {
+          const int64_t pos = sl.p0 + i;
+          if (EPI == EPI_FC1_GATED) {
+#pragma unroll
+            for (int g = 0; g < 2; g++) {
+              const float up = through_bf16(acc[t][2 * g][r] * scale[2 * g]), gate = through_bf16(acc[t][2 * g + 1][r] * scale[2 * g + 1]);
+              reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * g + r16] = bf16_of(silu(gate) * up);
+            }
+          } else {
+            const int64_t at = (EPI == EPI_FC2 ? (int64_t)p.order[pos] : pos) * p.out_stride + nb * 64 + r16;
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) {
+              const float y = acc[t][nt][r] * scale[nt];
+              if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
+                const float h = fmaxf(through_bf16(y), 0.f);
+                reinterpret_cast<uint16_t*>(p.out)[at + 16 * nt] = bf16_of(h * h);
+              } else if (EPI == EPI_DENSE || p.out_bf16) {
+                reinterpret_cast<uint16_t*>(p.out)[at + 16 * nt] = bf16_of(y);
+              } else {
+                reinterpret_cast<float*>(p.out)[at + 16 * nt] = y;
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// A dense call goes to the tile kernel when that is the faster of the two by a model fitted to measurements (both
+// costs are proportional to K): the weight stream takes about 23 us per 16 activation rows and 25600 output rows at
+// K = 5120; the tile kernel (no K split: one workgroup per 256 output rows and 128 activation rows, 512 resident) about
+// 130 us per round of workgroups.
+inline bool tile_serves_dense(int m, int n_blocks) {
+  const int64_t groups = (int64_t)((n_blocks + 3) / 4) * ((m + TILE_ROWS - 1) / TILE_ROWS), rounds = (groups + 511) / 512;
+  return m > 2 * ROWS_PER_SLOT && (int64_t)n_blocks * 64 * m > 2300000 * rounds;
+}
+
+// `slots`: the grid's second dimension (routed: the plan's upper bound; dense: ceil(m / TILE_ROWS)).
+template <class Fmt, int EPI>
+static int launch_tile(StreamParams& p, int64_t slots, hipStream_t stream) {
+  p.slot_rows = TILE_ROWS;
+  const dim3 grid((unsigned)((p.n_blocks + 3) / 4), (unsigned)slots);
+  HB_LAUNCH((tile_kernel<Fmt, EPI>), grid, dim3(256), 2 * TILE_BUF + TILE_ROWS * sizeof(int32_t), stream, p);
+  return HB_OK;
+}
+
+}  // namespace hb

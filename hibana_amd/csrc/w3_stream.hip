@@ -13,6 +13,7 @@
 #include <string.h>
 
 #include "stream_common.hpp"
+#include "tile_kernel.hpp"
 #include "w3_layout.hpp"
 
 namespace hb {
@@ -124,9 +125,41 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   finish_block<EPI, true>(p, sl, nb, active, ks, nbi, partial, acc0, acc1, acc2, acc3);
 }
 
+// ------------------------------------------------------------------------------------ the prefill kernel's W3 format
+struct TileW3 {
+  typedef hb::Chunk Chunk;
+  static constexpr int BLOCK_BYTES = W3_BLOCK_BYTES;
+  static constexpr bool SPLIT_A = false, PER_ROW = true;
+  static __device__ __forceinline__ void load(Chunk& ch, const uint8_t* blk, int lane, int r16) { load_chunk(ch, blk, lane, r16); }
+  // The B operand of 16-row tile nt, 32-group s, scaled by the group's E4M3 scale (a 4-bit level times a 4-bit scale:
+  // exact in BF16); the FP32 row scale stays in the epilogue.
+  static __device__ __forceinline__ bf16x8_t fragment(const Chunk& ch, int nt, int s, const Slot& sl) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_v;
+    const uint32_t q0 = nt == 0 ? ch.w0.x : nt == 1 ? ch.w0.w : nt == 2 ? ch.w1.z : ch.w2.y;
+    const uint32_t q1 = nt == 0 ? ch.w0.y : nt == 1 ? ch.w1.x : nt == 2 ? ch.w1.w : ch.w2.z;
+    const uint32_t q2 = nt == 0 ? ch.w0.z : nt == 1 ? ch.w1.y : nt == 2 ? ch.w2.x : ch.w2.w;
+    const uint32_t scales = nt == 0 ? ch.sc.x : nt == 1 ? ch.sc.y : nt == 2 ? ch.sc.z : ch.sc.w;
+    uint32_t sel[8];
+    w3_selectors(q0, q1, q2, sel);  // the six the step does not use fold away
+    const uint32_t f0 = __builtin_amdgcn_perm(sl.lut_hi, sl.lut_lo, sel[2 * s]);
+    const uint32_t f1 = __builtin_amdgcn_perm(sl.lut_hi, sl.lut_lo, sel[2 * s + 1]);
+    const float g = s == 0 ? __builtin_amdgcn_cvt_f32_fp8(scales, 0) : s == 1 ? __builtin_amdgcn_cvt_f32_fp8(scales, 1)
+                  : s == 2 ? __builtin_amdgcn_cvt_f32_fp8(scales, 2) : __builtin_amdgcn_cvt_f32_fp8(scales, 3);
+    const f32x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(f0, 1.0f, false), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(f0, 1.0f, true);
+    const f32x2_t c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(f1, 1.0f, false), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(f1, 1.0f, true);
+    u32x4_t packed;
+    packed.x = __builtin_bit_cast(uint32_t, bf16x2_v{(__bf16)(a.x * g), (__bf16)(a.y * g)});
+    packed.y = __builtin_bit_cast(uint32_t, bf16x2_v{(__bf16)(b.x * g), (__bf16)(b.y * g)});
+    packed.z = __builtin_bit_cast(uint32_t, bf16x2_v{(__bf16)(c.x * g), (__bf16)(c.y * g)});
+    packed.w = __builtin_bit_cast(uint32_t, bf16x2_v{(__bf16)(d.x * g), (__bf16)(d.y * g)});
+    return __builtin_bit_cast(bf16x8_t, packed);
+  }
+};
+
 // ---------------------------------------------------------------------------------------------------- host side
 struct Tuning {
-  int w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0;
+  int w3_tile = 0, w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0;
 };
 static Tuning g_tune;
 
@@ -160,7 +193,7 @@ extern "C" int hb_tune(const char* key, int value) {
   struct {
     const char* name;
     int* slot;
-  } table[] = {{"w3_ksplit", &g_tune.w3_ksplit},           {"w3_nbw", &g_tune.w3_nbw},
+  } table[] = {{"w3_tile", &g_tune.w3_tile}, {"w3_ksplit", &g_tune.w3_ksplit},           {"w3_nbw", &g_tune.w3_nbw},
                {"moe_fc1_ksplit", &g_tune.moe_fc1_ksplit}, {"moe_fc1_nbw", &g_tune.moe_fc1_nbw},
                {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}};
   for (auto& t : table)
@@ -187,6 +220,10 @@ extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* 
   p.m = m;
   p.out = y;
   p.out_stride = n;
+  if (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && tile_serves_dense(m, p.n_blocks))) {
+    if (int e = launch_tile<TileW3, EPI_DENSE>(p, (m + TILE_ROWS - 1) / TILE_ROWS, as_stream(stream))) return e;
+    return launch_status();
+  }
   const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
   if (slots > 65535) return HB_EINVAL;
   if (int e = launch_stream<EPI_DENSE>(p, slots, slots, Launch{g_tune.w3_ksplit, g_tune.w3_nbw}, as_stream(stream))) return e;
@@ -218,12 +255,16 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
                 const MoeWorkspace& ws, void* out_pairs, int pairs_bf16, hipStream_t stream, const Routing* route = nullptr) {
   const int64_t pairs = (int64_t)m * topk;
   const int shared_rows = shared ? m : 0;
-  const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows);
+  // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel
+  const bool dense = g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && pairs >= (int64_t)ex->experts * 2 * TILE_DENSE_ROWS);  // the pre-scaled expansion costs more here than the stream's
+  const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
+  const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows, slot_rows);
   if (slots > 65535) return HB_EINVAL;
   if (route) {
-    if (int e = moe_launch_route_plan(route->logits, m, route->e, topk, route->ids, route->weights, ex->base, ex->experts, shared_rows, ws, stream))
+    if (int e = moe_launch_route_plan(route->logits, m, route->e, topk, route->ids, route->weights, ex->base, ex->experts, shared_rows, ws, stream,
+                                      slot_rows))
       return e;
-  } else if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, shared_rows, ws, stream)) {
+  } else if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, shared_rows, ws, stream, slot_rows)) {
     return e;
   }
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
@@ -271,6 +312,11 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   f2.out = out_pairs;
   f2.out_stride = ex->hidden_out;
   f2.out_bf16 = pairs_bf16;
+  if (dense) {
+    if (int e = ex->gated ? launch_tile<TileW3, EPI_FC1_GATED>(p, slots, stream) : launch_tile<TileW3, EPI_FC1_RELU2>(p, slots, stream)) return e;
+    if (int e = launch_tile<TileW3, EPI_FC2>(f2, slots, stream)) return e;
+    return launch_status();
+  }
   const Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
   if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) return e;
   if (int e = launch_stream<EPI_FC2>(f2, slots, est, l2, stream)) return e;

@@ -12,6 +12,16 @@ from tests.util import MAX_REL, NORM_REL, errors
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["auto", "tile", "stream"], autouse=True)
+def kernel_choice(request):
+    """Every case runs with the library's own choice between the 128-row MFMA tile kernel and the 16-row weight stream,
+    and with each of them forced."""
+    from hibana_amd import _lib
+    assert _lib.lib().hb_tune(b'nvfp4_tile', {"auto": 0, "tile": 1, "stream": 2}[request.param]) == 0
+    yield request.param
+    _lib.lib().hb_tune(b'nvfp4_tile', 0)
+
+
 def _matrix(n, k, seed, lo=2 ** -6, hi=448.0):
     g = np.random.default_rng(seed)
     packed = g.integers(0, 256, (n, k // 2), dtype=np.uint8)

@@ -9,6 +9,16 @@ from tests.util import MAX_REL, NORM_REL, errors, random_w3, to_device_w3
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["auto", "tile", "stream"], autouse=True)
+def kernel_choice(request):
+    """Every case runs with the library's own choice between the 128-row MFMA tile kernel and the 16-row weight stream,
+    and with each of them forced."""
+    from hibana_amd import _lib
+    assert _lib.lib().hb_tune(b'w3_tile', {"auto": 0, "tile": 1, "stream": 2}[request.param]) == 0
+    yield request.param
+    _lib.lib().hb_tune(b'w3_tile', 0)
+
+
 @pytest.mark.parametrize("m", [1, 2, 5, 16, 17, 33, 64, 128])
 @pytest.mark.parametrize("n,k,codebook", [(128, 256, "uniform"), (512, 1024, "lloyd"), (1024, 640, "zero8"), (256, 2688, "lloyd")])
 def test_w3_linear_matches_the_oracle(m, n, k, codebook):

@@ -11,6 +11,16 @@ from tests.util import MAX_REL, NORM_REL, errors, oracle_expert_getter, random_e
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(params=["auto", "tile", "stream"], autouse=True)
+def kernel_choice(request):
+    """Every case runs with the library's own choice between the 128-row MFMA tile kernel and the 16-row weight stream,
+    and with each of them forced."""
+    from hibana_amd import _lib
+    assert _lib.lib().hb_tune(b'w3_tile', {"auto": 0, "tile": 1, "stream": 2}[request.param]) == 0
+    yield request.param
+    _lib.lib().hb_tune(b'w3_tile', 0)
+
 E, H, I, TOPK = 16, 256, 128, 10
 
 
