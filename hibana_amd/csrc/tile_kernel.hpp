@@ -41,16 +41,17 @@ __device__ __forceinline__ void stage_tile(const StreamParams& p, const int32_t*
   }
 }
 
-template <class Fmt, int EPI>
-__global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
-  extern __shared__ __align__(16) uint8_t tile_lds[];  // two activation buffers, then the row table
-  if (!epi_dense(EPI) && (int)blockIdx.y >= p.plan[0]) return;
-  const Slot sl = slot_of<EPI>(p, blockIdx.y);
+// ST: the slot's number of 16-row tiles when it is a compile-time constant (no test around a tile's MFMAs, so every
+// accumulator stays in place from chunk to chunk), or 0 for any count.
+template <class Fmt, int EPI, int ST>
+__device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl, uint8_t* tile_lds) {
+  constexpr bool FULL = ST > 0;
+  constexpr int MT = FULL ? ST : TILE_MT;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q = lane >> 4, r16 = lane & 15;
   const int nb = blockIdx.x * 4 + wave;
   const bool active = nb < p.n_blocks;
-  const int tiles = (sl.rows + 15) >> 4;
+  const int tiles = FULL ? ST : (sl.rows + 15) >> 4;
   int32_t* rowtab = reinterpret_cast<int32_t*>(tile_lds + 2 * TILE_BUF);
   if (threadIdx.x < TILE_ROWS) {  // the source row of each slot row (rows past the last repeat it)
     int64_t arow = sl.p0 + min((int)threadIdx.x, sl.rows - 1);
@@ -61,9 +62,9 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
     rowtab[threadIdx.x] = (int)arow;
   }
   __syncthreads();
-  f32x4_t acc[TILE_MT][4];
+  f32x4_t acc[MT][4];
 #pragma unroll
-  for (int t = 0; t < TILE_MT; t++)
+  for (int t = 0; t < MT; t++)
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) acc[t][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const uint8_t* blk = sl.w + (int64_t)(active ? nb : 0) * p.chunks * Fmt::BLOCK_BYTES;
@@ -88,8 +89,8 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
       const int slot_lo = ((4 * s + (q >> 1)) ^ r16) << 4, slot_hi = ((4 * s + 2 + (q >> 1)) ^ r16) << 4;
       const int slot_one = ((4 * s + q) ^ r16) << 4;
 #pragma unroll
-      for (int t = 0; t < TILE_MT; t++) {
-        if (t < tiles) {
+      for (int t = 0; t < MT; t++) {
+        if (FULL || t < tiles) {
           const uint8_t* row = buf + (16 * t + r16) * 256;
           u32x4_t a;
           if (Fmt::SPLIT_A) {
@@ -115,8 +116,8 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
 #pragma unroll
   for (int nt = 0; nt < 4; nt++) scale[nt] = Fmt::PER_ROW ? sl.rs[nb * 64 + 16 * nt + r16] : sl.scalar;
 #pragma unroll
-  for (int t = 0; t < TILE_MT; t++) {
-    if (t < tiles) {
+  for (int t = 0; t < MT; t++) {
+    if (FULL || t < tiles) {
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         const int i = 16 * t + 4 * q + r;
@@ -146,6 +147,20 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
         }
       }
     }
+  }
+}
+
+template <class Fmt, int EPI>
+__global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
+  extern __shared__ __align__(16) uint8_t tile_lds[];  // two activation buffers, then the row table
+  if (!epi_dense(EPI) && (int)blockIdx.y >= p.plan[0]) return;
+  const Slot sl = slot_of<EPI>(p, blockIdx.y);
+  // uniform over the workgroup; more compile-time counts than the full slot were tried: with a third body the
+  // compiler spills and every one of them gets slower
+  if (sl.rows > TILE_ROWS - 16) {
+    tile_slot<Fmt, EPI, TILE_MT>(p, sl, tile_lds);
+  } else {
+    tile_slot<Fmt, EPI, 0>(p, sl, tile_lds);
   }
 }
 
