@@ -200,9 +200,17 @@ __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
   finish_block<EPI, false>(p, sl, nb, active, ks, nbi, partial, acc0, acc1, acc2, acc3);
 }
 
+// experiments (hb_tune): the stream's workgroup shape ("nvfp4_ksplit", "nvfp4_nbw"); "nvfp4_tile": 1 forces the tile kernel, 2 the stream
+static int g_nvfp4_ksplit = 0, g_nvfp4_nbw = 0, g_nvfp4_tile = 0;
+
 template <int EPI>
 static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipStream_t stream) {
   pick_shape(p.n_blocks, p.chunks, busy_slots, 4096, &p.ks, &p.nbw);
+  if (g_nvfp4_ksplit) {
+    p.ks = g_nvfp4_ksplit;
+    p.nbw = g_nvfp4_nbw ? g_nvfp4_nbw : 1;
+  }
+  if (p.ks * p.nbw > 16 || p.ks > p.chunks || (p.ks & (p.ks - 1))) return HB_EINVAL;
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
   HB_LAUNCH(nvfp4_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
@@ -246,8 +254,6 @@ struct TileNvfp4 {
     return __builtin_bit_cast(bf16x8_t, packed);
   }
 };
-
-static int g_nvfp4_tile = 0;  // experiments: 1 forces the tile kernel, 2 the stream (hb_tune "nvfp4_tile")
 
 static inline unsigned grid_for(int64_t threads) { return (unsigned)((threads + 255) / 256); }
 
@@ -372,8 +378,9 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
 }  // namespace
 
 int hb::nvfp4_tune(const char* key, int value) {
-  if (strcmp(key, "nvfp4_tile")) return HB_EINVAL;
-  g_nvfp4_tile = value;
+  int* slot = !strcmp(key, "nvfp4_tile") ? &g_nvfp4_tile : !strcmp(key, "nvfp4_ksplit") ? &g_nvfp4_ksplit : !strcmp(key, "nvfp4_nbw") ? &g_nvfp4_nbw : nullptr;
+  if (!slot || value < 0 || value > 16) return HB_EINVAL;
+  *slot = value;
   return HB_OK;
 }
 
