@@ -20,6 +20,7 @@ from hibana_amd import _lib
 from hibana_amd.kernels import w3
 
 EXPERTS = 512
+RATIOS = tuple(round(0.5 + 0.025 * i, 3) for i in range(21))  # group scale = amax / max level * ratio, 0.5 .. 1.0
 ORDER_IN_KERNEL = 640  # kept for the reference's callers; the planner here orders any number of pairs on the device
 WIDE_ROWS = 1024
 
@@ -194,6 +195,78 @@ def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, 
                                                      _lib.ptr(logits.contiguous()), e_total, m, topk, _lib.ptr(ids), _lib.ptr(wt), _lib.ptr(out),
                                                      _lib.ptr(ws), need, _lib.stream()), "moe_layer_logits")
     return (out, ids, wt) if return_routing else out
+
+
+# ------------------------------------------------------------------ offline: 3-bit experts from NVFP4 experts
+
+@torch.no_grad()
+def fit_scales(weight: torch.Tensor, levels, ratios=RATIOS):
+    """float32 [N, K] -> (group scales float8_e4m3fn [N, K/32], row scales float32 [N]): per 32-group the stored scale,
+    among amax / max|level| * ratio on the ratio grid, with the smallest squared weight error at nearest-level codes;
+    the first of equal errors stays (hibana/weights/w3_calibration.py:17-37 with unit importance)."""
+    n, k = weight.shape
+    grouped = weight.float().reshape(n, k // w3.GROUP, w3.GROUP)
+    top = torch.tensor(max(abs(v) for v in levels), device=weight.device)
+    fp8_max = torch.tensor(w3.FP8_MAX, device=weight.device)
+    base = grouped.abs().amax(-1) / top
+    row_scale = (base.amax(-1) / fp8_max).clamp_min(1e-12)
+    lv = torch.tensor(levels, dtype=torch.float32, device=weight.device)
+    mids = (lv[1:] + lv[:-1]) / 2
+    best_loss = torch.full_like(base, float("inf"))
+    best = torch.zeros_like(base)
+    for ratio in ratios:
+        scale = (base * ratio / row_scale[:, None]).clamp(0, w3.FP8_MAX).to(torch.float8_e4m3fn).float()
+        effective = scale * row_scale[:, None]
+        q = torch.bucketize(grouped / effective.clamp_min(1e-30)[:, :, None], mids)
+        loss = (grouped - lv[q] * effective[:, :, None]).square().sum(-1)
+        improved = loss < best_loss
+        best_loss = torch.minimum(loss, best_loss)
+        best = torch.where(improved, scale, best)
+    return best.to(torch.float8_e4m3fn), row_scale
+
+
+@torch.no_grad()
+def quantize(weight: torch.Tensor, codebook="lloyd", ratios=RATIOS):
+    """float32 [N, K] -> (codes int32 [N, K], group scales float8_e4m3fn [N, K/32], row scales [N]): the group scale
+    minimizing the weight error on the ratio grid, nearest level (hibana/kernels/w3_moe.py:113-124)."""
+    levels = w3._codebook(codebook)
+    n, k = weight.shape
+    scales, row_scale = fit_scales(weight, levels, ratios)
+    effective = (scales.float() * row_scale[:, None]).clamp_min(1e-30)
+    lv = torch.tensor(levels, device=weight.device)
+    codes = torch.bucketize(weight.float().reshape(n, k // w3.GROUP, w3.GROUP) / effective[:, :, None], (lv[1:] + lv[:-1]) / 2, out_int32=True)
+    return codes.reshape(n, k), scales, row_scale
+
+
+@torch.no_grad()
+def calibrate(w13, s13, scale2_13, w2, s2, scale2_2, codebook="lloyd", ratios=RATIOS, chunk: int = 16):
+    """A layer's NVFP4 experts (w13 uint8 [E, 2I, H/2] with rows [up; gate], unswizzled float8 block scales
+    [E, 2I, H/16], FP32 scales [E]; w2 likewise) -> (W3Experts with fc1 rows in fc1_order, report with the relative
+    weight error of fc1 and fc2 against the NVFP4 values) (hibana/kernels/w3_moe.py:127-155). Runs on the GPU the
+    tensors are on."""
+    levels = w3._codebook(codebook)
+    order = fc1_order(w13.shape[1] // 2, w13.device)
+    parts, report = {}, {}
+    for key, (packed, scales, scale2, perm) in {"w13": (w13, s13, scale2_13, order), "w2": (w2, s2, scale2_2, None)}.items():
+        e, r = packed.shape[:2]
+        out, num, den = [], 0.0, 0.0
+        for lo in range(0, e, chunk):
+            hi = min(e, lo + chunk)
+            w = nvfp4_dequant(packed[lo:hi], scales[lo:hi], scale2[lo:hi])
+            if perm is not None:
+                w = w[:, perm]
+            w = w.reshape((hi - lo) * r, -1)
+            codes, sc, rs = quantize(w, levels, ratios)
+            m = w3.pack_codes(codes, sc, rs, levels, rows_per_chunk=r)
+            num += (w3.dequantize(m) - w).square().sum().item()
+            den += w.square().sum().item()
+            out.append(m)
+            del w, codes, sc, rs
+        k = packed.shape[2] * 2
+        cat = lambda a: torch.cat([getattr(m, a).view(torch.int32) if a == "planes" else getattr(m, a) for m in out])  # noqa: E731
+        parts[key] = w3.W3Weight(cat("planes").view(torch.uint32), cat("scales"), cat("row_scale"), e * r, k, levels, w3.lut_of(levels))
+        report[key] = (num / den) ** 0.5 if den else 0.0
+    return W3Experts.from_stacked(parts["w13"], parts["w2"], w13.shape[0]), report
 
 
 def unswizzle_batched(swizzled: torch.Tensor, rows: int, groups: int) -> torch.Tensor:

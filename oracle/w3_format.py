@@ -10,6 +10,7 @@ Follows hibana/kernels/w3.py of the reference:
   dequantize                            :239-242   levels[code] * group_scale, FP32, in this multiplication order
   pack (nearest level)                  :126-172   amax / max|level| scale, row scale, bucketize against midpoints
   interleave_rows                       :94-102    whole 32-row tiles moved in pair_order
+  fit_scales_ratio / quantize_groups    hibana/weights/w3_calibration.py:17-37, hibana/kernels/w3_moe.py:113-124 (ratio-grid group scales)
 
 Everything is written from the closed form of the layout (a weight's bit b sits at bit (4j + b + rot(s)) mod 32 of
 word bits*nt + b of lane 4g + t, n = 32nb + 8nt + g, k = 128kc + 16s + 4t + j, rot(s) = 16(s//4) + s%4) with explicit
@@ -26,6 +27,9 @@ Pinned by (tests/test_oracle_w3.py):
   pack                 codes == bucketize(w / scale, mids), extremes used, error < 0.22, byte count
                        (test_w3_pack.py:34-54); 2-bit variant and fitted scales (:57-76)
   interleave_rows      interleave_rows(pack(w)) == pack(w[pair_order]) (tests/unit/test_mlp_pairs.py:27-34)
+  fit_scales_ratio     with ratios (1.0,) it must reproduce pack's stored scales and codes exactly; per group the fitted
+                       loss is never above the ratio-1.0 loss and is the minimum over a brute-force loop on a tiny matrix;
+                       the reference's bounds (tests/unit/test_w3_moe_pack.py:35-47: error < 0.25, fitted <= nearest)
 
 PARITY UNPINNED: pack(fit_scales=True) picks, per group, the first of FIT_SCALES whose float32 squared error is strictly
 the least; the error sum's summation order differs between numpy and torch, so an exact tie could resolve differently
@@ -224,3 +228,44 @@ def interleave_rows(w3, block: int):
     out["scales"] = np.ascontiguousarray(w3["scales"][tiles])
     out["row_scale"] = np.ascontiguousarray(w3["row_scale"][rows])
     return out
+
+
+def fit_scales_ratio(weight, codebook=None, ratios=tuple(round(0.5 + 0.025 * i, 3) for i in range(21))):
+    """float32 [N, K] -> (scale bytes uint8 [N, K/32], row scales float32 [N]): per 32-group the stored E4M3 scale among
+    e4m3(amax / max|level| * ratio / row scale) over the ratio grid with the smallest squared error at nearest-level codes;
+    the first of equal losses stays (hibana/weights/w3_calibration.py:17-37, unit importance; the routed experts'
+    quantizer, hibana/kernels/w3_moe.py:113-124). With ratios == (1.0,) this is `pack`'s scale rule. PARITY UNPINNED for
+    which of two ratios wins when their float32 losses differ in the last bits (summation order)."""
+    w = np.asarray(weight, dtype=np.float32)
+    n, k = w.shape
+    levels = check_codebook(codebook)
+    lv = np.asarray(levels, dtype=np.float32)
+    mids = ((lv[1:] + lv[:-1]) / np.float32(2)).astype(np.float32)
+    g = w.reshape(n, k // GROUP, GROUP)
+    base = (np.abs(g).max(axis=-1) / np.float32(max(abs(v) for v in levels))).astype(np.float32)
+    row_scale = np.maximum(base.max(axis=-1) / np.float32(FP8_MAX), np.float32(1e-12)).astype(np.float32)
+    best_loss = np.full(base.shape, np.inf, dtype=np.float32)
+    best = np.zeros(base.shape, dtype=np.uint8)
+    for ratio in ratios:
+        raw = e4m3_bytes(np.clip((base * np.float32(ratio)).astype(np.float32) / row_scale[:, None], 0, FP8_MAX))
+        eff = (e4m3_floats(raw) * row_scale[:, None]).astype(np.float32)
+        q = _bucketize(g / np.maximum(eff, np.float32(1e-30))[:, :, None], mids)
+        err = (g - lv[q] * eff[:, :, None]).astype(np.float32)
+        loss = (err * err).sum(-1, dtype=np.float32)
+        better = loss < best_loss
+        best_loss = np.where(better, loss, best_loss)
+        best = np.where(better, raw, best)
+    return best.astype(np.uint8), row_scale
+
+
+def quantize_groups(weight, scale_bytes, row_scale, codebook=None):
+    """Nearest-level codes int64 [N, K] of float32 [N, K] under given stored scales (hibana/kernels/w3_moe.py:120-124)."""
+    w = np.asarray(weight, dtype=np.float32)
+    n, k = w.shape
+    levels = check_codebook(codebook)
+    lv = np.asarray(levels, dtype=np.float32)
+    mids = ((lv[1:] + lv[:-1]) / np.float32(2)).astype(np.float32)
+    eff = np.maximum((e4m3_floats(np.asarray(scale_bytes, dtype=np.uint8)) * np.asarray(row_scale, dtype=np.float32)[:, None]).astype(np.float32),
+                     np.float32(1e-30))
+    return _bucketize(w.reshape(n, k // GROUP, GROUP) / eff[:, :, None], mids).reshape(n, k)
+
