@@ -205,7 +205,7 @@ __device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 
 // time) into route.ids / route.weights, which `ids` then names.
 __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
                                                                 int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
-                                                                int route_rows, int slot_rows) {
+                                                                int route_rows, int slot_rows, int slot_cap) {
   extern __shared__ int lds[];
   if (route.logits) {
     for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
@@ -285,6 +285,12 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
     entry[3] = 0;
   }
   for (int r = threadIdx.x; r < shared_rows; r += PLAN_THREADS) order[kept + r] = pairs + r;
+  // entries the launches' grids reach beyond the last slot say "no rows": a workgroup learns that it has nothing to do
+  // from its own entry, without a second dependent read of the count
+  for (int s = slots + shared_slots + threadIdx.x; s < slot_cap; s += PLAN_THREADS) {
+    int32_t* entry = plan + PLAN_HEADER + 4 * s;
+    entry[0] = entry[1] = entry[2] = entry[3] = 0;
+  }
   if (threadIdx.x == 0) {
     plan[0] = slots + shared_slots;
     plan[1] = distinct;
@@ -445,7 +451,8 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream, int slot_rows) {
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
-  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0, slot_rows);
+  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0, slot_rows,
+            (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows));
   return HB_OK;
 }
 
@@ -469,7 +476,8 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   }
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
-  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, slot_rows);
+  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, slot_rows,
+            (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows));
   return HB_OK;
 }
 

@@ -163,8 +163,8 @@ __device__ __forceinline__ void fp4_chunk(const Fp4Chunk& ch, const uint16_t* ar
 template <int EPI>
 __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
   extern __shared__ float partial[];
-  if (!epi_dense(EPI) && (int)blockIdx.y >= p.plan[0]) return;  // a slot the plan did not fill
   const Slot sl = slot_of<EPI>(p, blockIdx.y);
+  if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q = lane >> 4, r16 = lane & 15;
   const int ks = wave % p.ks, nbi = wave / p.ks;

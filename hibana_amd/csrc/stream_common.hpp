@@ -104,7 +104,8 @@ __device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
   }
   s.w = expert < 0 ? p.w_shared : p.w + (int64_t)expert * p.expert_bytes;
   s.rs = expert < 0 ? p.rows_shared : p.rows + (int64_t)expert * p.expert_rows;
-  s.scalar = expert < 0 ? p.scalar_shared : p.scalars ? p.scalars[expert] : p.scalar;
+  // an entry without rows names no expert: nothing indexed by it is read
+  s.scalar = expert < 0 ? p.scalar_shared : (p.scalars && s.rows > 0) ? p.scalars[expert] : p.scalar;
   s.lut_lo = expert < 0 ? p.lut_lo_shared : p.lut_lo;
   s.lut_hi = expert < 0 ? p.lut_hi_shared : p.lut_hi;
   return s;

@@ -153,8 +153,8 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
 template <class Fmt, int EPI>
 __global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
   extern __shared__ __align__(16) uint8_t tile_lds[];  // two activation buffers, then the row table
-  if (!epi_dense(EPI) && (int)blockIdx.y >= p.plan[0]) return;
   const Slot sl = slot_of<EPI>(p, blockIdx.y);
+  if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
   // uniform over the workgroup; more compile-time counts than the full slot were tried: with a third body the
   // compiler spills and every one of them gets slower
   if (sl.rows > TILE_ROWS - 16) {
