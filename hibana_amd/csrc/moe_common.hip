@@ -335,10 +335,9 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
 // ---------------------------------------------------------------------------------------------------- combine
 //
 // out[r, c] = bf16( bf16(sum over the row's local slots, in selection order, of fma(w, y)) + g * shared ), one
-// workgroup per (row, 1024-column span). The reference's combine (hibana/kernels/csrc/w3_gemm.cu:1196-1213) when no
+// workgroup per (row, 512-column span). The reference's combine (hibana/kernels/csrc/w3_gemm.cu:1196-1213) when no
 // shared expert is given; with one, its fused form (hibana/kernels/flashnext_fused.py:530-571).
 constexpr int COMBINE_SPAN = 512;  // columns per workgroup (two per thread)
-constexpr int COMBINE_MAX_TOPK = 32;
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
   __shared__ float red[4];

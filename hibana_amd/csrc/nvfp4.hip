@@ -167,12 +167,13 @@ __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
   if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q = lane >> 4, r16 = lane & 15;
-  const int ks = wave % p.ks, nbi = wave / p.ks;
+  const WaveShare share = wave_share(p, wave);
+  const int ks = share.ks, nbi = share.nbi;
   const int nb = blockIdx.x * p.nbw + nbi;
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
   if (active) {
-    const int c0 = (int)((int64_t)ks * p.chunks / p.ks), c1 = (int)((int64_t)(ks + 1) * p.chunks / p.ks);
+    const int c0 = share.c0, c1 = share.c1;
     const uint16_t* aptr = activation_row<EPI>(p, sl, r16) + 4 * q + (int64_t)c0 * 128;
     const uint8_t* blk = sl.w + ((int64_t)nb * p.chunks + c0) * NVFP4_BLOCK_BYTES;
     if (c0 < c1) {
@@ -197,7 +198,7 @@ __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
       }
     }
   }
-  finish_block<EPI, false>(p, sl, nb, active, ks, nbi, partial, acc0, acc1, acc2, acc3);
+  finish_block<EPI, false>(p, sl, RowScales{}, nb, active, ks, nbi, partial, acc0, acc1, acc2, acc3);
 }
 
 // experiments (hb_tune): the stream's workgroup shape ("nvfp4_ksplit", "nvfp4_nbw"); "nvfp4_tile": 1 forces the tile kernel, 2 the stream
@@ -211,6 +212,7 @@ static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipS
     p.nbw = g_nvfp4_nbw ? g_nvfp4_nbw : 1;
   }
   if (p.ks * p.nbw > 16 || p.ks > p.chunks || (p.ks & (p.ks - 1))) return HB_EINVAL;
+  set_split(p);
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
   HB_LAUNCH(nvfp4_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);

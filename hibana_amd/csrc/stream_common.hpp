@@ -38,6 +38,8 @@ struct StreamParams {
   int64_t out_stride;     // elements between output rows
   int out_bf16;           // EPI_FC2: pair outputs in BF16 instead of FP32
   int ks, nbw;            // wavefronts per workgroup = ks (K splits) * nbw (64-row blocks)
+  int ks_inv, chunks_base, chunks_rem;  // set_split(): ceil(65536 / ks), chunks / ks, chunks % ks
+  int no_few;             // W3 stream: slots of at most four rows take the sixteen-row body too
 };
 
 // The epilogue's roundings use the hardware FP32 -> BF16 conversion (round to nearest even).
@@ -56,23 +58,39 @@ struct Slot {
   uint32_t lut_lo, lut_hi;
 };
 
+// The FP32 row scales of a 64-row block at this lane's row-in-tile, one per 16-row tile. A wavefront asks for them
+// before its first chunk: by the epilogue they have long arrived, where a load issued there would be a full memory
+// round trip at the end of every workgroup's life.
+struct RowScales {
+  float s[4];
+  __device__ __forceinline__ float of(int t) const { return t == 0 ? s[0] : t == 1 ? s[1] : t == 2 ? s[2] : s[3]; }
+};
+
+template <bool PER_ROW>
+__device__ __forceinline__ RowScales row_scales(const Slot& sl, int nb, int r16) {
+  RowScales rs;
+#pragma unroll
+  for (int t = 0; t < 4; t++) rs.s[t] = PER_ROW ? sl.rs[nb * 64 + 16 * t + r16] : 0.f;
+  return rs;
+}
+
 // One output element (or, gated, one up/gate pair) of the 64-row block: row tile `t` (gated: pair index), accumulator
 // register r of lane (q, r16); v0 / v1 are the K-complete sums before the FP32 scale (per output row with PER_ROW, else
 // one per matrix).
 template <int EPI, bool PER_ROW>
-__device__ __forceinline__ void emit(const StreamParams& p, const Slot& sl, int nb, int t, int r, int q, int r16, float v0, float v1) {
+__device__ __forceinline__ void emit(const StreamParams& p, const Slot& sl, const RowScales& rs, int nb, int t, int r, int q, int r16, float v0,
+                                     float v1) {
   if (r >= sl.rows) return;  // wave-uniform: this accumulator register holds no row of the slot in any lane
   const int i = 4 * q + r;   // activation row of the slot held by this accumulator register
   if (i >= sl.rows) return;
   const int64_t pos = sl.p0 + i;
   if (EPI == EPI_FC1_GATED) {
-    const int n_up = nb * 64 + 32 * t + r16;
-    const float up = through_bf16(v0 * (PER_ROW ? sl.rs[n_up] : sl.scalar));
-    const float gate = through_bf16(v1 * (PER_ROW ? sl.rs[n_up + 16] : sl.scalar));
+    const float up = through_bf16(v0 * (PER_ROW ? rs.of(2 * t) : sl.scalar));
+    const float gate = through_bf16(v1 * (PER_ROW ? rs.of(2 * t + 1) : sl.scalar));
     reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = bf16_of(silu(gate) * up);
   } else {
     const int n = nb * 64 + 16 * t + r16;
-    const float y = v0 * (PER_ROW ? sl.rs[n] : sl.scalar);
+    const float y = v0 * (PER_ROW ? rs.of(t) : sl.scalar);
     if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
       const float h = fmaxf(through_bf16(y), 0.f);
       reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(h * h);
@@ -111,6 +129,26 @@ __device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
   return s;
 }
 
+// Which K split (`ks`) and which of the workgroup's blocks (`nbi`) a wavefront is, and the chunks c0 .. c1 - 1 of its
+// split (the first chunks % ks splits have one chunk more). No division: wave / ks is a multiply by ceil(65536 / ks),
+// exact for the sixteen wavefronts a workgroup can have.
+struct WaveShare {
+  int ks, nbi, c0, c1;
+};
+__device__ __forceinline__ WaveShare wave_share(const StreamParams& p, int wave) {
+  WaveShare w;
+  w.nbi = (wave * p.ks_inv) >> 16;
+  w.ks = wave - w.nbi * p.ks;
+  w.c0 = w.ks * p.chunks_base + min(w.ks, p.chunks_rem);
+  w.c1 = w.c0 + p.chunks_base + (w.ks < p.chunks_rem ? 1 : 0);
+  return w;
+}
+inline void set_split(StreamParams& p) {  // after ks is chosen
+  p.ks_inv = (65536 + p.ks - 1) / p.ks;
+  p.chunks_base = p.chunks / p.ks;
+  p.chunks_rem = p.chunks % p.ks;
+}
+
 // The activation row this lane feeds to the MFMA A operand (row r16 of the slot). Lanes past the slot's last row read
 // that last row again: their MFMA output rows are never stored.
 template <int EPI>
@@ -124,10 +162,10 @@ __device__ __forceinline__ const uint16_t* activation_row(const StreamParams& p,
 }
 
 // The end of a 64-row block: K-complete sums straight from the registers (ks == 1), or the K split's partial sums
-// exchanged through LDS (`partial`: 4 KB per wavefront) and added in split order, then the epilogue. With ks > 1 every
-// wavefront of the workgroup must call it (one workgroup barrier).
-template <int EPI, bool PER_ROW>
-__device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& sl, int nb, bool active, int ks, int nbi, float* partial,
+// exchanged through LDS (`partial`: 4 KB at the start of each wavefront's STRIDE floats) and added in split order,
+// then the epilogue. With ks > 1 every wavefront of the workgroup must call it (one workgroup barrier).
+template <int EPI, bool PER_ROW, int STRIDE = 1024>
+__device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& sl, const RowScales& rs, int nb, bool active, int ks, int nbi, float* partial,
                                              const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2, const f32x4_t& acc3) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q = lane >> 4, r16 = lane & 15;
@@ -135,27 +173,27 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
   if (p.ks == 1) {
     if (!active) return;
     if (EPI == EPI_FC1_GATED) {
-      emit<EPI, PER_ROW>(p, sl, nb, 0, 0, q, r16, acc0.x, acc1.x);
-      emit<EPI, PER_ROW>(p, sl, nb, 0, 1, q, r16, acc0.y, acc1.y);
-      emit<EPI, PER_ROW>(p, sl, nb, 0, 2, q, r16, acc0.z, acc1.z);
-      emit<EPI, PER_ROW>(p, sl, nb, 0, 3, q, r16, acc0.w, acc1.w);
-      emit<EPI, PER_ROW>(p, sl, nb, 1, 0, q, r16, acc2.x, acc3.x);
-      emit<EPI, PER_ROW>(p, sl, nb, 1, 1, q, r16, acc2.y, acc3.y);
-      emit<EPI, PER_ROW>(p, sl, nb, 1, 2, q, r16, acc2.z, acc3.z);
-      emit<EPI, PER_ROW>(p, sl, nb, 1, 3, q, r16, acc2.w, acc3.w);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, 0, 0, q, r16, acc0.x, acc1.x);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, 0, 1, q, r16, acc0.y, acc1.y);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, 0, 2, q, r16, acc0.z, acc1.z);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, 0, 3, q, r16, acc0.w, acc1.w);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, 1, 0, q, r16, acc2.x, acc3.x);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, 1, 1, q, r16, acc2.y, acc3.y);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, 1, 2, q, r16, acc2.z, acc3.z);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, 1, 3, q, r16, acc2.w, acc3.w);
     } else {
       const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
 #pragma unroll
       for (int t = 0; t < 4; t++) {
-        emit<EPI, PER_ROW>(p, sl, nb, t, 0, q, r16, all[t].x, 0.f);
-        emit<EPI, PER_ROW>(p, sl, nb, t, 1, q, r16, all[t].y, 0.f);
-        emit<EPI, PER_ROW>(p, sl, nb, t, 2, q, r16, all[t].z, 0.f);
-        emit<EPI, PER_ROW>(p, sl, nb, t, 3, q, r16, all[t].w, 0.f);
+        emit<EPI, PER_ROW>(p, sl, rs, nb, t, 0, q, r16, all[t].x, 0.f);
+        emit<EPI, PER_ROW>(p, sl, rs, nb, t, 1, q, r16, all[t].y, 0.f);
+        emit<EPI, PER_ROW>(p, sl, rs, nb, t, 2, q, r16, all[t].z, 0.f);
+        emit<EPI, PER_ROW>(p, sl, rs, nb, t, 3, q, r16, all[t].w, 0.f);
       }
     }
     return;
   }
-  float* mine = partial + (int64_t)wave * 1024;
+  float* mine = partial + (int64_t)wave * STRIDE;
   {
     const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
 #pragma unroll
@@ -168,25 +206,25 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
   }
   __syncthreads();
   if (!active) return;
-  const float* first = partial + (int64_t)nbi * p.ks * 1024;
+  const float* first = partial + (int64_t)nbi * p.ks * STRIDE;
   if (EPI == EPI_FC1_GATED) {
     for (int idx = ks; idx < 8; idx += p.ks) {
       const int t = idx >> 2, r = idx & 3;
       if (r >= rows) continue;
       float up = 0.f, gate = 0.f;
       for (int s = 0; s < p.ks; s++) {
-        up += first[s * 1024 + ((2 * t) * 4 + r) * 64 + lane];
-        gate += first[s * 1024 + ((2 * t + 1) * 4 + r) * 64 + lane];
+        up += first[s * STRIDE + ((2 * t) * 4 + r) * 64 + lane];
+        gate += first[s * STRIDE + ((2 * t + 1) * 4 + r) * 64 + lane];
       }
-      emit<EPI, PER_ROW>(p, sl, nb, t, r, q, r16, up, gate);
+      emit<EPI, PER_ROW>(p, sl, rs, nb, t, r, q, r16, up, gate);
     }
   } else {
     for (int idx = ks; idx < 16; idx += p.ks) {
       const int t = idx >> 2, r = idx & 3;
       if (r >= rows) continue;
       float v = 0.f;
-      for (int s = 0; s < p.ks; s++) v += first[s * 1024 + (t * 4 + r) * 64 + lane];
-      emit<EPI, PER_ROW>(p, sl, nb, t, r, q, r16, v, 0.f);
+      for (int s = 0; s < p.ks; s++) v += first[s * STRIDE + (t * 4 + r) * 64 + lane];
+      emit<EPI, PER_ROW>(p, sl, rs, nb, t, r, q, r16, v, 0.f);
     }
   }
 }

@@ -1,15 +1,21 @@
 // The W3 weight stream on gfx950: dense linear and routed-expert grouped GEMMs for decode / verify sized calls.
 //
 // One wavefront owns a block column of the tile layout: 64 output rows x a range of 128-k chunks, for one "slot" of up
-// to 16 activation rows. Per chunk it issues three 128-bit loads of packed codes and one of scales (a contiguous
-// 3328-byte block), expands the codes in registers (v_perm_b32 over the 8-byte E4M3 codebook, then the hardware
-// FP8 -> BF16 pair conversion: exact), and feeds sixteen v_mfma_f32_16x16x32_bf16 (4 row tiles x 4 scale groups):
-// one MFMA is exactly one 32-group, so the group scale is folded into the FP32 accumulator after it
-// (acc += part * scale), as the reference kernel does per group (hibana/kernels/csrc/w3_gemm.cu:105-108); the FP32
-// row scale is applied in the epilogue (:209-210). Activations are BF16, read straight from global memory (they stay
-// in L2) as the MFMA A operand. The wavefronts of a workgroup split K (partials reduced through LDS in a fixed
-// order) and/or take neighbouring 64-row blocks. No atomics on floating point anywhere: results are bitwise
-// repeatable.
+// to 16 activation rows. A chunk is a contiguous 3328-byte block (packed codes, then scales); it travels from memory
+// into the wavefront's ring in LDS without passing through registers, two chunks ahead of the one being expanded.
+// The expansion happens in registers (v_perm_b32 over the 8-byte E4M3 codebook, then the hardware FP8 -> BF16 pair
+// conversion: exact) and feeds sixteen v_mfma_f32_16x16x32_bf16 (4 row tiles x 4 scale groups): one MFMA is exactly
+// one 32-group, so the group scale is folded into the FP32 accumulator after it (acc += part * scale), as the
+// reference kernel does per group (hibana/kernels/csrc/w3_gemm.cu:105-108); the FP32 row scale is applied in the
+// epilogue (:209-210). Activations are BF16, read straight from global memory (they stay in L2) as the MFMA A operand.
+// Slots of at most four rows (most of a decode or verify step) take a second body that packs the four groups into the
+// idle MFMA rows and so folds a quarter of the scales. The wavefronts of a workgroup split K (partials reduced through
+// LDS in a fixed order) and/or take neighbouring 64-row blocks. No atomics on floating point anywhere: results are
+// bitwise repeatable.
+//
+// Calls with many rows per weight block (prefill) go to the 128-row MFMA tile kernel of tile_kernel.hpp instead, through
+// the TileW3 policy below; the entry points choose (tile_serves_dense for a dense call, pairs per expert for a routed
+// one), and hb_tune("w3_tile", 1 | 2) forces one or the other.
 #include <string.h>
 
 #include "stream_common.hpp"
@@ -52,77 +58,280 @@ __device__ __forceinline__ bf16x8_t expand8(uint32_t sel_lo, uint32_t sel_hi, ui
   return __builtin_bit_cast(bf16x8_t, packed);
 }
 
-// One 16-row tile of a chunk: its three code dwords, its four scale bytes, the four activation fragments.
-__device__ __forceinline__ void compute_tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const Rows& ch, f32x4_t& acc,
-                                             uint32_t lut_lo, uint32_t lut_hi) {
+// Half of a 16-row tile of a chunk, sixteen activation rows: 32-groups 0 and 1 (HALF 0: their selectors come from the
+// tile's first two code dwords) or 2 and 3 (HALF 1). One MFMA is one group, so the group's scale is folded into the FP32
+// accumulator after it, in group order.
+template <int HALF>
+__device__ __forceinline__ void compute_half_tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const u32x4_t& a_lo, const u32x4_t& a_hi,
+                                                  f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi) {
   uint32_t sel[8];
-  w3_selectors(q0, q1, q2, sel);
+  w3_selectors(q0, q1, q2, sel);  // the four the half does not use fold away
   const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-  const f32x4_t p0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a0), expand8(sel[0], sel[1], lut_lo, lut_hi), zero, 0, 0, 0);
-  const f32x4_t p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a1), expand8(sel[2], sel[3], lut_lo, lut_hi), zero, 0, 0, 0);
-  const f32x4_t p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a2), expand8(sel[4], sel[5], lut_lo, lut_hi), zero, 0, 0, 0);
-  const f32x4_t p3 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a3), expand8(sel[6], sel[7], lut_lo, lut_hi), zero, 0, 0, 0);
-  const float s0 = __builtin_amdgcn_cvt_f32_fp8(scales, 0), s1 = __builtin_amdgcn_cvt_f32_fp8(scales, 1);
-  const float s2 = __builtin_amdgcn_cvt_f32_fp8(scales, 2), s3 = __builtin_amdgcn_cvt_f32_fp8(scales, 3);
-  acc.x = fmaf(p3.x, s3, fmaf(p2.x, s2, fmaf(p1.x, s1, fmaf(p0.x, s0, acc.x))));
-  acc.y = fmaf(p3.y, s3, fmaf(p2.y, s2, fmaf(p1.y, s1, fmaf(p0.y, s0, acc.y))));
-  acc.z = fmaf(p3.z, s3, fmaf(p2.z, s2, fmaf(p1.z, s1, fmaf(p0.z, s0, acc.z))));
-  acc.w = fmaf(p3.w, s3, fmaf(p2.w, s2, fmaf(p1.w, s1, fmaf(p0.w, s0, acc.w))));
+  const f32x4_t p0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a_lo), expand8(sel[4 * HALF], sel[4 * HALF + 1], lut_lo, lut_hi), zero, 0, 0, 0);
+  const f32x4_t p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a_hi), expand8(sel[4 * HALF + 2], sel[4 * HALF + 3], lut_lo, lut_hi), zero, 0, 0, 0);
+  const float s0 = HALF ? __builtin_amdgcn_cvt_f32_fp8(scales, 2) : __builtin_amdgcn_cvt_f32_fp8(scales, 0);
+  const float s1 = HALF ? __builtin_amdgcn_cvt_f32_fp8(scales, 3) : __builtin_amdgcn_cvt_f32_fp8(scales, 1);
+  acc.x = fmaf(p1.x, s1, fmaf(p0.x, s0, acc.x));
+  acc.y = fmaf(p1.y, s1, fmaf(p0.y, s0, acc.y));
+  acc.z = fmaf(p1.z, s1, fmaf(p0.z, s0, acc.z));
+  acc.w = fmaf(p1.w, s1, fmaf(p0.w, s0, acc.w));
 }
 
-__device__ __forceinline__ void compute_chunk(const Chunk& ch, const Rows& rows, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3,
-                                              uint32_t lut_lo, uint32_t lut_hi) {
-  compute_tile(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, rows, acc0, lut_lo, lut_hi);
-  compute_tile(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, rows, acc1, lut_lo, lut_hi);
-  compute_tile(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, rows, acc2, lut_lo, lut_hi);
-  compute_tile(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, rows, acc3, lut_lo, lut_hi);
+// The four tiles of a chunk over one half of its groups: once a half is done its two activation fragments are free for
+// the next chunk's.
+template <int HALF>
+__device__ __forceinline__ void compute_half_chunk(const Chunk& ch, const u32x4_t& a_lo, const u32x4_t& a_hi, f32x4_t& acc0, f32x4_t& acc1,
+                                                   f32x4_t& acc2, f32x4_t& acc3, uint32_t lut_lo, uint32_t lut_hi) {
+  compute_half_tile<HALF>(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, a_lo, a_hi, acc0, lut_lo, lut_hi);
+  compute_half_tile<HALF>(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, a_lo, a_hi, acc1, lut_lo, lut_hi);
+  compute_half_tile<HALF>(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, a_lo, a_hi, acc2, lut_lo, lut_hi);
+  compute_half_tile<HALF>(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, a_lo, a_hi, acc3, lut_lo, lut_hi);
+}
+
+// ------------------------------------------------------------------------------------------------ the weight ring
+//
+// Weight chunks do not wait in registers. A wavefront owns RING_CHUNKS block-sized slots of LDS and fills them with
+// LDS-direct loads (global_load_lds: memory to LDS, no register in between), two chunks ahead of the one it expands;
+// when a chunk's turn comes its block is read from the slot into sixteen registers and the slot is given to the chunk
+// two further on. Only the lanes that asked for a block read it back, so no barrier is involved: a wavefront waits on
+// its own vector-memory counter. A chunk in flight costs no registers this way: two of them stand behind the one
+// being expanded where register double-buffering affords one, and a wavefront's registers go to one chunk's codes, its
+// activations and the accumulators.
+//
+// The counter is shared by everything a wavefront has asked of memory, in order. A chunk's block is four LDS-direct
+// loads, asked for two chunks ahead, right after the slot it goes to has been read; the chunk's activation loads
+// (Acts::LOADS of them) are asked for one chunk later, when their registers are free. The compiler may move those
+// among the other requests made between two reads of the ring, but not across a read (the reads are volatile
+// statements that clobber memory). So when chunk i is due, everything asked for since the read before stands behind
+// its block: the block of chunk i + 1 and one chunk's activation loads at least. Waiting until at most that many
+// requests remain outstanding is waiting for chunk i, and hardly longer. The last chunk waits for everything. The
+// LDS-direct loads go through a buffer descriptor of the block row (the MUBUF form: around it the compiler keeps exact
+// count of its own loads, which it gives up around the FLAT form), and the ring is read with explicit ds_read_b128, so
+// the only waits on these transfers are the ones written here.
+constexpr int RING_CHUNKS = 2;
+constexpr int RING_BYTES = RING_CHUNKS * W3_BLOCK_BYTES;  // LDS per wavefront; its first 4 KB double as the K-split exchange
+constexpr int BLOCK_LOADS = 4;
+
+typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
+
+struct RingSource {
+  __amdgpu_buffer_rsrc_t row;  // the block row: chunks x W3_BLOCK_BYTES
+  uint32_t codes, scales;      // the lane's byte offsets in a block for the 16-byte and the 4-byte loads
+};
+
+__device__ __forceinline__ void request_chunk(const RingSource& src, int chunk, lds_ptr_t slot) {
+  const uint32_t at = (uint32_t)chunk * W3_BLOCK_BYTES;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 0, 2);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024, 2);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 2048, 2);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 4, src.scales, at, W3_SCALE_OFFSET, 2);
+  __builtin_amdgcn_sched_barrier(0);  // asked for here, not wherever the scheduler would sink it below the arithmetic
+}
+
+// `codes` / `scales`: LDS byte addresses of the lane's first code load and of its row-in-tile's scales in the ring's
+// slot 0; SLOT selects the slot through the instruction's offset.
+template <int BEHIND, int SLOT>  // BEHIND: requests that may stay outstanding
+__device__ __forceinline__ void take_chunk(Chunk& ch, uint32_t codes, uint32_t scales) {
+  asm volatile(
+      "s_waitcnt vmcnt(%6)\n\t"
+      "ds_read_b128 %0, %4 offset:%7\n\t"
+      "ds_read_b128 %1, %4 offset:%8\n\t"
+      "ds_read_b128 %2, %4 offset:%9\n\t"
+      "ds_read_b128 %3, %5 offset:%10\n\t"
+      "s_waitcnt lgkmcnt(0)"  // the slot is read: it may be given to another chunk
+      : "=&v"(ch.w0), "=&v"(ch.w1), "=&v"(ch.w2), "=&v"(ch.sc)
+      : "v"(codes), "v"(scales), "n"(BEHIND), "n"(SLOT * W3_BLOCK_BYTES), "n"(SLOT * W3_BLOCK_BYTES + 1024), "n"(SLOT * W3_BLOCK_BYTES + 2048),
+        "n"(SLOT * W3_BLOCK_BYTES + W3_SCALE_OFFSET)
+      : "memory");
+}
+
+// ------------------------------------------------------------------------------------------- slots of one to four rows
+//
+// Most slots of a decode or verify step hold a handful of rows (an expert a few tokens chose). Twelve of the sixteen
+// MFMA output rows are then idle, and they can carry the four 32-groups of a chunk instead: A row 4 j + i holds row i of
+// the slot over group j's k range only (zero elsewhere), so the four MFMAs of a tile, one per group, chain into ONE
+// accumulator whose rows 4 j .. 4 j + 3 are group j's partial sums. Lane (q, r16) then holds group q's sums for the
+// slot's four rows: one scale conversion and four multiply-adds per tile instead of four and sixteen, and sixteen bytes
+// of activations per lane and chunk instead of sixty-four. The four groups are added across the lanes once, after the
+// last chunk.
+constexpr int FEW_ROWS = 4;
+
+__device__ __forceinline__ void compute_tile_few(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const Rows& ch, f32x4_t& acc,
+                                                 uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
+  uint32_t sel[8];
+  w3_selectors(q0, q1, q2, sel);
+  f32x4_t part = {0.f, 0.f, 0.f, 0.f};
+  part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a0), expand8(sel[0], sel[1], lut_lo, lut_hi), part, 0, 0, 0);
+  part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a1), expand8(sel[2], sel[3], lut_lo, lut_hi), part, 0, 0, 0);
+  part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a2), expand8(sel[4], sel[5], lut_lo, lut_hi), part, 0, 0, 0);
+  part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a3), expand8(sel[6], sel[7], lut_lo, lut_hi), part, 0, 0, 0);
+  const float s = __builtin_amdgcn_cvt_f32_fp8(scales >> q8, 0);  // the scale of this lane's group
+  acc.x = fmaf(part.x, s, acc.x);
+  acc.y = fmaf(part.y, s, acc.y);
+  acc.z = fmaf(part.z, s, acc.z);
+  acc.w = fmaf(part.w, s, acc.w);
+}
+
+// `a`: the lane's sixteen activation bytes of the chunk (row r16 % 4 of the slot, the k range of group r16 / 4 that this
+// lane owns in the MFMA A operand); grp: that group.
+__device__ __forceinline__ void compute_few(const Chunk& ch, const u32x4_t& a, int grp, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
+                                            f32x4_t& acc3, uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
+  const u32x4_t none = {0u, 0u, 0u, 0u};
+  Rows rows;  // MFMA j's A operand: the lane's bytes in its own group, zero in the others
+  rows.a0 = grp == 0 ? a : none;
+  rows.a1 = grp == 1 ? a : none;
+  rows.a2 = grp == 2 ? a : none;
+  rows.a3 = grp == 3 ? a : none;
+  compute_tile_few(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, rows, acc0, lut_lo, lut_hi, q8);
+  compute_tile_few(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, rows, acc1, lut_lo, lut_hi, q8);
+  compute_tile_few(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, rows, acc2, lut_lo, lut_hi, q8);
+  compute_tile_few(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, rows, acc3, lut_lo, lut_hi, q8);
+}
+
+__device__ __forceinline__ void add_groups(f32x4_t& acc) {
+  acc.x += __shfl_xor(acc.x, 16);
+  acc.y += __shfl_xor(acc.y, 16);
+  acc.z += __shfl_xor(acc.z, 16);
+  acc.w += __shfl_xor(acc.w, 16);
+  acc.x += __shfl_xor(acc.x, 32);
+  acc.y += __shfl_xor(acc.y, 32);
+  acc.z += __shfl_xor(acc.z, 32);
+  acc.w += __shfl_xor(acc.w, 32);
+}
+
+// The two bodies of the stream differ in the activations: what registers they keep, when they ask for them, how a
+// chunk is computed. `step<ODD, MORE2, MORE1>` computes chunk i (ODD: its parity; MORE2 / MORE1: chunks i + 2 / i + 1
+// exist) and asks for the activations whose registers it frees.
+struct FewActs {
+  static constexpr int LOADS = 1;  // activation loads per chunk
+  u32x4_t held[2];                 // the lane's sixteen bytes of the next even and the next odd chunk
+  int grp;
+  uint32_t q8;
+  const uint16_t* at;              // the lane's sixteen bytes of the wavefront's first chunk
+  __device__ __forceinline__ u32x4_t load(int i) const { return *reinterpret_cast<const u32x4_t*>(at + (int64_t)i * 128); }
+  template <int EPI>
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int c0, int n, int lane) {
+    const int q = lane >> 4, r16 = lane & 15;
+    grp = r16 >> 2;
+    at = activation_row<EPI>(p, sl, r16 & 3) + (int64_t)c0 * 128 + 32 * grp + 8 * q;
+    q8 = 8 * q;
+    held[0] = load(0);
+    if (n > 1) held[1] = load(1);
+  }
+  template <int ODD, bool MORE2, bool MORE1>
+  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+    compute_few(ch, held[ODD], grp, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi, q8);
+    if (MORE2) held[ODD] = load(i + 2);
+  }
+  // On return every lane holds, in register r of each accumulator, the sum for the slot's row r: lanes q = 0 hold what
+  // the epilogue stores, and the rows the other lanes stand for are past the slot's end.
+  static __device__ __forceinline__ void finish(f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) {
+    add_groups(acc0);
+    add_groups(acc1);
+    add_groups(acc2);
+    add_groups(acc3);
+  }
+};
+
+struct FullActs {  // up to sixteen rows: lane (q, r16) feeds row r16, k 8 q .. 8 q + 7 of every group
+  static constexpr int LOADS = 4;
+  Rows held;           // one chunk's fragments; each half is asked for again as soon as its groups are done
+  const uint16_t* at;
+  template <int EPI>
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int c0, int, int lane) {
+    at = activation_row<EPI>(p, sl, lane & 15) + (int64_t)c0 * 128 + 8 * (lane >> 4);
+    load_rows(held, at);
+  }
+  template <int ODD, bool MORE2, bool MORE1>
+  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+    const uint16_t* next = at + (int64_t)(i + 1) * 128;
+    compute_half_chunk<0>(ch, held.a0, held.a1, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+    if (MORE1) {
+      held.a0 = *reinterpret_cast<const u32x4_t*>(next);
+      held.a1 = *reinterpret_cast<const u32x4_t*>(next + 32);
+    }
+    compute_half_chunk<1>(ch, held.a2, held.a3, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+    if (MORE1) {
+      held.a2 = *reinterpret_cast<const u32x4_t*>(next + 64);
+      held.a3 = *reinterpret_cast<const u32x4_t*>(next + 96);
+    }
+  }
+  static __device__ __forceinline__ void finish(f32x4_t&, f32x4_t&, f32x4_t&, f32x4_t&) {}
+};
+
+// Chunks c0 .. c1 - 1 (at least one) of block row `nb`, through the wavefront's ring.
+template <int EPI, class Acts>
+__device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& sl, int nb, int c0, int c1, int lane, uint8_t* ring,
+                                             f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) {
+  constexpr int BEHIND = BLOCK_LOADS + Acts::LOADS;
+  const int r16 = lane & 15, n = c1 - c0;
+  RingSource src;
+  src.row = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(sl.w + (int64_t)nb * p.chunks * W3_BLOCK_BYTES), 0, p.chunks * W3_BLOCK_BYTES,
+                                              0x00020000);
+  src.codes = 16u * lane;
+  src.scales = 4u * lane;
+  const lds_ptr_t slot0 = (lds_ptr_t)ring, slot1 = (lds_ptr_t)(ring + W3_BLOCK_BYTES);
+  const uint32_t codes = (uint32_t)(uintptr_t)slot0 + 16u * lane, scales = (uint32_t)(uintptr_t)slot0 + 16u * r16;
+  Acts acts;
+  Chunk ch;
+  request_chunk(src, c0, slot0);
+  asm volatile("" ::: "memory");  // whatever else the prologue asks for stands behind the first block
+  acts.template start<EPI>(p, sl, c0, n, lane);
+  if (n == 1) {
+    take_chunk<0, 0>(ch, codes, scales);
+    acts.template step<0, false, false>(ch, 0, acc0, acc1, acc2, acc3, sl);
+  } else {
+    request_chunk(src, c0 + 1, slot1);
+    int i = 0;
+    for (; i + 3 < n; i += 2) {  // chunks i and i + 1, asking for the blocks of i + 2 and i + 3
+      take_chunk<BEHIND, 0>(ch, codes, scales);
+      request_chunk(src, c0 + i + 2, slot0);
+      acts.template step<0, true, true>(ch, i, acc0, acc1, acc2, acc3, sl);
+      take_chunk<BEHIND, 1>(ch, codes, scales);
+      request_chunk(src, c0 + i + 3, slot1);
+      acts.template step<1, true, true>(ch, i + 1, acc0, acc1, acc2, acc3, sl);
+    }
+    if (i + 3 == n) {  // three left: the block of i + 2 is still to ask for
+      take_chunk<BEHIND, 0>(ch, codes, scales);
+      request_chunk(src, c0 + i + 2, slot0);
+      acts.template step<0, true, true>(ch, i, acc0, acc1, acc2, acc3, sl);
+      take_chunk<BEHIND, 1>(ch, codes, scales);
+      acts.template step<1, false, true>(ch, i + 1, acc0, acc1, acc2, acc3, sl);
+      take_chunk<0, 0>(ch, codes, scales);
+      acts.template step<0, false, false>(ch, i + 2, acc0, acc1, acc2, acc3, sl);
+    } else {  // two left, both asked for
+      take_chunk<BEHIND, 0>(ch, codes, scales);
+      acts.template step<0, false, true>(ch, i, acc0, acc1, acc2, acc3, sl);
+      take_chunk<0, 1>(ch, codes, scales);
+      acts.template step<1, false, false>(ch, i + 1, acc0, acc1, acc2, acc3, sl);
+    }
+  }
+  Acts::finish(acc0, acc1, acc2, acc3);
 }
 
 // General kernel, any K: one workgroup per (run of p.nbw 64-row blocks, slot), K split p.ks ways across its wavefronts.
-// Weights and activations of chunk i + 1 are requested together before chunk i is expanded (two register buffers).
 template <int EPI>
 __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
-  extern __shared__ float partial[];
+  extern __shared__ __align__(16) uint8_t rings[];
   const Slot sl = slot_of<EPI>(p, blockIdx.y);
   if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int q = lane >> 4, r16 = lane & 15;
-  const int ks = wave % p.ks, nbi = wave / p.ks;
-  const int nb = blockIdx.x * p.nbw + nbi;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: kept in scalars
+  const WaveShare share = wave_share(p, wave);
+  const int ks = share.ks, nbi = share.nbi, nb = blockIdx.x * p.nbw + nbi;
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
+  RowScales rs{};
   if (active) {
-    const int c0 = (int)((int64_t)ks * p.chunks / p.ks), c1 = (int)((int64_t)(ks + 1) * p.chunks / p.ks);
-    const uint8_t* blk = sl.w + ((int64_t)nb * p.chunks + c0) * W3_BLOCK_BYTES;
-    if (c0 < c1) {
-      Chunk we, wo;
-      Rows ae, ao;
-      load_chunk(we, blk, lane, r16);
-      const uint16_t* aptr = activation_row<EPI>(p, sl, r16) + 8 * q + (int64_t)c0 * 128;
-      load_rows(ae, aptr);
-      int left = c1 - c0 - 1;  // chunks not yet requested
-      while (left >= 2) {
-        load_chunk(wo, blk + W3_BLOCK_BYTES, lane, r16);
-        load_rows(ao, aptr + 128);
-        compute_chunk(we, ae, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
-        blk += 2 * W3_BLOCK_BYTES;
-        aptr += 256;
-        load_chunk(we, blk, lane, r16);
-        load_rows(ae, aptr);
-        compute_chunk(wo, ao, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
-        left -= 2;
-      }
-      if (left == 1) {
-        load_chunk(wo, blk + W3_BLOCK_BYTES, lane, r16);
-        load_rows(ao, aptr + 128);
-        compute_chunk(we, ae, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
-        compute_chunk(wo, ao, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
-      } else {
-        compute_chunk(we, ae, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
-      }
+    const int c0 = share.c0, c1 = share.c1;  // at least one chunk: the launch keeps ks <= chunks
+    uint8_t* ring = rings + wave * RING_BYTES;
+    if (sl.rows <= FEW_ROWS && !p.no_few) {
+      stream_block<EPI, FewActs>(p, sl, nb, c0, c1, lane, ring, acc0, acc1, acc2, acc3);
+    } else {
+      stream_block<EPI, FullActs>(p, sl, nb, c0, c1, lane, ring, acc0, acc1, acc2, acc3);
     }
+    rs = row_scales<true>(sl, nb, lane & 15);
   }
-  finish_block<EPI, true>(p, sl, nb, active, ks, nbi, partial, acc0, acc1, acc2, acc3);
+  finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
 }
 
 // ------------------------------------------------------------------------------------ the prefill kernel's W3 format
@@ -159,7 +368,7 @@ struct TileW3 {
 
 // ---------------------------------------------------------------------------------------------------- host side
 struct Tuning {
-  int w3_tile = 0, w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0;
+  int w3_tile = 0, w3_few = 0, w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0;
 };
 static Tuning g_tune;
 
@@ -178,9 +387,11 @@ static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Lau
   }
   if (want.nbw) p.nbw = want.nbw;
   if (p.ks * p.nbw > 16 || p.ks > p.chunks) return HB_EINVAL;
+  set_split(p);
+  p.no_few = g_tune.w3_few == 2;  // every slot takes the sixteen-row body
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
-  HB_LAUNCH(w3_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
+  HB_LAUNCH(w3_stream_kernel<EPI>, grid, dim3(64 * waves), (size_t)waves * RING_BYTES, stream, p);
   return HB_OK;
 }
 
@@ -193,12 +404,12 @@ extern "C" int hb_tune(const char* key, int value) {
   struct {
     const char* name;
     int* slot;
-  } table[] = {{"w3_tile", &g_tune.w3_tile}, {"w3_ksplit", &g_tune.w3_ksplit},           {"w3_nbw", &g_tune.w3_nbw},
+  } table[] = {{"w3_tile", &g_tune.w3_tile}, {"w3_few", &g_tune.w3_few}, {"w3_ksplit", &g_tune.w3_ksplit},           {"w3_nbw", &g_tune.w3_nbw},
                {"moe_fc1_ksplit", &g_tune.moe_fc1_ksplit}, {"moe_fc1_nbw", &g_tune.moe_fc1_nbw},
                {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}};
   for (auto& t : table)
     if (!strcmp(t.name, key)) {
-      if (value < 0 || value > 16 || (value & (value - 1))) return HB_EINVAL;
+      if (value < 0 || value > 16) return HB_EINVAL;
       *t.slot = value;
       return HB_OK;
     }

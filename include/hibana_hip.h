@@ -32,8 +32,11 @@ enum {
 int hb_version(void);
 const char* hb_error_string(int code);
 
-/* Tuning knobs for experiments ("w3_ksplit", "w3_nbw", "moe_fc1_ksplit", ...); value 0 restores the built-in choice.
- * Returns HB_EINVAL for an unknown key. Not thread-safe against concurrent launches. */
+/* Tuning knobs for experiments and tests; value 0 restores the built-in choice. "w3_ksplit" / "w3_nbw",
+ * "moe_fc1_ksplit" / "moe_fc1_nbw", "moe_fc2_ksplit" / "moe_fc2_nbw", "nvfp4_ksplit" / "nvfp4_nbw": K splits and 64-row
+ * blocks per workgroup (their product at most 16); "w3_tile" / "nvfp4_tile": 1 forces the MFMA tile kernel, 2 the weight
+ * stream; "w3_few": 2 switches off the stream's body for slots of at most four rows. Returns HB_EINVAL for an unknown
+ * key or a value out of range. Not thread-safe against concurrent launches. */
 int hb_tune(const char* key, int value);
 
 /* Measurement hook (no counterpart in the reference): `events` are hipEvent_t handles the caller created, taken in

@@ -9,18 +9,22 @@ from tests.util import MAX_REL, NORM_REL, errors, random_w3, to_device_w3
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["auto", "tile", "stream"], autouse=True)
+@pytest.fixture(params=["auto", "tile", "stream", "stream16"], autouse=True)
 def kernel_choice(request):
     """Every case runs with the library's own choice between the 128-row MFMA tile kernel and the 16-row weight stream,
-    and with each of them forced."""
+    with each of them forced, and with the stream's body for slots of at most four rows switched off (so those slots
+    take the sixteen-row body, as they do when the activation matrix is too large for a buffer descriptor)."""
     from hibana_amd import _lib
-    assert _lib.lib().hb_tune(b'w3_tile', {"auto": 0, "tile": 1, "stream": 2}[request.param]) == 0
+    tile, few = {"auto": (0, 0), "tile": (1, 0), "stream": (2, 0), "stream16": (2, 2)}[request.param]
+    assert _lib.lib().hb_tune(b'w3_tile', tile) == 0 and _lib.lib().hb_tune(b'w3_few', few) == 0
     yield request.param
     _lib.lib().hb_tune(b'w3_tile', 0)
+    _lib.lib().hb_tune(b'w3_few', 0)
 
 
-@pytest.mark.parametrize("m", [1, 2, 5, 16, 17, 33, 64, 128])
-@pytest.mark.parametrize("n,k,codebook", [(128, 256, "uniform"), (512, 1024, "lloyd"), (1024, 640, "zero8"), (256, 2688, "lloyd")])
+@pytest.mark.parametrize("m", [1, 2, 4, 5, 16, 17, 33, 64, 128])  # 4 | 5: the last slot the few-row body takes, the first it does not
+@pytest.mark.parametrize("n,k,codebook", [(128, 256, "uniform"), (512, 1024, "lloyd"), (1024, 640, "zero8"), (256, 2688, "lloyd"),
+                                          (128, 128, "lloyd"), (256, 384, "uniform")])  # one and three chunks: the ring's short tails
 def test_w3_linear_matches_the_oracle(m, n, k, codebook):
     from hibana_amd.kernels import w3
     packed, *_ = random_w3(n, k, 7, codebook)
@@ -42,14 +46,15 @@ def test_every_k_split_gives_close_results_and_the_unsplit_bits_repeat():
     from hibana_amd.kernels import w3
     packed, *_ = random_w3(256, 2048, 8)
     dev = to_device_w3(packed)
-    x = torch.randn(16, 2048, generator=torch.Generator().manual_seed(1)).bfloat16()
-    want = layers.dense_ref(x, ow3.dequantize(packed))
     try:
-        for ks, nbw in ((1, 1), (1, 4), (2, 2), (4, 1), (8, 1), (16, 1), (4, 4), (0, 0)):
-            assert _lib.lib().hb_tune(b"w3_ksplit", ks) == 0 and _lib.lib().hb_tune(b"w3_nbw", nbw) == 0
-            got = w3.w3_linear(x.cuda(), dev)
-            mx, nr = errors(got, want)
-            assert mx < MAX_REL and nr < NORM_REL, (ks, nbw, mx, nr)
+        for m in (3, 16):  # both bodies of the stream; from 16 chunks a wavefront down to 1, even and odd counts
+            x = torch.randn(m, 2048, generator=torch.Generator().manual_seed(m)).bfloat16()
+            want = layers.dense_ref(x, ow3.dequantize(packed))
+            for ks, nbw in ((1, 1), (1, 4), (2, 2), (3, 1), (4, 1), (5, 3), (7, 2), (8, 1), (16, 1), (4, 4), (0, 0)):
+                assert _lib.lib().hb_tune(b"w3_ksplit", ks) == 0 and _lib.lib().hb_tune(b"w3_nbw", nbw) == 0
+                got = w3.w3_linear(x.cuda(), dev)
+                mx, nr = errors(got, want)
+                assert mx < MAX_REL and nr < NORM_REL, (m, ks, nbw, mx, nr)
     finally:
         _lib.lib().hb_tune(b"w3_ksplit", 0)
         _lib.lib().hb_tune(b"w3_nbw", 0)
