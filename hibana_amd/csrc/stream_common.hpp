@@ -58,9 +58,7 @@ struct Slot {
   uint32_t lut_lo, lut_hi;
 };
 
-// The FP32 row scales of a 64-row block at this lane's row-in-tile, one per 16-row tile. A wavefront asks for them
-// before its first chunk: by the epilogue they have long arrived, where a load issued there would be a full memory
-// round trip at the end of every workgroup's life.
+// The FP32 row scales of a 64-row block at this lane's row-in-tile, one per 16-row tile.
 struct RowScales {
   float s[4];
   __device__ __forceinline__ float of(int t) const { return t == 0 ? s[0] : t == 1 ? s[1] : t == 2 ? s[2] : s[3]; }
@@ -74,36 +72,44 @@ __device__ __forceinline__ RowScales row_scales(const Slot& sl, int nb, int r16)
   return rs;
 }
 
-// One output element (or, gated, one up/gate pair) of the 64-row block: row tile `t` (gated: pair index), accumulator
-// register r of lane (q, r16); v0 / v1 are the K-complete sums before the FP32 scale (per output row with PER_ROW, else
-// one per matrix).
+// Stores one output element (gated: one up/gate pair) of the 64-row block: row tile `t` (gated: pair index), column r16
+// of it, slot row i. y0 / y1 are the K-complete sums times their FP32 scale; the roundings are the reference's.
+template <int EPI>
+__device__ __forceinline__ void store_out(const StreamParams& p, const Slot& sl, int nb, int t, int i, int r16, float y0, float y1) {
+  const int64_t pos = sl.p0 + i;
+  if (EPI == EPI_FC1_GATED) {
+    const float up = through_bf16(y0), gate = through_bf16(y1);
+    reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = bf16_of(silu(gate) * up);
+  } else {
+    const int n = nb * 64 + 16 * t + r16;
+    if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
+      const float h = fmaxf(through_bf16(y0), 0.f);
+      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(h * h);
+    } else if (EPI == EPI_DENSE) {
+      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(y0);
+    } else {
+      const int64_t pair = p.order[pos];
+      if (p.out_bf16) {
+        reinterpret_cast<uint16_t*>(p.out)[pair * p.out_stride + n] = bf16_of(y0);
+      } else {
+        reinterpret_cast<float*>(p.out)[pair * p.out_stride + n] = y0;
+      }
+    }
+  }
+}
+
+// One output element (or, gated, one up/gate pair) from accumulator register r of lane (q, r16); v0 / v1 are the
+// K-complete sums before the FP32 scale (per output row with PER_ROW, else one per matrix).
 template <int EPI, bool PER_ROW>
 __device__ __forceinline__ void emit(const StreamParams& p, const Slot& sl, const RowScales& rs, int nb, int t, int r, int q, int r16, float v0,
                                      float v1) {
   if (r >= sl.rows) return;  // wave-uniform: this accumulator register holds no row of the slot in any lane
   const int i = 4 * q + r;   // activation row of the slot held by this accumulator register
   if (i >= sl.rows) return;
-  const int64_t pos = sl.p0 + i;
   if (EPI == EPI_FC1_GATED) {
-    const float up = through_bf16(v0 * (PER_ROW ? rs.of(2 * t) : sl.scalar));
-    const float gate = through_bf16(v1 * (PER_ROW ? rs.of(2 * t + 1) : sl.scalar));
-    reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = bf16_of(silu(gate) * up);
+    store_out<EPI>(p, sl, nb, t, i, r16, v0 * (PER_ROW ? rs.of(2 * t) : sl.scalar), v1 * (PER_ROW ? rs.of(2 * t + 1) : sl.scalar));
   } else {
-    const int n = nb * 64 + 16 * t + r16;
-    const float y = v0 * (PER_ROW ? rs.of(t) : sl.scalar);
-    if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
-      const float h = fmaxf(through_bf16(y), 0.f);
-      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(h * h);
-    } else if (EPI == EPI_DENSE) {
-      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(y);
-    } else {
-      const int64_t pair = p.order[pos];
-      if (p.out_bf16) {
-        reinterpret_cast<uint16_t*>(p.out)[pair * p.out_stride + n] = bf16_of(y);
-      } else {
-        reinterpret_cast<float*>(p.out)[pair * p.out_stride + n] = y;
-      }
-    }
+    store_out<EPI>(p, sl, nb, t, i, r16, v0 * (PER_ROW ? rs.of(t) : sl.scalar), 0.f);
   }
 }
 

@@ -152,8 +152,8 @@ __device__ __forceinline__ void take_chunk(Chunk& ch, uint32_t codes, uint32_t s
 // the slot over group j's k range only (zero elsewhere), so the four MFMAs of a tile, one per group, chain into ONE
 // accumulator whose rows 4 j .. 4 j + 3 are group j's partial sums. Lane (q, r16) then holds group q's sums for the
 // slot's four rows: one scale conversion and four multiply-adds per tile instead of four and sixteen, and sixteen bytes
-// of activations per lane and chunk instead of sixty-four. The four groups are added across the lanes once, after the
-// last chunk.
+// of activations per lane and chunk instead of sixty-four. The four groups are added once, after the last chunk, in the
+// exchange through LDS that the K splits are added in.
 constexpr int FEW_ROWS = 4;
 
 __device__ __forceinline__ void compute_tile_few(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const Rows& ch, f32x4_t& acc,
@@ -188,17 +188,6 @@ __device__ __forceinline__ void compute_few(const Chunk& ch, const u32x4_t& a, i
   compute_tile_few(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, rows, acc3, lut_lo, lut_hi, q8);
 }
 
-__device__ __forceinline__ void add_groups(f32x4_t& acc) {
-  acc.x += __shfl_xor(acc.x, 16);
-  acc.y += __shfl_xor(acc.y, 16);
-  acc.z += __shfl_xor(acc.z, 16);
-  acc.w += __shfl_xor(acc.w, 16);
-  acc.x += __shfl_xor(acc.x, 32);
-  acc.y += __shfl_xor(acc.y, 32);
-  acc.z += __shfl_xor(acc.z, 32);
-  acc.w += __shfl_xor(acc.w, 32);
-}
-
 // The two bodies of the stream differ in the activations: what registers they keep, when they ask for them, how a
 // chunk is computed. `step<ODD, MORE2, MORE1>` computes chunk i (ODD: its parity; MORE2 / MORE1: chunks i + 2 / i + 1
 // exist) and asks for the activations whose registers it frees.
@@ -222,14 +211,6 @@ struct FewActs {
   __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
     compute_few(ch, held[ODD], grp, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi, q8);
     if (MORE2) held[ODD] = load(i + 2);
-  }
-  // On return every lane holds, in register r of each accumulator, the sum for the slot's row r: lanes q = 0 hold what
-  // the epilogue stores, and the rows the other lanes stand for are past the slot's end.
-  static __device__ __forceinline__ void finish(f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) {
-    add_groups(acc0);
-    add_groups(acc1);
-    add_groups(acc2);
-    add_groups(acc3);
   }
 };
 
@@ -256,7 +237,6 @@ struct FullActs {  // up to sixteen rows: lane (q, r16) feeds row r16, k 8 q .. 
       held.a3 = *reinterpret_cast<const u32x4_t*>(next + 96);
     }
   }
-  static __device__ __forceinline__ void finish(f32x4_t&, f32x4_t&, f32x4_t&, f32x4_t&) {}
 };
 
 // Chunks c0 .. c1 - 1 (at least one) of block row `nb`, through the wavefront's ring.
@@ -306,7 +286,50 @@ __device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& 
       acts.template step<1, false, false>(ch, i + 1, acc0, acc1, acc2, acc3, sl);
     }
   }
-  Acts::finish(acc0, acc1, acc2, acc3);
+}
+
+// The end of a 64-row block for a slot of at most four rows. Lane (g, r16) of each of the block's K splits holds, in
+// register r of accumulator t, group g's part of (tile t, slot row r, column r16): sixteen values a lane, each to be
+// added over the four groups and the splits. They go to LDS, and the workgroup's 64 x ks lanes share the 16 x 16
+// results of the block: lane (q, r16) of split `ks` takes tile q, column r16, of slot rows ks, ks + p.ks, ... It
+// multiplies by its tile's row scale (`scale`, asked for before the first chunk); a gated pair's gate comes from the
+// neighbouring tile's lane. Every wavefront of the workgroup must call it when K is split (one workgroup barrier).
+template <int EPI>
+__device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl, float scale, int nb, bool active, int wave, int ks, int nbi,
+                                           float* partial, const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2, const f32x4_t& acc3) {
+  constexpr int STRIDE = RING_BYTES / 4;
+  const int lane = threadIdx.x & 63, q = lane >> 4, r16 = lane & 15;
+  float* mine = partial + wave * STRIDE;
+  const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    mine[(t * 4 + 0) * 64 + lane] = all[t].x;
+    mine[(t * 4 + 1) * 64 + lane] = all[t].y;
+    mine[(t * 4 + 2) * 64 + lane] = all[t].z;
+    mine[(t * 4 + 3) * 64 + lane] = all[t].w;
+  }
+  if (p.ks > 1) {
+    __syncthreads();
+  } else {
+    __builtin_amdgcn_wave_barrier();  // the lanes of one wavefront: its LDS operations execute in program order
+  }
+  if (!active) return;
+  const float* first = partial + nbi * p.ks * STRIDE + r16;
+  for (int r = ks; r < sl.rows; r += p.ks) {
+    const float* at = first + (q * 4 + r) * 64;
+    float v = 0.f;
+    for (int s = 0; s < p.ks; s++) {
+      v += (at[0] + at[16]) + (at[32] + at[48]);
+      at += STRIDE;
+    }
+    const float y = v * scale;
+    if (EPI == EPI_FC1_GATED) {
+      const float gate = __shfl_xor(y, 16);  // tiles 2 t and 2 t + 1 are a pair's up and gate rows
+      if ((q & 1) == 0) store_out<EPI>(p, sl, nb, q >> 1, r, r16, y, gate);
+    } else {
+      store_out<EPI>(p, sl, nb, q, r, r16, y, 0.f);
+    }
+  }
 }
 
 // General kernel, any K: one workgroup per (run of p.nbw 64-row blocks, slot), K split p.ks ways across its wavefronts.
@@ -320,18 +343,22 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   const int ks = share.ks, nbi = share.nbi, nb = blockIdx.x * p.nbw + nbi;
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
-  RowScales rs{};
-  if (active) {
-    const int c0 = share.c0, c1 = share.c1;  // at least one chunk: the launch keeps ks <= chunks
-    uint8_t* ring = rings + wave * RING_BYTES;
-    if (sl.rows <= FEW_ROWS && !p.no_few) {
-      stream_block<EPI, FewActs>(p, sl, nb, c0, c1, lane, ring, acc0, acc1, acc2, acc3);
-    } else {
-      stream_block<EPI, FullActs>(p, sl, nb, c0, c1, lane, ring, acc0, acc1, acc2, acc3);
+  uint8_t* ring = rings + wave * RING_BYTES;
+  if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
+    float scale = 0.f;
+    if (active) {
+      scale = sl.rs[nb * 64 + lane];  // row 16 q + r16 of the block: asked for ahead of the chunks, there when the epilogue wants it
+      stream_block<EPI, FewActs>(p, sl, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);  // at least one chunk: ks <= chunks
     }
-    rs = row_scales<true>(sl, nb, lane & 15);
+    finish_few<EPI>(p, sl, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+  } else {
+    RowScales rs{};
+    if (active) {
+      stream_block<EPI, FullActs>(p, sl, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      rs = row_scales<true>(sl, nb, lane & 15);
+    }
+    finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
   }
-  finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
 }
 
 // ------------------------------------------------------------------------------------ the prefill kernel's W3 format
