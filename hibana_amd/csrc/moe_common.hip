@@ -153,7 +153,8 @@ static void launch_route(const RouteParams& p, int m, hipStream_t stream) {
 // distinct local experts in ascending id, each expert's pairs in ascending pair index (a stable sort), cut into slots
 // of at most 16 rows. One workgroup; any number of pairs. Integer atomics on LDS counters only (order-independent).
 //   plan[0] = slots, plan[1] = distinct experts, plan[2] = kept routed pairs,
-//   plan[16 + 4 s ..] = { local expert id (-1: the shared expert), first sorted position, rows, 0 }
+//   plan[16 + 4 s ..] = { local expert id (-1: the shared expert), first sorted position, rows, 0 }: the shared
+//                        expert's slots first, then the routed experts' (the heavily loaded ones before the others)
 //   order[pos] = pair index (row * topk + slot; shared expert rows: pairs + row)
 constexpr int PLAN_THREADS = 1024;
 constexpr int PLAN_WAVES = PLAN_THREADS / 64;
@@ -241,44 +242,42 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
       if (e[j] >= 0 && e[j] < e_n) atomicAdd(&seg_count[wave * e_n + e[j]], 1);
   }
   __syncthreads();
-  // per expert: total count, exclusive positions; slots of 16 rows
-  int kept = 0, distinct = 0, slots = 0;
-  for (int base = 0; base < e_n; base += PLAN_THREADS) {  // experts in ascending id, PLAN_THREADS at a time
-    const int e = base + threadIdx.x;
-    int count = 0;
-    if (e < e_n)
-      for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
-    const int my_slots = (count + slot_rows - 1) / slot_rows;
-    Scan3 tot;
-    const Scan3 at = block_exclusive_scan3(Scan3{count, count > 0 ? 1 : 0, my_slots}, scratch, &tot);
-    const int my_start = kept + at.a, my_slot = slots + at.c;
-    const int tot_count = tot.a, tot_distinct = tot.b, tot_slots = tot.c;
-    if (e < e_n) {
-      start[e] = my_start;
-      for (int s = 0; s < my_slots; s++) {
-        int32_t* entry = plan + PLAN_HEADER + 4 * (my_slot + s);
-        entry[0] = e;
-        entry[1] = my_start + s * slot_rows;
-        entry[2] = min(slot_rows, count - s * slot_rows);
-        entry[3] = 0;
-      }
-      // turn the per-segment counts into the first position of each segment's run
-      int run = my_start;
-      for (int wv = 0; wv < PLAN_WAVES; wv++) {
-        const int c = seg_count[wv * e_n + e];
-        seg_count[wv * e_n + e] = run;
-        run += c;
-      }
+  // Slot order is the order the hardware starts a launch's workgroups in, so the long-running slots go first: the
+  // shared expert's (full slots), then the experts with more than a quarter slot of rows, then the rest, each class in
+  // ascending expert id. Sorted positions are another matter: ascending expert id, the shared rows after the routed
+  // pairs.
+  const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
+  const int e = threadIdx.x;  // one thread an expert: the launch keeps e_n <= PLAN_THREADS
+  int count = 0;
+  if (e < e_n)
+    for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
+  const int my_slots = (count + slot_rows - 1) / slot_rows;
+  const bool heavy = 4 * count > slot_rows;
+  Scan3 tot;  // a: rows; b: heavy slots, and distinct experts in the upper half (neither sum reaches 65536); c: light slots
+  const Scan3 at = block_exclusive_scan3(Scan3{count, (heavy ? my_slots : 0) | (count > 0 ? 1 << 16 : 0), heavy ? 0 : my_slots}, scratch, &tot);
+  const int kept = tot.a, distinct = tot.b >> 16, heavy_slots = tot.b & 0xffff;
+  const int slots = shared_slots + heavy_slots + tot.c;
+  if (e < e_n) {
+    const int my_start = at.a, my_slot = shared_slots + (heavy ? (at.b & 0xffff) : heavy_slots + at.c);
+    start[e] = my_start;
+    for (int s = 0; s < my_slots; s++) {
+      int32_t* entry = plan + PLAN_HEADER + 4 * (my_slot + s);
+      entry[0] = e;
+      entry[1] = my_start + s * slot_rows;
+      entry[2] = min(slot_rows, count - s * slot_rows);
+      entry[3] = 0;
     }
-    kept += tot_count;
-    distinct += tot_distinct;
-    slots += tot_slots;
+    // turn the per-segment counts into the first position of each segment's run
+    int run = my_start;
+    for (int wv = 0; wv < PLAN_WAVES; wv++) {
+      const int c = seg_count[wv * e_n + e];
+      seg_count[wv * e_n + e] = run;
+      run += c;
+    }
   }
   __syncthreads();
-  // the shared expert's rows follow the routed pairs
-  const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
   for (int s = threadIdx.x; s < shared_slots; s += PLAN_THREADS) {
-    int32_t* entry = plan + PLAN_HEADER + 4 * (slots + s);
+    int32_t* entry = plan + PLAN_HEADER + 4 * s;
     entry[0] = -1;
     entry[1] = kept + s * slot_rows;
     entry[2] = min(slot_rows, shared_rows - s * slot_rows);
@@ -287,12 +286,12 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   for (int r = threadIdx.x; r < shared_rows; r += PLAN_THREADS) order[kept + r] = pairs + r;
   // entries the launches' grids reach beyond the last slot say "no rows": a workgroup learns that it has nothing to do
   // from its own entry, without a second dependent read of the count
-  for (int s = slots + shared_slots + threadIdx.x; s < slot_cap; s += PLAN_THREADS) {
+  for (int s = slots + threadIdx.x; s < slot_cap; s += PLAN_THREADS) {
     int32_t* entry = plan + PLAN_HEADER + 4 * s;
     entry[0] = entry[1] = entry[2] = entry[3] = 0;
   }
   if (threadIdx.x == 0) {
-    plan[0] = slots + shared_slots;
+    plan[0] = slots;
     plan[1] = distinct;
     plan[2] = kept;
   }
@@ -449,7 +448,7 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
 
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream, int slot_rows) {
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
-  if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
+  if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
   HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0, slot_rows,
             (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows));
   return HB_OK;
@@ -474,7 +473,7 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
     return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, slot_rows);
   }
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
-  if (plan_lds > 64 * 1024 || pairs > 0x3fffffff) return HB_EINVAL;
+  if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
   HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, slot_rows,
             (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows));
   return HB_OK;
