@@ -429,7 +429,7 @@ int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows, int slot_rows
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int hidden_out, int shared) {
+MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int hidden_out, int shared, int hidden) {
   const int64_t pairs = (int64_t)m * topk, rows = pairs + (shared ? m : 0);
   MoeWorkspace w{};
   size_t off = 0;
@@ -442,6 +442,12 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
   w.order = static_cast<int32_t*>(take(rows * sizeof(int32_t)));
   w.h = static_cast<uint16_t*>(take((size_t)rows * inter * sizeof(uint16_t)));
   w.y = static_cast<float*>(take((size_t)rows * hidden_out * sizeof(float)));
+  if (hidden) {
+    w.xq = static_cast<uint8_t*>(take((size_t)m * hidden));
+    w.xs = static_cast<float*>(take((size_t)m * (hidden / 32) * sizeof(float)));
+    w.hq = static_cast<uint8_t*>(take((size_t)rows * inter));
+    w.hs = static_cast<float*>(take((size_t)rows * (inter / 32) * sizeof(float)));
+  }
   w.bytes = off;
   return w;
 }

@@ -29,6 +29,8 @@ struct StreamParams {
   int chunks;             // K / 128
   const uint16_t* a;      // BF16 activations
   int64_t a_stride;       // elements between rows
+  const uint8_t* aq;      // E4M3 activation mode: codes [rows, a_stride] ...
+  const float* aq_scale;  // ... and their scales [rows, a_stride / 32]
   const int32_t* plan;    // grouped calls: slot table
   const int32_t* order;   // grouped calls: sorted position -> pair index
   int m;                  // dense calls: rows
@@ -155,16 +157,22 @@ inline void set_split(StreamParams& p) {  // after ks is chosen
   p.chunks_rem = p.chunks % p.ks;
 }
 
-// The activation row this lane feeds to the MFMA A operand (row r16 of the slot). Lanes past the slot's last row read
-// that last row again: their MFMA output rows are never stored.
+// The row of the activation matrix that is row r of the slot. Rows past the slot's last read that last row again: their
+// MFMA output rows are never stored.
 template <int EPI>
-__device__ __forceinline__ const uint16_t* activation_row(const StreamParams& p, const Slot& s, int r16) {
-  int64_t arow = s.p0 + min(r16, s.rows - 1);
+__device__ __forceinline__ int64_t activation_row_index(const StreamParams& p, const Slot& s, int r) {
+  int64_t arow = s.p0 + min(r, s.rows - 1);
   if (epi_gathers(EPI)) {
     const int pair = p.order[arow];
     arow = pair < p.pairs ? pair / p.topk : pair - p.pairs;
   }
-  return p.a + arow * p.a_stride;
+  return arow;
+}
+
+// The activation row this lane feeds to the MFMA A operand (row r16 of the slot).
+template <int EPI>
+__device__ __forceinline__ const uint16_t* activation_row(const StreamParams& p, const Slot& s, int r16) {
+  return p.a + activation_row_index<EPI>(p, s, r16) * p.a_stride;
 }
 
 // The end of a 64-row block: K-complete sums straight from the registers (ks == 1), or the K split's partial sums
@@ -243,11 +251,15 @@ struct MoeWorkspace {
   int32_t* order;
   uint16_t* h;   // [(pairs + shared rows), inter] BF16, in sorted order
   float* y;      // [(pairs + shared rows), hidden_out] FP32 (or BF16 pairs), by pair index
+  uint8_t* xq;   // E4M3 activation mode: codes of x [m, hidden] ...
+  float* xs;     // ... and their scales [m, hidden / 32]
+  uint8_t* hq;   // the same for h: [(pairs + shared rows), inter], [.., inter / 32]
+  float* hs;
   size_t bytes;
 };
 
 int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows, int slot_rows = ROWS_PER_SLOT);
-MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int hidden_out, int shared);
+MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int hidden_out, int shared, int hidden = 0);  // hidden: also the E4M3 activation buffers
 // Enqueue the plan kernel; HB_EINVAL if the expert count does not fit its LDS.
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream,
                     int slot_rows = ROWS_PER_SLOT);

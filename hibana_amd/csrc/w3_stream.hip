@@ -172,6 +172,40 @@ __device__ __forceinline__ void compute_tile_few(uint32_t q0, uint32_t q1, uint3
   acc.w = fmaf(part.w, s, acc.w);
 }
 
+// The E4M3-activation form of the four-row body (the arithmetic of the reference kernel, hibana/kernels/csrc/
+// w3_gemm.cu:105-108: FP8 x FP8 products, FP32 sums a group, the two group scales folded into the accumulator). The
+// codebook's E4M3 bytes are the MFMA operand as they come out of v_perm_b32: no conversion. `a`: the lane's eight
+// activation codes of the chunk; xs: the activation scales of the slot's four rows at this lane's group.
+__device__ __forceinline__ long fp8x8(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
+
+__device__ __forceinline__ void compute_tile_few8(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const long a[4], const f32x4_t& xs,
+                                                  f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
+  uint32_t sel[8];
+  w3_selectors(q0, q1, q2, sel);
+  f32x4_t part = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const long b = fp8x8(__builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j]), __builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j + 1]));
+    part = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[j], b, part, 0, 0, 0);
+  }
+  const float s = __builtin_amdgcn_cvt_f32_fp8(scales >> q8, 0);  // the weight scale of this lane's group
+  acc.x = fmaf(part.x, xs.x * s, acc.x);
+  acc.y = fmaf(part.y, xs.y * s, acc.y);
+  acc.z = fmaf(part.z, xs.z * s, acc.z);
+  acc.w = fmaf(part.w, xs.w * s, acc.w);
+}
+
+__device__ __forceinline__ void compute_few8(const Chunk& ch, long a, const f32x4_t& xs, int grp, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
+                                             f32x4_t& acc3, uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
+  long rows[4];  // MFMA j's A operand: the lane's codes in its own group, zero in the others
+#pragma unroll
+  for (int j = 0; j < 4; j++) rows[j] = grp == j ? a : 0L;
+  compute_tile_few8(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, rows, xs, acc0, lut_lo, lut_hi, q8);
+  compute_tile_few8(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, rows, xs, acc1, lut_lo, lut_hi, q8);
+  compute_tile_few8(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, rows, xs, acc2, lut_lo, lut_hi, q8);
+  compute_tile_few8(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, rows, xs, acc3, lut_lo, lut_hi, q8);
+}
+
 // `a`: the lane's sixteen activation bytes of the chunk (row r16 % 4 of the slot, the k range of group r16 / 4 that this
 // lane owns in the MFMA A operand); grp: that group.
 __device__ __forceinline__ void compute_few(const Chunk& ch, const u32x4_t& a, int grp, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
@@ -199,10 +233,10 @@ struct FewActs {
   const uint16_t* at;              // the lane's sixteen bytes of the wavefront's first chunk
   __device__ __forceinline__ u32x4_t load(int i) const { return *reinterpret_cast<const u32x4_t*>(at + (int64_t)i * 128); }
   template <int EPI>
-  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int c0, int n, int lane) {
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int row0, int c0, int n, int lane) {
     const int q = lane >> 4, r16 = lane & 15;
     grp = r16 >> 2;
-    at = activation_row<EPI>(p, sl, r16 & 3) + (int64_t)c0 * 128 + 32 * grp + 8 * q;
+    at = activation_row<EPI>(p, sl, row0 + (r16 & 3)) + (int64_t)c0 * 128 + 32 * grp + 8 * q;
     q8 = 8 * q;
     held[0] = load(0);
     if (n > 1) held[1] = load(1);
@@ -214,12 +248,44 @@ struct FewActs {
   }
 };
 
+struct FewActs8 {  // E4M3 activations: eight codes a lane and chunk, and the scales of the slot's four rows at the lane's output group
+  static constexpr int LOADS = 5;
+  long held[2];
+  f32x4_t scale[2];
+  int grp;
+  uint32_t q8;
+  const uint8_t* at;       // the lane's eight codes of the wavefront's first chunk
+  const float* scales;     // the scale matrix
+  uint32_t soff[4];        // in it, the scale of slot row row0 + i at group q of that chunk (the launch keeps the matrix under 2^32 scales)
+  __device__ __forceinline__ void load(int slot, int i) {
+    held[slot] = *reinterpret_cast<const long*>(at + (int64_t)i * 128);
+    scale[slot] = f32x4_t{scales[soff[0] + 4 * i], scales[soff[1] + 4 * i], scales[soff[2] + 4 * i], scales[soff[3] + 4 * i]};
+  }
+  template <int EPI>
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int row0, int c0, int n, int lane) {
+    const int q = lane >> 4, r16 = lane & 15;
+    grp = r16 >> 2;
+    at = p.aq + activation_row_index<EPI>(p, sl, row0 + (r16 & 3)) * p.a_stride + (int64_t)c0 * 128 + 32 * grp + 8 * q;
+    scales = p.aq_scale;
+#pragma unroll
+    for (int i = 0; i < 4; i++) soff[i] = (uint32_t)(activation_row_index<EPI>(p, sl, row0 + i) * (p.a_stride >> 5)) + 4 * c0 + q;
+    q8 = 8 * q;
+    load(0, 0);
+    if (n > 1) load(1, 1);
+  }
+  template <int ODD, bool MORE2, bool MORE1>
+  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+    compute_few8(ch, held[ODD], scale[ODD], grp, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi, q8);
+    if (MORE2) load(ODD, i + 2);
+  }
+};
+
 struct FullActs {  // up to sixteen rows: lane (q, r16) feeds row r16, k 8 q .. 8 q + 7 of every group
   static constexpr int LOADS = 4;
   Rows held;           // one chunk's fragments; each half is asked for again as soon as its groups are done
   const uint16_t* at;
   template <int EPI>
-  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int c0, int, int lane) {
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int, int c0, int, int lane) {
     at = activation_row<EPI>(p, sl, lane & 15) + (int64_t)c0 * 128 + 8 * (lane >> 4);
     load_rows(held, at);
   }
@@ -239,9 +305,10 @@ struct FullActs {  // up to sixteen rows: lane (q, r16) feeds row r16, k 8 q .. 
   }
 };
 
-// Chunks c0 .. c1 - 1 (at least one) of block row `nb`, through the wavefront's ring.
+// Chunks c0 .. c1 - 1 (at least one) of block row `nb`, through the wavefront's ring, for the slot's rows from row0 (the
+// four-row bodies: row0 .. row0 + 3; the sixteen-row body: all, row0 = 0).
 template <int EPI, class Acts>
-__device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& sl, int nb, int c0, int c1, int lane, uint8_t* ring,
+__device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& sl, int row0, int nb, int c0, int c1, int lane, uint8_t* ring,
                                              f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) {
   constexpr int BEHIND = BLOCK_LOADS + Acts::LOADS;
   const int r16 = lane & 15, n = c1 - c0;
@@ -256,7 +323,7 @@ __device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& 
   Chunk ch;
   request_chunk(src, c0, slot0);
   asm volatile("" ::: "memory");  // whatever else the prologue asks for stands behind the first block
-  acts.template start<EPI>(p, sl, c0, n, lane);
+  acts.template start<EPI>(p, sl, row0, c0, n, lane);
   if (n == 1) {
     take_chunk<0, 0>(ch, codes, scales);
     acts.template step<0, false, false>(ch, 0, acc0, acc1, acc2, acc3, sl);
@@ -291,12 +358,13 @@ __device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& 
 // The end of a 64-row block for a slot of at most four rows. Lane (g, r16) of each of the block's K splits holds, in
 // register r of accumulator t, group g's part of (tile t, slot row r, column r16): sixteen values a lane, each to be
 // added over the four groups and the splits. They go to LDS, and the workgroup's 64 x ks lanes share the 16 x 16
-// results of the block: lane (q, r16) of split `ks` takes tile q, column r16, of slot rows ks, ks + p.ks, ... It
+// results of the block: lane (q, r16) of split `ks` takes tile q, column r16, of slot rows row0 + ks, row0 + ks + p.ks, ... It
 // multiplies by its tile's row scale (`scale`, asked for before the first chunk); a gated pair's gate comes from the
 // neighbouring tile's lane. Every wavefront of the workgroup must call it when K is split (one workgroup barrier).
 template <int EPI>
-__device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl, float scale, int nb, bool active, int wave, int ks, int nbi,
-                                           float* partial, const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2, const f32x4_t& acc3) {
+__device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl, int row0, float scale, int nb, bool active, int wave, int ks,
+                                           int nbi, float* partial, const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2,
+                                           const f32x4_t& acc3) {
   constexpr int STRIDE = RING_BYTES / 4;
   const int lane = threadIdx.x & 63, q = lane >> 4, r16 = lane & 15;
   float* mine = partial + wave * STRIDE;
@@ -315,7 +383,8 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
   }
   if (!active) return;
   const float* first = partial + nbi * p.ks * STRIDE + r16;
-  for (int r = ks; r < sl.rows; r += p.ks) {
+  const int rows = min(FEW_ROWS, sl.rows - row0);
+  for (int r = ks; r < rows; r += p.ks) {
     const float* at = first + (q * 4 + r) * 64;
     float v = 0.f;
     for (int s = 0; s < p.ks; s++) {
@@ -325,15 +394,17 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
     const float y = v * scale;
     if (EPI == EPI_FC1_GATED) {
       const float gate = __shfl_xor(y, 16);  // tiles 2 t and 2 t + 1 are a pair's up and gate rows
-      if ((q & 1) == 0) store_out<EPI>(p, sl, nb, q >> 1, r, r16, y, gate);
+      if ((q & 1) == 0) store_out<EPI>(p, sl, nb, q >> 1, row0 + r, r16, y, gate);
     } else {
-      store_out<EPI>(p, sl, nb, q, r, r16, y, 0.f);
+      store_out<EPI>(p, sl, nb, q, row0 + r, r16, y, 0.f);
     }
   }
 }
 
 // General kernel, any K: one workgroup per (run of p.nbw 64-row blocks, slot), K split p.ks ways across its wavefronts.
-template <int EPI>
+// A8: E4M3 activations (p.aq, p.aq_scale); every slot goes through the four-row body, four of its rows at a time (the
+// later passes find the block row in L2).
+template <int EPI, bool A8>
 __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   extern __shared__ __align__(16) uint8_t rings[];
   const Slot sl = slot_of<EPI>(p, blockIdx.y);
@@ -344,17 +415,25 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
   uint8_t* ring = rings + wave * RING_BYTES;
-  if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
+  if (A8) {
+    const float scale = active ? sl.rs[nb * 64 + lane] : 0.f;
+    for (int row0 = 0; row0 < sl.rows; row0 += FEW_ROWS) {  // uniform over the workgroup
+      acc0 = acc1 = acc2 = acc3 = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (active) stream_block<EPI, FewActs8>(p, sl, row0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      finish_few<EPI>(p, sl, row0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+      if (p.ks > 1) __syncthreads();  // the exchange is read before the next pass fills the rings it lies in
+    }
+  } else if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
     float scale = 0.f;
     if (active) {
       scale = sl.rs[nb * 64 + lane];  // row 16 q + r16 of the block: asked for ahead of the chunks, there when the epilogue wants it
-      stream_block<EPI, FewActs>(p, sl, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);  // at least one chunk: ks <= chunks
+      stream_block<EPI, FewActs>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);  // at least one chunk: ks <= chunks
     }
-    finish_few<EPI>(p, sl, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+    finish_few<EPI>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
   } else {
     RowScales rs{};
     if (active) {
-      stream_block<EPI, FullActs>(p, sl, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      stream_block<EPI, FullActs>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
       rs = row_scales<true>(sl, nb, lane & 15);
     }
     finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
@@ -393,6 +472,46 @@ struct TileW3 {
   }
 };
 
+// ------------------------------------------------------------------------------------------ activation rounding
+//
+// BF16 [m, k] -> E4M3 codes [m, k] and one FP32 scale per (row, 32-group): s = max(amax / 448, 1e-12),
+// q = e4m3(clamp(x / s, -448, 448)), both quotients IEEE FP32 divisions (the reference's torch statement of its
+// quantizer, hibana/kernels/w3_moe.py:187-190; its CUDA kernel, hibana/kernels/csrc/w3_gemm.cu:291-327, multiplies by
+// an approximate reciprocal instead). One lane takes eight consecutive values, four lanes a group.
+__global__ __launch_bounds__(256) void w3_quant_groups_kernel(const uint16_t* __restrict__ x, int64_t lanes, uint8_t* __restrict__ q,
+                                                              float* __restrict__ scales) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= lanes) return;  // whole groups: k is a multiple of 32, so a group's four lanes are in or out together
+  const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(x + 8 * i);
+  float v[8];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    v[2 * j] = __uint_as_float(raw[j] << 16);
+    v[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(v[j]));
+  amax = fmaxf(amax, __shfl_xor(amax, 1));
+  amax = fmaxf(amax, __shfl_xor(amax, 2));
+  const float s = fmaxf(amax / 448.0f, 1e-12f);
+#pragma unroll
+  for (int j = 0; j < 8; j++) v[j] = fminf(fmaxf(v[j] / s, -448.0f), 448.0f);
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], hi, true);
+  typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+  *reinterpret_cast<i32x2_t*>(q + 8 * i) = i32x2_t{lo, hi};
+  if ((i & 3) == 0) scales[i >> 2] = s;
+}
+
+static void launch_quant_groups(const void* x, int64_t rows, int k, uint8_t* q, float* scales, hipStream_t stream) {
+  const int64_t lanes = rows * k / 8;
+  HB_LAUNCH(w3_quant_groups_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream, static_cast<const uint16_t*>(x), lanes, q, scales);
+}
+
 // ---------------------------------------------------------------------------------------------------- host side
 struct Tuning {
   int w3_tile = 0, w3_few = 0, w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0;
@@ -418,7 +537,11 @@ static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Lau
   p.no_few = g_tune.w3_few == 2;  // every slot takes the sixteen-row body
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
-  HB_LAUNCH(w3_stream_kernel<EPI>, grid, dim3(64 * waves), (size_t)waves * RING_BYTES, stream, p);
+  if (p.aq) {
+    HB_LAUNCH((w3_stream_kernel<EPI, true>), grid, dim3(64 * waves), (size_t)waves * RING_BYTES, stream, p);
+  } else {
+    HB_LAUNCH((w3_stream_kernel<EPI, false>), grid, dim3(64 * waves), (size_t)waves * RING_BYTES, stream, p);
+  }
   return HB_OK;
 }
 
@@ -468,6 +591,36 @@ extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* 
   return launch_status();
 }
 
+extern "C" int hb_w3_quant_groups(const void* x, int64_t m, int k, void* q, float* scales, void* stream) {
+  if (!x || !q || !scales) return HB_ENULL;
+  if (m <= 0 || k <= 0 || k % 32) return HB_EINVAL;
+  launch_quant_groups(x, m, k, static_cast<uint8_t*>(q), scales, as_stream(stream));
+  return launch_status();
+}
+
+extern "C" int hb_w3_gemm_e4m3(const void* xq, const float* x_scale, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k,
+                               void* y, void* stream) {
+  if (!xq || !x_scale || !tiled || !row_scale || !y) return HB_ENULL;
+  if (m <= 0 || n <= 0 || k <= 0 || n % W3_BLOCK_ROWS || k % W3_CHUNK || (int64_t)m * (k / 32) > 0xffffffffll) return HB_EINVAL;
+  StreamParams p{};
+  p.w = static_cast<const uint8_t*>(tiled);
+  p.rows = row_scale;
+  p.lut_lo = (uint32_t)((uint64_t)lut & 0xffffffffu);
+  p.lut_hi = (uint32_t)((uint64_t)lut >> 32);
+  p.n_blocks = n / W3_BLOCK_ROWS;
+  p.chunks = k / W3_CHUNK;
+  p.aq = static_cast<const uint8_t*>(xq);
+  p.aq_scale = x_scale;
+  p.a_stride = k;
+  p.m = m;
+  p.out = y;
+  p.out_stride = n;
+  const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
+  if (slots > 65535) return HB_EINVAL;
+  if (int e = launch_stream<EPI_DENSE>(p, slots, slots, Launch{g_tune.w3_ksplit, g_tune.w3_nbw}, as_stream(stream))) return e;
+  return launch_status();
+}
+
 // ------------------------------------------------------------------------------------------------ routed experts
 namespace {
 
@@ -490,11 +643,13 @@ struct Routing {  // set: the chain routes `logits` [m, e] itself into the calle
 };
 
 int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void* x, const int32_t* ids, int m, int topk,
-                const MoeWorkspace& ws, void* out_pairs, int pairs_bf16, hipStream_t stream, const Routing* route = nullptr) {
+                const MoeWorkspace& ws, void* out_pairs, int pairs_bf16, hipStream_t stream, const Routing* route = nullptr,
+                bool e4m3 = false) {
   const int64_t pairs = (int64_t)m * topk;
   const int shared_rows = shared ? m : 0;
   // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel
-  const bool dense = g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && pairs >= (int64_t)ex->experts * 2 * TILE_DENSE_ROWS);  // the pre-scaled expansion costs more here than the stream's
+  // (E4M3 activations: the stream only)
+  const bool dense = !e4m3 && (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && pairs >= (int64_t)ex->experts * 2 * TILE_DENSE_ROWS));  // the pre-scaled expansion costs more here than the stream's
   const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
   const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows, slot_rows);
   if (slots > 65535) return HB_EINVAL;
@@ -556,7 +711,16 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
     return launch_status();
   }
   const Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
+  if (e4m3) {  // x and h go through the activation rounding: x_q -> fc1 -> h (BF16) -> h_q -> fc2
+    launch_quant_groups(x, m, ex->hidden, ws.xq, ws.xs, stream);
+    p.aq = ws.xq;
+    p.aq_scale = ws.xs;
+    f2.aq = ws.hq;
+    f2.aq_scale = ws.hs;
+  }
   if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) return e;
+  // rows of h past the kept pairs are never written: the quantizer reads them and nobody reads what it makes of them
+  if (e4m3) launch_quant_groups(ws.h, pairs + shared_rows, ex->inter, ws.hq, ws.hs, stream);
   if (int e = launch_stream<EPI_FC2>(f2, slots, est, l2, stream)) return e;
   return launch_status();
 }
@@ -565,18 +729,20 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
 
 extern "C" size_t hb_w3_moe_workspace_bytes(int m, int topk, const hb_w3_experts* routed, int shared) {
   if (!routed || m <= 0 || topk <= 0 || check_experts(routed) != HB_OK) return 0;
-  return moe_carve(nullptr, m, topk, routed->experts, routed->inter, routed->hidden_out, shared).bytes;
+  return moe_carve(nullptr, m, topk, routed->experts, routed->inter, routed->hidden_out, shared, routed->hidden).bytes;
 }
 
 extern "C" int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32_t* ids, const float* weights, int m, int topk, int mode,
                          void* out, void* workspace, size_t workspace_bytes, void* stream) {
   if (int e = check_experts(routed)) return e;
   if (!x || !ids || !weights || !out || !workspace) return HB_ENULL;
+  const bool e4m3 = (mode & HB_MOE_E4M3) != 0;
+  mode &= ~HB_MOE_E4M3;
   if (m <= 0 || topk <= 0 || mode < HB_MOE_SUM || mode > HB_MOE_PAIRS_BF16) return HB_EINVAL;
-  const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, 0);
+  const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
   void* pairs_out = mode == HB_MOE_SUM ? static_cast<void*>(ws.y) : out;
-  if (int e = run_experts(routed, nullptr, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16, as_stream(stream))) return e;
+  if (int e = run_experts(routed, nullptr, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16, as_stream(stream), nullptr, e4m3)) return e;
   if (mode == HB_MOE_SUM) {
     CombineParams c{};
     c.pairs = ws.y;
@@ -605,7 +771,7 @@ static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, c
   }
   if (!x || !ids || !weights || !out || !workspace) return HB_ENULL;
   if (m <= 0 || topk <= 0) return HB_EINVAL;
-  const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, shared ? 1 : 0);
+  const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, shared ? 1 : 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
   if (int e = run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream), route)) return e;
   CombineParams c{};

@@ -231,26 +231,53 @@ def interleave_rows(weight: W3Weight, block: int) -> W3Weight:
                    row_scale=weight.row_scale[rows].contiguous(), tiled=None)
 
 
-def quant_groups(x: torch.Tensor):
-    raise NotImplementedError("E4M3 activation quantization is not part of the weight-only kernels (activations stay BF16)")
+def quant_rows(x: torch.Tensor):
+    """One E4M3 scale per row (hibana/kernels/w3.py:326-330): the reference keeps it for comparison only (it loses the
+    small channels next to an outlier) and serves `quant_groups`; not built here."""
+    raise NotImplementedError("per-row E4M3 activation quantization is not built; use quant_groups")
 
 
-quant_rows = quant_groups
+def quant_groups(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-(row, 32-group) E4M3 quantization of a BF16 [M, K] matrix: (x_q float8_e4m3fn [M, K], scale float32
+    [M, K/32]), scale = max(amax / 448, 1e-12), x_q = e4m3(x / scale) (hibana/kernels/w3.py:333-337, with the exact
+    divisions of its torch statement, hibana/kernels/w3_moe.py:187-190)."""
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % GROUP:
+        raise ValueError("quant_groups: BF16 [M, K] with K a multiple of 32")
+    _lib.need_gpu(x)
+    m, k = x.shape
+    q = torch.empty((m, k), dtype=torch.float8_e4m3fn, device=x.device)
+    scale = torch.empty((m, k // GROUP), dtype=torch.float32, device=x.device)
+    if m:
+        _lib.check(_lib.lib().hb_w3_quant_groups(_lib.ptr(x.contiguous()), m, k, _lib.ptr(q), _lib.ptr(scale), _lib.stream()), "quant_groups")
+    return q, scale
 
 
 def w3_linear(x: torch.Tensor, w3: W3Weight, x_scale: torch.Tensor | None = None, splits: int | None = None) -> torch.Tensor:
-    """y = x @ W^T for x [M, K] BF16, M <= MAX_ROWS; returns BF16 [M, N] (hibana/kernels/w3.py:340-365).
+    """y = x @ W^T for x [M, K], M <= MAX_ROWS; returns BF16 [M, N] (hibana/kernels/w3.py:340-365). BF16 x: the
+    weight-only product (x is NOT re-quantized, unlike the reference). E4M3 x with its scale (one per tensor, per row or
+    per (row, 32-group), as `quant_groups` makes them): the reference kernel's arithmetic on those codes.
     `splits` is accepted for signature compatibility; the K split is chosen by the library."""
     m, k = x.shape
     if m > MAX_ROWS or k != w3.in_features:
         raise ValueError("w3_linear: unsupported call")
-    if x.dtype != torch.bfloat16:
-        raise ValueError("w3_linear: the weight-only kernels take BF16 activations")
+    if x.dtype == torch.float8_e4m3fn:
+        if x_scale is None:
+            raise ValueError("FP8 activations need their scale")
+    elif x.dtype != torch.bfloat16:
+        raise ValueError("w3_linear: BF16 activations, or E4M3 ones with their scale")
     _lib.need_gpu(x)
     tile(w3)
     x = x.contiguous()
     y = torch.empty((m, w3.out_features), dtype=torch.bfloat16, device=x.device)
     if m == 0:
+        return y
+    if x.dtype == torch.float8_e4m3fn:
+        groups = k // GROUP
+        if x_scale.numel() not in (1, m, m * groups):
+            raise ValueError("w3_linear: x_scale must have 1, M or M * K/32 elements")
+        scale = x_scale.float().reshape(-1, groups if x_scale.numel() == m * groups else 1).expand(m, groups).contiguous()
+        _lib.check(_lib.lib().hb_w3_gemm_e4m3(_lib.ptr(x), _lib.ptr(scale), m, _lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut,
+                                              w3.out_features, k, _lib.ptr(y), _lib.stream()), "w3_linear")
         return y
     _lib.check(_lib.lib().hb_w3_gemm(_lib.ptr(x), m, _lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut, w3.out_features, k,
                                      _lib.ptr(y), _lib.stream()), "w3_linear")

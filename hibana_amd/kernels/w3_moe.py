@@ -124,13 +124,17 @@ def _check_call(experts: W3Experts, x, ids, weights):
     _lib.need_gpu(x, ids, weights)
 
 
+MOE_E4M3 = 16  # hb_w3_moe mode flag: activations through the reference's E4M3 rounding
+
+
 def w3_moe(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, pairs: bool = False,
-           pairs_bf16: bool = False) -> torch.Tensor:
+           pairs_bf16: bool = False, e4m3: bool = False) -> torch.Tensor:
     """Routed experts for x [M, H] BF16 with the router's ids [M, k] and weights [M, k] -> BF16 [M, H_out], the
     weighted sum in selection order (no shared expert). An id outside this object's range base .. base + E - 1 (another
     rank's expert, or the "no expert" id 512) adds nothing. With `pairs`, the FP32 (`pairs_bf16`: BF16) output of each
     (row, k) pair [M * k, H_out], unsummed; rows of skipped pairs are unspecified
-    (hibana/kernels/w3_moe.py:158-179)."""
+    (hibana/kernels/w3_moe.py:158-179). `e4m3`: x and h are rounded to E4M3 per (row, 32-group) before their products, as
+    the reference kernel does (its torch statement: hibana/kernels/w3_moe.py:193-214); default: weight-only."""
     _check_call(experts, x, ids, weights)
     m, k = ids.shape
     h_out = experts.shape2[0]
@@ -144,6 +148,7 @@ def w3_moe(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: torc
     ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     ids32 = ids.to(torch.int32).contiguous()
     wt = weights.float().contiguous()
+    mode |= MOE_E4M3 if e4m3 else 0
     _lib.check(_lib.lib().hb_w3_moe(C.byref(st), _lib.ptr(x.contiguous()), _lib.ptr(ids32), _lib.ptr(wt), m, k, mode, _lib.ptr(out),
                                     _lib.ptr(ws), need, _lib.stream()), "w3_moe")
     return out

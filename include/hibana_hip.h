@@ -92,6 +92,22 @@ int hb_w3_dequant(const void* tiled, const float* row_scale, int64_t lut, int64_
 int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, void* y,
                void* stream);
 
+/* The reference's activation rounding: x BF16 [m, k] (k % 32 == 0) -> q E4M3 bytes [m, k], scales float32 [m, k / 32]:
+ * s = max(amax / 448, 1e-12) per (row, 32-group), q = e4m3(clamp(x / s, -448, 448)), IEEE FP32 divisions.
+ * ref: w3.quant_groups, hibana/kernels/w3.py:333-337 (quant_groups_kernel, hibana/kernels/csrc/w3_gemm.cu:291-327), as
+ * its torch statement defines it (hibana/kernels/w3_moe.py:187-190): the CUDA kernel multiplies by an approximate
+ * reciprocal, whose bits are NVIDIA's. */
+int hb_w3_quant_groups(const void* x, int64_t m, int k, void* q, float* scales, void* stream);
+
+/* hb_w3_gemm on rounded activations, the reference kernel's own arithmetic:
+ * y[m, n] = bf16( row_scale[n] * sum_g (x_scale[m, g] * scale[n, g]) * sum_{k in g} xq[m, k] * level[code[n, k]] ),
+ * FP8 x FP8 products summed in FP32 a group. xq E4M3 [m, k], x_scale float32 [m, k / 32] as hb_w3_quant_groups makes
+ * them. Served by the weight stream at any m (the reference stops at 128 rows).
+ * ref: w3_gemm, hibana/kernels/csrc/w3_gemm.cu:105-108,209-210,1299-1331 (w3.w3_linear with E4M3 x, hibana/kernels/
+ * w3.py:340-365). */
+int hb_w3_gemm_e4m3(const void* xq, const float* x_scale, int m, const void* tiled, const float* row_scale, int64_t lut,
+                    int n, int k, void* y, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * Routed experts on W3 weights (gated SiLU when fc1 has 2*inter rows per expert in the reference's fc1_order, ReLU^2
  * when it has inter rows).
@@ -108,7 +124,7 @@ typedef struct hb_w3_experts {
   int gated;
 } hb_w3_experts;
 
-enum { HB_MOE_SUM = 0, HB_MOE_PAIRS_F32 = 1, HB_MOE_PAIRS_BF16 = 2 };
+enum { HB_MOE_SUM = 0, HB_MOE_PAIRS_F32 = 1, HB_MOE_PAIRS_BF16 = 2, HB_MOE_E4M3 = 16 /* flag: or it into a mode */ };
 
 /* Workspace bytes for hb_w3_moe / hb_w3_moe_layer with up to m rows of top-k ids (shared: 1 if a shared expert rides
  * along). */
@@ -118,8 +134,10 @@ size_t hb_w3_moe_workspace_bytes(int m, int topk, const hb_w3_experts* routed, i
  * y = fc2_e( act( bf16(fc1_e x_r) ) ) in FP32, h rounded to BF16. ids int32 [m, topk]; an id outside
  * [base, base + experts) adds nothing. mode HB_MOE_SUM: out BF16 [m, hidden_out]; HB_MOE_PAIRS_F32 / _BF16: out is
  * the unsummed pair outputs [m * topk, hidden_out] (rows of dropped pairs are left untouched).
- * ref: w3_moe, hibana/kernels/csrc/w3_gemm.cu:1366-1382 (run<S> :1215-1292; Python hibana/kernels/w3_moe.py:158-179),
- * weight-only form. */
+ * With HB_MOE_E4M3 or-ed into mode, x and h go through the reference's activation rounding (hb_w3_quant_groups) before
+ * their products, as in the reference kernel (y = fc2_e(Q(act(bf16(fc1_e Q(x_r)))))); without it the weight-only form.
+ * ref: w3_moe, hibana/kernels/csrc/w3_gemm.cu:1366-1382 (run<S> :1215-1292; Python hibana/kernels/w3_moe.py:158-179;
+ * its torch statement w3_moe.reference, :193-214). */
 int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32_t* ids, const float* weights, int m, int topk,
               int mode, void* out, void* workspace, size_t workspace_bytes, void* stream);
 

@@ -21,11 +21,20 @@ points of the reference kept.
                          sigmoid + bias (ties to the lower id), weights from the plain sigmoid, renormalized, scaled
   latent_moe_ref         tests/nemotron_reference.py:568-593 (ReLU^2 latent experts, BF16 linears, FP32 accumulate)
   silu_and_mul           hibana/kernels/ops.py:86-92
+  quant_e4m3_groups      hibana/kernels/w3_moe.py:187-190 (the torch mirror of the activation rounding, the definition
+                         to follow; the CUDA quantizer of hibana/kernels/csrc/w3_gemm.cu:291-327 multiplies by an
+                         approximate reciprocal instead of dividing, so its bits are PARITY UNPINNED here): per (row,
+                         32-group) s = max(amax / 448, 1e-12) in FP32, q = e4m3(clamp(x / s, -448, 448))
+  dense_a8_ref           hibana/kernels/w3.py:340-365 with quantized activations (the reference kernel's own math,
+                         hibana/kernels/csrc/w3_gemm.cu:105-108,209-210): x is replaced by q * s
+  `quant=` of the expert functions: hibana/kernels/w3_moe.py:193-214 with quant = quant_e4m3 (x and h both rounded)
 
 Pinned by (tests/test_oracle_layers.py): special cases that reduce to textbook routines (one token, one expert, weight
 one == two dense products; all weights zero == zero; a permutation of slots with equal weights), brute-force
 per-pair Python loops on tiny shapes written from the formula in w3_moe.py:205-213, torch.topk/softmax for the
-routing, and sortedness/CSR invariants for the plan.
+routing, and sortedness/CSR invariants for the plan. quant_e4m3_groups: a brute-force nearest-value search over the
+256-entry E4M3 table (ties to the even code) on random and hand-made groups, the group maximum landing on +-448 * s, and
+groups that are already E4M3 multiples of their scale coming back unchanged.
 """
 from __future__ import annotations
 
@@ -52,6 +61,31 @@ def nvfp4_dense_ref(x: torch.Tensor, w_unscaled, scale2: float, relu2: bool = Fa
     if relu2:
         y = bf16(torch.relu(y.float()).square())
     return y
+
+
+def quant_e4m3_groups(t: torch.Tensor):
+    """t [M, K] (K % 32 == 0) -> (E4M3 bytes uint8 [M, K], scales float32 [M, K/32])."""
+    m, k = t.shape
+    g = t.float().reshape(m, k // 32, 32)
+    s = (g.abs().amax(-1, keepdim=True) / 448.0).clamp_min(1e-12)
+    q = (g / s).clamp(-448, 448).to(torch.float8_e4m3fn)
+    return q.view(torch.uint8).reshape(m, k), s.reshape(m, k // 32)
+
+
+def dequant_e4m3_groups(q: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
+    """float32 [M, K] = e4m3(q) * s, a group's scale over its 32 columns."""
+    m, k = q.shape
+    return (q.view(torch.float8_e4m3fn).float().reshape(m, k // 32, 32) * s.reshape(m, k // 32, 1)).reshape(m, k)
+
+
+def rounded_e4m3(t: torch.Tensor) -> torch.Tensor:
+    """t through the activation rounding and back: what the E4M3-activation kernels multiply with."""
+    return dequant_e4m3_groups(*quant_e4m3_groups(t))
+
+
+def dense_a8_ref(x: torch.Tensor, w_deq) -> torch.Tensor:
+    """x [M, K] rounded to E4M3 per (row, 32-group), times w_deq float32 [N, K], one rounding to BF16."""
+    return bf16((rounded_e4m3(x).double() @ torch.as_tensor(w_deq).double().T).float())
 
 
 def fc1_order(inter: int) -> np.ndarray:
@@ -85,20 +119,22 @@ def silu_and_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:
     return torch.nn.functional.silu(gate_up[..., :half]) * gate_up[..., half:]
 
 
-def expert_pairs_ref(x: torch.Tensor, rows: np.ndarray, w13, w2, gated: bool) -> torch.Tensor:
+def expert_pairs_ref(x: torch.Tensor, rows: np.ndarray, w13, w2, gated: bool, quant=None) -> torch.Tensor:
     """One expert on the token rows `rows` of x: w13 float32 [N1, K] with rows in checkpoint order ([up; gate] when
-    gated, up alone otherwise), w2 float32 [H, I] -> FP32 [len(rows), H]."""
+    gated, up alone otherwise), w2 float32 [H, I] -> FP32 [len(rows), H]. `quant` (None: weight-only) rounds x and h
+    before their products, as the reference's `quant` argument does."""
     w13, w2 = torch.as_tensor(w13).double(), torch.as_tensor(w2).double()
-    h1 = bf16((x[torch.as_tensor(rows)].double() @ w13.T).float()).float()
+    xr = x[torch.as_tensor(rows)]
+    h1 = bf16(((quant(xr) if quant else xr).double() @ w13.T).float()).float()
     if gated:
         inter = w13.shape[0] // 2
         h = bf16(torch.nn.functional.silu(h1[:, inter:]) * h1[:, :inter])
     else:
         h = bf16(torch.relu(h1).square())
-    return (h.double() @ w2.T).float()
+    return ((quant(h) if quant else h).double() @ w2.T).float()
 
 
-def routed_experts_ref(x: torch.Tensor, ids: np.ndarray, get_expert, gated: bool, e_lo: int = 0, e_n: int = 512):
+def routed_experts_ref(x: torch.Tensor, ids: np.ndarray, get_expert, gated: bool, e_lo: int = 0, e_n: int = 512, quant=None):
     """FP32 pair outputs [M*k, H] (rows of dropped pairs are zero). get_expert(local id) -> (w13 [N1, K] float32 in
     checkpoint row order, w2 [H, I] float32)."""
     ids = np.asarray(ids)
@@ -108,7 +144,7 @@ def routed_experts_ref(x: torch.Tensor, ids: np.ndarray, get_expert, gated: bool
     for d, e in enumerate(experts):
         q = order[starts[d]:starts[d + 1]]
         w13, w2 = get_expert(int(e))
-        y = expert_pairs_ref(x, q // k, w13, w2, gated)
+        y = expert_pairs_ref(x, q // k, w13, w2, gated, quant)
         if pairs is None:
             pairs = torch.zeros(m * k, y.shape[1], dtype=torch.float32)
         pairs[torch.as_tensor(q)] = y

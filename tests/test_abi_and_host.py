@@ -35,7 +35,7 @@ def test_validation_without_a_gpu():
     assert lib.hb_w3_tiled_bytes(96, 2048) == 0 and lib.hb_w3_tiled_bytes(128, 100) == 0
     assert lib.hb_nvfp4_tiled_bytes(128, 256) == 128 * 256 // 2 + 128 * 256 // 16
     assert lib.hb_nvfp4_tiled_bytes(128, 64) == 0
-    assert lib.hb_tune(b"no_such_knob", 1) == _lib.HB_EINVAL and lib.hb_tune(b"w3_ksplit", 3) == _lib.HB_EINVAL
+    assert lib.hb_tune(b"no_such_knob", 1) == _lib.HB_EINVAL and lib.hb_tune(b"w3_ksplit", 17) == _lib.HB_EINVAL
     assert lib.hb_tune(b"w3_ksplit", 4) == 0 and lib.hb_tune(b"w3_ksplit", 0) == 0
     assert lib.hb_w3_repack(None, None, 128, 128, 3, None, None) == _lib.HB_ENULL
     assert lib.hb_w3_gemm(None, 1, None, None, 0, 128, 128, None, None) == _lib.HB_ENULL
@@ -94,7 +94,11 @@ def test_host_logic_mirrors_the_reference_interface(monkeypatch):
     with pytest.raises(ValueError):
         w3.pack_codes(torch.full((128, 128), 9, dtype=torch.uint8), torch.zeros(128, 4).to(torch.float8_e4m3fn), torch.ones(128))
     with pytest.raises(NotImplementedError):
-        w3.quant_groups(torch.zeros(1, 32))
+        w3.quant_rows(torch.zeros(1, 32))
+    with pytest.raises(ValueError):
+        w3.quant_groups(torch.zeros(1, 32))  # not BF16
+    with pytest.raises(RuntimeError):
+        w3.quant_groups(torch.zeros(1, 32, dtype=torch.bfloat16))  # no CPU path
 
 
 def test_bench_refuses_more_than_one_gpu():

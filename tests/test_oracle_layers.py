@@ -144,3 +144,81 @@ def test_silu_and_mul_layouts():
     assert torch.allclose(plain, torch.nn.functional.silu(gu[:, :128]) * gu[:, 128:])
     order = torch.arange(256).view(2, 2, 64).transpose(0, 1).reshape(-1)  # pair_order(256, 64)
     assert torch.allclose(L.silu_and_mul(gu[:, order], pairs=64), plain)
+
+
+# ------------------------------------------------------------------------------------------ E4M3 activation rounding
+def _e4m3_table():
+    """Every finite E4M3 value from the bit fields (1 sign, 4 exponent bits with bias 7, 3 mantissa bits, no infinities,
+    0x7f / 0xff NaN), written out here rather than taken from a dtype cast."""
+    vals = []
+    for byte in range(256):
+        sign, exp, man = byte >> 7, (byte >> 3) & 15, byte & 7
+        if exp == 15 and man == 7:
+            vals.append(float("nan"))
+            continue
+        mag = man / 8.0 * 2.0 ** -6 if exp == 0 else (1 + man / 8.0) * 2.0 ** (exp - 7)
+        vals.append(-mag if sign else mag)
+    return np.array(vals, dtype=np.float64)
+
+
+def _nearest_e4m3(v: float, table: np.ndarray) -> int:
+    """The code whose value is nearest to v; of two equally near, the one with the even code (round to nearest even)."""
+    dist = np.abs(table - v)
+    dist[np.isnan(dist)] = np.inf
+    best = np.flatnonzero(dist == dist.min())
+    best = [b for b in best if (b < 128) == (v >= 0 or table[b] == 0)] or list(best)  # the zero of v's sign
+    if v == 0:
+        return 0x80 if np.signbit(v) else 0
+    return int(min(best, key=lambda b: (b & 1, b)))
+
+
+def test_quant_e4m3_groups_is_nearest_value_rounding_under_the_group_scale():
+    table = _e4m3_table()
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(6, 96, generator=g) * torch.tensor([1e-3, 0.1, 1.0, 30.0, 3e3, 1.0])[:, None]).bfloat16()
+    x[5, :32] = 0  # an all-zero group: scale 1e-12, codes zero
+    x[5, 40] = -0.0
+    q, s = L.quant_e4m3_groups(x)
+    assert q.dtype == torch.uint8 and q.shape == (6, 96) and s.shape == (6, 3) and s.dtype == torch.float32
+    xf = x.float().numpy()
+    for r in range(6):
+        for grp in range(3):
+            vals = xf[r, 32 * grp:32 * grp + 32]
+            amax = np.float32(np.abs(vals).max())
+            scale = max(np.float32(amax / np.float32(448.0)), np.float32(1e-12))
+            assert s[r, grp].item() == scale
+            for i, v in enumerate(vals):
+                ratio = float(np.float32(v) / scale)  # the FP32 quotient, as the definition divides in FP32
+                want = _nearest_e4m3(min(max(ratio, -448.0), 448.0), table)
+                got = int(q[r, 32 * grp + i])
+                assert table[got] == table[want] and (got == want or table[got] == 0), (r, grp, i, v, got, want)
+            if amax > 0:  # the group's largest magnitude lands on the largest code
+                top = int(np.argmax(np.abs(vals)))
+                assert abs(table[int(q[r, 32 * grp + top])]) == 448.0
+    back = L.dequant_e4m3_groups(q, s)
+    assert torch.all(back[5, :32] == 0)
+
+
+def test_quant_e4m3_groups_keeps_what_is_already_representable():
+    table = _e4m3_table()
+    codes = torch.randint(0, 127, (4, 64), generator=torch.Generator().manual_seed(1))
+    codes[:, 0] = 126  # 448 in every group: the scale is exactly the multiplier
+    codes[:, 32] = 126
+    vals = torch.tensor(table[codes.numpy()], dtype=torch.float32) * 0.25  # a power-of-two scale: bf16-exact
+    q, s = L.quant_e4m3_groups(vals.bfloat16())
+    assert torch.all(s == 0.25) and torch.equal(q.long(), codes)
+    assert torch.equal(L.rounded_e4m3(vals.bfloat16()), vals)
+
+
+def test_dense_a8_ref_is_the_dense_product_of_the_rounded_activations():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(3, 64, generator=g).bfloat16()
+    w = torch.randn(5, 64, generator=g)
+    want = L.dense_ref(L.rounded_e4m3(x), w.numpy())  # rounded values are FP32: dense_ref takes any float x
+    assert torch.equal(L.dense_a8_ref(x, w.numpy()), want)
+    # one expert, one token, weight one: the routed sum with quant is two dense products with both inputs rounded
+    w13, w2 = torch.randn(64, 64, generator=g), torch.randn(64, 32, generator=g)
+    y = L.expert_pairs_ref(x[:1], np.array([0]), w13.numpy(), w2.numpy(), True, quant=L.rounded_e4m3)
+    h1 = L.bf16((L.rounded_e4m3(x[:1]).double() @ w13.double().T).float()).float()
+    h = L.bf16(torch.nn.functional.silu(h1[:, 32:]) * h1[:, :32])
+    assert torch.equal(y, (L.rounded_e4m3(h).double() @ w2.double().T).float())
