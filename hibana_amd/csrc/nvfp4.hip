@@ -11,6 +11,7 @@
 // Codes expand with v_cvt_scalef32_pk_bf16_fp4 (two weights per instruction, exact).
 #include <string.h>
 
+#include "ring.hpp"
 #include "stream_common.hpp"
 #include "tile_kernel.hpp"
 
@@ -91,11 +92,11 @@ __global__ __launch_bounds__(256) void nvfp4_dequant_kernel(const uint8_t* __res
   }
 }
 
-struct Fp4Chunk {  // the weight side of a chunk: prefetched one chunk ahead
+struct Fp4Chunk {  // the weight side of a chunk: four 16-row tiles of codes, their block scales
   u32x4_t w0, w1, w2, w3, s0, s1;
 };
 
-struct Fp4Rows {  // the activation side: read from L2 when the chunk is computed
+struct Fp4Rows {  // the activation side: eight MFMA A fragments (one per 16-block), read from L2
   u32x2_t a0, a1, a2, a3, a4, a5, a6, a7;
 };
 
@@ -107,17 +108,6 @@ __device__ __forceinline__ void load_fp4_chunk(Fp4Chunk& ch, const uint8_t* blk,
   ch.w3 = __builtin_nontemporal_load(b + 192 + lane);
   ch.s0 = __builtin_nontemporal_load(b + 256 + 2 * r16);
   ch.s1 = __builtin_nontemporal_load(b + 257 + 2 * r16);
-}
-
-__device__ __forceinline__ void load_fp4_rows(Fp4Rows& ch, const uint16_t* arow) {
-  ch.a0 = *reinterpret_cast<const u32x2_t*>(arow);
-  ch.a1 = *reinterpret_cast<const u32x2_t*>(arow + 16);
-  ch.a2 = *reinterpret_cast<const u32x2_t*>(arow + 32);
-  ch.a3 = *reinterpret_cast<const u32x2_t*>(arow + 48);
-  ch.a4 = *reinterpret_cast<const u32x2_t*>(arow + 64);
-  ch.a5 = *reinterpret_cast<const u32x2_t*>(arow + 80);
-  ch.a6 = *reinterpret_cast<const u32x2_t*>(arow + 96);
-  ch.a7 = *reinterpret_cast<const u32x2_t*>(arow + 112);
 }
 
 // One 16-block: two conversions, one MFMA, the block scale folded into the accumulator.
@@ -137,72 +127,217 @@ __device__ __forceinline__ void load_fp4_rows(Fp4Rows& ch, const uint16_t* arow)
 
 typedef __attribute__((ext_vector_type(4))) short bf16x4_t_s;  // the 16x16x16 builtin takes its BF16 operands as 4 x i16
 
-__device__ __forceinline__ void fp4_tile(const u32x4_t& w, uint32_t sc_lo, uint32_t sc_hi, const Fp4Rows& ch, f32x4_t& acc) {
-  HB_FP4_BLOCK(w.x, 0, ch.a0, sc_lo, 0, acc)
-  HB_FP4_BLOCK(w.x, 2, ch.a1, sc_lo, 1, acc)
-  HB_FP4_BLOCK(w.y, 0, ch.a2, sc_lo, 2, acc)
-  HB_FP4_BLOCK(w.y, 2, ch.a3, sc_lo, 3, acc)
-  HB_FP4_BLOCK(w.z, 0, ch.a4, sc_hi, 0, acc)
-  HB_FP4_BLOCK(w.z, 2, ch.a5, sc_hi, 1, acc)
-  HB_FP4_BLOCK(w.w, 0, ch.a6, sc_hi, 2, acc)
-  HB_FP4_BLOCK(w.w, 2, ch.a7, sc_hi, 3, acc)
+// Half of a 16-row tile of a chunk: 16-blocks 0 .. 3 (two code dwords, one scale dword, four activation fragments) or
+// 4 .. 7; the blocks of a chunk fold into the accumulator in ascending order either way.
+__device__ __forceinline__ void fp4_half_tile(uint32_t c01, uint32_t c23, uint32_t sc, const u32x2_t& a0, const u32x2_t& a1, const u32x2_t& a2,
+                                              const u32x2_t& a3, f32x4_t& acc) {
+  HB_FP4_BLOCK(c01, 0, a0, sc, 0, acc)
+  HB_FP4_BLOCK(c01, 2, a1, sc, 1, acc)
+  HB_FP4_BLOCK(c23, 0, a2, sc, 2, acc)
+  HB_FP4_BLOCK(c23, 2, a3, sc, 3, acc)
 }
 
-__device__ __forceinline__ void fp4_chunk(const Fp4Chunk& ch, const uint16_t* arow, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
-                                          f32x4_t& acc3) {
-  Fp4Rows rows;
-  load_fp4_rows(rows, arow);
-  fp4_tile(ch.w0, ch.s0.x, ch.s0.y, rows, acc0);
-  fp4_tile(ch.w1, ch.s0.z, ch.s0.w, rows, acc1);
-  fp4_tile(ch.w2, ch.s1.x, ch.s1.y, rows, acc2);
-  fp4_tile(ch.w3, ch.s1.z, ch.s1.w, rows, acc3);
+// ------------------------------------------------------------------------------------------------ the weight ring
+// (ring.hpp) for NVFP4 blocks: four 16-byte loads a lane of codes, two 4-byte loads a lane of scales.
+struct Fp4Ring {
+  typedef Fp4Chunk Chunk;
+  static constexpr int BLOCK_BYTES = NVFP4_BLOCK_BYTES, LOADS = 6;
+  static __device__ __forceinline__ void lanes(RingSource& src, int lane, int r16, uint32_t slot0, uint32_t& codes, uint32_t& scales) {
+    src.codes = 16u * lane;
+    src.scales = 4u * lane;
+    codes = slot0 + 16u * lane;
+    scales = slot0 + 32u * r16;
+  }
+  static __device__ __forceinline__ void request(const RingSource& src, int chunk, lds_ptr_t slot) {
+    const uint32_t at = (uint32_t)chunk * NVFP4_BLOCK_BYTES;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 0, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 2048, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 3072, 2);
+    // the instruction's offset field (which moves both ends) stops at 4095: the scales' place is given by hand
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot + NVFP4_SCALE_OFFSET, 4, src.scales, at + NVFP4_SCALE_OFFSET, 0, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot + NVFP4_SCALE_OFFSET, 4, src.scales, at + NVFP4_SCALE_OFFSET, 256, 2);
+    __builtin_amdgcn_sched_barrier(0);  // asked for here, not wherever the scheduler would sink it below the arithmetic
+  }
+  template <int BEHIND, int SLOT>
+  static __device__ __forceinline__ void take(Chunk& ch, uint32_t codes, uint32_t scales) {
+    asm volatile(
+        "s_waitcnt vmcnt(%8)\n\t"
+        "ds_read_b128 %0, %6 offset:%9\n\t"
+        "ds_read_b128 %1, %6 offset:%10\n\t"
+        "ds_read_b128 %2, %6 offset:%11\n\t"
+        "ds_read_b128 %3, %6 offset:%12\n\t"
+        "ds_read_b128 %4, %7 offset:%13\n\t"
+        "ds_read_b128 %5, %7 offset:%14\n\t"
+        "s_waitcnt lgkmcnt(0)"  // the slot is read: it may be given to another chunk
+        : "=&v"(ch.w0), "=&v"(ch.w1), "=&v"(ch.w2), "=&v"(ch.w3), "=&v"(ch.s0), "=&v"(ch.s1)
+        : "v"(codes), "v"(scales), "n"(BEHIND), "n"(SLOT * NVFP4_BLOCK_BYTES), "n"(SLOT * NVFP4_BLOCK_BYTES + 1024),
+          "n"(SLOT * NVFP4_BLOCK_BYTES + 2048), "n"(SLOT * NVFP4_BLOCK_BYTES + 3072), "n"(SLOT * NVFP4_BLOCK_BYTES + NVFP4_SCALE_OFFSET),
+          "n"(SLOT * NVFP4_BLOCK_BYTES + NVFP4_SCALE_OFFSET + 16)
+        : "memory");
+  }
+};
+constexpr int FP4_RING_BYTES = ring_bytes<Fp4Ring>();  // LDS per wavefront; its first 4 KB double as the K-split exchange
+
+// The stream's activations: lane (q, r16) feeds row r16, k 4 q .. 4 q + 3 of every 16-block. One chunk's fragments are
+// held; each half is asked for again (for the next chunk) as soon as its blocks are done.
+struct Fp4Acts {
+  static constexpr int LOADS = 8;
+  Fp4Rows held;
+  const uint16_t* at;
+  __device__ __forceinline__ void load_lo(const uint16_t* from) {
+    held.a0 = *reinterpret_cast<const u32x2_t*>(from);
+    held.a1 = *reinterpret_cast<const u32x2_t*>(from + 16);
+    held.a2 = *reinterpret_cast<const u32x2_t*>(from + 32);
+    held.a3 = *reinterpret_cast<const u32x2_t*>(from + 48);
+  }
+  __device__ __forceinline__ void load_hi(const uint16_t* from) {
+    held.a4 = *reinterpret_cast<const u32x2_t*>(from + 64);
+    held.a5 = *reinterpret_cast<const u32x2_t*>(from + 80);
+    held.a6 = *reinterpret_cast<const u32x2_t*>(from + 96);
+    held.a7 = *reinterpret_cast<const u32x2_t*>(from + 112);
+  }
+  template <int EPI>
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int, int c0, int, int lane) {
+    at = activation_row<EPI>(p, sl, lane & 15) + (int64_t)c0 * 128 + 4 * (lane >> 4);
+    load_lo(at);
+    load_hi(at);
+  }
+  template <int ODD, bool MORE2, bool MORE1>
+  __device__ __forceinline__ void step(const Fp4Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot&) {
+    const uint16_t* next = at + (int64_t)(i + 1) * 128;
+    fp4_half_tile(ch.w0.x, ch.w0.y, ch.s0.x, held.a0, held.a1, held.a2, held.a3, acc0);
+    fp4_half_tile(ch.w1.x, ch.w1.y, ch.s0.z, held.a0, held.a1, held.a2, held.a3, acc1);
+    fp4_half_tile(ch.w2.x, ch.w2.y, ch.s1.x, held.a0, held.a1, held.a2, held.a3, acc2);
+    fp4_half_tile(ch.w3.x, ch.w3.y, ch.s1.z, held.a0, held.a1, held.a2, held.a3, acc3);
+    if (MORE1) load_lo(next);
+    fp4_half_tile(ch.w0.z, ch.w0.w, ch.s0.y, held.a4, held.a5, held.a6, held.a7, acc0);
+    fp4_half_tile(ch.w1.z, ch.w1.w, ch.s0.w, held.a4, held.a5, held.a6, held.a7, acc1);
+    fp4_half_tile(ch.w2.z, ch.w2.w, ch.s1.y, held.a4, held.a5, held.a6, held.a7, acc2);
+    fp4_half_tile(ch.w3.z, ch.w3.w, ch.s1.w, held.a4, held.a5, held.a6, held.a7, acc3);
+    if (MORE1) load_hi(next);
+  }
+};
+
+// ---------------------------------------------------------------------------------------- slots of one to eight rows
+//
+// With at most eight rows in the slot the sixteen MFMA rows carry two 16-blocks at once: A row 8 p + i holds row i of
+// the slot over the k of block 2 j + p only (zero over the other block's), so one v_mfma_f32_16x16x32_bf16 does the
+// blocks 2 j and 2 j + 1 of a tile (one code dword: four conversions) and leaves block 2 j + p's partial sums in its
+// output rows 8 p .. 8 p + 7. Half the MFMAs, scale conversions and folds of the sixteen-row body, and four 8-byte
+// activation loads a chunk instead of eight. Lane (q, r16) ends up with block parity q / 2 of slot rows 4 (q % 2) ..
+// + 3: the two parities are added across the lanes after the last chunk, which leaves the sixteen-row layout.
+constexpr int FP4_FEW_ROWS = 8;
+
+struct Fp4Pieces {  // the lane's four 8-byte pieces of a chunk, one per block pair
+  u32x2_t p0, p1, p2, p3;
+};
+
+struct Fp4FewActs {
+  static constexpr int LOADS = 4;
+  Fp4Pieces even, odd;  // of the next even and the next odd chunk
+  bool upper;           // this lane's A row belongs to the odd blocks (p = 1)
+  uint32_t shift;       // 8 * (q / 2): where this lane's OUTPUT rows find their block's scale in a scale dword
+  const uint16_t* at;   // the lane's piece of block pair 0 of the wavefront's first chunk
+  __device__ __forceinline__ void load(Fp4Pieces& to, int i) const {
+    const uint16_t* from = at + (int64_t)i * 128;
+    to.p0 = *reinterpret_cast<const u32x2_t*>(from);
+    to.p1 = *reinterpret_cast<const u32x2_t*>(from + 32);
+    to.p2 = *reinterpret_cast<const u32x2_t*>(from + 64);
+    to.p3 = *reinterpret_cast<const u32x2_t*>(from + 96);
+  }
+  template <int EPI>
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int, int c0, int n, int lane) {
+    const int q = lane >> 4, r16 = lane & 15;
+    upper = r16 >= 8;
+    shift = 8 * (q >> 1);
+    at = activation_row<EPI>(p, sl, r16 & 7) + (int64_t)c0 * 128 + (upper ? 16 : 0) + 4 * q;
+    load(even, 0);
+    if (n > 1) load(odd, 1);
+  }
+  // MFMA j's A operand: the lane's piece in its own block's half, zero in the other
+  __device__ __forceinline__ u32x4_t operand(const u32x2_t& piece) const {
+    u32x4_t a;  // word by word: a select between two vectors built from the same piece is compiled through memory
+    a.x = upper ? 0u : piece.x;
+    a.y = upper ? 0u : piece.y;
+    a.z = upper ? piece.x : 0u;
+    a.w = upper ? piece.y : 0u;
+    return a;
+  }
+  // One tile over one block pair: the pair's code dword, the scale dword holding its two scales in bytes BYTE, BYTE + 1.
+  template <int BYTE>
+  __device__ __forceinline__ void pair(uint32_t codes, uint32_t sc, const u32x4_t& a, f32x4_t& acc) const {
+    u32x4_t b;
+    b.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, 1.0f, 0));
+    b.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, 1.0f, 1));
+    b.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, 1.0f, 2));
+    b.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, 1.0f, 3));
+    const f32x4_t part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                                 f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    const float s = __builtin_amdgcn_cvt_f32_fp8(sc >> shift, BYTE);  // the scale of block BYTE + q / 2 of the dword
+    acc.x = fmaf(part.x, s, acc.x);
+    acc.y = fmaf(part.y, s, acc.y);
+    acc.z = fmaf(part.z, s, acc.z);
+    acc.w = fmaf(part.w, s, acc.w);
+  }
+  __device__ __forceinline__ void tile(const u32x4_t& w, uint32_t sc_lo, uint32_t sc_hi, const u32x4_t& a0, const u32x4_t& a1, const u32x4_t& a2,
+                                       const u32x4_t& a3, f32x4_t& acc) const {
+    pair<0>(w.x, sc_lo, a0, acc);
+    pair<2>(w.y, sc_lo, a1, acc);
+    pair<0>(w.z, sc_hi, a2, acc);
+    pair<2>(w.w, sc_hi, a3, acc);
+  }
+  template <int ODD, bool MORE2, bool MORE1>
+  __device__ __forceinline__ void step(const Fp4Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot&) {
+    Fp4Pieces& held = ODD ? odd : even;
+    const u32x4_t a0 = operand(held.p0), a1 = operand(held.p1), a2 = operand(held.p2), a3 = operand(held.p3);
+    tile(ch.w0, ch.s0.x, ch.s0.y, a0, a1, a2, a3, acc0);
+    __builtin_amdgcn_sched_barrier(0);  // a tile at a time: interleaving the four costs more registers than there are
+    tile(ch.w1, ch.s0.z, ch.s0.w, a0, a1, a2, a3, acc1);
+    __builtin_amdgcn_sched_barrier(0);
+    tile(ch.w2, ch.s1.x, ch.s1.y, a0, a1, a2, a3, acc2);
+    __builtin_amdgcn_sched_barrier(0);
+    tile(ch.w3, ch.s1.z, ch.s1.w, a0, a1, a2, a3, acc3);
+    if (MORE2) load(held, i + 2);
+  }
+};
+
+__device__ __forceinline__ void add_parities(f32x4_t& acc) {
+  acc.x += __shfl_xor(acc.x, 32);
+  acc.y += __shfl_xor(acc.y, 32);
+  acc.z += __shfl_xor(acc.z, 32);
+  acc.w += __shfl_xor(acc.w, 32);
 }
 
 // y = x Wq^T, dense or grouped by the expert plan: one wavefront per (64-row block, K range, slot of 16 activation rows),
-// the same launch shape, slot table, K-split exchange and epilogues as the W3 stream.
+// the same launch shape, slot table, weight ring, K-split exchange and epilogues as the W3 stream.
 template <int EPI>
 __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
-  extern __shared__ float partial[];
+  extern __shared__ __align__(16) uint8_t rings[];
   const Slot sl = slot_of<EPI>(p, blockIdx.y);
   if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int q = lane >> 4, r16 = lane & 15;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: kept in scalars
   const WaveShare share = wave_share(p, wave);
-  const int ks = share.ks, nbi = share.nbi;
-  const int nb = blockIdx.x * p.nbw + nbi;
+  const int ks = share.ks, nbi = share.nbi, nb = blockIdx.x * p.nbw + nbi;
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
-  if (active) {
-    const int c0 = share.c0, c1 = share.c1;
-    const uint16_t* aptr = activation_row<EPI>(p, sl, r16) + 4 * q + (int64_t)c0 * 128;
-    const uint8_t* blk = sl.w + ((int64_t)nb * p.chunks + c0) * NVFP4_BLOCK_BYTES;
-    if (c0 < c1) {
-      Fp4Chunk even, odd;
-      load_fp4_chunk(even, blk, lane, r16);
-      int left = c1 - c0 - 1;
-      while (left >= 2) {
-        load_fp4_chunk(odd, blk + NVFP4_BLOCK_BYTES, lane, r16);
-        fp4_chunk(even, aptr, acc0, acc1, acc2, acc3);
-        blk += 2 * NVFP4_BLOCK_BYTES;
-        load_fp4_chunk(even, blk, lane, r16);
-        fp4_chunk(odd, aptr + 128, acc0, acc1, acc2, acc3);
-        aptr += 256;
-        left -= 2;
-      }
-      if (left == 1) {
-        load_fp4_chunk(odd, blk + NVFP4_BLOCK_BYTES, lane, r16);
-        fp4_chunk(even, aptr, acc0, acc1, acc2, acc3);
-        fp4_chunk(odd, aptr + 128, acc0, acc1, acc2, acc3);
-      } else {
-        fp4_chunk(even, aptr, acc0, acc1, acc2, acc3);
-      }
+  if (active) {  // at least one chunk: the launch keeps ks <= chunks
+    uint8_t* ring = rings + wave * FP4_RING_BYTES;
+    if (sl.rows <= FP4_FEW_ROWS && !p.no_few) {  // uniform over the workgroup
+      stream_block<EPI, Fp4FewActs, Fp4Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      add_parities(acc0);  // lanes q = 0, 1 now hold slot rows 0 .. 7 as the epilogue expects them; q = 2, 3 stand for rows past the slot's end
+      add_parities(acc1);
+      add_parities(acc2);
+      add_parities(acc3);
+    } else {
+      stream_block<EPI, Fp4Acts, Fp4Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
     }
   }
-  finish_block<EPI, false>(p, sl, RowScales{}, nb, active, ks, nbi, partial, acc0, acc1, acc2, acc3);
+  finish_block<EPI, false, FP4_RING_BYTES / 4>(p, sl, RowScales{}, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
 }
 
 // experiments (hb_tune): the stream's workgroup shape ("nvfp4_ksplit", "nvfp4_nbw"); "nvfp4_tile": 1 forces the tile kernel, 2 the stream
-static int g_nvfp4_ksplit = 0, g_nvfp4_nbw = 0, g_nvfp4_tile = 0;
+static int g_nvfp4_ksplit = 0, g_nvfp4_nbw = 0, g_nvfp4_tile = 0, g_nvfp4_few = 0;  // "nvfp4_few": 2 switches off the body for slots of at most eight rows
 
 template <int EPI>
 static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipStream_t stream) {
@@ -213,9 +348,10 @@ static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipS
   }
   if (p.ks * p.nbw > 16 || p.ks > p.chunks || (p.ks & (p.ks - 1))) return HB_EINVAL;
   set_split(p);
+  p.no_few = g_nvfp4_few == 2;
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
-  HB_LAUNCH(nvfp4_stream_kernel<EPI>, grid, dim3(64 * waves), p.ks > 1 ? (size_t)waves * 4096 : 0, stream, p);
+  HB_LAUNCH(nvfp4_stream_kernel<EPI>, grid, dim3(64 * waves), (size_t)waves * FP4_RING_BYTES, stream, p);
   return HB_OK;
 }
 
@@ -380,7 +516,8 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
 }  // namespace
 
 int hb::nvfp4_tune(const char* key, int value) {
-  int* slot = !strcmp(key, "nvfp4_tile") ? &g_nvfp4_tile : !strcmp(key, "nvfp4_ksplit") ? &g_nvfp4_ksplit : !strcmp(key, "nvfp4_nbw") ? &g_nvfp4_nbw : nullptr;
+  int* slot = !strcmp(key, "nvfp4_tile") ? &g_nvfp4_tile : !strcmp(key, "nvfp4_ksplit") ? &g_nvfp4_ksplit : !strcmp(key, "nvfp4_nbw") ? &g_nvfp4_nbw
+              : !strcmp(key, "nvfp4_few") ? &g_nvfp4_few : nullptr;
   if (!slot || value < 0 || value > 16) return HB_EINVAL;
   *slot = value;
   return HB_OK;

@@ -18,6 +18,7 @@
 // one), and hb_tune("w3_tile", 1 | 2) forces one or the other.
 #include <string.h>
 
+#include "ring.hpp"
 #include "stream_common.hpp"
 #include "tile_kernel.hpp"
 #include "w3_layout.hpp"
@@ -89,61 +90,41 @@ __device__ __forceinline__ void compute_half_chunk(const Chunk& ch, const u32x4_
 }
 
 // ------------------------------------------------------------------------------------------------ the weight ring
-//
-// Weight chunks do not wait in registers. A wavefront owns RING_CHUNKS block-sized slots of LDS and fills them with
-// LDS-direct loads (global_load_lds: memory to LDS, no register in between), two chunks ahead of the one it expands;
-// when a chunk's turn comes its block is read from the slot into sixteen registers and the slot is given to the chunk
-// two further on. Only the lanes that asked for a block read it back, so no barrier is involved: a wavefront waits on
-// its own vector-memory counter. A chunk in flight costs no registers this way: two of them stand behind the one
-// being expanded where register double-buffering affords one, and a wavefront's registers go to one chunk's codes, its
-// activations and the accumulators.
-//
-// The counter is shared by everything a wavefront has asked of memory, in order. A chunk's block is four LDS-direct
-// loads, asked for two chunks ahead, right after the slot it goes to has been read; the chunk's activation loads
-// (Acts::LOADS of them) are asked for one chunk later, when their registers are free. The compiler may move those
-// among the other requests made between two reads of the ring, but not across a read (the reads are volatile
-// statements that clobber memory). So when chunk i is due, everything asked for since the read before stands behind
-// its block: the block of chunk i + 1 and one chunk's activation loads at least. Waiting until at most that many
-// requests remain outstanding is waiting for chunk i, and hardly longer. The last chunk waits for everything. The
-// LDS-direct loads go through a buffer descriptor of the block row (the MUBUF form: around it the compiler keeps exact
-// count of its own loads, which it gives up around the FLAT form), and the ring is read with explicit ds_read_b128, so
-// the only waits on these transfers are the ones written here.
-constexpr int RING_CHUNKS = 2;
-constexpr int RING_BYTES = RING_CHUNKS * W3_BLOCK_BYTES;  // LDS per wavefront; its first 4 KB double as the K-split exchange
-constexpr int BLOCK_LOADS = 4;
-
-typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
-
-struct RingSource {
-  __amdgpu_buffer_rsrc_t row;  // the block row: chunks x W3_BLOCK_BYTES
-  uint32_t codes, scales;      // the lane's byte offsets in a block for the 16-byte and the 4-byte loads
+// (ring.hpp) for W3 blocks: three 16-byte loads a lane of codes, one 4-byte load a lane of scales.
+struct W3Ring {
+  typedef hb::Chunk Chunk;
+  static constexpr int BLOCK_BYTES = W3_BLOCK_BYTES, LOADS = 4;
+  // the lane's byte offsets in a block for the 16-byte and the 4-byte loads, and where it reads them back
+  static __device__ __forceinline__ void lanes(RingSource& src, int lane, int r16, uint32_t slot0, uint32_t& codes, uint32_t& scales) {
+    src.codes = 16u * lane;
+    src.scales = 4u * lane;
+    codes = slot0 + 16u * lane;
+    scales = slot0 + 16u * r16;
+  }
+  static __device__ __forceinline__ void request(const RingSource& src, int chunk, lds_ptr_t slot) {
+    const uint32_t at = (uint32_t)chunk * W3_BLOCK_BYTES;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 0, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 2048, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 4, src.scales, at, W3_SCALE_OFFSET, 2);
+    __builtin_amdgcn_sched_barrier(0);  // asked for here, not wherever the scheduler would sink it below the arithmetic
+  }
+  template <int BEHIND, int SLOT>  // BEHIND: requests that may stay outstanding
+  static __device__ __forceinline__ void take(Chunk& ch, uint32_t codes, uint32_t scales) {
+    asm volatile(
+        "s_waitcnt vmcnt(%6)\n\t"
+        "ds_read_b128 %0, %4 offset:%7\n\t"
+        "ds_read_b128 %1, %4 offset:%8\n\t"
+        "ds_read_b128 %2, %4 offset:%9\n\t"
+        "ds_read_b128 %3, %5 offset:%10\n\t"
+        "s_waitcnt lgkmcnt(0)"  // the slot is read: it may be given to another chunk
+        : "=&v"(ch.w0), "=&v"(ch.w1), "=&v"(ch.w2), "=&v"(ch.sc)
+        : "v"(codes), "v"(scales), "n"(BEHIND), "n"(SLOT * W3_BLOCK_BYTES), "n"(SLOT * W3_BLOCK_BYTES + 1024), "n"(SLOT * W3_BLOCK_BYTES + 2048),
+          "n"(SLOT * W3_BLOCK_BYTES + W3_SCALE_OFFSET)
+        : "memory");
+  }
 };
-
-__device__ __forceinline__ void request_chunk(const RingSource& src, int chunk, lds_ptr_t slot) {
-  const uint32_t at = (uint32_t)chunk * W3_BLOCK_BYTES;
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 0, 2);
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024, 2);
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 2048, 2);
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 4, src.scales, at, W3_SCALE_OFFSET, 2);
-  __builtin_amdgcn_sched_barrier(0);  // asked for here, not wherever the scheduler would sink it below the arithmetic
-}
-
-// `codes` / `scales`: LDS byte addresses of the lane's first code load and of its row-in-tile's scales in the ring's
-// slot 0; SLOT selects the slot through the instruction's offset.
-template <int BEHIND, int SLOT>  // BEHIND: requests that may stay outstanding
-__device__ __forceinline__ void take_chunk(Chunk& ch, uint32_t codes, uint32_t scales) {
-  asm volatile(
-      "s_waitcnt vmcnt(%6)\n\t"
-      "ds_read_b128 %0, %4 offset:%7\n\t"
-      "ds_read_b128 %1, %4 offset:%8\n\t"
-      "ds_read_b128 %2, %4 offset:%9\n\t"
-      "ds_read_b128 %3, %5 offset:%10\n\t"
-      "s_waitcnt lgkmcnt(0)"  // the slot is read: it may be given to another chunk
-      : "=&v"(ch.w0), "=&v"(ch.w1), "=&v"(ch.w2), "=&v"(ch.sc)
-      : "v"(codes), "v"(scales), "n"(BEHIND), "n"(SLOT * W3_BLOCK_BYTES), "n"(SLOT * W3_BLOCK_BYTES + 1024), "n"(SLOT * W3_BLOCK_BYTES + 2048),
-        "n"(SLOT * W3_BLOCK_BYTES + W3_SCALE_OFFSET)
-      : "memory");
-}
+constexpr int RING_BYTES = ring_bytes<W3Ring>();  // LDS per wavefront; its first 4 KB double as the K-split exchange
 
 // ------------------------------------------------------------------------------------------- slots of one to four rows
 //
@@ -305,56 +286,6 @@ struct FullActs {  // up to sixteen rows: lane (q, r16) feeds row r16, k 8 q .. 
   }
 };
 
-// Chunks c0 .. c1 - 1 (at least one) of block row `nb`, through the wavefront's ring, for the slot's rows from row0 (the
-// four-row bodies: row0 .. row0 + 3; the sixteen-row body: all, row0 = 0).
-template <int EPI, class Acts>
-__device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& sl, int row0, int nb, int c0, int c1, int lane, uint8_t* ring,
-                                             f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) {
-  constexpr int BEHIND = BLOCK_LOADS + Acts::LOADS;
-  const int r16 = lane & 15, n = c1 - c0;
-  RingSource src;
-  src.row = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(sl.w + (int64_t)nb * p.chunks * W3_BLOCK_BYTES), 0, p.chunks * W3_BLOCK_BYTES,
-                                              0x00020000);
-  src.codes = 16u * lane;
-  src.scales = 4u * lane;
-  const lds_ptr_t slot0 = (lds_ptr_t)ring, slot1 = (lds_ptr_t)(ring + W3_BLOCK_BYTES);
-  const uint32_t codes = (uint32_t)(uintptr_t)slot0 + 16u * lane, scales = (uint32_t)(uintptr_t)slot0 + 16u * r16;
-  Acts acts;
-  Chunk ch;
-  request_chunk(src, c0, slot0);
-  asm volatile("" ::: "memory");  // whatever else the prologue asks for stands behind the first block
-  acts.template start<EPI>(p, sl, row0, c0, n, lane);
-  if (n == 1) {
-    take_chunk<0, 0>(ch, codes, scales);
-    acts.template step<0, false, false>(ch, 0, acc0, acc1, acc2, acc3, sl);
-  } else {
-    request_chunk(src, c0 + 1, slot1);
-    int i = 0;
-    for (; i + 3 < n; i += 2) {  // chunks i and i + 1, asking for the blocks of i + 2 and i + 3
-      take_chunk<BEHIND, 0>(ch, codes, scales);
-      request_chunk(src, c0 + i + 2, slot0);
-      acts.template step<0, true, true>(ch, i, acc0, acc1, acc2, acc3, sl);
-      take_chunk<BEHIND, 1>(ch, codes, scales);
-      request_chunk(src, c0 + i + 3, slot1);
-      acts.template step<1, true, true>(ch, i + 1, acc0, acc1, acc2, acc3, sl);
-    }
-    if (i + 3 == n) {  // three left: the block of i + 2 is still to ask for
-      take_chunk<BEHIND, 0>(ch, codes, scales);
-      request_chunk(src, c0 + i + 2, slot0);
-      acts.template step<0, true, true>(ch, i, acc0, acc1, acc2, acc3, sl);
-      take_chunk<BEHIND, 1>(ch, codes, scales);
-      acts.template step<1, false, true>(ch, i + 1, acc0, acc1, acc2, acc3, sl);
-      take_chunk<0, 0>(ch, codes, scales);
-      acts.template step<0, false, false>(ch, i + 2, acc0, acc1, acc2, acc3, sl);
-    } else {  // two left, both asked for
-      take_chunk<BEHIND, 0>(ch, codes, scales);
-      acts.template step<0, false, true>(ch, i, acc0, acc1, acc2, acc3, sl);
-      take_chunk<0, 1>(ch, codes, scales);
-      acts.template step<1, false, false>(ch, i + 1, acc0, acc1, acc2, acc3, sl);
-    }
-  }
-}
-
 // The end of a 64-row block for a slot of at most four rows. Lane (g, r16) of each of the block's K splits holds, in
 // register r of accumulator t, group g's part of (tile t, slot row r, column r16): sixteen values a lane, each to be
 // added over the four groups and the splits. They go to LDS, and the workgroup's 64 x ks lanes share the 16 x 16
@@ -419,7 +350,7 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
     const float scale = active ? sl.rs[nb * 64 + lane] : 0.f;
     for (int row0 = 0; row0 < sl.rows; row0 += FEW_ROWS) {  // uniform over the workgroup
       acc0 = acc1 = acc2 = acc3 = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      if (active) stream_block<EPI, FewActs8>(p, sl, row0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      if (active) stream_block<EPI, FewActs8, W3Ring>(p, sl, row0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
       finish_few<EPI>(p, sl, row0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
       if (p.ks > 1) __syncthreads();  // the exchange is read before the next pass fills the rings it lies in
     }
@@ -427,13 +358,13 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
     float scale = 0.f;
     if (active) {
       scale = sl.rs[nb * 64 + lane];  // row 16 q + r16 of the block: asked for ahead of the chunks, there when the epilogue wants it
-      stream_block<EPI, FewActs>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);  // at least one chunk: ks <= chunks
+      stream_block<EPI, FewActs, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);  // at least one chunk: ks <= chunks
     }
     finish_few<EPI>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
   } else {
     RowScales rs{};
     if (active) {
-      stream_block<EPI, FullActs>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      stream_block<EPI, FullActs, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
       rs = row_scales<true>(sl, nb, lane & 15);
     }
     finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);

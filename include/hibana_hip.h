@@ -35,7 +35,8 @@ const char* hb_error_string(int code);
 /* Tuning knobs for experiments and tests; value 0 restores the built-in choice. "w3_ksplit" / "w3_nbw",
  * "moe_fc1_ksplit" / "moe_fc1_nbw", "moe_fc2_ksplit" / "moe_fc2_nbw", "nvfp4_ksplit" / "nvfp4_nbw": K splits and 64-row
  * blocks per workgroup (their product at most 16); "w3_tile" / "nvfp4_tile": 1 forces the MFMA tile kernel, 2 the weight
- * stream; "w3_few": 2 switches off the stream's body for slots of at most four rows. Returns HB_EINVAL for an unknown
+ * stream; "w3_few" / "nvfp4_few": 2 switches off the stream's body for slots of few rows (W3: at most four, NVFP4: at
+ * most eight). Returns HB_EINVAL for an unknown
  * key or a value out of range. Not thread-safe against concurrent launches. */
 int hb_tune(const char* key, int value);
 

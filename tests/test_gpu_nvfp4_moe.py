@@ -12,15 +12,17 @@ from tests.util import MAX_REL, NORM_REL, errors
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["auto", "tile", "stream"], autouse=True)
+@pytest.fixture(params=["auto", "tile", "stream", "stream16"], autouse=True)
 def kernel_choice(request):
-    """Every case runs with the library's own choice between the 128-row tile kernel and the 16-row weight stream, and
-    with each of them forced."""
+    """Every case runs with the library's own choice between the 128-row tile kernel and the 16-row weight stream, with
+    each of them forced, and with the stream's body for slots of at most eight rows switched off (so those slots take the
+    sixteen-row body)."""
     from hibana_amd import _lib
-    value = {"auto": 0, "tile": 1, "stream": 2}[request.param]
-    assert _lib.lib().hb_tune(b"nvfp4_tile", value) == 0
+    tile, few = {"auto": (0, 0), "tile": (1, 0), "stream": (2, 0), "stream16": (2, 2)}[request.param]
+    assert _lib.lib().hb_tune(b"nvfp4_tile", tile) == 0 and _lib.lib().hb_tune(b"nvfp4_few", few) == 0
     yield request.param
     _lib.lib().hb_tune(b"nvfp4_tile", 0)
+    _lib.lib().hb_tune(b"nvfp4_few", 0)
 
 
 def _stack(e, rows, k, seed):
