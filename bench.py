@@ -113,7 +113,7 @@ def latent_prefill(args) -> int:
         block(x)
     torch.cuda.synchronize()
     hip = Hip()
-    names = ["route", "plan", "fc1", "fc2", "combine"]
+    names = ["route", "plan count", "plan scan", "plan place", "fc1", "fc2", "combine"]  # 45 056 pairs: the plan is three launches
     per_kernel = {n: [] for n in names}
     for rep in range(4):
         evs = hip.events(2 * len(names))

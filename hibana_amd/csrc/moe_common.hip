@@ -159,6 +159,8 @@ static void launch_route(const RouteParams& p, int m, hipStream_t stream) {
 constexpr int PLAN_THREADS = 1024;
 constexpr int PLAN_WAVES = PLAN_THREADS / 64;
 constexpr int PLAN_BATCH = 8;  // tiles of 64 pairs whose ids a wavefront requests at once
+constexpr int PLAN_WIDE_PAIRS = 8192;   // from this many pairs the plan is shared among workgroups (three launches)
+constexpr int PLAN_WIDE_GROUPS = 64;
 constexpr int ROUTE_FUSED_ROWS = 16;  // up to this many rows the plan workgroup routes them itself (one a wavefront)
 
 struct Scan3 {
@@ -204,9 +206,15 @@ __device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 
 
 // With `route.logits` set the workgroup first routes the route.m rows itself (softmax top-k, a row a wavefront at a
 // time) into route.ids / route.weights, which `ids` then names.
+//
+// Many pairs (a prefill chunk) are shared among `groups` workgroups in three launches of this kernel, `wide` [groups, e_n]
+// between them: phase 1, each group counts its share of the pairs per expert; phase 2, one workgroup adds the groups'
+// counts, writes the slot table and turns `wide` into the first sorted position of each group's run of each expert;
+// phase 3, each group places its share. Phase 0 is all of it in one workgroup.
 __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
                                                                 int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
-                                                                int route_rows, int slot_rows, int slot_cap) {
+                                                                int route_rows, int slot_rows, int slot_cap, int32_t* __restrict__ wide, int groups,
+                                                                int phase) {
   extern __shared__ int lds[];
   if (route.logits) {
     for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
@@ -221,14 +229,17 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   int* seg_count = lds;                         // [PLAN_WAVES][e_n]: pairs of expert e in segment w, then running positions
   int* start = lds + PLAN_WAVES * e_n;          // [e_n]: first sorted position of expert e
   int* scratch = start + e_n;                   // [3 * (PLAN_WAVES + 1)]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int i = threadIdx.x; i < PLAN_WAVES * e_n; i += PLAN_THREADS) seg_count[i] = 0;
-  __syncthreads();
-  // segment w = pairs [w * seg, (w + 1) * seg), seg a multiple of 64
-  const int seg = ((pairs + PLAN_WAVES - 1) / PLAN_WAVES + 63) / 64 * 64;
-  const int lo = wave * seg, hi = min(pairs, lo + seg);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, group = blockIdx.x;
+  // segment (group, w) = pairs [(group * PLAN_WAVES + w) * seg, ... + seg), seg a multiple of 64
+  const int seg = (((pairs + groups - 1) / groups + PLAN_WAVES - 1) / PLAN_WAVES + 63) / 64 * 64;
+  const int lo = min(pairs, (group * PLAN_WAVES + wave) * seg), hi = min(pairs, lo + seg);
   const int batch = seg > 64 ? PLAN_BATCH : 1;  // long segments: the ids of a batch of tiles are requested together
-  for (int i0 = lo + lane; i0 < hi; i0 += 64 * batch) {
+  const int e = threadIdx.x;  // one thread an expert: the launch keeps e_n <= PLAN_THREADS
+  if (phase != 2) {
+    for (int i = threadIdx.x; i < PLAN_WAVES * e_n; i += PLAN_THREADS) seg_count[i] = 0;
+    __syncthreads();
+  }
+  for (int i0 = lo + lane; phase != 2 && i0 < hi; i0 += 64 * batch) {
     if (batch == 1) {
       const int e = ids[i0] - e_lo;
       if (e >= 0 && e < e_n) atomicAdd(&seg_count[wave * e_n + e], 1);
@@ -242,15 +253,42 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
       if (e[j] >= 0 && e[j] < e_n) atomicAdd(&seg_count[wave * e_n + e[j]], 1);
   }
   __syncthreads();
+  if (phase == 1) {  // this group's pairs of each expert
+    if (e < e_n) {
+      int count = 0;
+      for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
+      wide[group * e_n + e] = count;
+    }
+    return;
+  }
+  if (phase == 3) {  // the first position of each of this group's segments' runs, from the group's own
+    if (e < e_n) {
+      int run = wide[group * e_n + e];
+      for (int wv = 0; wv < PLAN_WAVES; wv++) {
+        const int c = seg_count[wv * e_n + e];
+        seg_count[wv * e_n + e] = run;
+        run += c;
+      }
+    }
+    __syncthreads();
+  } else {
   // Slot order is the order the hardware starts a launch's workgroups in, so the long-running slots go first: the
   // shared expert's (full slots), then the experts with more than a quarter slot of rows, then the rest, each class in
   // ascending expert id. Sorted positions are another matter: ascending expert id, the shared rows after the routed
   // pairs.
   const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
-  const int e = threadIdx.x;  // one thread an expert: the launch keeps e_n <= PLAN_THREADS
   int count = 0;
-  if (e < e_n)
-    for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
+  int of_group[PLAN_WIDE_GROUPS];  // phase 2: the groups' counts of this thread's expert, all asked for at once
+  if (e < e_n) {
+    if (phase == 0) {
+      for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
+    } else {
+#pragma unroll
+      for (int g = 0; g < PLAN_WIDE_GROUPS; g++) of_group[g] = g < groups ? wide[g * e_n + e] : 0;
+#pragma unroll
+      for (int g = 0; g < PLAN_WIDE_GROUPS; g++) count += of_group[g];
+    }
+  }
   const int my_slots = (count + slot_rows - 1) / slot_rows;
   const bool heavy = 4 * count > slot_rows;
   Scan3 tot;  // a: rows; b: heavy slots, and distinct experts in the upper half (neither sum reaches 65536); c: light slots
@@ -267,12 +305,20 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
       entry[2] = min(slot_rows, count - s * slot_rows);
       entry[3] = 0;
     }
-    // turn the per-segment counts into the first position of each segment's run
+    // turn the per-segment (phase 2: per-group) counts into the first position of each segment's (group's) run
     int run = my_start;
-    for (int wv = 0; wv < PLAN_WAVES; wv++) {
-      const int c = seg_count[wv * e_n + e];
-      seg_count[wv * e_n + e] = run;
-      run += c;
+    if (phase == 0) {
+      for (int wv = 0; wv < PLAN_WAVES; wv++) {
+        const int c = seg_count[wv * e_n + e];
+        seg_count[wv * e_n + e] = run;
+        run += c;
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < PLAN_WIDE_GROUPS; g++) {
+        if (g < groups) wide[g * e_n + e] = run;
+        run += of_group[g];
+      }
     }
   }
   __syncthreads();
@@ -294,6 +340,8 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
     plan[0] = slots;
     plan[1] = distinct;
     plan[2] = kept;
+  }
+  if (phase == 2) return;
   }
   // stable placement: each wavefront walks its segment 64 pairs at a time; a lane's position is its expert's running
   // position in this segment plus the number of lower lanes of the tile with the same expert
@@ -439,6 +487,7 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
     return ptr;
   };
   w.plan = static_cast<int32_t*>(take((PLAN_HEADER + 4 * moe_max_slots(pairs, experts, shared ? m : 0, ROWS_PER_SLOT)) * sizeof(int32_t)));
+  w.plan_wide = static_cast<int32_t*>(take((size_t)PLAN_WIDE_GROUPS * experts * sizeof(int32_t)));
   w.order = static_cast<int32_t*>(take(rows * sizeof(int32_t)));
   w.h = static_cast<uint16_t*>(take((size_t)rows * inter * sizeof(uint16_t)));
   w.y = static_cast<float*>(take((size_t)rows * hidden_out * sizeof(float)));
@@ -455,8 +504,16 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream, int slot_rows) {
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
+  const int slot_cap = (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows);
+  if (pairs >= PLAN_WIDE_PAIRS) {  // a share of about a thousand pairs a workgroup
+    const int groups = (int)std::min<int64_t>(PLAN_WIDE_GROUPS, pairs / 1024);
+    for (int phase = 1; phase <= 3; phase++)
+      HB_LAUNCH(moe_plan_kernel, dim3(phase == 2 ? 1 : groups), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan,
+                ws.order, RouteParams{}, 0, slot_rows, slot_cap, ws.plan_wide, groups, phase);
+    return HB_OK;
+  }
   HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0, slot_rows,
-            (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows));
+            slot_cap, ws.plan_wide, 1, 0);
   return HB_OK;
 }
 
@@ -481,7 +538,7 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
   HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, slot_rows,
-            (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows));
+            (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows), ws.plan_wide, 1, 0);
   return HB_OK;
 }
 

@@ -248,6 +248,7 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
 // Workspace of a routed call, carved from one caller-owned buffer.
 struct MoeWorkspace {
   int32_t* plan;
+  int32_t* plan_wide;  // [64, experts]: the plan's counts a workgroup when many pairs are shared among several
   int32_t* order;
   uint16_t* h;   // [(pairs + shared rows), inter] BF16, in sorted order
   float* y;      // [(pairs + shared rows), hidden_out] FP32 (or BF16 pairs), by pair index

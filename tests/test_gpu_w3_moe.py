@@ -209,9 +209,11 @@ def test_graph_replay_gives_the_eager_bits(gated):
         assert torch.equal(captured, eager)
 
 
-def test_plan_orders_many_pairs_on_the_device(gated):
-    """2,000 rows x 10: 20,000 pairs sorted by the planning kernel itself, against the oracle."""
-    _check(*gated, *_inputs(2000, TOPK, 1234))
+@pytest.mark.parametrize("m", [819, 820, 2000])
+def test_plan_orders_many_pairs_on_the_device(gated, m):
+    """8,190 pairs (the last count one workgroup plans alone), 8,200 and 20,000 (shared among 8 and 19 workgroups in
+    three launches), sorted by the planning kernel itself, against the oracle."""
+    _check(*gated, *_inputs(m, TOPK, 1234 + m))
 
 
 def test_bad_calls_raise(gated):
