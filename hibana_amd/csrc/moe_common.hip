@@ -211,10 +211,12 @@ __device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 
 // between them: phase 1, each group counts its share of the pairs per expert; phase 2, one workgroup adds the groups'
 // counts, writes the slot table and turns `wide` into the first sorted position of each group's run of each expert;
 // phase 3, each group places its share. Phase 0 is all of it in one workgroup.
+template <bool WIDE>  // false: one workgroup (phase 0) and nothing of the shared form compiled in
 __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
                                                                 int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
-                                                                int route_rows, int slot_rows, int slot_cap, int32_t* __restrict__ wide, int groups,
-                                                                int phase) {
+                                                                int route_rows, int slot_rows, int slot_cap, int32_t* __restrict__ wide, int groups_,
+                                                                int phase_) {
+  const int groups = WIDE ? groups_ : 1, phase = WIDE ? phase_ : 0;
   extern __shared__ int lds[];
   if (route.logits) {
     for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
@@ -508,12 +510,12 @@ int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int sh
   if (pairs >= PLAN_WIDE_PAIRS) {  // a share of about a thousand pairs a workgroup
     const int groups = (int)std::min<int64_t>(PLAN_WIDE_GROUPS, pairs / 1024);
     for (int phase = 1; phase <= 3; phase++)
-      HB_LAUNCH(moe_plan_kernel, dim3(phase == 2 ? 1 : groups), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan,
+      HB_LAUNCH(moe_plan_kernel<true>, dim3(phase == 2 ? 1 : groups), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan,
                 ws.order, RouteParams{}, 0, slot_rows, slot_cap, ws.plan_wide, groups, phase);
     return HB_OK;
   }
-  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0, slot_rows,
-            slot_cap, ws.plan_wide, 1, 0);
+  HB_LAUNCH(moe_plan_kernel<false>, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0,
+            slot_rows, slot_cap, ws.plan_wide, 1, 0);
   return HB_OK;
 }
 
@@ -537,7 +539,7 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   }
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
-  HB_LAUNCH(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, slot_rows,
+  HB_LAUNCH(moe_plan_kernel<false>, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, slot_rows,
             (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows), ws.plan_wide, 1, 0);
   return HB_OK;
 }
