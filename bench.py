@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Headline benchmark: the w3 MoE layer at the speculative-verify batch (BASELINE config 3: 32 tokens, hidden 2048,
+"""Headline benchmark (the default, `--config 3`): the w3 MoE layer at the speculative-verify batch (BASELINE config 3: 32 tokens, hidden 2048,
 512 experts of intermediate 512 + 1 shared expert, top-10 with Zipf(1.1)-skewed routing, SiLU-gated, 3-bit weights).
 
 A step is one MoE layer call (softmax top-k routing of given logits, expert plan, fc1, fc2, combine with the shared
@@ -9,6 +9,10 @@ are one HIP-graph replay (the way a serving engine issues them), bracketed by sy
 
 Prints one JSON line: tokens/s, the HBM roofline of the dominant kernel (the fc1 stream) measured live with HIP events,
 and the CPU oracle timed on this host's cores on a bounded sample of the same workload.
+
+The other BASELINE configs are `--config 2` (the same layer at M = 1), `--config 0` / `--config 1` (the w3 / NVFP4 dense
+decode projection, `--rows` for M) and `--config 4` (the NVFP4 latent-MoE layer on a 2048-token prefill chunk, MFMA
+roofline); they print the same kind of line without the CPU leg (config 2 keeps it).
 """
 from __future__ import annotations
 
@@ -80,8 +84,8 @@ def cpu_baseline(layer, x, ids, weights, budget_s: float = 15.0):
         c_port.moe_layer(routed, xb, idn, wn, sh)
         spent += time.perf_counter() - t0
         calls += 1
-    info = {"value": M * calls / spent, "unit": "tokens/s", "cores": c_port.threads(), "kind": "port",
-            "sample": f"{calls} whole layer calls of {M} tokens on layer 0 ({distinct} distinct experts + shared): C/OpenMP oracle, "
+    info = {"value": x.shape[0] * calls / spent, "unit": "tokens/s", "cores": c_port.threads(), "kind": "port",
+            "sample": f"{calls} whole layer calls of {x.shape[0]} tokens on layer 0 ({distinct} distinct experts + shared): C/OpenMP oracle, "
                       f"unpack from the checkpoint layout + FP32 matmul"}
     return info, torch.from_numpy(out.view(np.int16).copy()).view(torch.bfloat16)
 
@@ -155,6 +159,86 @@ def latent_prefill(args) -> int:
     return 0
 
 
+def dense_decode(args) -> int:
+    """BASELINE configs 0 and 1 (not the headline line): one dense decode projection a step - config 0 the w3 linear
+    5120 x 5120 at M = 1, config 1 the NVFP4 up-projection 25600 x 5120 at M = --rows (1, 8 or 64) - cycling through six
+    copies of the matrix so that every step streams its weights from HBM. The roofline entry is that one kernel against
+    the HBM peak, its duration from the kernel's own start / stop events."""
+    import torch
+
+    from hibana_amd import _lib, synthetic
+    from hibana_amd.kernels import w3
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.lib()
+    m = args.rows
+    if args.config == 0:
+        n = k = 5120
+        mats = [w3.tile(synthetic.w3_matrix(n, k, 40 + i, dev, "uniform"), release=True) for i in range(args.layers)]
+        nbytes = w3_bytes(n, k)
+        x = torch.randn(m, k, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
+
+        def step(i: int):
+            return w3.w3_linear(x, mats[i % args.layers])
+
+        kernel, what = "w3_stream_kernel<dense>", f"BASELINE config 0: w3 dense linear {n} x {k}, M = {m}, uniform codebook"
+    else:
+        n, k = 25600, 5120
+        size = lib.hb_nvfp4_tiled_bytes(n, k)
+        g = torch.Generator(device=dev).manual_seed(7)
+        mats = [torch.randint(0, 256, (size,), dtype=torch.uint8, device=dev, generator=g) for _ in range(args.layers)]
+        for t in mats:  # every scale byte a finite positive E4M3 value
+            blocks = t.view(-1, 4608)[:, 4096:]
+            blocks.copy_(blocks % 120 + 1)
+        nbytes = n * k // 2 + n * k // 16
+        x = torch.randn(m, k, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
+        y = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+
+        def step(i: int):
+            _lib.check(lib.hb_nvfp4_gemm(_lib.ptr(x), m, _lib.ptr(mats[i % args.layers]), 1.0 / 448.0, n, k, 0, _lib.ptr(y), _lib.stream()), "nvfp4 gemm")
+            return y
+
+        kernel, what = "nvfp4_stream_kernel<dense>", f"BASELINE config 1: NVFP4 dense linear {n} x {k}, M = {m} (codes and block scales random, global scale 1/448)"
+    for i in range(max(args.warmup, args.layers)):
+        step(i)
+    torch.cuda.synchronize()
+    hip = Hip()
+    times = []
+    for rep in range(5):
+        for i in range(args.layers):
+            evs = hip.events(2)
+            _lib.check(lib.hb_debug_events(evs, 2), "events")
+            step(i)
+            lib.hb_debug_events(None, 0)
+            torch.cuda.synchronize()
+            if rep:
+                times.append(hip.elapsed_ms(evs[0], evs[1]))
+    kernel_ms = sum(times) / len(times)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = [step(i) for i in range(args.steps)]
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    del outs
+    achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+    line = {
+        "metric": "dense decode projection tokens/s, with achieved HBM GB/s", "value": m * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": what, "matrices_cycled": args.layers, "timed_as": "one HIP-graph replay of all steps"},
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": None, "launch_bytes": nbytes, "launch_ms": kernel_ms},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -162,7 +246,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--layers", type=int, default=6, help="distinct layers the steps cycle through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--config", type=int, default=3, choices=(3, 4), help="3: the headline w3 verify-batch layer; 4: the NVFP4 prefill layer")
+    ap.add_argument("--config", type=int, default=3, choices=(0, 1, 2, 3, 4),
+                    help="3: the headline w3 verify-batch layer; 2: the same layer at M = 1 with N(0,1) logits; 0 / 1: the w3 / NVFP4 dense decode "
+                         "projection; 4: the NVFP4 prefill layer")
+    ap.add_argument("--rows", type=int, default=1, help="configs 0 and 1: activation rows M")
     ap.add_argument("--copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (a known-size "
                     "reference for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
@@ -179,6 +266,10 @@ def main() -> int:
         return 2
     if args.config == 4:
         return latent_prefill(args)
+    if args.config in (0, 1):
+        return dense_decode(args)
+    decode = args.config == 2  # the layer at batch 1: logits from N(0, 1), ten experts and the shared one a step
+    m = 1 if decode else M
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     layers = []
@@ -186,8 +277,11 @@ def main() -> int:
         keep = i == 0 and not args.no_cpu  # the CPU leg reads layer 0 in the checkpoint layout
         layers.append((synthetic.w3_experts(EXPERTS, HIDDEN, INTER, True, 100 + i, dev, release=not keep),
                        synthetic.w3_experts(1, HIDDEN, INTER, True, 900 + i, dev, release=not keep)))
-    logits = [synthetic.zipf_logits(M, EXPERTS, ZIPF, 3000 + i, dev) for i in range(args.layers)]
-    x = torch.randn(M, HIDDEN, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
+    if decode:
+        logits = [torch.randn(m, EXPERTS, generator=torch.Generator().manual_seed(3000 + i)).to(dev) for i in range(args.layers)]
+    else:
+        logits = [synthetic.zipf_logits(m, EXPERTS, ZIPF, 3000 + i, dev) for i in range(args.layers)]
+    x = torch.randn(m, HIDDEN, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
     torch.cuda.synchronize()
 
     def step(i: int):
@@ -201,7 +295,7 @@ def main() -> int:
     # live kernel timing: each kernel of the chain is launched with its own (start, stop) HIP event pair, which the
     # runtime stamps with that kernel's begin and end on the stream it runs on
     hip = Hip()
-    names = ["route", "plan", "fc1", "fc2", "combine"]
+    names = ["route + plan", "fc1", "fc2", "combine"] if decode else ["route", "plan", "fc1", "fc2", "combine"]  # up to 16 rows are routed by the plan's workgroup
     per_kernel = {n: [] for n in names}
     reps = 5
     for rep in range(reps):
@@ -232,7 +326,7 @@ def main() -> int:
     elapsed = time.perf_counter() - t0
     del outs
     ms_per_step = elapsed / args.steps * 1e3
-    step_bytes = mean([(distinct[i % args.layers] + 1) * EXPERT_BYTES + 2 * M * HIDDEN * 2 for i in range(args.steps)])
+    step_bytes = mean([(distinct[i % args.layers] + 1) * EXPERT_BYTES + 2 * m * HIDDEN * 2 for i in range(args.steps)])
     chain_gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     if args.copy_mib:
@@ -248,18 +342,20 @@ def main() -> int:
         check = {"max_rel_vs_cpu_oracle": float((got - want.float()).abs().max() / want.float().abs().max()),
                  "norm_rel_vs_cpu_oracle": float((got - want.float()).norm() / want.float().norm())}
     line = {
-        "metric": "w3 MoE layer tokens/s at the verify batch (M=32), with achieved HBM GB/s",
-        "value": M * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": "w3 MoE layer tokens/s at decode (M=1), with achieved HBM GB/s" if decode else "w3 MoE layer tokens/s at the verify batch (M=32), with achieved HBM GB/s",
+        "value": m * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "BASELINE config 3: w3 MoE layer, 32 tokens (4 seq x 8 draft), hidden 2048, 512 experts x inter 512 + 1 shared, "
-                               "top-10 Zipf(1.1) routing, SiLU-gated, codebook lloyd",
+        "config": {"workload": ("BASELINE config 2: w3 MoE layer, 1 token, hidden 2048, 512 experts x inter 512 + 1 shared, top-10 of N(0,1) logits, "
+                                "SiLU-gated, codebook lloyd") if decode else
+                               ("BASELINE config 3: w3 MoE layer, 32 tokens (4 seq x 8 draft), hidden 2048, 512 experts x inter 512 + 1 shared, "
+                                "top-10 Zipf(1.1) routing, SiLU-gated, codebook lloyd"),
                    "layers_cycled": args.layers, "distinct_experts_per_step": mean(distinct), "timed_as": "one HIP-graph replay of all steps"},
         "roofline": {"bound": "hbm", "kernel": "w3_stream_kernel<fc1 gated>", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      # HBM bytes a launch: the ratio of scaled FETCH_SIZE + WRITE_SIZE to the algorithmic bytes measured with
                      # rocprofv3 --pmc on this workload (summary kept under profiles/), applied to this run's bytes
-                     "traffic": FC1_TRAFFIC_RATIO * fc1_launch_bytes, "launch_bytes": fc1_launch_bytes, "launch_ms": fc1_ms},
+                     "traffic": None if decode else FC1_TRAFFIC_RATIO * fc1_launch_bytes, "launch_bytes": fc1_launch_bytes, "launch_ms": fc1_ms},
         "layer_chain": {"algorithmic_bytes_per_step": step_bytes, "achieved_GBs": chain_gbs, "frac_of_hbm_peak": chain_gbs / HBM_PEAK_GBS,
                         "kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
         "cpu_baseline": cpu,

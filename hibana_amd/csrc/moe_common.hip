@@ -204,6 +204,74 @@ __device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 
   return Scan3{scratch[wave] + inc.a - v.a, scratch[PLAN_WAVES + 1 + wave] + inc.b - v.b, scratch[2 * (PLAN_WAVES + 1) + wave] + inc.c - v.c};
 }
 
+// The plan of at most 64 pairs (a decode step), by one wavefront, a pair a lane: no counters per expert, no scan over
+// the experts. Lanes with the same expert find each other by ballots over the id's bits; what precedes an expert in
+// either order (sorted positions: ascending id; slot table: shared, heavily loaded, the rest) is summed in a loop over
+// the lanes. Writes exactly what the general form writes.
+__device__ __forceinline__ void plan_few_pairs(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows, int32_t* __restrict__ plan,
+                                               int32_t* __restrict__ order, int slot_rows, int slot_cap) {
+  const int lane = threadIdx.x & 63;
+  int e = lane < pairs ? ids[lane] - e_lo : -1;
+  if (e < 0 || e >= e_n) e = -1;
+  int id_bits = 1;
+  while ((1 << id_bits) < e_n) id_bits++;
+  uint64_t same = __ballot(e >= 0);
+  const int kept = __popcll(same);
+  for (int b = 0; b < id_bits; b++) {
+    const uint64_t m = __ballot((e >> b) & 1);
+    same &= ((e >> b) & 1) ? m : ~m;
+  }
+  const int rank = __popcll(same & ((1ull << lane) - 1ull)), count = e >= 0 ? __popcll(same) : 0;
+  const bool first = e >= 0 && rank == 0;
+  const int my_slots = (count + slot_rows - 1) / slot_rows;
+  const bool heavy = 4 * count > slot_rows;
+  int start = 0, heavy_before = 0, light_before = 0, heavy_total = 0, light_total = 0, distinct = 0;
+  for (int j = 0; j < pairs; j++) {  // uniform: lane j's expert, if lane j is the first of it
+    const int ej = __builtin_amdgcn_readlane(first ? e : -1, j);
+    if (ej < 0) continue;
+    const int cj = __builtin_amdgcn_readlane(count, j), sj = __builtin_amdgcn_readlane(my_slots, j);
+    const bool hj = 4 * cj > slot_rows;
+    distinct++;
+    heavy_total += hj ? sj : 0;
+    light_total += hj ? 0 : sj;
+    if (ej < e) {
+      start += cj;
+      heavy_before += hj ? sj : 0;
+      light_before += hj ? 0 : sj;
+    }
+  }
+  const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
+  const int slots = shared_slots + heavy_total + light_total;
+  if (e >= 0) order[start + rank] = lane;
+  if (first) {
+    const int my_slot = shared_slots + (heavy ? heavy_before : heavy_total + light_before);
+    for (int s = 0; s < my_slots; s++) {
+      int32_t* entry = plan + PLAN_HEADER + 4 * (my_slot + s);
+      entry[0] = e;
+      entry[1] = start + s * slot_rows;
+      entry[2] = min(slot_rows, count - s * slot_rows);
+      entry[3] = 0;
+    }
+  }
+  for (int s = lane; s < shared_slots; s += 64) {
+    int32_t* entry = plan + PLAN_HEADER + 4 * s;
+    entry[0] = -1;
+    entry[1] = kept + s * slot_rows;
+    entry[2] = min(slot_rows, shared_rows - s * slot_rows);
+    entry[3] = 0;
+  }
+  for (int r = lane; r < shared_rows; r += 64) order[kept + r] = pairs + r;
+  for (int s = slots + lane; s < slot_cap; s += 64) {
+    int32_t* entry = plan + PLAN_HEADER + 4 * s;
+    entry[0] = entry[1] = entry[2] = entry[3] = 0;
+  }
+  if (lane == 0) {
+    plan[0] = slots;
+    plan[1] = distinct;
+    plan[2] = kept;
+  }
+}
+
 // With `route.logits` set the workgroup first routes the route.m rows itself (softmax top-k, a row a wavefront at a
 // time) into route.ids / route.weights, which `ids` then names.
 //
@@ -227,6 +295,10 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
       }
     }
     __syncthreads();
+  }
+  if (!WIDE && pairs <= 64) {  // a decode step: one wavefront plans it
+    if (threadIdx.x < 64) plan_few_pairs(ids, pairs, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap);
+    return;
   }
   int* seg_count = lds;                         // [PLAN_WAVES][e_n]: pairs of expert e in segment w, then running positions
   int* start = lds + PLAN_WAVES * e_n;          // [e_n]: first sorted position of expert e
