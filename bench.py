@@ -149,7 +149,7 @@ def latent_prefill(args) -> int:
         "data": "synthetic",
         "config": {"workload": "BASELINE config 4: NVFP4 latent-MoE layer, 2048 tokens, hidden 4096 -> latent 1024, 512 experts x inter 2688, "
                                "ReLU^2, top-22 sigmoid routing of N(0,1) logits, no shared expert", "timed_as": "one HIP-graph replay of all steps"},
-        "roofline": {"bound": "mfma", "kernel": "nvfp4_tile_kernel<fc1 relu2>", "achieved": gemm_flops / (fc1_ms * 1e-3) / 1e12,
+        "roofline": {"bound": "mfma", "kernel": "tile_kernel<TileNvfp4, fc1 relu2>", "achieved": gemm_flops / (fc1_ms * 1e-3) / 1e12,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": None, "launch_flops": gemm_flops, "launch_ms": fc1_ms},
         "layer_chain": {"kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
