@@ -692,7 +692,7 @@ extern "C" int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32
 
 static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x, const int32_t* ids,
                      const float* weights, int m, int topk, void* out, void* workspace, size_t workspace_bytes, void* stream,
-                     const Routing* route) {
+                     const Routing* route, bool e4m3 = false) {
   if (int e = check_experts(routed)) return e;
   if (shared) {
     if (int e = check_experts(shared)) return e;
@@ -704,7 +704,7 @@ static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, c
   if (m <= 0 || topk <= 0) return HB_EINVAL;
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, shared ? 1 : 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
-  if (int e = run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream), route)) return e;
+  if (int e = run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream), route, e4m3)) return e;
   CombineParams c{};
   c.pairs = ws.y;
   c.ids = ids;
@@ -731,6 +731,12 @@ extern "C" int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts*
                                const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
                                size_t workspace_bytes, void* stream) {
   return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, nullptr);
+}
+
+extern "C" int hb_w3_moe_layer_e4m3(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                                    const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, nullptr, true);
 }
 
 extern "C" int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,

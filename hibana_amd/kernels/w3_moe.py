@@ -155,10 +155,11 @@ def w3_moe(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: torc
 
 
 def moe_layer(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, shared: W3Experts | None = None,
-              gate_vec: torch.Tensor | None = None) -> torch.Tensor:
+              gate_vec: torch.Tensor | None = None, e4m3: bool = False) -> torch.Tensor:
     """The MoE layer on 3-bit weights in one chain of launches: routed sum + the shared expert (`shared`: a one-expert
     W3Experts of the same geometry) combined as bf16(bf16(routed) + g * bf16(shared)), g = sigmoid(x . gate_vec) or 1
-    (hibana/model/flashnext/moe.py:177-192)."""
+    (hibana/model/flashnext/moe.py:177-192). `e4m3`: x and h of every expert are rounded to E4M3 per (row, 32-group)
+    before their products, as in `w3_moe`."""
     _check_call(experts, x, ids, weights)
     m, k = ids.shape
     out = torch.empty((m, experts.shape2[0]), dtype=torch.bfloat16, device=x.device)
@@ -171,8 +172,9 @@ def moe_layer(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: t
     ids32 = ids.to(torch.int32).contiguous()
     wt = weights.float().contiguous()
     gv = None if gate_vec is None else gate_vec.float().contiguous()
-    _lib.check(_lib.lib().hb_w3_moe_layer(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(x.contiguous()),
-                                          _lib.ptr(ids32), _lib.ptr(wt), m, k, _lib.ptr(out), _lib.ptr(ws), need, _lib.stream()), "moe_layer")
+    entry = _lib.lib().hb_w3_moe_layer_e4m3 if e4m3 else _lib.lib().hb_w3_moe_layer
+    _lib.check(entry(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(x.contiguous()),
+                     _lib.ptr(ids32), _lib.ptr(wt), m, k, _lib.ptr(out), _lib.ptr(ws), need, _lib.stream()), "moe_layer")
     return out
 
 

@@ -151,6 +151,14 @@ int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, co
                     const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
                     size_t workspace_bytes, void* stream);
 
+/* hb_w3_moe_layer in the reference kernel's own arithmetic: x and h of the routed experts and of the shared expert go
+ * through the activation rounding (hb_w3_quant_groups) before their products, as with HB_MOE_E4M3 in hb_w3_moe; the
+ * combine is the same.
+ * ref: as hb_w3_moe_layer, with w3_moe.reference's `quant`, hibana/kernels/w3_moe.py:187-214. */
+int hb_w3_moe_layer_e4m3(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                         const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
 /* The same layer from the router's logits (float32 [m, experts_total]): softmax top-k routing as
  * hb_route_softmax_topk, written to ids int32 [m, topk] and weights float32 [m, topk] (caller's buffers), then the
  * chain of hb_w3_moe_layer. Up to 16 rows the routing runs inside the planning workgroup (one launch fewer).

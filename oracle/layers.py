@@ -176,17 +176,18 @@ def combine_shared_ref(routed: torch.Tensor, shared: torch.Tensor, x: torch.Tens
     return bf16(r + g * s)
 
 
-def moe_layer_ref(x, ids, weights, get_expert, gated: bool, shared=None, gate_vec=None, e_lo: int = 0, e_n: int = 512):
+def moe_layer_ref(x, ids, weights, get_expert, gated: bool, shared=None, gate_vec=None, e_lo: int = 0, e_n: int = 512, quant=None):
     """The gated-MoE layer of hibana/model/flashnext/moe.py:177-192 on 3-bit experts: routed sum, plus the shared
-    expert (w13, w2 in checkpoint row order) rounded to BF16 on its own, combined as combine_shared_ref."""
-    pairs = routed_experts_ref(x, ids, get_expert, gated, e_lo, e_n)
+    expert (w13, w2 in checkpoint row order) rounded to BF16 on its own, combined as combine_shared_ref. `quant`: the
+    activation rounding of the expert functions, for every expert."""
+    pairs = routed_experts_ref(x, ids, get_expert, gated, e_lo, e_n, quant)
     if pairs is None:
         width = shared[1].shape[0] if shared is not None else x.shape[1]
         pairs = torch.zeros(np.asarray(ids).size, width)
     routed = combine_ref(pairs, ids, weights, e_lo, e_n)
     if shared is None:
         return routed
-    s = bf16(expert_pairs_ref(x, np.arange(x.shape[0]), shared[0], shared[1], gated))
+    s = bf16(expert_pairs_ref(x, np.arange(x.shape[0]), shared[0], shared[1], gated, quant))
     return combine_shared_ref(routed, s, x, gate_vec)
 
 

@@ -105,3 +105,25 @@ def test_routed_experts_on_rounded_activations(gated, m, topk):
     # and it is a different function from the weight-only one: the rounding of x alone moves the result
     plain = w3_moe.w3_moe(ex, x.cuda(), ids.cuda(), wt.cuda())
     assert not torch.equal(plain, got)
+
+
+@pytest.mark.parametrize("m,with_gate", [(1, False), (5, True), (33, True)])
+def test_layer_with_shared_expert_on_rounded_activations(m, with_gate):
+    """The whole layer in the E4M3 activation mode: the routed experts and the shared expert both round x and h."""
+    from hibana_amd.kernels import w3_moe
+    e, hidden, inter, topk = 8, 256, 128, 3
+    ex, per = random_experts(e, hidden, inter, True, 41)
+    shared_ex, shared_per = random_experts(1, hidden, inter, True, 42)
+    get, shared_get = oracle_expert_getter(per, True, inter), oracle_expert_getter(shared_per, True, inter)
+    g = torch.Generator().manual_seed(50 + m)
+    x = torch.randn(m, hidden, generator=g).bfloat16()
+    ids = torch.stack([torch.randperm(e, generator=g)[:topk] for _ in range(m)]).to(torch.int32)
+    wt = torch.softmax(torch.randn(m, topk, generator=g), -1)
+    gate = torch.randn(hidden, generator=g) * 0.05 if with_gate else None
+    want = layers.moe_layer_ref(x, ids.numpy(), wt, get, True, shared=shared_get(0), gate_vec=gate, e_n=e, quant=layers.rounded_e4m3)
+    run = lambda **kw: w3_moe.moe_layer(ex, x.cuda(), ids.cuda(), wt.cuda(), shared=shared_ex, gate_vec=None if gate is None else gate.cuda(), **kw)
+    got = run(e4m3=True)
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    assert torch.equal(run(e4m3=True), got)
+    assert not torch.equal(run(), got)  # the weight-only layer is another function
