@@ -286,6 +286,76 @@ struct FullActs {  // up to sixteen rows: lane (q, r16) feeds row r16, k 8 q .. 
   }
 };
 
+// The sixteen-row body on E4M3 activations: lane (q, r16) feeds row r16's eight codes of every group (the FP8 MFMA's A
+// operand) and folds, per group, the product of the weight scale and the activation scales of the four rows its
+// accumulator registers hold (rows 4 q .. 4 q + 3). Both are asked for again by halves, as FullActs does.
+struct FullActs8 {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  static constexpr int LOADS = 12;
+  long a[4];            // the lane's codes of groups 0..3
+  f32x2_t xs_lo[4];     // activation scales of rows 4 q + r at groups 0, 1
+  f32x2_t xs_hi[4];     // ... at groups 2, 3
+  const uint8_t* at;    // the lane's codes of group 0 of the wavefront's first chunk
+  const float* scales;
+  uint32_t soff[4];     // the scale of slot row 4 q + r at group 0 of that chunk
+  __device__ __forceinline__ void load_half(int half, int i) {
+    a[2 * half] = *reinterpret_cast<const long*>(at + (int64_t)i * 128 + 64 * half);
+    a[2 * half + 1] = *reinterpret_cast<const long*>(at + (int64_t)i * 128 + 64 * half + 32);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const f32x2_t v = *reinterpret_cast<const f32x2_t*>(scales + soff[r] + 4 * i + 2 * half);
+      if (half) {
+        xs_hi[r] = v;
+      } else {
+        xs_lo[r] = v;
+      }
+    }
+  }
+  template <int EPI>
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int, int c0, int, int lane) {
+    const int q = lane >> 4, r16 = lane & 15;
+    at = p.aq + activation_row_index<EPI>(p, sl, r16) * p.a_stride + (int64_t)c0 * 128 + 8 * q;
+    scales = p.aq_scale;
+#pragma unroll
+    for (int r = 0; r < 4; r++) soff[r] = (uint32_t)(activation_row_index<EPI>(p, sl, 4 * q + r) * (p.a_stride >> 5)) + 4 * c0;
+    load_half(0, 0);
+    load_half(1, 0);
+  }
+  // groups 2 HALF and 2 HALF + 1 of the four tiles
+  template <int HALF>
+  __device__ __forceinline__ void half_chunk(const Chunk& ch, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, uint32_t lut_lo,
+                                             uint32_t lut_hi) const {
+    const uint32_t q0[4] = {ch.w0.x, ch.w0.w, ch.w1.z, ch.w2.y}, q1[4] = {ch.w0.y, ch.w1.x, ch.w1.w, ch.w2.z};
+    const uint32_t q2[4] = {ch.w0.z, ch.w1.y, ch.w2.x, ch.w2.w}, sc[4] = {ch.sc.x, ch.sc.y, ch.sc.z, ch.sc.w};
+    f32x4_t* acc[4] = {&acc0, &acc1, &acc2, &acc3};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      uint32_t sel[8];
+      w3_selectors(q0[t], q1[t], q2[t], sel);  // the four the half does not use fold away
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++) {
+        const int j = 2 * HALF + jj;
+        const long b = fp8x8(__builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j]), __builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j + 1]));
+        const f32x4_t part = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[j], b, f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        const float ws = j == 0 ? __builtin_amdgcn_cvt_f32_fp8(sc[t], 0) : j == 1 ? __builtin_amdgcn_cvt_f32_fp8(sc[t], 1)
+                       : j == 2 ? __builtin_amdgcn_cvt_f32_fp8(sc[t], 2) : __builtin_amdgcn_cvt_f32_fp8(sc[t], 3);
+        const f32x2_t* xs = HALF ? xs_hi : xs_lo;
+        acc[t]->x = fmaf(part.x, (jj ? xs[0].y : xs[0].x) * ws, acc[t]->x);
+        acc[t]->y = fmaf(part.y, (jj ? xs[1].y : xs[1].x) * ws, acc[t]->y);
+        acc[t]->z = fmaf(part.z, (jj ? xs[2].y : xs[2].x) * ws, acc[t]->z);
+        acc[t]->w = fmaf(part.w, (jj ? xs[3].y : xs[3].x) * ws, acc[t]->w);
+      }
+    }
+  }
+  template <int ODD, bool MORE2, bool MORE1>
+  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+    half_chunk<0>(ch, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+    if (MORE1) load_half(0, i + 1);
+    half_chunk<1>(ch, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
+    if (MORE1) load_half(1, i + 1);
+  }
+};
+
 // The end of a 64-row block for a slot of at most four rows. Lane (g, r16) of each of the block's K splits holds, in
 // register r of accumulator t, group g's part of (tile t, slot row r, column r16): sixteen values a lane, each to be
 // added over the four groups and the splits. They go to LDS, and the workgroup's 64 x ks lanes share the 16 x 16
@@ -333,8 +403,7 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
 }
 
 // General kernel, any K: one workgroup per (run of p.nbw 64-row blocks, slot), K split p.ks ways across its wavefronts.
-// A8: E4M3 activations (p.aq, p.aq_scale); every slot goes through the four-row body, four of its rows at a time (the
-// later passes find the block row in L2).
+// A8: E4M3 activations (p.aq, p.aq_scale), with the two bodies' FP8 forms.
 template <int EPI, bool A8>
 __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   extern __shared__ __align__(16) uint8_t rings[];
@@ -347,12 +416,20 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
   uint8_t* ring = rings + wave * RING_BYTES;
   if (A8) {
-    const float scale = active ? sl.rs[nb * 64 + lane] : 0.f;
-    for (int row0 = 0; row0 < sl.rows; row0 += FEW_ROWS) {  // uniform over the workgroup
-      acc0 = acc1 = acc2 = acc3 = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      if (active) stream_block<EPI, FewActs8, W3Ring>(p, sl, row0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
-      finish_few<EPI>(p, sl, row0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
-      if (p.ks > 1) __syncthreads();  // the exchange is read before the next pass fills the rings it lies in
+    if (sl.rows <= FEW_ROWS) {  // uniform over the workgroup
+      float scale = 0.f;
+      if (active) {
+        scale = sl.rs[nb * 64 + lane];
+        stream_block<EPI, FewActs8, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      }
+      finish_few<EPI>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+    } else {
+      RowScales rs{};
+      if (active) {
+        stream_block<EPI, FullActs8, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+        rs = row_scales<true>(sl, nb, lane & 15);
+      }
+      finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
     }
   } else if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
     float scale = 0.f;
