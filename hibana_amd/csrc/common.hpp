@@ -17,6 +17,9 @@ constexpr int WAVE = 64;
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// Device pointers the kernels read or write with 16-byte (activations, tile layouts, workspace) or 4-byte accesses.
+inline bool aligned(const void* p, size_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? HB_OK : HB_ELAUNCH; }
 
 // float32 -> bfloat16 bits, round to nearest even (NaN kept quiet).

@@ -630,6 +630,8 @@ extern "C" int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int
   if (!pairs || !ids || !weights || !out) return HB_ENULL;
   if (gate_vec && shared && !x) return HB_ENULL;
   if (m <= 0 || topk <= 0 || h <= 0 || h % 2) return HB_EINVAL;
+  if (!aligned(pairs, 8) || !aligned(ids, 4) || !aligned(weights, 4) || !aligned(shared, 4) || !aligned(x, 2) || !aligned(gate_vec, 4) || !aligned(out, 4))
+    return HB_EINVAL;
   CombineParams c{};
   c.pairs = pairs;
   c.pairs_bf16 = pairs_bf16;

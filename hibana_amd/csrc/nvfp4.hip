@@ -429,6 +429,7 @@ extern "C" int hb_nvfp4_dequant(const void* tiled, float global_scale, int64_t r
 extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y, void* stream) {
   if (!x || !tiled || !y) return HB_ENULL;
   if (m <= 0 || n <= 0 || k <= 0 || n % 64 || k % 128) return HB_EINVAL;
+  if (!aligned(x, 16) || !aligned(tiled, 16) || !aligned(y, 2)) return HB_EINVAL;
   StreamParams p{};
   p.w = static_cast<const uint8_t*>(tiled);
   p.scalar = global_scale;
@@ -462,6 +463,7 @@ int check_experts(const hb_nvfp4_experts* ex) {
   if (ex->experts <= 0 || ex->hidden <= 0 || ex->inter <= 0 || ex->hidden_out <= 0) return HB_EINVAL;
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
   if (ex->hidden % 128 || ex->inter % 128 || n1 % 64 || ex->hidden_out % 64) return HB_EINVAL;
+  if (!aligned(ex->fc1, 16) || !aligned(ex->fc2, 16) || !aligned(ex->fc1_scale2, 4) || !aligned(ex->fc2_scale2, 4)) return HB_EINVAL;
   return HB_OK;
 }
 
@@ -533,6 +535,7 @@ extern "C" int hb_nvfp4_moe(const hb_nvfp4_experts* routed, const void* x, const
   if (int e = check_experts(routed)) return e;
   if (!x || !ids || !weights || !out || !workspace) return HB_ENULL;
   if (m <= 0 || topk <= 0 || mode < HB_MOE_SUM || mode > HB_MOE_PAIRS_BF16) return HB_EINVAL;
+  if (!aligned(x, 16) || !aligned(ids, 4) || !aligned(weights, 4) || !aligned(out, 8) || !aligned(workspace, 16)) return HB_EINVAL;
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, 0);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
   const bool sum = mode == HB_MOE_SUM;

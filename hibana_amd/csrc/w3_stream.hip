@@ -577,6 +577,7 @@ extern "C" int hb_tune(const char* key, int value) {
 extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, void* y, void* stream) {
   if (!x || !tiled || !row_scale || !y) return HB_ENULL;
   if (m <= 0 || n <= 0 || k <= 0 || n % W3_BLOCK_ROWS || k % W3_CHUNK) return HB_EINVAL;
+  if (!aligned(x, 16) || !aligned(tiled, 16) || !aligned(row_scale, 4) || !aligned(y, 2)) return HB_EINVAL;
   StreamParams p{};
   p.w = static_cast<const uint8_t*>(tiled);
   p.rows = row_scale;
@@ -602,6 +603,7 @@ extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* 
 extern "C" int hb_w3_quant_groups(const void* x, int64_t m, int k, void* q, float* scales, void* stream) {
   if (!x || !q || !scales) return HB_ENULL;
   if (m <= 0 || k <= 0 || k % 32) return HB_EINVAL;
+  if (!aligned(x, 16) || !aligned(q, 8) || !aligned(scales, 4)) return HB_EINVAL;
   launch_quant_groups(x, m, k, static_cast<uint8_t*>(q), scales, as_stream(stream));
   return launch_status();
 }
@@ -610,6 +612,7 @@ extern "C" int hb_w3_gemm_e4m3(const void* xq, const float* x_scale, int m, cons
                                void* y, void* stream) {
   if (!xq || !x_scale || !tiled || !row_scale || !y) return HB_ENULL;
   if (m <= 0 || n <= 0 || k <= 0 || n % W3_BLOCK_ROWS || k % W3_CHUNK || (int64_t)m * (k / 32) > 0xffffffffll) return HB_EINVAL;
+  if (!aligned(xq, 8) || !aligned(x_scale, 8) || !aligned(tiled, 16) || !aligned(row_scale, 4) || !aligned(y, 2)) return HB_EINVAL;
   StreamParams p{};
   p.w = static_cast<const uint8_t*>(tiled);
   p.rows = row_scale;
@@ -638,6 +641,7 @@ int check_experts(const hb_w3_experts* ex) {
   if (ex->experts <= 0 || ex->hidden <= 0 || ex->inter <= 0 || ex->hidden_out <= 0) return HB_EINVAL;
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
   if (ex->hidden % W3_CHUNK || ex->inter % W3_CHUNK || n1 % W3_BLOCK_ROWS || ex->hidden_out % W3_BLOCK_ROWS) return HB_EINVAL;
+  if (!aligned(ex->fc1, 16) || !aligned(ex->fc2, 16) || !aligned(ex->fc1_rows, 4) || !aligned(ex->fc2_rows, 4)) return HB_EINVAL;
   return HB_OK;
 }
 
@@ -747,6 +751,7 @@ extern "C" int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32
   const bool e4m3 = (mode & HB_MOE_E4M3) != 0;
   mode &= ~HB_MOE_E4M3;
   if (m <= 0 || topk <= 0 || mode < HB_MOE_SUM || mode > HB_MOE_PAIRS_BF16) return HB_EINVAL;
+  if (!aligned(x, 16) || !aligned(ids, 4) || !aligned(weights, 4) || !aligned(out, 8) || !aligned(workspace, 16)) return HB_EINVAL;
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
   void* pairs_out = mode == HB_MOE_SUM ? static_cast<void*>(ws.y) : out;
@@ -779,6 +784,7 @@ static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, c
   }
   if (!x || !ids || !weights || !out || !workspace) return HB_ENULL;
   if (m <= 0 || topk <= 0) return HB_EINVAL;
+  if (!aligned(x, 16) || !aligned(ids, 4) || !aligned(weights, 4) || !aligned(out, 4) || !aligned(workspace, 16) || !aligned(gate_vec, 4)) return HB_EINVAL;
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, shared ? 1 : 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
   if (int e = run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream), route, e4m3)) return e;
@@ -820,6 +826,7 @@ extern "C" int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_e
                                       const float* logits, int experts_total, int m, int topk, int32_t* ids, float* weights, void* out,
                                       void* workspace, size_t workspace_bytes, void* stream) {
   if (!logits) return HB_ENULL;
+  if (!aligned(logits, 4)) return HB_EINVAL;
   const Routing route{logits, experts_total, ids, weights};
   return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, &route);
 }

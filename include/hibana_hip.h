@@ -22,7 +22,9 @@ extern "C" {
 
 enum {
   HB_OK = 0,
-  HB_EINVAL = -1,     /* a shape, alignment or flag the kernels do not take (the Python layer raises ValueError) */
+  HB_EINVAL = -1,     /* a shape, alignment or flag the kernels do not take (the Python layer raises ValueError):
+                         activations, tile layouts and workspaces must lie on 16-byte boundaries, FP32 / int32 arrays on
+                         4-byte ones (any allocator's blocks do; the calls check) */
   HB_ENULL = -2,      /* a required pointer is NULL */
   HB_EWORKSPACE = -3, /* workspace smaller than hb_*_workspace_bytes() says */
   HB_ELAUNCH = -4     /* the HIP runtime refused a launch (hipGetLastError is left set for the caller) */

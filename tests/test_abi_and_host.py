@@ -41,12 +41,18 @@ def test_validation_without_a_gpu():
     assert lib.hb_w3_gemm(None, 1, None, None, 0, 128, 128, None, None) == _lib.HB_ENULL
     assert lib.hb_nvfp4_gemm(None, 1, None, 1.0, 128, 128, 0, None, None) == _lib.HB_ENULL
     assert lib.hb_w3_moe_workspace_bytes(4, 2, None, 0) == 0
-    ex = _lib.HbW3Experts(1, 1, 1, 1, 0, 0, 8, 0, 256, 128, 256, 1)
+    ex = _lib.HbW3Experts(256, 256, 256, 256, 0, 0, 8, 0, 256, 128, 256, 1)  # (no call below reads through the pointers)
     need = lib.hb_w3_moe_workspace_bytes(32, 10, C.byref(ex), 1)
     assert need >= (320 + 32) * (128 * 2 + 256 * 4)
-    bad = _lib.HbW3Experts(1, 1, 1, 1, 0, 0, 8, 0, 200, 128, 256, 1)  # hidden not a multiple of 128
+    bad = _lib.HbW3Experts(256, 256, 256, 256, 0, 0, 8, 0, 200, 128, 256, 1)  # hidden not a multiple of 128
     assert lib.hb_w3_moe_workspace_bytes(32, 10, C.byref(bad), 1) == 0
     assert lib.hb_w3_moe(C.byref(bad), None, None, None, 1, 1, 0, None, None, 0, None) == _lib.HB_EINVAL
+    # pointers off the boundaries the kernels' vector accesses need are refused before anything is launched
+    odd = _lib.HbW3Experts(264, 256, 256, 256, 0, 0, 8, 0, 256, 128, 256, 1)  # fc1 on an 8-byte boundary only
+    assert lib.hb_w3_moe_workspace_bytes(32, 10, C.byref(odd), 1) == 0
+    assert lib.hb_w3_gemm(258, 1, 256, 256, 0, 128, 128, 256, None) == _lib.HB_EINVAL  # x on a 2-byte boundary
+    assert lib.hb_w3_moe(C.byref(ex), 256, 256, 256, 1, 1, 0, 256, 264, 1 << 30, None) == _lib.HB_EINVAL  # workspace on 8
+    assert lib.hb_nvfp4_gemm(256, 1, 260, 1.0, 128, 128, 0, 256, None) == _lib.HB_EINVAL  # tile layout on 4
     with pytest.raises(ValueError):
         _lib.check(_lib.HB_EINVAL, "x")
     with pytest.raises(RuntimeError):
