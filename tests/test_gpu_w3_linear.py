@@ -94,3 +94,25 @@ def test_unsupported_calls_raise():
         w3.w3_linear(torch.zeros(4, 128, dtype=torch.bfloat16, device="cuda"), dev)
     with pytest.raises(RuntimeError):
         w3.w3_linear(torch.zeros(4, 256, dtype=torch.bfloat16), dev)
+
+
+@pytest.mark.parametrize("m", [1, 16, 128])
+@pytest.mark.parametrize("n,k", [(10240, 5120), (5120, 17408)])
+def test_the_references_full_size_shapes(n, k, m):
+    """The shapes of the reference's own GPU test of the dense linear (tests/gpu/test_w3_calibration.py:23-45: rows 1 to
+    128 on 10240 x 5120 and 5120 x 17408, norm-relative error below 0.004): the kernel against x @ dequantize(W)^T in
+    FP32 on the GPU, the dequantization being pinned bit-exact against the oracle on the smaller shapes; bitwise
+    repeatable, as that test demands of a graph replay."""
+    from hibana_amd.kernels import w3
+    g = torch.Generator(device="cuda").manual_seed(n + k + m)
+    q = torch.randint(0, 8, (n, k), device="cuda", dtype=torch.uint8, generator=g)
+    s = torch.rand(n, k // 32, device="cuda", generator=g) * 0.03 + 1e-3
+    row = (s.amax(dim=1) / 448.0).clamp_min(1e-12)
+    stored = (s / row[:, None]).to(torch.float8_e4m3fn)
+    weight = w3.pack_codes(q, stored, row, "lloyd")
+    x = torch.randn(m, k, device="cuda", generator=g).bfloat16()
+    want = (x.float() @ w3.dequantize(weight).T).bfloat16()
+    got = w3.w3_linear(x, weight)
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    assert torch.equal(w3.w3_linear(x, weight), got)
