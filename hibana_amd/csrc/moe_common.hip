@@ -275,6 +275,8 @@ __device__ __forceinline__ void plan_few_pairs(const int32_t* ids, int pairs, in
 // With `route.logits` set the workgroup first routes the route.m rows itself (softmax top-k, a row a wavefront at a
 // time) into route.ids / route.weights, which `ids` then names.
 //
+// With `job.lanes` set the launch has further workgroups, which round the job's activations to E4M3 and plan nothing.
+//
 // Many pairs (a prefill chunk) are shared among `groups` workgroups in three launches of this kernel, `wide` [groups, e_n]
 // between them: phase 1, each group counts its share of the pairs per expert; phase 2, one workgroup adds the groups'
 // counts, writes the slot table and turns `wide` into the first sorted position of each group's run of each expert;
@@ -283,9 +285,14 @@ template <bool WIDE>  // false: one workgroup (phase 0) and nothing of the share
 __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
                                                                 int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
                                                                 int route_rows, int slot_rows, int slot_cap, int32_t* __restrict__ wide, int groups_,
-                                                                int phase_) {
+                                                                int phase_, QuantJob job) {
   const int groups = WIDE ? groups_ : 1, phase = WIDE ? phase_ : 0;
   extern __shared__ int lds[];
+  if (!WIDE && blockIdx.x > 0) {  // the workgroups beside the plan's: the activation rounding, PLAN_THREADS lanes each
+    const int64_t i = (int64_t)(blockIdx.x - 1) * PLAN_THREADS + threadIdx.x;
+    if (i < job.lanes) quant_groups_lane(job.x, i, job.q, job.scales);  // whole groups: four lanes in or out together
+    return;
+  }
   if (route.logits) {
     for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
       if (route.per <= 8) {
@@ -575,26 +582,39 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
   return w;
 }
 
-int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream, int slot_rows) {
+__global__ __launch_bounds__(256) void quant_groups_kernel(QuantJob job) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < job.lanes) quant_groups_lane(job.x, i, job.q, job.scales);
+}
+
+void moe_launch_quant_groups(const QuantJob& job, hipStream_t stream) {
+  HB_LAUNCH(quant_groups_kernel, dim3((unsigned)((job.lanes + 255) / 256)), dim3(256), 0, stream, job);
+}
+
+static unsigned plan_groups(const QuantJob* job) { return 1u + (job ? (unsigned)((job->lanes + PLAN_THREADS - 1) / PLAN_THREADS) : 0u); }
+
+int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream, int slot_rows,
+                    const QuantJob* job) {
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
   const int slot_cap = (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows);
   if (pairs >= PLAN_WIDE_PAIRS) {  // a share of about a thousand pairs a workgroup
     const int groups = (int)std::min<int64_t>(PLAN_WIDE_GROUPS, pairs / 1024);
+    if (job) moe_launch_quant_groups(*job, stream);
     for (int phase = 1; phase <= 3; phase++)
       HB_LAUNCH(moe_plan_kernel<true>, dim3(phase == 2 ? 1 : groups), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan,
-                ws.order, RouteParams{}, 0, slot_rows, slot_cap, ws.plan_wide, groups, phase);
+                ws.order, RouteParams{}, 0, slot_rows, slot_cap, ws.plan_wide, groups, phase, QuantJob{});
     return HB_OK;
   }
-  HB_LAUNCH(moe_plan_kernel<false>, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, RouteParams{}, 0,
-            slot_rows, slot_cap, ws.plan_wide, 1, 0);
+  HB_LAUNCH(moe_plan_kernel<false>, dim3(plan_groups(job)), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order,
+            RouteParams{}, 0, slot_rows, slot_cap, ws.plan_wide, 1, 0, job ? *job : QuantJob{});
   return HB_OK;
 }
 
 int moe_check_route(int m, int e, int k) { return m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE ? HB_EINVAL : HB_OK; }
 
 int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
-                          const MoeWorkspace& ws, hipStream_t stream, int slot_rows) {
+                          const MoeWorkspace& ws, hipStream_t stream, int slot_rows, const QuantJob* job) {
   if (int err = moe_check_route(m, e, topk)) return err;
   RouteParams rp{};
   rp.logits = logits;
@@ -607,12 +627,12 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   const int64_t pairs = (int64_t)m * topk;
   if (m > ROUTE_FUSED_ROWS) {  // many rows: a wavefront a row over the whole device, then the plan
     launch_route<false>(rp, m, stream);
-    return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, slot_rows);
+    return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, slot_rows, job);
   }
   const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
   if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
-  HB_LAUNCH(moe_plan_kernel<false>, dim3(1), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order, rp, m, slot_rows,
-            (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows), ws.plan_wide, 1, 0);
+  HB_LAUNCH(moe_plan_kernel<false>, dim3(plan_groups(job)), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order,
+            rp, m, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows), ws.plan_wide, 1, 0, job ? *job : QuantJob{});
   return HB_OK;
 }
 

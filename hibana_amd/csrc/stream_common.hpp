@@ -38,6 +38,8 @@ struct StreamParams {
   int topk, pairs;        // grouped calls: pair q < pairs belongs to token q / topk, q >= pairs to token q - pairs
   void* out;
   int64_t out_stride;     // elements between output rows
+  uint8_t* oq;            // fc1 in the E4M3 activation mode: h leaves as codes [rows, out_stride] ...
+  float* oq_scale;        // ... and scales [rows, out_stride / 32] instead of BF16 in `out`
   int out_bf16;           // EPI_FC2: pair outputs in BF16 instead of FP32
   int ks, nbw;            // wavefronts per workgroup = ks (K splits) * nbw (64-row blocks)
   int ks_inv, chunks_base, chunks_rem;  // set_split(): ceil(65536 / ks), chunks / ks, chunks % ks
@@ -74,19 +76,26 @@ __device__ __forceinline__ RowScales row_scales(const Slot& sl, int nb, int r16)
   return rs;
 }
 
+// What fc1 hands to fc2 for one element, as the FP32 value of its BF16 rounding: y0 / y1 are the K-complete sums times
+// their FP32 scale (gated: the up and the gate row); the roundings are the reference's.
+template <int EPI>
+__device__ __forceinline__ float fc1_value(float y0, float y1) {
+  if (EPI == EPI_FC1_GATED) return through_bf16(silu(through_bf16(y1)) * through_bf16(y0));
+  const float h = fmaxf(through_bf16(y0), 0.f);
+  return through_bf16(h * h);
+}
+
 // Stores one output element (gated: one up/gate pair) of the 64-row block: row tile `t` (gated: pair index), column r16
-// of it, slot row i. y0 / y1 are the K-complete sums times their FP32 scale; the roundings are the reference's.
+// of it, slot row i.
 template <int EPI>
 __device__ __forceinline__ void store_out(const StreamParams& p, const Slot& sl, int nb, int t, int i, int r16, float y0, float y1) {
   const int64_t pos = sl.p0 + i;
   if (EPI == EPI_FC1_GATED) {
-    const float up = through_bf16(y0), gate = through_bf16(y1);
-    reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = bf16_of(silu(gate) * up);
+    reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = bf16_of(fc1_value<EPI>(y0, y1));
   } else {
     const int n = nb * 64 + 16 * t + r16;
     if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
-      const float h = fmaxf(through_bf16(y0), 0.f);
-      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(h * h);
+      reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(fc1_value<EPI_FC1_RELU2>(y0, 0.f));
     } else if (EPI == EPI_DENSE) {
       reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(y0);
     } else {
@@ -98,6 +107,26 @@ __device__ __forceinline__ void store_out(const StreamParams& p, const Slot& sl,
       }
     }
   }
+}
+
+// The largest of a value over the sixteen lanes of a DPP row, in each of them. Lanes that are switched off
+// contribute 0 (the values are magnitudes).
+__device__ __forceinline__ float row16_max(float x) {
+  x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false)));   // lane ^ 1
+  x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false)));   // lane ^ 2
+  x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false)));  // mirror within 8
+  x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, false)));  // mirror within 16
+  return x;
+}
+
+// The activation rounding of one element of h inside fc1's epilogue: `h` = fc1_value of column `col` of sorted row
+// `pos`, `amax` the largest magnitude of the column's 32-group. s = max(amax / 448, 1e-12), code = e4m3(h / s), IEEE
+// divisions: the arithmetic of the separate quantizer (quant_groups_lane below), value for value.
+__device__ __forceinline__ void store_quantized(const StreamParams& p, int64_t pos, int col, float h, float amax, bool first_of_group) {
+  const float s = fmaxf(amax / 448.0f, 1e-12f);
+  const float v = fminf(fmaxf(h / s, -448.0f), 448.0f);
+  p.oq[pos * p.out_stride + col] = (uint8_t)__builtin_amdgcn_cvt_pk_fp8_f32(v, 0.f, 0, false);
+  if (first_of_group) p.oq_scale[pos * (p.out_stride >> 5) + (col >> 5)] = s;
 }
 
 // One output element (or, gated, one up/gate pair) from accumulator register r of lane (q, r16); v0 / v1 are the
@@ -112,6 +141,33 @@ __device__ __forceinline__ void emit(const StreamParams& p, const Slot& sl, cons
     store_out<EPI>(p, sl, nb, t, i, r16, v0 * (PER_ROW ? rs.of(2 * t) : sl.scalar), v1 * (PER_ROW ? rs.of(2 * t + 1) : sl.scalar));
   } else {
     store_out<EPI>(p, sl, nb, t, i, r16, v0 * (PER_ROW ? rs.of(t) : sl.scalar), 0.f);
+  }
+}
+
+// The E4M3 form of emit for fc1: the four K-complete sums of accumulator register r of lane (q, r16), one per 16-row
+// tile, become this slot row's codes of the block's h columns (gated: 32 columns, one group; else 64, two groups). A
+// group's columns are the sixteen lanes of this lane's DPP row times two tiles; the row's lanes hold the same slot row,
+// so they stay or leave together.
+template <int EPI>
+__device__ __forceinline__ void quant_emit(const StreamParams& p, const Slot& sl, const RowScales& rs, int nb, int r, int q, int r16, float v0, float v1,
+                                           float v2, float v3) {
+  if (r >= sl.rows) return;  // wave-uniform
+  const int i = 4 * q + r;
+  if (i >= sl.rows) return;
+  const int64_t pos = sl.p0 + i;
+  const float y0 = v0 * rs.of(0), y1 = v1 * rs.of(1), y2 = v2 * rs.of(2), y3 = v3 * rs.of(3);
+  if (EPI == EPI_FC1_GATED) {
+    const float h0 = fc1_value<EPI>(y0, y1), h1 = fc1_value<EPI>(y2, y3);
+    const float amax = row16_max(fmaxf(fabsf(h0), fabsf(h1)));
+    store_quantized(p, pos, nb * 32 + r16, h0, amax, r16 == 0);
+    store_quantized(p, pos, nb * 32 + 16 + r16, h1, amax, false);
+  } else {
+    const float h0 = fc1_value<EPI>(y0, 0.f), h1 = fc1_value<EPI>(y1, 0.f), h2 = fc1_value<EPI>(y2, 0.f), h3 = fc1_value<EPI>(y3, 0.f);
+    const float lo = row16_max(fmaxf(fabsf(h0), fabsf(h1))), hi = row16_max(fmaxf(fabsf(h2), fabsf(h3)));
+    store_quantized(p, pos, nb * 64 + r16, h0, lo, r16 == 0);
+    store_quantized(p, pos, nb * 64 + 16 + r16, h1, lo, false);
+    store_quantized(p, pos, nb * 64 + 32 + r16, h2, hi, r16 == 0);
+    store_quantized(p, pos, nb * 64 + 48 + r16, h3, hi, false);
   }
 }
 
@@ -177,8 +233,10 @@ __device__ __forceinline__ const uint16_t* activation_row(const StreamParams& p,
 
 // The end of a 64-row block: K-complete sums straight from the registers (ks == 1), or the K split's partial sums
 // exchanged through LDS (`partial`: 4 KB at the start of each wavefront's STRIDE floats) and added in split order,
-// then the epilogue. With ks > 1 every wavefront of the workgroup must call it (one workgroup barrier).
-template <int EPI, bool PER_ROW, int STRIDE = 1024>
+// then the epilogue. With ks > 1 every wavefront of the workgroup must call it (one workgroup barrier). QUANT (fc1 in
+// the E4M3 activation mode): the epilogue is quant_emit, a split taking whole accumulator registers (all four tiles
+// of slot rows r, r + 4, ...), since a group's maximum needs two tiles.
+template <int EPI, bool PER_ROW, int STRIDE = 1024, bool QUANT = false>
 __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& sl, const RowScales& rs, int nb, bool active, int ks, int nbi, float* partial,
                                              const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2, const f32x4_t& acc3) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -186,7 +244,12 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
   const int rows = sl.rows;
   if (p.ks == 1) {
     if (!active) return;
-    if (EPI == EPI_FC1_GATED) {
+    if (QUANT) {
+      quant_emit<EPI>(p, sl, rs, nb, 0, q, r16, acc0.x, acc1.x, acc2.x, acc3.x);
+      quant_emit<EPI>(p, sl, rs, nb, 1, q, r16, acc0.y, acc1.y, acc2.y, acc3.y);
+      quant_emit<EPI>(p, sl, rs, nb, 2, q, r16, acc0.z, acc1.z, acc2.z, acc3.z);
+      quant_emit<EPI>(p, sl, rs, nb, 3, q, r16, acc0.w, acc1.w, acc2.w, acc3.w);
+    } else if (EPI == EPI_FC1_GATED) {
       emit<EPI, PER_ROW>(p, sl, rs, nb, 0, 0, q, r16, acc0.x, acc1.x);
       emit<EPI, PER_ROW>(p, sl, rs, nb, 0, 1, q, r16, acc0.y, acc1.y);
       emit<EPI, PER_ROW>(p, sl, rs, nb, 0, 2, q, r16, acc0.z, acc1.z);
@@ -221,7 +284,17 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
   __syncthreads();
   if (!active) return;
   const float* first = partial + (int64_t)nbi * p.ks * STRIDE;
-  if (EPI == EPI_FC1_GATED) {
+  if (QUANT) {
+    for (int r = ks; r < 4; r += p.ks) {
+      if (r >= rows) continue;
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int s = 0; s < p.ks; s++) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) v[t] += first[s * STRIDE + (t * 4 + r) * 64 + lane];
+      }
+      quant_emit<EPI>(p, sl, rs, nb, r, q, r16, v[0], v[1], v[2], v[3]);
+    }
+  } else if (EPI == EPI_FC1_GATED) {
     for (int idx = ks; idx < 8; idx += p.ks) {
       const int t = idx >> 2, r = idx & 3;
       if (r >= rows) continue;
@@ -244,6 +317,47 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
 }
 
 
+// ------------------------------------------------------------------------------------------ activation rounding
+//
+// BF16 [m, k] -> E4M3 codes [m, k] and one FP32 scale per (row, 32-group): s = max(amax / 448, 1e-12),
+// q = e4m3(clamp(x / s, -448, 448)), both quotients IEEE FP32 divisions (the reference's torch statement of its
+// quantizer, hibana/kernels/w3_moe.py:187-190; its CUDA kernel, hibana/kernels/csrc/w3_gemm.cu:291-327, multiplies by
+// an approximate reciprocal instead). Lane i takes the eight consecutive values from 8 i, four lanes a group; the
+// four lanes of a group are neighbours in one wavefront and must all be switched on.
+__device__ __forceinline__ void quant_groups_lane(const uint16_t* __restrict__ x, int64_t i, uint8_t* __restrict__ q, float* __restrict__ scales) {
+  const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(x + 8 * i);
+  float v[8];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    v[2 * j] = __uint_as_float(raw[j] << 16);
+    v[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(v[j]));
+  amax = fmaxf(amax, __shfl_xor(amax, 1));
+  amax = fmaxf(amax, __shfl_xor(amax, 2));
+  const float s = fmaxf(amax / 448.0f, 1e-12f);
+#pragma unroll
+  for (int j = 0; j < 8; j++) v[j] = fminf(fmaxf(v[j] / s, -448.0f), 448.0f);
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], hi, true);
+  typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+  *reinterpret_cast<i32x2_t*>(q + 8 * i) = i32x2_t{lo, hi};
+  if ((i & 3) == 0) scales[i >> 2] = s;
+}
+
+// A rounding to run beside a plan: `lanes` = values / 8 (0: none).
+struct QuantJob {
+  const uint16_t* x;
+  int64_t lanes;
+  uint8_t* q;
+  float* scales;
+};
+
 // ---------------------------------------------------------------------------------------------------- host side
 // Workspace of a routed call, carved from one caller-owned buffer.
 struct MoeWorkspace {
@@ -262,13 +376,15 @@ struct MoeWorkspace {
 int64_t moe_max_slots(int64_t pairs, int experts, int shared_rows, int slot_rows = ROWS_PER_SLOT);
 MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int hidden_out, int shared, int hidden = 0);  // hidden: also the E4M3 activation buffers
 // Enqueue the plan kernel; HB_EINVAL if the expert count does not fit its LDS.
+// A rounding job rides in the plan's launch (further workgroups beside the one that plans).
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream,
-                    int slot_rows = ROWS_PER_SLOT);
+                    int slot_rows = ROWS_PER_SLOT, const QuantJob* job = nullptr);
+void moe_launch_quant_groups(const QuantJob& job, hipStream_t stream);  // the rounding alone
 
 // Softmax top-k routing of `m` rows of `e` logits into ids / weights [m, topk], then the plan of those ids: one launch
 // for up to a few dozen rows, two beyond.
 int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
-                          const MoeWorkspace& ws, hipStream_t stream, int slot_rows = ROWS_PER_SLOT);
+                          const MoeWorkspace& ws, hipStream_t stream, int slot_rows = ROWS_PER_SLOT, const QuantJob* job = nullptr);
 
 struct CombineParams {
   const void* pairs;      // [m * topk (+ m), h] FP32 or BF16

@@ -362,7 +362,8 @@ struct FullActs8 {
 // results of the block: lane (q, r16) of split `ks` takes tile q, column r16, of slot rows row0 + ks, row0 + ks + p.ks, ... It
 // multiplies by its tile's row scale (`scale`, asked for before the first chunk); a gated pair's gate comes from the
 // neighbouring tile's lane. Every wavefront of the workgroup must call it when K is split (one workgroup barrier).
-template <int EPI>
+// QUANT (fc1 in the E4M3 activation mode): h leaves as codes and scales; a 32-group is two of the wavefront's DPP rows.
+template <int EPI, bool QUANT = false>
 __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl, int row0, float scale, int nb, bool active, int wave, int ks,
                                            int nbi, float* partial, const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2,
                                            const f32x4_t& acc3) {
@@ -395,7 +396,20 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
     const float y = v * scale;
     if (EPI == EPI_FC1_GATED) {
       const float gate = __shfl_xor(y, 16);  // tiles 2 t and 2 t + 1 are a pair's up and gate rows
-      if ((q & 1) == 0) store_out<EPI>(p, sl, nb, q >> 1, row0 + r, r16, y, gate);
+      if (QUANT) {  // the pairs are in tiles 0 and 2: their two rows of lanes are the group
+        const bool pair = (q & 1) == 0;
+        const float h = pair ? fc1_value<EPI>(y, gate) : 0.f;
+        float amax = row16_max(fabsf(h));
+        amax = fmaxf(amax, __shfl_xor(amax, 32));
+        if (pair) store_quantized(p, sl.p0 + row0 + r, nb * 32 + 8 * q + r16, h, amax, lane == 0);
+      } else if ((q & 1) == 0) {
+        store_out<EPI>(p, sl, nb, q >> 1, row0 + r, r16, y, gate);
+      }
+    } else if (QUANT) {  // tiles 0, 1 and tiles 2, 3 are the block's two groups
+      const float h = fc1_value<EPI>(y, 0.f);
+      float amax = row16_max(fabsf(h));
+      amax = fmaxf(amax, __shfl_xor(amax, 16));
+      store_quantized(p, sl.p0 + row0 + r, nb * 64 + 16 * q + r16, h, amax, (lane & 31) == 0);
     } else {
       store_out<EPI>(p, sl, nb, q, row0 + r, r16, y, 0.f);
     }
@@ -403,7 +417,8 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
 }
 
 // General kernel, any K: one workgroup per (run of p.nbw 64-row blocks, slot), K split p.ks ways across its wavefronts.
-// A8: E4M3 activations (p.aq, p.aq_scale), with the two bodies' FP8 forms.
+// A8: E4M3 activations (p.aq, p.aq_scale), with the two bodies' FP8 forms; fc1 then writes h as E4M3 codes and
+// scales (p.oq, p.oq_scale), the activation rounding done in its epilogue.
 template <int EPI, bool A8>
 __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   extern __shared__ __align__(16) uint8_t rings[];
@@ -415,6 +430,7 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
   uint8_t* ring = rings + wave * RING_BYTES;
+  constexpr bool QUANT = A8 && epi_gathers(EPI);  // fc1 on E4M3 activations hands fc2 E4M3 activations
   if (A8) {
     if (sl.rows <= FEW_ROWS) {  // uniform over the workgroup
       float scale = 0.f;
@@ -422,14 +438,14 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
         scale = sl.rs[nb * 64 + lane];
         stream_block<EPI, FewActs8, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
       }
-      finish_few<EPI>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+      finish_few<EPI, QUANT>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
     } else {
       RowScales rs{};
       if (active) {
         stream_block<EPI, FullActs8, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
         rs = row_scales<true>(sl, nb, lane & 15);
       }
-      finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+      finish_block<EPI, true, RING_BYTES / 4, QUANT>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
     }
   } else if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
     float scale = 0.f;
@@ -479,46 +495,6 @@ struct TileW3 {
     return __builtin_bit_cast(bf16x8_t, packed);
   }
 };
-
-// ------------------------------------------------------------------------------------------ activation rounding
-//
-// BF16 [m, k] -> E4M3 codes [m, k] and one FP32 scale per (row, 32-group): s = max(amax / 448, 1e-12),
-// q = e4m3(clamp(x / s, -448, 448)), both quotients IEEE FP32 divisions (the reference's torch statement of its
-// quantizer, hibana/kernels/w3_moe.py:187-190; its CUDA kernel, hibana/kernels/csrc/w3_gemm.cu:291-327, multiplies by
-// an approximate reciprocal instead). One lane takes eight consecutive values, four lanes a group.
-__global__ __launch_bounds__(256) void w3_quant_groups_kernel(const uint16_t* __restrict__ x, int64_t lanes, uint8_t* __restrict__ q,
-                                                              float* __restrict__ scales) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= lanes) return;  // whole groups: k is a multiple of 32, so a group's four lanes are in or out together
-  const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(x + 8 * i);
-  float v[8];
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    v[2 * j] = __uint_as_float(raw[j] << 16);
-    v[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
-  }
-  float amax = 0.f;
-#pragma unroll
-  for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(v[j]));
-  amax = fmaxf(amax, __shfl_xor(amax, 1));
-  amax = fmaxf(amax, __shfl_xor(amax, 2));
-  const float s = fmaxf(amax / 448.0f, 1e-12f);
-#pragma unroll
-  for (int j = 0; j < 8; j++) v[j] = fminf(fmaxf(v[j] / s, -448.0f), 448.0f);
-  int lo = 0, hi = 0;
-  lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], lo, false);
-  lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], lo, true);
-  hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], hi, false);
-  hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], hi, true);
-  typedef __attribute__((ext_vector_type(2))) int i32x2_t;
-  *reinterpret_cast<i32x2_t*>(q + 8 * i) = i32x2_t{lo, hi};
-  if ((i & 3) == 0) scales[i >> 2] = s;
-}
-
-static void launch_quant_groups(const void* x, int64_t rows, int k, uint8_t* q, float* scales, hipStream_t stream) {
-  const int64_t lanes = rows * k / 8;
-  HB_LAUNCH(w3_quant_groups_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream, static_cast<const uint16_t*>(x), lanes, q, scales);
-}
 
 // ---------------------------------------------------------------------------------------------------- host side
 struct Tuning {
@@ -604,7 +580,7 @@ extern "C" int hb_w3_quant_groups(const void* x, int64_t m, int k, void* q, floa
   if (!x || !q || !scales) return HB_ENULL;
   if (m <= 0 || k <= 0 || k % 32) return HB_EINVAL;
   if (!aligned(x, 16) || !aligned(q, 8) || !aligned(scales, 4)) return HB_EINVAL;
-  launch_quant_groups(x, m, k, static_cast<uint8_t*>(q), scales, as_stream(stream));
+  moe_launch_quant_groups(QuantJob{static_cast<const uint16_t*>(x), m * k / 8, static_cast<uint8_t*>(q), scales}, as_stream(stream));
   return launch_status();
 }
 
@@ -665,11 +641,13 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
   const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows, slot_rows);
   if (slots > 65535) return HB_EINVAL;
+  // E4M3 activations: x is rounded by further workgroups of the plan's launch, h in fc1's epilogue
+  const QuantJob xjob{static_cast<const uint16_t*>(x), (int64_t)m * ex->hidden / 8, ws.xq, ws.xs};
   if (route) {
     if (int e = moe_launch_route_plan(route->logits, m, route->e, topk, route->ids, route->weights, ex->base, ex->experts, shared_rows, ws, stream,
-                                      slot_rows))
+                                      slot_rows, e4m3 ? &xjob : nullptr))
       return e;
-  } else if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, shared_rows, ws, stream, slot_rows)) {
+  } else if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, shared_rows, ws, stream, slot_rows, e4m3 ? &xjob : nullptr)) {
     return e;
   }
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
@@ -723,16 +701,15 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
     return launch_status();
   }
   const Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
-  if (e4m3) {  // x and h go through the activation rounding: x_q -> fc1 -> h (BF16) -> h_q -> fc2
-    launch_quant_groups(x, m, ex->hidden, ws.xq, ws.xs, stream);
+  if (e4m3) {  // x and h go through the activation rounding: x_q -> fc1 -> h_q -> fc2
     p.aq = ws.xq;
     p.aq_scale = ws.xs;
+    p.oq = ws.hq;
+    p.oq_scale = ws.hs;
     f2.aq = ws.hq;
     f2.aq_scale = ws.hs;
   }
   if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) return e;
-  // rows of h past the kept pairs are never written: the quantizer reads them and nobody reads what it makes of them
-  if (e4m3) launch_quant_groups(ws.h, pairs + shared_rows, ex->inter, ws.hq, ws.hs, stream);
   if (int e = launch_stream<EPI_FC2>(f2, slots, est, l2, stream)) return e;
   return launch_status();
 }
@@ -829,4 +806,13 @@ extern "C" int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_e
   if (!aligned(logits, 4)) return HB_EINVAL;
   const Routing route{logits, experts_total, ids, weights};
   return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, &route);
+}
+
+extern "C" int hb_w3_moe_layer_logits_e4m3(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                                           const float* logits, int experts_total, int m, int topk, int32_t* ids, float* weights, void* out,
+                                           void* workspace, size_t workspace_bytes, void* stream) {
+  if (!logits) return HB_ENULL;
+  if (!aligned(logits, 4)) return HB_EINVAL;
+  const Routing route{logits, experts_total, ids, weights};
+  return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, &route, true);
 }

@@ -179,10 +179,11 @@ def moe_layer(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: t
 
 
 def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, topk: int, shared: W3Experts | None = None,
-                     gate_vec: torch.Tensor | None = None, return_routing: bool = False):
+                     gate_vec: torch.Tensor | None = None, return_routing: bool = False, e4m3: bool = False):
     """`moe_layer` from the router's FP32 logits [M, E_total]: softmax top-k routing (ops.route_topk's arithmetic) runs
     in the same chain - inside the planning workgroup up to 16 rows, so that a decode step is four launches -
-    (hibana/model/flashnext/moe.py:122-144,177-192). With `return_routing`, also the ids and weights it used."""
+    (hibana/model/flashnext/moe.py:122-144,177-192). With `return_routing`, also the ids and weights it used.
+    `e4m3`: the experts' activations are rounded to E4M3 as in `moe_layer`."""
     if x.dtype != torch.bfloat16 or x.ndim != 2 or x.shape[1] != experts.shape13[1]:
         raise ValueError("moe_layer_logits: x must be BF16 [M, hidden]")
     if logits.ndim != 2 or logits.shape[0] != x.shape[0] or logits.dtype != torch.float32:
@@ -198,9 +199,10 @@ def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, 
         need = _lib.lib().hb_w3_moe_workspace_bytes(m, topk, C.byref(st), int(shared is not None))
         ws = torch.empty(need, dtype=torch.uint8, device=x.device)
         gv = None if gate_vec is None else gate_vec.float().contiguous()
-        _lib.check(_lib.lib().hb_w3_moe_layer_logits(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(x.contiguous()),
-                                                     _lib.ptr(logits.contiguous()), e_total, m, topk, _lib.ptr(ids), _lib.ptr(wt), _lib.ptr(out),
-                                                     _lib.ptr(ws), need, _lib.stream()), "moe_layer_logits")
+        entry = _lib.lib().hb_w3_moe_layer_logits_e4m3 if e4m3 else _lib.lib().hb_w3_moe_layer_logits
+        _lib.check(entry(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(x.contiguous()),
+                         _lib.ptr(logits.contiguous()), e_total, m, topk, _lib.ptr(ids), _lib.ptr(wt), _lib.ptr(out),
+                         _lib.ptr(ws), need, _lib.stream()), "moe_layer_logits")
     return (out, ids, wt) if return_routing else out
 
 

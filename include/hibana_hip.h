@@ -154,8 +154,9 @@ int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, co
                     size_t workspace_bytes, void* stream);
 
 /* hb_w3_moe_layer in the reference kernel's own arithmetic: x and h of the routed experts and of the shared expert go
- * through the activation rounding (hb_w3_quant_groups) before their products, as with HB_MOE_E4M3 in hb_w3_moe; the
- * combine is the same.
+ * through the activation rounding (hb_w3_quant_groups' arithmetic) before their products, as with HB_MOE_E4M3 in
+ * hb_w3_moe; the combine is the same. No launch of its own for either rounding: x is rounded by further workgroups of
+ * the planning launch, h in fc1's epilogue.
  * ref: as hb_w3_moe_layer, with w3_moe.reference's `quant`, hibana/kernels/w3_moe.py:187-214. */
 int hb_w3_moe_layer_e4m3(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
                          const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
@@ -168,6 +169,13 @@ int hb_w3_moe_layer_e4m3(const hb_w3_experts* routed, const hb_w3_experts* share
 int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec,
                            const void* x, const float* logits, int experts_total, int m, int topk, int32_t* ids,
                            float* weights, void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* hb_w3_moe_layer_logits with the activation rounding of hb_w3_moe_layer_e4m3 (the routing itself reads the FP32
+ * logits and is the same).
+ * ref: as hb_w3_moe_layer_logits, with w3_moe.reference's `quant`, hibana/kernels/w3_moe.py:187-214. */
+int hb_w3_moe_layer_logits_e4m3(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec,
+                                const void* x, const float* logits, int experts_total, int m, int topk, int32_t* ids,
+                                float* weights, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* out = bf16( bf16(sum over the row's local slots of w * pairs) + g * shared ) from unsummed pair outputs (FP32 or,
  * pairs_bf16 != 0, BF16) [m * topk, h]; shared BF16 [m, h] or NULL; gate_vec float32 [h] or NULL (then g = 1; x

@@ -127,3 +127,48 @@ def test_layer_with_shared_expert_on_rounded_activations(m, with_gate):
     assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
     assert torch.equal(run(e4m3=True), got)
     assert not torch.equal(run(), got)  # the weight-only layer is another function
+
+
+@pytest.mark.parametrize("gated", [True, False])
+def test_fc1_rounds_h_in_its_epilogue_under_every_split(gated):
+    """h leaves fc1 as E4M3 codes: both bodies of the stream (expert 1 has twelve rows, the others at most four), K
+    unsplit and split two to eight ways, one to four blocks a workgroup."""
+    from hibana_amd import _lib
+    from hibana_amd.kernels import w3_moe
+    e, hidden, inter, m, topk = 4, 1024, 256, 12, 2
+    ex, per = random_experts(e, hidden, inter, gated, 61)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(m, hidden, generator=g).bfloat16()
+    x[:, ::53] *= 25
+    ids = torch.stack([1 + torch.randperm(e - 1, generator=g)[:topk] for _ in range(m)]).to(torch.int32)
+    ids[:, 0] = 1
+    ids[:, 1] = torch.tensor([0, 2, 3] * 4)
+    wt = torch.rand(m, topk, generator=g) + 0.1
+    want = layers.routed_experts_ref(x, ids.numpy(), oracle_expert_getter(per, gated, inter), gated, 0, e, quant=layers.rounded_e4m3)
+    try:
+        for ks, nbw in ((1, 1), (1, 4), (2, 2), (3, 1), (4, 1), (5, 2), (8, 1), (0, 0)):
+            assert _lib.lib().hb_tune(b"moe_fc1_ksplit", ks) == 0 and _lib.lib().hb_tune(b"moe_fc1_nbw", nbw) == 0
+            got = w3_moe.w3_moe(ex, x.cuda(), ids.cuda(), wt.cuda(), pairs=True, e4m3=True)
+            mx, nr = errors(got, want)
+            assert mx < MAX_REL and nr < NORM_REL, (ks, nbw, mx, nr)
+    finally:
+        _lib.lib().hb_tune(b"moe_fc1_ksplit", 0)
+        _lib.lib().hb_tune(b"moe_fc1_nbw", 0)
+
+
+@pytest.mark.parametrize("m", [3, 16, 24])  # up to 16 rows the planning workgroup routes them itself
+def test_layer_from_logits_on_rounded_activations(m):
+    """Routing from the FP32 logits is the weight-only layer's; the experts then see rounded activations: the same
+    output as the E4M3 layer called with the ids and weights the routing chose."""
+    from hibana_amd.kernels import w3_moe
+    e, hidden, inter, topk = 8, 256, 128, 3
+    ex, _ = random_experts(e, hidden, inter, True, 41)
+    shared_ex, _ = random_experts(1, hidden, inter, True, 42)
+    g = torch.Generator().manual_seed(90 + m)
+    x = torch.randn(m, hidden, generator=g).bfloat16().cuda()
+    logits = torch.randn(m, e, generator=g).cuda()
+    gate = (torch.randn(hidden, generator=g) * 0.05).cuda()
+    got, ids, wt = w3_moe.moe_layer_logits(ex, x, logits, topk, shared=shared_ex, gate_vec=gate, return_routing=True, e4m3=True)
+    _, ids_plain, wt_plain = w3_moe.moe_layer_logits(ex, x, logits, topk, shared=shared_ex, gate_vec=gate, return_routing=True)
+    assert torch.equal(ids, ids_plain) and torch.equal(wt, wt_plain)
+    assert torch.equal(got, w3_moe.moe_layer(ex, x, ids, wt, shared=shared_ex, gate_vec=gate, e4m3=True))
