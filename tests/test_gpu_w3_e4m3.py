@@ -172,3 +172,22 @@ def test_layer_from_logits_on_rounded_activations(m):
     _, ids_plain, wt_plain = w3_moe.moe_layer_logits(ex, x, logits, topk, shared=shared_ex, gate_vec=gate, return_routing=True)
     assert torch.equal(ids, ids_plain) and torch.equal(wt, wt_plain)
     assert torch.equal(got, w3_moe.moe_layer(ex, x, ids, wt, shared=shared_ex, gate_vec=gate, e4m3=True))
+
+
+def test_many_pairs_on_rounded_activations_agree_with_the_call_in_halves():
+    """From 8192 pairs the plan is shared among workgroups and the rounding of x is a launch of its own: the same rows
+    as two calls of half the tokens, whose plans are one workgroup with the rounding beside it (the slots group the rows
+    differently, so sums may differ in their last bits)."""
+    from hibana_amd.kernels import w3_moe
+    e, hidden, inter, m, topk = 8, 256, 128, 2048, 4
+    ex, _ = random_experts(e, hidden, inter, True, 71)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(m, hidden, generator=g).bfloat16().cuda()
+    ids = torch.stack([torch.randperm(e, generator=g)[:topk] for _ in range(m)]).to(torch.int32).cuda()
+    wt = (torch.rand(m, topk, generator=g) + 0.1).cuda()
+    whole = w3_moe.w3_moe(ex, x, ids, wt, e4m3=True)
+    half = m // 2
+    halves = torch.cat([w3_moe.w3_moe(ex, x[:half], ids[:half], wt[:half], e4m3=True), w3_moe.w3_moe(ex, x[half:], ids[half:], wt[half:], e4m3=True)])
+    mx, nr = errors(whole, halves.cpu())
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    assert torch.equal(whole, w3_moe.w3_moe(ex, x, ids, wt, e4m3=True))
