@@ -250,6 +250,8 @@ def main() -> int:
                     help="3: the headline w3 verify-batch layer; 2: the same layer at M = 1 with N(0,1) logits; 0 / 1: the w3 / NVFP4 dense decode "
                          "projection; 4: the NVFP4 prefill layer")
     ap.add_argument("--rows", type=int, default=1, help="configs 0 and 1: activation rows M")
+    ap.add_argument("--e4m3", action="store_true", help="configs 2 and 3: the reference kernel's own arithmetic (activations rounded to E4M3 per "
+                    "32-group, FP8 MFMA) instead of the weight-only form; no CPU leg")
     ap.add_argument("--copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (a known-size "
                     "reference for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
@@ -268,6 +270,8 @@ def main() -> int:
         return latent_prefill(args)
     if args.config in (0, 1):
         return dense_decode(args)
+    if args.e4m3:
+        args.no_cpu = True  # the C oracle states the weight-only form
     decode = args.config == 2  # the layer at batch 1: logits from N(0, 1), ten experts and the shared one a step
     m = 1 if decode else M
     dev = torch.device("cuda:0")
@@ -285,7 +289,7 @@ def main() -> int:
     torch.cuda.synchronize()
 
     def step(i: int):
-        return w3_moe.moe_layer_logits(layers[i % args.layers][0], x, logits[i % args.layers], TOPK, shared=layers[i % args.layers][1])
+        return w3_moe.moe_layer_logits(layers[i % args.layers][0], x, logits[i % args.layers], TOPK, shared=layers[i % args.layers][1], e4m3=args.e4m3)
 
     distinct = [int(torch.unique(ops.route_topk(lg, TOPK)[0]).numel()) for lg in logits]
     for i in range(max(args.warmup, args.layers)):  # untimed: also builds every layer's tiled weights and warms the allocator
@@ -342,20 +346,21 @@ def main() -> int:
         check = {"max_rel_vs_cpu_oracle": float((got - want.float()).abs().max() / want.float().abs().max()),
                  "norm_rel_vs_cpu_oracle": float((got - want.float()).norm() / want.float().norm())}
     line = {
-        "metric": "w3 MoE layer tokens/s at decode (M=1), with achieved HBM GB/s" if decode else "w3 MoE layer tokens/s at the verify batch (M=32), with achieved HBM GB/s",
+        "metric": ("w3 MoE layer tokens/s at decode (M=1), with achieved HBM GB/s" if decode else
+                   "w3 MoE layer tokens/s at the verify batch (M=32), with achieved HBM GB/s") + (" [E4M3 activation mode]" if args.e4m3 else ""),
         "value": m * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8" if args.e4m3 else "bf16",
         "data": "synthetic",
         "config": {"workload": ("BASELINE config 2: w3 MoE layer, 1 token, hidden 2048, 512 experts x inter 512 + 1 shared, top-10 of N(0,1) logits, "
                                 "SiLU-gated, codebook lloyd") if decode else
                                ("BASELINE config 3: w3 MoE layer, 32 tokens (4 seq x 8 draft), hidden 2048, 512 experts x inter 512 + 1 shared, "
                                 "top-10 Zipf(1.1) routing, SiLU-gated, codebook lloyd"),
                    "layers_cycled": args.layers, "distinct_experts_per_step": mean(distinct), "timed_as": "one HIP-graph replay of all steps"},
-        "roofline": {"bound": "hbm", "kernel": "w3_stream_kernel<fc1 gated>", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "roofline": {"bound": "hbm", "kernel": "w3_stream_kernel<fc1 gated, E4M3>" if args.e4m3 else "w3_stream_kernel<fc1 gated>", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      # HBM bytes a launch: the ratio of scaled FETCH_SIZE + WRITE_SIZE to the algorithmic bytes measured with
                      # rocprofv3 --pmc on this workload (summary kept under profiles/), applied to this run's bytes
-                     "traffic": None if decode else FC1_TRAFFIC_RATIO * fc1_launch_bytes, "launch_bytes": fc1_launch_bytes, "launch_ms": fc1_ms},
+                     "traffic": None if decode or args.e4m3 else FC1_TRAFFIC_RATIO * fc1_launch_bytes, "launch_bytes": fc1_launch_bytes, "launch_ms": fc1_ms},
         "layer_chain": {"algorithmic_bytes_per_step": step_bytes, "achieved_GBs": chain_gbs, "frac_of_hbm_peak": chain_gbs / HBM_PEAK_GBS,
                         "kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
         "cpu_baseline": cpu,
