@@ -22,21 +22,27 @@ namespace hb {
 
 constexpr int TILE_ROWS = 128;
 constexpr int TILE_MT = TILE_ROWS / 16;
-constexpr int TILE_BUF = TILE_ROWS * 256;  // bytes of one activation buffer
+// A 16-row tile of an activation buffer is 4 KB and 16 bytes of padding: with the tiles a multiple of 512 bytes apart
+// the compiler pairs the 8-byte reads of neighbouring tiles into one instruction and then moves registers to put a
+// fragment's two halves side by side (a quarter of the loop's VALU instructions); off that grid every half is its own
+// read, straight into its place.
+constexpr int TILE_PITCH = 16 * 256 + 16;
+constexpr int TILE_BUF = TILE_MT * TILE_PITCH;  // bytes of one activation buffer
 constexpr int TILE_DENSE_ROWS = 24;        // average rows an expert from which the tile kernel serves a routed call
 typedef __attribute__((ext_vector_type(2))) uint32_t tile_u32x2_t;
 
-__device__ __forceinline__ void stage_tile(const StreamParams& p, const int32_t* rowtab, uint8_t* buf, int chunk, int tiles, int wave, int lane) {
-  // a wavefront brings rows wave * 32 .. + 31 in eight instructions of four rows each: lane l lands at byte 16 l of the
-  // instruction's kilobyte, i.e. row (l >> 4), slot (l & 15) of it, and therefore fetches piece slot ^ (row & 15)
-  const int sub = lane >> 4, slot = lane & 15;
+// Brings chunk `chunk` of the slot's activation tile into `buf`: a wavefront takes rows wave * 32 .. + 31 in eight
+// instructions of four rows each; lane l lands at byte 16 l of the instruction's kilobyte, i.e. row (l >> 4), slot
+// (l & 15) of it, and therefore fetches piece slot ^ (row & 15) of its row. `piece[j]`: that piece's byte offset from
+// the activation matrix's start for chunk 0 (32 bits: the launch refuses matrices of 4 GiB and more); the chunk moves
+// the scalar base, so a chunk's staging is eight loads and no arithmetic.
+__device__ __forceinline__ void stage_tile(const StreamParams& p, const uint32_t (&piece)[8], uint8_t* buf, int chunk, int tiles, int wave) {
+  const uint8_t* base = reinterpret_cast<const uint8_t*>(p.a) + (int64_t)chunk * 256;
 #pragma unroll
   for (int j = 0; j < 8; j++) {
-    const int row = wave * 32 + j * 4 + sub;
     if (wave * 32 + j * 4 < tiles * 16) {  // wave-uniform: whole 16-row tiles past the slot's rows are never read
-      const uint16_t* src = p.a + (int64_t)rowtab[row] * p.a_stride + (int64_t)chunk * 128 + ((slot ^ (row & 15)) << 3);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src),
-                                       (__attribute__((address_space(3))) void*)(buf + (wave * 32 + j * 4) * 256), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + piece[j]),
+                                       (__attribute__((address_space(3))) void*)(buf + (wave * 2 + (j >> 2)) * TILE_PITCH + (j & 3) * 1024), 16, 0, 0);
     }
   }
 }
@@ -47,7 +53,7 @@ template <class Fmt, int EPI, int ST>
 __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl, uint8_t* tile_lds) {
   constexpr bool FULL = ST > 0;
   constexpr int MT = FULL ? ST : TILE_MT;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: kept in scalars
   const int q = lane >> 4, r16 = lane & 15;
   const int nb = blockIdx.x * 4 + wave;
   const bool active = nb < p.n_blocks;
@@ -62,6 +68,12 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
     rowtab[threadIdx.x] = (int)arow;
   }
   __syncthreads();
+  uint32_t piece[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const int row = wave * 32 + j * 4 + (lane >> 4);
+    piece[j] = (uint32_t)rowtab[row] * (uint32_t)(p.a_stride * 2) + (uint32_t)((((lane & 15) ^ (row & 15))) << 4);
+  }
   f32x4_t acc[MT][4];
 #pragma unroll
   for (int t = 0; t < MT; t++)
@@ -70,14 +82,14 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
   const uint8_t* blk = sl.w + (int64_t)(active ? nb : 0) * p.chunks * Fmt::BLOCK_BYTES;
   typename Fmt::Chunk cur, nxt;
   Fmt::load(cur, blk, lane, r16);
-  stage_tile(p, rowtab, tile_lds, 0, tiles, wave, lane);
+  stage_tile(p, piece, tile_lds, 0, tiles, wave);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   for (int c = 0; c < p.chunks; c++) {
     uint8_t* buf = tile_lds + (c & 1) * TILE_BUF;
     if (c + 1 < p.chunks) {
       Fmt::load(nxt, blk + (int64_t)(c + 1) * Fmt::BLOCK_BYTES, lane, r16);
-      stage_tile(p, rowtab, tile_lds + ((c + 1) & 1) * TILE_BUF, c + 1, tiles, wave, lane);
+      stage_tile(p, piece, tile_lds + ((c + 1) & 1) * TILE_BUF, c + 1, tiles, wave);
     }
 #pragma unroll
     for (int s = 0; s < 4; s++) {  // 32-k steps of the chunk
@@ -91,7 +103,7 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
 #pragma unroll
       for (int t = 0; t < MT; t++) {
         if (FULL || t < tiles) {
-          const uint8_t* row = buf + (16 * t + r16) * 256;
+          const uint8_t* row = buf + t * TILE_PITCH + r16 * 256;
           u32x4_t a;
           if (Fmt::SPLIT_A) {
             const tile_u32x2_t lo = *reinterpret_cast<const tile_u32x2_t*>(row + half + slot_lo);
@@ -173,9 +185,15 @@ inline bool tile_serves_dense(int m, int n_blocks) {
   return m > 2 * ROWS_PER_SLOT && (int64_t)n_blocks * 64 * m > 2300000 * rounds;
 }
 
-// `slots`: the grid's second dimension (routed: the plan's upper bound; dense: ceil(m / TILE_ROWS)).
+// Whether an activation matrix of `rows` rows is one the tile kernel takes: it addresses the matrix with 32-bit byte
+// offsets.
+inline bool tile_takes(int64_t rows, int64_t a_stride) { return rows * a_stride * 2 <= 0xffffffffll; }
+
+// `slots`: the grid's second dimension (routed: the plan's upper bound; dense: ceil(m / TILE_ROWS)); `a_rows`: rows of
+// the activation matrix.
 template <class Fmt, int EPI>
-static int launch_tile(StreamParams& p, int64_t slots, hipStream_t stream) {
+static int launch_tile(StreamParams& p, int64_t slots, int64_t a_rows, hipStream_t stream) {
+  if (!tile_takes(a_rows, p.a_stride)) return HB_EINVAL;
   p.slot_rows = TILE_ROWS;
   const dim3 grid((unsigned)((p.n_blocks + 3) / 4), (unsigned)slots);
   HB_LAUNCH((tile_kernel<Fmt, EPI>), grid, dim3(256), 2 * TILE_BUF + TILE_ROWS * sizeof(int32_t), stream, p);

@@ -567,7 +567,7 @@ extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* 
   p.out = y;
   p.out_stride = n;
   if (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && tile_serves_dense(m, p.n_blocks))) {
-    if (int e = launch_tile<TileW3, EPI_DENSE>(p, (m + TILE_ROWS - 1) / TILE_ROWS, as_stream(stream))) return e;
+    if (int e = launch_tile<TileW3, EPI_DENSE>(p, (m + TILE_ROWS - 1) / TILE_ROWS, m, as_stream(stream))) return e;
     return launch_status();
   }
   const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
@@ -637,7 +637,8 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   const int shared_rows = shared ? m : 0;
   // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel
   // (E4M3 activations: the stream only)
-  const bool dense = !e4m3 && (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && pairs >= (int64_t)ex->experts * 2 * TILE_DENSE_ROWS));  // the pre-scaled expansion costs more here than the stream's
+  const bool dense = !e4m3 && tile_takes(m, ex->hidden) && tile_takes(pairs + shared_rows, ex->inter) &&
+                     (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && pairs >= (int64_t)ex->experts * 2 * TILE_DENSE_ROWS));  // the pre-scaled expansion costs more here than the stream's
   const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
   const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows, slot_rows);
   if (slots > 65535) return HB_EINVAL;
@@ -696,8 +697,8 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   f2.out_stride = ex->hidden_out;
   f2.out_bf16 = pairs_bf16;
   if (dense) {
-    if (int e = ex->gated ? launch_tile<TileW3, EPI_FC1_GATED>(p, slots, stream) : launch_tile<TileW3, EPI_FC1_RELU2>(p, slots, stream)) return e;
-    if (int e = launch_tile<TileW3, EPI_FC2>(f2, slots, stream)) return e;
+    if (int e = ex->gated ? launch_tile<TileW3, EPI_FC1_GATED>(p, slots, m, stream) : launch_tile<TileW3, EPI_FC1_RELU2>(p, slots, m, stream)) return e;
+    if (int e = launch_tile<TileW3, EPI_FC2>(f2, slots, pairs + shared_rows, stream)) return e;
     return launch_status();
   }
   const Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
