@@ -299,7 +299,7 @@ def main() -> int:
     # live kernel timing: each kernel of the chain is launched with its own (start, stop) HIP event pair, which the
     # runtime stamps with that kernel's begin and end on the stream it runs on
     hip = Hip()
-    names = ["route + plan", "fc1", "fc2", "combine"] if decode else ["route", "plan", "fc1", "fc2", "combine"]  # up to 16 rows are routed by the plan's workgroup
+    names = (["route + plan", "fc1", "fc2 + combine"] if decode else ["route", "plan", "fc1", "fc2", "combine"])  # up to 4 rows are routed by the plan's workgroup; one token's fc2 and combine are one launch
     per_kernel = {n: [] for n in names}
     reps = 5
     for rep in range(reps):

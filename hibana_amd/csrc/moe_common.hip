@@ -161,7 +161,10 @@ constexpr int PLAN_WAVES = PLAN_THREADS / 64;
 constexpr int PLAN_BATCH = 8;  // tiles of 64 pairs whose ids a wavefront requests at once
 constexpr int PLAN_WIDE_PAIRS = 8192;   // from this many pairs the plan is shared among workgroups (three launches)
 constexpr int PLAN_WIDE_GROUPS = 64;
-constexpr int ROUTE_FUSED_ROWS = 16;  // up to this many rows the plan workgroup routes them itself (one a wavefront)
+// Up to this many rows the plan workgroup routes them itself (one a wavefront): a row's selection is some 700 dependent
+// VALU instructions, so on ONE compute unit more than four rows take longer than a launch of their own over the device
+// (measured, whole layer: 22.1 against 22.5 us at one row, even at four, 50.7 against 46.8 us at sixteen).
+constexpr int ROUTE_FUSED_ROWS = 4;
 
 struct Scan3 {
   int a, b, c;
@@ -472,14 +475,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
   const int r = blockIdx.x;
   float g = 1.0f;
   if (p.gate_vec && p.shared) {
-    float dot = 0.f;
-    for (int i = threadIdx.x; i < p.hx; i += 256) dot += bf16_bits_to_f32(p.x[(int64_t)r * p.hx + i]) * p.gate_vec[i];
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) dot += __shfl_xor(dot, d);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = dot;
+    combine_gate_partial(p.x, p.gate_vec, p.hx, r, threadIdx.x, red);
     __syncthreads();
-    dot = (red[0] + red[1]) + (red[2] + red[3]);
-    g = 1.0f / (1.0f + expf(-dot));
+    g = combine_gate_value(red);
   }
   const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
   if (c >= p.h) return;
@@ -518,15 +516,15 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
     float s0, s1;
     if (p.shared_f32) {
       const float2 two = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.shared) + at);
-      s0 = round_bf16(two.x);
-      s1 = round_bf16(two.y);
+      s0 = two.x;
+      s1 = two.y;
     } else {
       const uint32_t two = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.shared) + at);
       s0 = __uint_as_float(two << 16);
       s1 = __uint_as_float(two & 0xffff0000u);
     }
-    v0 = round_bf16(v0) + g * s0;
-    v1 = round_bf16(v1) + g * s1;
+    v0 = combine_shared(v0, g, s0);
+    v1 = combine_shared(v1, g, s1);
   }
   *reinterpret_cast<uint32_t*>(p.out + (int64_t)r * p.h + c) = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
 }

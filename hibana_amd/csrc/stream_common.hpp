@@ -402,6 +402,23 @@ struct CombineParams {
 };
 void moe_launch_combine(const CombineParams& c, hipStream_t stream);
 
+// The pieces of the combine that every kernel doing it shares, so that each gives the other's bits.
+// g = sigmoid(x[r] . gate_vec): 256 threads (t = 0 .. 255, four whole wavefronts) each add their share and leave four
+// partial sums in `red` (LDS); after a barrier any thread reads g from them.
+__device__ __forceinline__ void combine_gate_partial(const uint16_t* x, const float* gate_vec, int hx, int64_t r, int t, float* red) {
+  float dot = 0.f;
+  for (int i = t; i < hx; i += 256) dot += bf16_bits_to_f32(x[r * hx + i]) * gate_vec[i];
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) dot += __shfl_xor(dot, d);
+  if ((t & 63) == 0) red[t >> 6] = dot;
+}
+__device__ __forceinline__ float combine_gate_value(const float* red) {
+  const float dot = (red[0] + red[1]) + (red[2] + red[3]);
+  return 1.0f / (1.0f + expf(-dot));
+}
+// routed: the FP32 chain over the row's slots; shared: the shared expert's FP32 (or BF16) output
+__device__ __forceinline__ float combine_shared(float routed, float g, float shared) { return round_bf16(routed) + g * round_bf16(shared); }
+
 // Measurement hook: the caller's next (start, stop) event pair, if any is armed. A kernel launched through HB_LAUNCH
 // then carries the pair: the runtime stamps the two events with that kernel's own begin and end.
 bool moe_next_events(hipEvent_t* start, hipEvent_t* stop);

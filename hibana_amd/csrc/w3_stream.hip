@@ -18,6 +18,8 @@
 // one), and hb_tune("w3_tile", 1 | 2) forces one or the other.
 #include <string.h>
 
+#include <algorithm>
+
 #include "ring.hpp"
 #include "stream_common.hpp"
 #include "tile_kernel.hpp"
@@ -136,6 +138,25 @@ constexpr int RING_BYTES = ring_bytes<W3Ring>();  // LDS per wavefront; its firs
 // of activations per lane and chunk instead of sixty-four. The four groups are added once, after the last chunk, in the
 // exchange through LDS that the K splits are added in.
 constexpr int FEW_ROWS = 4;
+
+// fc2 stores by pair index, which it reads from the sorted list: asked for ahead of the weights, so that the epilogue
+// does not wait on memory once more.
+struct FewPairs {
+  int pair[FEW_ROWS];
+  __device__ __forceinline__ void ask(const StreamParams& p, const Slot& sl, int row0) {
+#pragma unroll
+    for (int r = 0; r < FEW_ROWS; r++) pair[r] = p.order[sl.p0 + min(row0 + r, sl.rows - 1)];
+  }
+  __device__ __forceinline__ int of(int r) const { return r == 0 ? pair[0] : r == 1 ? pair[1] : r == 2 ? pair[2] : pair[3]; }
+};
+
+__device__ __forceinline__ void store_pair(const StreamParams& p, int64_t pair, int n, float y) {
+  if (p.out_bf16) {
+    reinterpret_cast<uint16_t*>(p.out)[pair * p.out_stride + n] = bf16_of(y);
+  } else {
+    reinterpret_cast<float*>(p.out)[pair * p.out_stride + n] = y;
+  }
+}
 
 __device__ __forceinline__ void compute_tile_few(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const Rows& ch, f32x4_t& acc,
                                                  uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
@@ -366,7 +387,7 @@ struct FullActs8 {
 template <int EPI, bool QUANT = false>
 __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl, int row0, float scale, int nb, bool active, int wave, int ks,
                                            int nbi, float* partial, const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2,
-                                           const f32x4_t& acc3) {
+                                           const f32x4_t& acc3, const FewPairs& pairs = FewPairs{}) {
   constexpr int STRIDE = RING_BYTES / 4;
   const int lane = threadIdx.x & 63, q = lane >> 4, r16 = lane & 15;
   float* mine = partial + wave * STRIDE;
@@ -410,6 +431,8 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
       float amax = row16_max(fabsf(h));
       amax = fmaxf(amax, __shfl_xor(amax, 16));
       store_quantized(p, sl.p0 + row0 + r, nb * 64 + 16 * q + r16, h, amax, (lane & 31) == 0);
+    } else if (EPI == EPI_FC2) {
+      store_pair(p, pairs.of(r), nb * 64 + lane, y);  // lane (q, r16) is column 16 q + r16 of the block
     } else {
       store_out<EPI>(p, sl, nb, q, row0 + r, r16, y, 0.f);
     }
@@ -434,11 +457,13 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   if (A8) {
     if (sl.rows <= FEW_ROWS) {  // uniform over the workgroup
       float scale = 0.f;
+      FewPairs pairs{};
       if (active) {
         scale = sl.rs[nb * 64 + lane];
+        if (EPI == EPI_FC2) pairs.ask(p, sl, 0);
         stream_block<EPI, FewActs8, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
       }
-      finish_few<EPI, QUANT>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+      finish_few<EPI, QUANT>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs);
     } else {
       RowScales rs{};
       if (active) {
@@ -449,11 +474,13 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
     }
   } else if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
     float scale = 0.f;
+    FewPairs pairs{};
     if (active) {
       scale = sl.rs[nb * 64 + lane];  // row 16 q + r16 of the block: asked for ahead of the chunks, there when the epilogue wants it
+      if (EPI == EPI_FC2) pairs.ask(p, sl, 0);
       stream_block<EPI, FewActs, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);  // at least one chunk: ks <= chunks
     }
-    finish_few<EPI>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+    finish_few<EPI>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs);
   } else {
     RowScales rs{};
     if (active) {
@@ -462,6 +489,76 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
     }
     finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
   }
+}
+
+// One token (a decode step): fc2 and the combine in one launch. A workgroup owns a 64-row block of the output; each of
+// its first `slots` wavefronts takes one slot of the plan (an expert the token chose, or the shared expert) through all
+// of K on the four-row body, adds its groups as finish_few does without a K split, and leaves the slot's 64 outputs in
+// LDS under the pair's selection index; with a gate, four more wavefronts meanwhile make its dot product. The first
+// wavefront then runs the combine's chain, a column a lane. Every sum is the one the two separate launches make (fc2
+// with one K split, then moe_combine_kernel), so the bits are theirs; what goes away is the round trip of the pair
+// outputs through memory and a launch.
+constexpr int ONE_GATE_WAVES = 4;  // the gate's dot product is laid out over 256 threads
+constexpr int ONE_MAX_WAVES = 16;
+
+__global__ __launch_bounds__(1024) void w3_fc2_combine_one_kernel(StreamParams p, CombineParams c, int slots) {
+  extern __shared__ __align__(16) uint8_t rings[];  // a ring a streaming wavefront, then ys [topk + 1][64], then the gate's four partial sums
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nb = blockIdx.x, q = lane >> 4, r16 = lane & 15;
+  float* ys = reinterpret_cast<float*>(rings + slots * RING_BYTES);
+  float* red = ys + (p.topk + 1) * 64;
+  // the chain's operands, a selection a lane, asked for now; a pair whose expert is not local has no slot: its place
+  // in ys is never written and never read
+  float w_mine = 0.f;
+  bool keep_mine = false;
+  if (wave == 0 && lane < p.topk) {
+    const int e = c.ids[lane] - c.e_lo;
+    keep_mine = e >= 0 && e < c.e_n;
+    w_mine = c.weights[lane];
+  }
+  if (wave >= slots) {  // only with a gate
+    combine_gate_partial(c.x, c.gate_vec, c.hx, 0, (int)threadIdx.x - 64 * slots, red);
+  } else {
+    const Slot sl = slot_of<EPI_FC2>(p, wave);
+    if (sl.rows > 0) {  // uniform over the wavefront
+      const float scale = sl.rs[nb * 64 + lane];
+      float* mine = reinterpret_cast<float*>(rings + wave * RING_BYTES);
+      for (int row0 = 0; row0 < sl.rows; row0 += FEW_ROWS) {  // more than one row: the caller named an expert twice
+        f32x4_t acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        FewPairs pairs;
+        pairs.ask(p, sl, row0);
+        stream_block<EPI_FC2, FewActs, W3Ring>(p, sl, row0, nb, 0, p.chunks, lane, reinterpret_cast<uint8_t*>(mine), acc[0], acc[1], acc[2], acc[3]);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          mine[(t * 4 + 0) * 64 + lane] = acc[t].x;
+          mine[(t * 4 + 1) * 64 + lane] = acc[t].y;
+          mine[(t * 4 + 2) * 64 + lane] = acc[t].z;
+          mine[(t * 4 + 3) * 64 + lane] = acc[t].w;
+        }
+        __builtin_amdgcn_wave_barrier();  // the lanes of one wavefront: its LDS operations execute in program order
+        const int rows = min(FEW_ROWS, sl.rows - row0);
+        for (int r = 0; r < rows; r++) {
+          const float* at = mine + (q * 4 + r) * 64 + r16;
+          float v = 0.f;
+          v += (at[0] + at[16]) + (at[32] + at[48]);
+          ys[min(pairs.of(r), p.topk) * 64 + lane] = v * scale;  // lane (q, r16) is column 16 q + r16 of the block; the shared expert's row follows the pairs
+        }
+        __builtin_amdgcn_wave_barrier();  // read before the next pass's blocks land in the ring
+      }
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float v = 0.f;
+  for (int s = 0; s < p.topk; s++) {
+    const bool keep = __builtin_amdgcn_readlane((int)keep_mine, s) != 0;
+    const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w_mine), s));
+    v = fmaf(keep ? w : 0.f, keep ? ys[s * 64 + lane] : 0.f, v);
+  }
+  if (c.shared) v = combine_shared(v, c.gate_vec ? combine_gate_value(red) : 1.0f, ys[p.topk * 64 + lane]);
+  c.out[nb * 64 + lane] = f32_to_bf16_bits(v);
 }
 
 // ------------------------------------------------------------------------------------ the prefill kernel's W3 format
@@ -498,7 +595,7 @@ struct TileW3 {
 
 // ---------------------------------------------------------------------------------------------------- host side
 struct Tuning {
-  int w3_tile = 0, w3_few = 0, w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0;
+  int w3_tile = 0, w3_few = 0, w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0, moe_one = 0;
 };
 static Tuning g_tune;
 
@@ -540,7 +637,7 @@ extern "C" int hb_tune(const char* key, int value) {
     int* slot;
   } table[] = {{"w3_tile", &g_tune.w3_tile}, {"w3_few", &g_tune.w3_few}, {"w3_ksplit", &g_tune.w3_ksplit},           {"w3_nbw", &g_tune.w3_nbw},
                {"moe_fc1_ksplit", &g_tune.moe_fc1_ksplit}, {"moe_fc1_nbw", &g_tune.moe_fc1_nbw},
-               {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}};
+               {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}, {"moe_one", &g_tune.moe_one}};
   for (auto& t : table)
     if (!strcmp(t.name, key)) {
       if (value < 0 || value > 16) return HB_EINVAL;
@@ -621,8 +718,8 @@ int check_experts(const hb_w3_experts* ex) {
   return HB_OK;
 }
 
-// plan -> fc1 -> fc2 (-> combine): `out_pairs` receives fc2's per-pair outputs (the workspace's y unless the caller
-// wants the pairs themselves).
+// plan -> fc1 -> fc2 (-> combine, when `combine` is given): `out_pairs` receives fc2's per-pair outputs (the
+// workspace's y unless the caller wants the pairs themselves). One token's fc2 and combine are one launch.
 struct Routing {  // set: the chain routes `logits` [m, e] itself into the caller's ids / weights
   const float* logits;
   int e;
@@ -632,7 +729,7 @@ struct Routing {  // set: the chain routes `logits` [m, e] itself into the calle
 
 int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void* x, const int32_t* ids, int m, int topk,
                 const MoeWorkspace& ws, void* out_pairs, int pairs_bf16, hipStream_t stream, const Routing* route = nullptr,
-                bool e4m3 = false) {
+                bool e4m3 = false, const CombineParams* combine = nullptr) {
   const int64_t pairs = (int64_t)m * topk;
   const int shared_rows = shared ? m : 0;
   // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel
@@ -699,6 +796,7 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   if (dense) {
     if (int e = ex->gated ? launch_tile<TileW3, EPI_FC1_GATED>(p, slots, m, stream) : launch_tile<TileW3, EPI_FC1_RELU2>(p, slots, m, stream)) return e;
     if (int e = launch_tile<TileW3, EPI_FC2>(f2, slots, pairs + shared_rows, stream)) return e;
+    if (combine) moe_launch_combine(*combine, stream);
     return launch_status();
   }
   const Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
@@ -711,7 +809,20 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
     f2.aq_scale = ws.hs;
   }
   if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) return e;
+  int fc2_ks = l2.ks, fc2_nbw;
+  if (!fc2_ks) pick_shape(f2.n_blocks, f2.chunks, est, 8192, &fc2_ks, &fc2_nbw);
+  // one token, and a separate fc2 would not split K either: the fused launch makes the same sums
+  const int one_waves = (int)slots + (combine && combine->gate_vec && combine->shared ? ONE_GATE_WAVES : 0);
+  if (combine && m == 1 && !e4m3 && one_waves <= ONE_MAX_WAVES && fc2_ks == 1 && g_tune.moe_one != 2) {
+    f2.ks = 1;
+    f2.nbw = 1;
+    set_split(f2);
+    HB_LAUNCH(w3_fc2_combine_one_kernel, dim3((unsigned)f2.n_blocks), dim3(64 * one_waves), (size_t)slots * RING_BYTES + (topk + 1) * 256 + 16, stream, f2,
+              *combine, (int)slots);
+    return launch_status();
+  }
   if (int e = launch_stream<EPI_FC2>(f2, slots, est, l2, stream)) return e;
+  if (combine) moe_launch_combine(*combine, stream);
   return launch_status();
 }
 
@@ -733,21 +844,18 @@ extern "C" int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
   void* pairs_out = mode == HB_MOE_SUM ? static_cast<void*>(ws.y) : out;
-  if (int e = run_experts(routed, nullptr, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16, as_stream(stream), nullptr, e4m3)) return e;
-  if (mode == HB_MOE_SUM) {
-    CombineParams c{};
-    c.pairs = ws.y;
-    c.ids = ids;
-    c.weights = weights;
-    c.e_lo = routed->base;
-    c.e_n = routed->experts;
-    c.m = m;
-    c.topk = topk;
-    c.h = routed->hidden_out;
-    c.out = static_cast<uint16_t*>(out);
-    moe_launch_combine(c, as_stream(stream));
-  }
-  return launch_status();
+  CombineParams c{};
+  c.pairs = ws.y;
+  c.ids = ids;
+  c.weights = weights;
+  c.e_lo = routed->base;
+  c.e_n = routed->experts;
+  c.m = m;
+  c.topk = topk;
+  c.h = routed->hidden_out;
+  c.out = static_cast<uint16_t*>(out);
+  return run_experts(routed, nullptr, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16, as_stream(stream), nullptr, e4m3,
+                     mode == HB_MOE_SUM ? &c : nullptr);
 }
 
 static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x, const int32_t* ids,
@@ -765,7 +873,6 @@ static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, c
   if (!aligned(x, 16) || !aligned(ids, 4) || !aligned(weights, 4) || !aligned(out, 4) || !aligned(workspace, 16) || !aligned(gate_vec, 4)) return HB_EINVAL;
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, shared ? 1 : 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
-  if (int e = run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream), route, e4m3)) return e;
   CombineParams c{};
   c.pairs = ws.y;
   c.ids = ids;
@@ -784,8 +891,7 @@ static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, c
   c.topk = topk;
   c.h = routed->hidden_out;
   c.out = static_cast<uint16_t*>(out);
-  moe_launch_combine(c, as_stream(stream));
-  return launch_status();
+  return run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream), route, e4m3, &c);
 }
 
 extern "C" int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,

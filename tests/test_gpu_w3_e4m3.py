@@ -156,7 +156,7 @@ def test_fc1_rounds_h_in_its_epilogue_under_every_split(gated):
         _lib.lib().hb_tune(b"moe_fc1_nbw", 0)
 
 
-@pytest.mark.parametrize("m", [3, 16, 24])  # up to 16 rows the planning workgroup routes them itself
+@pytest.mark.parametrize("m", [3, 4, 5, 16, 24])  # up to four rows the planning workgroup routes them itself
 def test_layer_from_logits_on_rounded_activations(m):
     """Routing from the FP32 logits is the weight-only layer's; the experts then see rounded activations: the same
     output as the E4M3 layer called with the ids and weights the routing chose."""

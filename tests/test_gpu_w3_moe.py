@@ -160,9 +160,9 @@ def test_layer_with_shared_expert(gated, m, with_gate):
     assert torch.equal(w3_moe.moe_layer(ex, x.cuda(), ids.cuda(), weights.cuda()), w3_moe.w3_moe(ex, x.cuda(), ids.cuda(), weights.cuda()))
 
 
-@pytest.mark.parametrize("m", [1, 16, 17, 32, 200])
+@pytest.mark.parametrize("m", [1, 4, 5, 16, 17, 32, 200])
 def test_layer_from_logits_is_route_then_layer(gated, m):
-    """Routing inside the chain (in the planning workgroup up to 16 rows, its own launch beyond) gives the bits of
+    """Routing inside the chain (in the planning workgroup up to four rows, its own launch beyond) gives the bits of
     ops.route_topk followed by moe_layer."""
     from hibana_amd.kernels import ops, w3_moe
     ex, _ = gated
@@ -175,6 +175,72 @@ def test_layer_from_logits_is_route_then_layer(gated, m):
     got, got_ids, got_w = w3_moe.moe_layer_logits(ex, x, logits, TOPK, shared=shared_ex, return_routing=True)
     assert torch.equal(got_ids, ids) and torch.equal(got_w, wts) and torch.equal(got, want)
     assert torch.equal(w3_moe.moe_layer_logits(ex, x, logits, TOPK), w3_moe.moe_layer(ex, x, ids, wts))
+
+
+def _one_token_both_ways(call):
+    """`call()` with one token's fc2 and combine as one launch (the library's choice) and as two."""
+    from hibana_amd import _lib
+    fused = call()
+    assert _lib.lib().hb_tune(b"moe_one", 2) == 0
+    try:
+        apart = call()
+    finally:
+        _lib.lib().hb_tune(b"moe_one", 0)
+    return fused, apart
+
+
+@pytest.mark.parametrize("k", [1, 3, TOPK, 15])
+@pytest.mark.parametrize("shape", ["routed", "shared", "gate"])
+def test_one_token_fc2_and_combine_in_one_launch_give_the_bits_of_two(gated, k, shape):
+    """A decode step (one token) runs fc2 and the combine as one launch: bit for bit what the two launches give, with
+    and without the shared expert and its gate, with ids past the local experts, on an expert-parallel half, and when
+    the caller names an expert twice or five times (slots of more than one row, and of more than the body's four)."""
+    from hibana_amd.kernels import w3_moe
+    ex, get = gated
+    shared_ex, shared_per = random_experts(1, H, I, True, 79)
+    shared_get = oracle_expert_getter(shared_per, True, I)
+    gate = (torch.randn(H, generator=torch.Generator().manual_seed(4)) * 0.05).cuda()
+    kw = {"routed": {}, "shared": {"shared": shared_ex}, "gate": {"shared": shared_ex, "gate_vec": gate}}[shape]
+    x, ids, weights = _inputs(1, k, 900 + k)
+    cases = [ids.clone()]
+    if k > 1:
+        cases.append(ids.clone())
+        cases[-1][0, -1] = w3_moe.EXPERTS  # a pair without an expert
+        cases.append(ids.clone())
+        cases[-1][0, 1] = cases[-1][0, 0]  # an expert named twice
+    if k >= 5:
+        cases.append(ids.clone())
+        cases[-1][0, :5] = 3
+    for case in cases:
+        fused, apart = _one_token_both_ways(lambda: w3_moe.moe_layer(ex, x.cuda(), case.cuda(), weights.cuda(), **kw))
+        assert torch.equal(fused, apart)
+        want = layers.moe_layer_ref(x, case.numpy(), weights, get, True, e_n=E, shared=shared_get(0) if kw else None,
+                                    gate_vec=gate.cpu() if shape == "gate" else None)
+        mx, nr = errors(fused, want)
+        assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    from dataclasses import replace
+    half = E // 2
+    hi = replace(ex, planes13=ex.planes13[half:], scales13=ex.scales13[half:], row13=ex.row13[half:], planes2=ex.planes2[half:],
+                 scales2=ex.scales2[half:], row2=ex.row2[half:], base=half, tiled13=None, tiled2=None)
+    fused, apart = _one_token_both_ways(lambda: w3_moe.w3_moe(hi, x.cuda(), ids.cuda(), weights.cuda()))
+    assert torch.equal(fused, apart)
+
+
+def test_one_token_at_the_decode_geometry_and_relu2(relu2):
+    """The same at the benchmark layer's geometry (fc2 of four chunks, 32 output blocks) and on ReLU^2 experts."""
+    from hibana_amd.kernels import w3_moe
+    ex, _ = random_experts(24, 2048, 512, True, 81)
+    shared_ex, _ = random_experts(1, 2048, 512, True, 82)
+    g = torch.Generator().manual_seed(83)
+    x = torch.randn(1, 2048, generator=g).bfloat16().cuda()
+    logits = torch.randn(1, 24, generator=g).cuda()
+    gate = (torch.randn(2048, generator=g) * 0.02).cuda()
+    fused, apart = _one_token_both_ways(lambda: w3_moe.moe_layer_logits(ex, x, logits, TOPK, shared=shared_ex, gate_vec=gate))
+    assert torch.equal(fused, apart) and fused.float().abs().max() > 0
+    rex, _ = relu2
+    xr, ids, weights = _inputs(1, 6, 84, experts=8)
+    fused, apart = _one_token_both_ways(lambda: w3_moe.w3_moe(rex, xr.cuda(), ids.cuda(), weights.cuda()))
+    assert torch.equal(fused, apart)
 
 
 @pytest.mark.parametrize("m", [1, 16, 150])
