@@ -38,8 +38,8 @@ const char* hb_error_string(int code);
  * "moe_fc1_ksplit" / "moe_fc1_nbw", "moe_fc2_ksplit" / "moe_fc2_nbw", "nvfp4_ksplit" / "nvfp4_nbw": K splits and 64-row
  * blocks per workgroup (their product at most 16); "w3_tile" / "nvfp4_tile": 1 forces the MFMA tile kernel, 2 the weight
  * stream; "w3_few" / "nvfp4_few": 2 switches off the stream's body for slots of few rows (W3: at most four, NVFP4: at
- * most eight). Returns HB_EINVAL for an unknown
- * key or a value out of range. Not thread-safe against concurrent launches. */
+ * most eight); "moe_one": 2 switches off the single launch that does one token's fc2 and combine. Returns HB_EINVAL for
+ * an unknown key or a value out of range. Not thread-safe against concurrent launches. */
 int hb_tune(const char* key, int value);
 
 /* Measurement hook (no counterpart in the reference): `events` are hipEvent_t handles the caller created, taken in
