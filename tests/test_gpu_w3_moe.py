@@ -257,10 +257,11 @@ def test_relu2_experts_with_their_own_fc2_codebook(relu2, m):
     _check(ex, get, x, ids, weights, is_gated=False)
 
 
-def test_graph_replay_gives_the_eager_bits(gated):
+@pytest.mark.parametrize("m", [1, 32])  # one token: fc2 and the combine are one launch
+def test_graph_replay_gives_the_eager_bits(gated, m):
     from hibana_amd.kernels import w3_moe
     ex, _ = gated
-    x, ids, weights = _inputs(32, TOPK, 900)
+    x, ids, weights = _inputs(m, TOPK, 900)
     xd, idd, wd = x.cuda(), ids.cuda(), weights.cuda()
     eager = w3_moe.w3_moe(ex, xd, idd, wd)
     torch.cuda.synchronize()
