@@ -318,15 +318,20 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   const int seg = (((pairs + groups - 1) / groups + PLAN_WAVES - 1) / PLAN_WAVES + 63) / 64 * 64;
   const int lo = min(pairs, (group * PLAN_WAVES + wave) * seg), hi = min(pairs, lo + seg);
   const int batch = seg > 64 ? PLAN_BATCH : 1;  // long segments: the ids of a batch of tiles are requested together
+  const int nseg = WIDE ? PLAN_WAVES : min(PLAN_WAVES, (pairs + seg - 1) / seg);  // segments that hold pairs: the others' counters are neither cleared nor read
   const int e = threadIdx.x;  // one thread an expert: the launch keeps e_n <= PLAN_THREADS
   if (phase != 2) {
-    for (int i = threadIdx.x; i < PLAN_WAVES * e_n; i += PLAN_THREADS) seg_count[i] = 0;
+    for (int i = threadIdx.x; i < nseg * e_n; i += PLAN_THREADS) seg_count[i] = 0;
     __syncthreads();
   }
+  int only = -1;  // seg == 64: the local expert of this lane's one pair, kept for the placement (no second read of the ids)
   for (int i0 = lo + lane; phase != 2 && i0 < hi; i0 += 64 * batch) {
     if (batch == 1) {
       const int e = ids[i0] - e_lo;
-      if (e >= 0 && e < e_n) atomicAdd(&seg_count[wave * e_n + e], 1);
+      if (e >= 0 && e < e_n) {
+        atomicAdd(&seg_count[wave * e_n + e], 1);
+        only = e;
+      }
       continue;
     }
     int e[PLAN_BATCH];
@@ -365,7 +370,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   int of_group[PLAN_WIDE_GROUPS];  // phase 2: the groups' counts of this thread's expert, all asked for at once
   if (e < e_n) {
     if (phase == 0) {
-      for (int wv = 0; wv < PLAN_WAVES; wv++) count += seg_count[wv * e_n + e];
+      for (int wv = 0; wv < nseg; wv++) count += seg_count[wv * e_n + e];
     } else {
 #pragma unroll
       for (int g = 0; g < PLAN_WIDE_GROUPS; g++) of_group[g] = g < groups ? wide[g * e_n + e] : 0;
@@ -392,7 +397,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
     // turn the per-segment (phase 2: per-group) counts into the first position of each segment's (group's) run
     int run = my_start;
     if (phase == 0) {
-      for (int wv = 0; wv < PLAN_WAVES; wv++) {
+      for (int wv = 0; wv < nseg; wv++) {
         const int c = seg_count[wv * e_n + e];
         seg_count[wv * e_n + e] = run;
         run += c;
@@ -436,8 +441,13 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
 #pragma unroll
     for (int j = 0; j < PLAN_BATCH; j++) {
       const int i = i0 + 64 * j + lane;
-      int e = j < batch && i < hi ? ids[i] - e_lo : -1;
-      if (e < 0 || e >= e_n) e = -1;
+      int e;
+      if (seg == 64) {  // uniform: one tile a wavefront, read when it was counted
+        e = j == 0 ? only : -1;
+      } else {
+        e = j < batch && i < hi ? ids[i] - e_lo : -1;
+        if (e < 0 || e >= e_n) e = -1;
+      }
       eb[j] = e;
     }
 #pragma unroll
