@@ -42,7 +42,7 @@ struct RouteParams {
   const float* logits;   // [m, stride]: e logits a row (sigmoid: followed by `latent` FP32 columns)
   int64_t stride;
   const float* bias;     // sigmoid: [e] added to the scores for the choice only
-  const int32_t* slots;  // sigmoid: row r is real iff slots[r / steps] != 0 (null: every row)
+  const int32_t* slots;  // row r is real iff slots[r / steps] != 0 (null: every row)
   int steps, repeat;
   int e, k, per, latent;
   int32_t* ids;
@@ -53,12 +53,11 @@ struct RouteParams {
 template <bool SIGMOID, int PER>
 __device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane) {
   const int e = p.e, per = p.per, first = lane * per;
-  bool padded = false;
   if (SIGMOID) {
     const float* src = p.logits + (int64_t)r * p.stride + e;
     for (int c = lane; c < p.latent; c += 64) p.lat[(int64_t)r * p.latent + c] = __builtin_bit_cast(uint16_t, (__bf16)src[c]);
-    padded = p.slots && p.slots[r / p.steps] == 0;
   }
+  const bool padded = p.slots && p.slots[r / p.steps] == 0;
   const float* row = p.logits + (int64_t)(padded ? 0 : r) * p.stride;  // a padded row repeats row 0's first choice
   float val[PER];   // the weight an expert would get before renormalization
   uint32_t key[PER];
@@ -595,6 +594,51 @@ __global__ __launch_bounds__(256) void quant_groups_kernel(QuantJob job) {
   if (i < job.lanes) quant_groups_lane(job.x, i, job.q, job.scales);
 }
 
+// BF16 [m, k] (k % 8 == 0) -> E4M3 codes [m, k] and ONE FP32 scale a row: s = max(amax / 448, 1e-12),
+// q = e4m3(clamp(x / s, -448, 448)), IEEE divisions as in quant_groups_lane (the reference's per-row quantizer,
+// hibana/kernels/csrc/w3_gemm.cu:244-288, which multiplies by a reciprocal). One workgroup a row: the row's largest
+// magnitude over the four wavefronts through LDS, then every lane rounds its runs of eight values.
+__global__ __launch_bounds__(256) void quant_rows_kernel(const uint16_t* __restrict__ x, int k, uint8_t* __restrict__ q, float* __restrict__ scales) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const uint16_t* xr = x + row * k;
+  float amax = 0.f;
+  for (int c = 8 * threadIdx.x; c < k; c += 8 * 256) {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(xr + c);
+#pragma unroll
+    for (int j = 0; j < 4; j++) amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(raw[j] << 16)), fabsf(__uint_as_float(raw[j] & 0xffff0000u))));
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float s = fmaxf(amax / 448.0f, 1e-12f);
+  if (threadIdx.x == 0) scales[row] = s;
+  for (int c = 8 * threadIdx.x; c < k; c += 8 * 256) {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(xr + c);
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      v[2 * j] = __uint_as_float(raw[j] << 16);
+      v[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = fminf(fmaxf(v[j] / s, -448.0f), 448.0f);
+    int lo = 0, hi = 0;
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], lo, false);
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], lo, true);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], hi, false);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], hi, true);
+    typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+    *reinterpret_cast<i32x2_t*>(q + row * k + c) = i32x2_t{lo, hi};
+  }
+}
+
+void moe_launch_quant_rows(const uint16_t* x, int64_t m, int k, uint8_t* q, float* scales, hipStream_t stream) {
+  HB_LAUNCH(quant_rows_kernel, dim3((unsigned)m), dim3(256), 0, stream, x, k, q, scales);
+}
+
 void moe_launch_quant_groups(const QuantJob& job, hipStream_t stream) {
   HB_LAUNCH(quant_groups_kernel, dim3((unsigned)((job.lanes + 255) / 256)), dim3(256), 0, stream, job);
 }
@@ -630,6 +674,7 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   rp.e = e;
   rp.k = topk;
   rp.per = (e + 63) / 64;
+  rp.steps = 1;
   rp.ids = ids;
   rp.weights = weights;
   const int64_t pairs = (int64_t)m * topk;
@@ -680,12 +725,45 @@ extern "C" int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int
   return launch_status();
 }
 
-extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, int32_t* ids, float* weights, void* stream) {
+// out[r, c] = bf16( bf16(silu(gate)) * up ) of BF16 rows holding `half` gate and `half` up columns: [gate | up]
+// (pairs == 0) or alternating blocks of `pairs` gate columns and their `pairs` up columns. The roundings are those of
+// the BF16 tensor expression silu(gate) * up (hibana/kernels/ops.py:86-92 of the reference). Two columns a thread.
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __restrict__ x, int64_t rows, int half, int pairs, uint16_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // column pair i % (half / 2) of row i / (half / 2)
+  const int per_row = half >> 1;
+  if (i >= rows * per_row) return;
+  const int64_t r = i / per_row;
+  const int c = 2 * (int)(i - r * per_row);
+  const int gate_at = pairs ? (c / pairs) * 2 * pairs + c % pairs : c, up_at = pairs ? gate_at + pairs : half + c;
+  const uint16_t* row = x + r * 2 * half;
+  const uint32_t g2 = *reinterpret_cast<const uint32_t*>(row + gate_at), u2 = *reinterpret_cast<const uint32_t*>(row + up_at);
+  const float g0 = __uint_as_float(g2 << 16), g1 = __uint_as_float(g2 & 0xffff0000u);
+  const float u0 = __uint_as_float(u2 << 16), u1 = __uint_as_float(u2 & 0xffff0000u);
+  const float s0 = round_bf16(g0 / (1.0f + expf(-g0))), s1 = round_bf16(g1 / (1.0f + expf(-g1)));
+  *reinterpret_cast<uint32_t*>(out + r * half + c) = (uint32_t)f32_to_bf16_bits(s0 * u0) | ((uint32_t)f32_to_bf16_bits(s1 * u1) << 16);
+}
+
+extern "C" int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int pairs, void* out, void* stream) {
+  if (!gate_up || !out) return HB_ENULL;
+  if (rows <= 0 || half <= 0 || half % 2 || pairs < 0 || (pairs && (pairs % 2 || half % pairs))) return HB_EINVAL;
+  if (!aligned(gate_up, 4) || !aligned(out, 4)) return HB_EINVAL;
+  const int64_t threads = rows * (half / 2);
+  hipLaunchKernelGGL(silu_and_mul_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint16_t*>(gate_up), rows, half, pairs, static_cast<uint16_t*>(out));
+  return launch_status();
+}
+
+extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, const int32_t* slots, int steps, int repeat, int32_t* ids,
+                                     float* weights, void* stream) {
   if (!logits || !ids || !weights) return HB_ENULL;
-  if (m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE) return HB_EINVAL;
+  if (m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE || steps <= 0) return HB_EINVAL;
+  if (!aligned(logits, 4) || !aligned(slots, 4) || !aligned(ids, 4) || !aligned(weights, 4)) return HB_EINVAL;
   RouteParams p{};
   p.logits = logits;
   p.stride = e;
+  p.slots = slots;
+  p.steps = steps;
+  p.repeat = repeat;
   p.e = e;
   p.k = k;
   p.per = (e + 63) / 64;

@@ -380,6 +380,7 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream,
                     int slot_rows = ROWS_PER_SLOT, const QuantJob* job = nullptr);
 void moe_launch_quant_groups(const QuantJob& job, hipStream_t stream);  // the rounding alone
+void moe_launch_quant_rows(const uint16_t* x, int64_t m, int k, uint8_t* q, float* scales, hipStream_t stream);  // one scale a row
 
 // Softmax top-k routing of `m` rows of `e` logits into ids / weights [m, topk], then the plan of those ids: one launch
 // for up to a few dozen rows, two beyond.

@@ -681,6 +681,14 @@ extern "C" int hb_w3_quant_groups(const void* x, int64_t m, int k, void* q, floa
   return launch_status();
 }
 
+extern "C" int hb_w3_quant_rows(const void* x, int64_t m, int k, void* q, float* scales, void* stream) {
+  if (!x || !q || !scales) return HB_ENULL;
+  if (m <= 0 || m > 0x7fffffff || k <= 0 || k % 8) return HB_EINVAL;
+  if (!aligned(x, 16) || !aligned(q, 8) || !aligned(scales, 4)) return HB_EINVAL;
+  moe_launch_quant_rows(static_cast<const uint16_t*>(x), m, k, static_cast<uint8_t*>(q), scales, as_stream(stream));
+  return launch_status();
+}
+
 extern "C" int hb_w3_gemm_e4m3(const void* xq, const float* x_scale, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k,
                                void* y, void* stream) {
   if (!xq || !x_scale || !tiled || !row_scale || !y) return HB_ENULL;

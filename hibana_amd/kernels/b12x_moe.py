@@ -84,6 +84,7 @@ class B12xExperts:
         ws = torch.empty(need, dtype=torch.uint8, device=x.device)
         ids32 = ids.to(torch.int32).contiguous()
         wt = weights.float().contiguous()
-        _lib.check(_lib.lib().hb_nvfp4_moe(C.byref(st), _lib.ptr(x.contiguous()), _lib.ptr(ids32), _lib.ptr(wt), m, topk, int(pairs),
+        xc = x.contiguous()
+        _lib.check(_lib.lib().hb_nvfp4_moe(C.byref(st), _lib.ptr(xc), _lib.ptr(ids32), _lib.ptr(wt), m, topk, int(pairs),
                                            _lib.ptr(out), _lib.ptr(ws), need, _lib.stream()), "nvfp4 experts")
         return out

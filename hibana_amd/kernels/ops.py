@@ -16,7 +16,8 @@ def w3_decode(lin, m: int, rows: int | None = None) -> bool:
 
 def nvfp4_linear(x: torch.Tensor, lin, prequantized=None, relu2: bool = False) -> torch.Tensor:
     """BF16 x [M, K] -> BF16 [M, N] on NVFP4 weights, weight-only: bf16((x Wq^T)_fp32 * global scale); the 3-bit copy
-    serves the call when one is attached and enabled (hibana/kernels/ops.py:56-83)."""
+    serves the call when one is attached and enabled (hibana/kernels/ops.py:56-83). No host synchronization on the
+    call path once `lin.tile()` has run (it caches the global scale as a host float), so the call can be captured."""
     if prequantized is not None:
         raise ValueError("nvfp4_linear: NVFP4 activations are not taken by the weight-only kernels")
     if x.dtype == torch.bfloat16 and w3_decode(lin, x.shape[0]) and not relu2:
@@ -28,31 +29,39 @@ def nvfp4_linear(x: torch.Tensor, lin, prequantized=None, relu2: bool = False) -
     m = x.shape[0]
     y = torch.empty((m, lin.out_features), dtype=torch.bfloat16, device=x.device)
     if m:
-        _lib.check(_lib.lib().hb_nvfp4_gemm(_lib.ptr(x.contiguous()), m, _lib.ptr(lin.tiled), lin.global_scale, lin.out_features,
+        xc = x.contiguous()  # held until the launch is enqueued: a temporary's block could be handed out again before that
+        _lib.check(_lib.lib().hb_nvfp4_gemm(_lib.ptr(xc), m, _lib.ptr(lin.tiled), lin.global_scale, lin.out_features,
                                             lin.in_features, int(relu2), _lib.ptr(y), _lib.stream()), "nvfp4_linear")
     return y
 
 
 def silu_and_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:
-    """silu(gate) * up of [..., gate | up], or (`pairs`) of gate and up alternating in blocks of `pairs` columns
-    (hibana/kernels/ops.py:86-92)."""
+    """silu(gate) * up of BF16 [..., gate | up], or (`pairs`) of gate and up alternating in blocks of `pairs` columns
+    (hibana/kernels/ops.py:86-92), on the GPU; the roundings are those of the BF16 tensor expression."""
+    if gate_up.dtype != torch.bfloat16 or gate_up.shape[-1] % 4 or (pairs and (pairs % 2 or (gate_up.shape[-1] // 2) % pairs)):
+        raise ValueError("silu_and_mul: BF16 [..., 2 * half], half even (and a multiple of an even `pairs`)")
+    _lib.need_gpu(gate_up)
     half = gate_up.shape[-1] // 2
-    if pairs:
-        blocks = gate_up.unflatten(-1, (half // pairs, 2, pairs))
-        return (torch.nn.functional.silu(blocks[..., 0, :]) * blocks[..., 1, :]).flatten(-2)
-    return torch.nn.functional.silu(gate_up[..., :half]) * gate_up[..., half:]
+    flat = gate_up.reshape(-1, 2 * half).contiguous()
+    out = torch.empty((flat.shape[0], half), dtype=torch.bfloat16, device=gate_up.device)
+    if flat.shape[0]:
+        _lib.check(_lib.lib().hb_silu_and_mul(_lib.ptr(flat), flat.shape[0], half, pairs, _lib.ptr(out), _lib.stream()), "silu_and_mul")
+    return out.reshape(*gate_up.shape[:-1], half)
 
 
-def route_topk(logits: torch.Tensor, k: int):
-    """[M, E] FP32 logits -> (int32 ids [M, k], FP32 renormalized softmax weights [M, k]), largest first
-    (hibana/kernels/flashnext_fused.py:308-319, without the padded-slot table)."""
-    _lib.need_gpu(logits)
+def route_topk(logits: torch.Tensor, k: int, slots: torch.Tensor | None = None, steps: int = 1, repeat: bool = False):
+    """[M, E] FP32 logits -> (int32 ids [M, k], FP32 renormalized softmax weights [M, k]), largest first. With `slots`,
+    row r is real iff slots[r // steps] != 0; a padded row takes expert E at weight 0 (the 3-bit experts skip it) or,
+    `repeat`, row 0's first choice at weight 0 (hibana/kernels/flashnext_fused.py:308-319)."""
+    _lib.need_gpu(logits, slots)
     m, e = logits.shape
-    logits = logits.float().contiguous()
+    lg = logits.float().contiguous()
+    sl = None if slots is None else slots.to(torch.int32).contiguous()
     ids = torch.empty((m, k), dtype=torch.int32, device=logits.device)
     w = torch.empty((m, k), dtype=torch.float32, device=logits.device)
     if m:
-        _lib.check(_lib.lib().hb_route_softmax_topk(_lib.ptr(logits), m, e, k, _lib.ptr(ids), _lib.ptr(w), _lib.stream()), "route_topk")
+        _lib.check(_lib.lib().hb_route_softmax_topk(_lib.ptr(lg), m, e, k, _lib.ptr(sl), steps, int(repeat), _lib.ptr(ids), _lib.ptr(w),
+                                                    _lib.stream()), "route_topk")
     return ids, w
 
 
@@ -69,10 +78,12 @@ def moe_combine_pairs(y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
         return out
     if y.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("moe_combine_pairs: pairs must be FP32 or BF16")
+    # every converted operand is bound to a name until the launch is enqueued
+    yc, ids32, wt = y.contiguous(), ids.to(torch.int32).contiguous(), weights.float().contiguous()
     sh = None if shared is None else shared.to(torch.bfloat16).contiguous()
     xx = None if x is None else x.to(torch.bfloat16).contiguous()
-    gw = None if gate_w is None else gate_w.float().contiguous()
-    _lib.check(_lib.lib().hb_moe_combine_pairs(_lib.ptr(y.contiguous()), int(y.dtype == torch.bfloat16), _lib.ptr(ids.to(torch.int32).contiguous()),
-                                               _lib.ptr(weights.float().contiguous()), _lib.ptr(sh), _lib.ptr(xx), _lib.ptr(gw), e_lo, e_n, m, topk, h,
-                                               _lib.ptr(out), _lib.stream()), "moe_combine_pairs")
+    gw = None if gate_w is None else gate_w.float().reshape(-1).contiguous()
+    _lib.check(_lib.lib().hb_moe_combine_pairs(_lib.ptr(yc), int(y.dtype == torch.bfloat16), _lib.ptr(ids32), _lib.ptr(wt), _lib.ptr(sh),
+                                               _lib.ptr(xx), _lib.ptr(gw), e_lo, e_n, m, topk, h, _lib.ptr(out), _lib.stream()),
+               "moe_combine_pairs")
     return out

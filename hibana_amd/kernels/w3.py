@@ -16,7 +16,6 @@ Every function here that touches packed data runs on the GPU and raises on CPU t
 from __future__ import annotations
 
 import os
-import struct
 from dataclasses import dataclass, replace
 
 import torch
@@ -75,16 +74,22 @@ class W3Weight:
 
 
 def lut_of(codebook: tuple[float, ...]) -> int:
-    raw = torch.tensor(codebook, dtype=torch.float32).to(torch.float8_e4m3fn).view(torch.uint8).tolist()
-    return struct.unpack("<q", bytes(raw + [0] * (8 - len(raw))))[0]
+    """The codebook as the kernels take it: level i as an E4M3 byte in byte i of a little-endian signed 64-bit integer,
+    a four-level book zero-filled (hibana/kernels/w3.py:105-107)."""
+    e4m3 = torch.tensor(codebook, dtype=torch.float32).to(torch.float8_e4m3fn).view(torch.uint8)
+    return int.from_bytes(bytes(e4m3.tolist()).ljust(8, b"\0"), "little", signed=True)
 
 
 def _codebook(codebook) -> tuple[float, ...]:
-    name = DEFAULT_CODEBOOK if codebook is None else codebook
-    levels = CODEBOOKS[name] if isinstance(name, str) else tuple(float(v) for v in name)
-    if len(levels) not in (4, 8) or any(b < a for a, b in zip(levels, levels[1:])):
+    """A codebook by name (None: the default) or as a sequence of levels, checked (hibana/kernels/w3.py:110-118)."""
+    if codebook is None:
+        codebook = DEFAULT_CODEBOOK
+    levels = tuple(CODEBOOKS[codebook]) if isinstance(codebook, str) else tuple(map(float, codebook))
+    ascending = all(lo <= hi for lo, hi in zip(levels, levels[1:]))
+    if len(levels) not in (4, 8) or not ascending:
         raise ValueError("a codebook is eight (or, two-bit, four) ascending levels")
-    if torch.tensor(levels).to(torch.float8_e4m3fn).float().tolist() != list(levels):
+    through_e4m3 = torch.tensor(levels).to(torch.float8_e4m3fn).float()
+    if not torch.equal(through_e4m3, torch.tensor(levels)):
         raise ValueError("codebook levels must be exactly representable in E4M3")
     return levels
 
@@ -134,43 +139,87 @@ def pack_codes(q: torch.Tensor, scale_fp8: torch.Tensor, row_scale: torch.Tensor
     return W3Weight(planes, scales, row_scale.float().contiguous(), n, k, levels, lut_of(levels))
 
 
+def sum32(values: torch.Tensor) -> torch.Tensor:
+    """FP32 sum over a last axis of 32 in a FIXED order, the one the reference's CPU `.sum(-1)` takes: element i into
+    partial sum i % 8 (ascending i), then the eight partial sums in ascending order. Which candidate scale a group gets
+    is decided by strict comparisons of such sums, so the order is part of the format's definition here, not left to
+    the device's reduction."""
+    lanes = values.unflatten(-1, (4, 8))
+    part = ((lanes[..., 0, :] + lanes[..., 1, :]) + lanes[..., 2, :]) + lanes[..., 3, :]
+    total = part[..., 0]
+    for j in range(1, 8):
+        total = total + part[..., j]
+    return total
+
+
+class _Levels:
+    """A codebook on a device: its levels, the midpoints that separate them, its largest magnitude."""
+
+    def __init__(self, levels: tuple[float, ...], device):
+        self.values = torch.tensor(levels, dtype=torch.float32, device=device)
+        self.mids = (self.values[1:] + self.values[:-1]) / 2
+        # divisors as tensors: torch divides by a Python scalar on the GPU through its reciprocal, which is off by an ulp
+        self.top = torch.tensor(max(abs(v) for v in levels), device=device)
+        self.fp8_max = torch.tensor(FP8_MAX, device=device)
+
+    def nearest(self, groups: torch.Tensor, effective: torch.Tensor) -> torch.Tensor:
+        """Codes of [N, G, 32] weights under effective group scales [N, G]: a value on a midpoint takes the lower level."""
+        return torch.bucketize(groups / effective.clamp_min(1e-30).unsqueeze(-1), self.mids)
+
+    def loss(self, groups: torch.Tensor, effective: torch.Tensor) -> torch.Tensor:
+        """Squared error [N, G] of the nearest-level copy under `effective`."""
+        copy = self.values[self.nearest(groups, effective)] * effective.unsqueeze(-1)
+        return sum32((copy - groups).square())
+
+    def row_scale(self, group_scale: torch.Tensor) -> torch.Tensor:
+        return (group_scale.amax(dim=-1) / self.fp8_max).clamp_min(1e-12)
+
+    @staticmethod
+    def stored(group_scale: torch.Tensor, row: torch.Tensor) -> torch.Tensor:
+        return (group_scale / row.unsqueeze(1)).clamp(0, FP8_MAX).to(torch.float8_e4m3fn)
+
+
+def first_best(candidates):
+    """Of (loss [N, G], payload [N, G]) pairs in order, per group the payload of the FIRST pair whose loss is strictly
+    below every earlier one's (the rule of both fitted-scale searches of the reference, hibana/kernels/w3.py:154-164 and
+    hibana/weights/w3_calibration.py:28-36)."""
+    best_loss = best = None
+    for loss, payload in candidates:
+        if best is None:
+            best_loss, best = loss, payload
+            continue
+        wins = loss < best_loss
+        best_loss = torch.where(wins, loss, best_loss)
+        best = torch.where(wins, payload, best)
+    return best
+
+
+def quantize_rows(rows: torch.Tensor, book: _Levels, fit_scales: bool):
+    """float [n, K] -> (codes uint8 [n, K], stored scales float8_e4m3fn [n, K/32], row scales [n]) by the nearest-level
+    rule of hibana/kernels/w3.py:146-172: group scale = largest magnitude / largest level - or, `fit_scales`, the
+    multiple of it among FIT_SCALES with the least squared error -, row scale = largest group scale / 448, the group
+    scale stored as the E4M3 of their ratio, codes nearest under the scale as stored."""
+    groups = rows.float().unflatten(1, (rows.shape[1] // GROUP, GROUP))
+    scale = groups.abs().amax(dim=-1) / book.top
+    if fit_scales:
+        scale = first_best((book.loss(groups, cand), cand) for cand in (scale * mult for mult in FIT_SCALES))
+    row = book.row_scale(scale)
+    stored = book.stored(scale, row)
+    codes = book.nearest(groups, stored.float() * row.unsqueeze(1)).flatten(1)
+    return codes.to(torch.uint8), stored, row
+
+
 def pack(weight: torch.Tensor, codebook=None, rows_per_chunk: int = 4096, fit_scales: bool = False) -> W3Weight:
-    """Nearest-level quantization of a [N, K] float matrix (N, K multiples of 128), hibana/kernels/w3.py:126-172:
-    group scale = amax / largest level (or, `fit_scales`, the best of FIT_SCALES times that), row scale = largest
-    group scale / 448, group scale stored as E4M3 of the ratio, code = the nearest level of w / effective scale."""
+    """Nearest-level quantization of a [N, K] float matrix (N, K multiples of 128) into the fragment order,
+    hibana/kernels/w3.py:126-143; `rows_per_chunk` rows at a time (the temporaries of the lm_head would not fit
+    otherwise). The arithmetic is quantize_rows'."""
     n, k = weight.shape
     if k % CHUNK or n % 128:
         raise ValueError("N and K must be multiples of 128")
     levels = _codebook(codebook)
-    lv = torch.tensor(levels, device=weight.device)
-    mids = (lv[1:] + lv[:-1]) / 2
-    # divisors as tensors: torch divides by a Python scalar on the GPU through its reciprocal, which is off by an ulp
-    top = torch.tensor(max(abs(v) for v in levels), device=weight.device)
-    fp8_max = torch.tensor(FP8_MAX, device=weight.device)
-    parts = []
-    for r0 in range(0, n, rows_per_chunk):
-        g = weight[r0:r0 + rows_per_chunk].float().unflatten(1, (k // GROUP, GROUP))
-        scale = g.abs().amax(dim=-1) / top
-        if fit_scales:
-            best_err = best = None
-            for mult in FIT_SCALES:
-                cand = scale * mult
-                deq = lv[torch.bucketize(g / cand.clamp_min(1e-30).unsqueeze(-1), mids)] * cand.unsqueeze(-1)
-                err = (deq - g).square().sum(-1)
-                if best is None:
-                    best_err, best = err, cand
-                else:
-                    take = err < best_err
-                    best_err, best = torch.where(take, err, best_err), torch.where(take, cand, best)
-            scale = best
-        row = (scale.amax(dim=-1) / fp8_max).clamp_min(1e-12)
-        stored = (scale / row.unsqueeze(1)).clamp(0, FP8_MAX).to(torch.float8_e4m3fn)
-        eff = stored.float() * row.unsqueeze(1)
-        q = torch.bucketize((g / eff.clamp_min(1e-30).unsqueeze(-1)).flatten(1), mids)
-        parts.append((q.to(torch.uint8), stored, row))
-    q = torch.cat([p[0] for p in parts])
-    stored = torch.cat([p[1] for p in parts])
-    row = torch.cat([p[2] for p in parts])
+    book = _Levels(levels, weight.device)
+    pieces = [quantize_rows(weight[r0:r0 + rows_per_chunk], book, fit_scales) for r0 in range(0, n, rows_per_chunk)]
+    q, stored, row = (torch.cat(column) for column in zip(*pieces))
     return pack_codes(q, stored, row, levels)
 
 
@@ -184,7 +233,8 @@ def _unpack(w3: W3Weight, want_codes: bool, want_scales: bool):
     if w3.tiled is not None:
         _lib.check(_lib.lib().hb_w3_unpack(_lib.ptr(w3.tiled), n, k, _lib.ptr(codes8), _lib.ptr(raw), _lib.stream()), "w3 unpack")
     else:
-        _lib.check(_lib.lib().hb_w3_unpack_planes(_lib.ptr(w3.planes.contiguous()), _lib.ptr(w3.scales.contiguous()), n, k, w3.bits,
+        planes, scales = w3.planes.contiguous(), w3.scales.contiguous()
+        _lib.check(_lib.lib().hb_w3_unpack_planes(_lib.ptr(planes), _lib.ptr(scales), n, k, w3.bits,
                                                   _lib.ptr(codes8), _lib.ptr(raw), _lib.stream()), "w3 unpack")
     return codes8, raw
 
@@ -214,41 +264,60 @@ def dequantize(w3: W3Weight) -> torch.Tensor:
 
 
 def pair_order(rows: int, block: int) -> torch.Tensor:
-    """Row order that interleaves [gate; up] in blocks of `block` rows (hibana/weights/modelopt.py:84-86)."""
-    half = torch.arange(rows // 2).unflatten(0, (rows // 2 // block, block))
-    return torch.stack((half, half + rows // 2), dim=1).reshape(-1)
+    """Row order that interleaves [gate; up] in blocks of `block` rows: gate block 0, up block 0, gate block 1, ...
+    (hibana/weights/modelopt.py:84-86)."""
+    half = rows // 2
+    gate = torch.arange(half).reshape(half // block, block)
+    return torch.cat((gate, gate + half), dim=1).reshape(-1)
 
 
 def interleave_rows(weight: W3Weight, block: int) -> W3Weight:
-    """`weight`'s rows in pair_order (an MLP's gate|up interleaved in blocks of `block`, a multiple of 32): planes and
-    scales move in whole 32-row tiles (hibana/kernels/w3.py:94-102). The tiled copy, if any, is rebuilt on demand."""
+    """`weight`'s rows in pair_order (an MLP's gate|up interleaved in blocks of `block`, a multiple of 32): dim 0 of
+    planes and scales counts 32-row tiles, so they move as `block / 32` tiles at a time and the row scales row by row
+    (hibana/kernels/w3.py:94-102). The tiled copy, if any, is rebuilt on demand."""
     if weight.planes is None:
         raise ValueError("interleave_rows needs the fragment-order tensors (they were released)")
-    tiles = pair_order(weight.out_features // 32, block // 32).to(weight.planes.device)
-    rows = pair_order(weight.out_features, block).to(weight.row_scale.device)
-    planes = weight.planes.view(torch.int32)[tiles].view(torch.uint32)
-    return replace(weight, planes=planes.contiguous(), scales=weight.scales[tiles].contiguous(),
-                   row_scale=weight.row_scale[rows].contiguous(), tiled=None)
+    if block % 32:
+        raise ValueError("rows move in whole 32-row tiles")
+    tile_order = pair_order(weight.out_features // 32, block // 32).to(weight.planes.device)
+    row_order = pair_order(weight.out_features, block).to(weight.row_scale.device)
+    moved = weight.planes.view(torch.int32).index_select(0, tile_order).view(torch.uint32)  # no uint32 gather on the device
+    return replace(weight, planes=moved.contiguous(), scales=weight.scales.index_select(0, tile_order).contiguous(),
+                   row_scale=weight.row_scale.index_select(0, row_order).contiguous(), tiled=None)
 
 
-def quant_rows(x: torch.Tensor):
-    """One E4M3 scale per row (hibana/kernels/w3.py:326-330): the reference keeps it for comparison only (it loses the
-    small channels next to an outlier) and serves `quant_groups`; not built here."""
-    raise NotImplementedError("per-row E4M3 activation quantization is not built; use quant_groups")
+def _quant_check(x: torch.Tensor, multiple: int, name: str) -> None:
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % multiple:
+        raise ValueError(f"{name}: BF16 [M, K] with K a multiple of {multiple}")
+    _lib.need_gpu(x)
+
+
+def quant_rows(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-row E4M3 quantization of a BF16 [M, K] matrix: (x_q float8_e4m3fn [M, K], scale float32 [M]), scale =
+    max(amax of the row / 448, 1e-12), x_q = e4m3(x / scale) (hibana/kernels/w3.py:326-330; exact divisions, as
+    `quant_groups`). The reference keeps it for comparison (one scale a row loses the small channels next to an outlier)
+    and serves `quant_groups`; `w3_linear` takes either."""
+    _quant_check(x, 8, "quant_rows")
+    m, k = x.shape
+    q = torch.empty((m, k), dtype=torch.float8_e4m3fn, device=x.device)
+    scale = torch.empty((m,), dtype=torch.float32, device=x.device)
+    if m:
+        xc = x.contiguous()
+        _lib.check(_lib.lib().hb_w3_quant_rows(_lib.ptr(xc), m, k, _lib.ptr(q), _lib.ptr(scale), _lib.stream()), "quant_rows")
+    return q, scale
 
 
 def quant_groups(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """Per-(row, 32-group) E4M3 quantization of a BF16 [M, K] matrix: (x_q float8_e4m3fn [M, K], scale float32
     [M, K/32]), scale = max(amax / 448, 1e-12), x_q = e4m3(x / scale) (hibana/kernels/w3.py:333-337, with the exact
     divisions of its torch statement, hibana/kernels/w3_moe.py:187-190)."""
-    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % GROUP:
-        raise ValueError("quant_groups: BF16 [M, K] with K a multiple of 32")
-    _lib.need_gpu(x)
+    _quant_check(x, GROUP, "quant_groups")
     m, k = x.shape
     q = torch.empty((m, k), dtype=torch.float8_e4m3fn, device=x.device)
     scale = torch.empty((m, k // GROUP), dtype=torch.float32, device=x.device)
     if m:
-        _lib.check(_lib.lib().hb_w3_quant_groups(_lib.ptr(x.contiguous()), m, k, _lib.ptr(q), _lib.ptr(scale), _lib.stream()), "quant_groups")
+        xc = x.contiguous()
+        _lib.check(_lib.lib().hb_w3_quant_groups(_lib.ptr(xc), m, k, _lib.ptr(q), _lib.ptr(scale), _lib.stream()), "quant_groups")
     return q, scale
 
 
@@ -284,30 +353,48 @@ def w3_linear(x: torch.Tensor, w3: W3Weight, x_scale: torch.Tensor | None = None
     return y
 
 
+def _missing(linears):
+    return [(name, lin) for name, lin in linears if getattr(lin, "w3", None) is None]
+
+
 def attach(linears, codebook=DEFAULT_CODEBOOK) -> tuple[int, int]:
     """Nearest-level 3-bit copies for (name, linear) pairs that have none; returns (matrices packed, bytes)
     (hibana/kernels/w3.py:370-378)."""
-    count = total = 0
-    for _, lin in linears:
-        if getattr(lin, "w3", None) is None:
-            lin.w3 = tile(pack(lin.dequantize(), codebook))
-            total += lin.w3.bytes
-            count += 1
-    return count, total
+    todo = _missing(linears)
+    for _, lin in todo:
+        lin.w3 = tile(pack(lin.dequantize(), codebook))
+    return len(todo), sum(lin.w3.bytes for _, lin in todo)
 
 
-def attach_model(model, log=print, codebook=DEFAULT_CODEBOOK) -> dict:
-    """Pack 3-bit decode copies for every projection `model.linears()` lists (hibana/kernels/w3.py:381-404, without
-    the calibrated-checkpoint branch)."""
-    count, total = attach(list(model.linears()), codebook)
+def attach_model(model, log=print, codebook=DEFAULT_CODEBOOK, checkpoint=None, revision: str | None = None) -> dict:
+    """3-bit decode copies for every projection `model.linears()` lists (hibana/kernels/w3.py:381-404): calibrated ones
+    from a W3 checkpoint when one is given - `checkpoint` a directory or a `CalibratedWeights` (default: the directory
+    HIBANA_W3_CHECKPOINT names, for the target at `revision`), which must hold exactly the model's projections -,
+    nearest-level copies otherwise. Each copy is tiled for the kernels as it is attached."""
+    from hibana_amd.weights.w3_checkpoint import REPLICATED, CalibratedWeights
+    source = checkpoint if checkpoint is not None else (os.environ.get("HIBANA_W3_CHECKPOINT") or None)
+    if source is not None and not isinstance(source, CalibratedWeights):
+        source = CalibratedWeights(source, revision if revision is not None else getattr(model, "revision", None))
+    linears = list(model.linears())
+    if source is not None and set(source.weights) != {name for name, _ in linears}:
+        raise ValueError("calibrated W3 checkpoint must contain every target layer projection")
+    todo = _missing(linears)
+    if source is None:
+        count, total = attach(todo, codebook)
+    else:
+        wanted = ((name, lin, getattr(lin, "shard", REPLICATED)) for name, lin in todo)
+        for (_, lin), copy in zip(todo, source.load_many(wanted)):
+            lin.w3 = tile(copy)
+        count, total = len(todo), sum(lin.w3.bytes for _, lin in todo)
     torch.cuda.synchronize()
-    model.w3_identity = "nearest:" + str(codebook)
+    model.w3_identity = source.identity if source is not None else f"nearest:{codebook}"
     log(f"  w3: packed {count} matrices, {total / 2**30:.2f} GiB of 3-bit decode weights (codebook {codebook})")
     return {"matrices": count, "bytes": total}
 
 
 def attach_draft(draft, log=print, codebook=DEFAULT_CODEBOOK) -> dict:
-    count, total = attach(draft.fp8_weights.items(), codebook)
+    """3-bit copies of a parallel draft model's FP8 matrices, `draft.fp8_weights` name -> linear (hibana/kernels/w3.py:407-412)."""
+    count, total = attach(list(draft.fp8_weights.items()), codebook)
     torch.cuda.synchronize()
     log(f"  w3: packed {count} draft matrices, {total / 2**30:.2f} GiB")
     return {"matrices": count, "bytes": total}

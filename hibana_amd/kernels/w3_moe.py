@@ -57,30 +57,35 @@ class W3Experts:
         (n1, h), (h2, i) = self.shape13, self.shape2
         return self.experts * (n1 * h * 3 // 8 + n1 * h // 32 + n1 * 4 + h2 * i * 3 // 8 + h2 * i // 32 + h2 * 4)
 
+    def _side(self, fc1: bool):
+        """(planes, scales, row scales, (rows, k), codebook, lut, tiled) of the fc1 or the fc2 stack."""
+        if fc1:
+            return self.planes13, self.scales13, self.row13, self.shape13, self.codebook, self.lut, self.tiled13
+        return self.planes2, self.scales2, self.row2, self.shape2, self.fc2_codebook, self.fc2_lut, self.tiled2
+
     def matrix(self, e: int, fc1: bool) -> w3.W3Weight:
         """Expert e's fc1 (rows in fc1_order) or fc2 as a W3Weight (views, no copy)."""
-        p, s, r = (self.planes13, self.scales13, self.row13) if fc1 else (self.planes2, self.scales2, self.row2)
-        n, k = self.shape13 if fc1 else self.shape2
-        book = (self.codebook, self.lut) if fc1 else (self.fc2_codebook, self.fc2_lut)
-        tiled = self.tiled13 if fc1 else self.tiled2
-        part = None if tiled is None else tiled.view(self.experts, -1)[e]
-        return w3.W3Weight(None if p is None else p[e], None if s is None else s[e], r[e], n, k, *book, tiled=part)
+        planes, scales, rows, (n, k), book, lut, tiled = self._side(fc1)
+        pick = lambda t: None if t is None else t[e]  # noqa: E731
+        return w3.W3Weight(pick(planes), pick(scales), rows[e], n, k, book, lut,
+                           tiled=None if tiled is None else tiled.view(self.experts, -1)[e])
 
     def stacked(self, fc1: bool) -> w3.W3Weight:
-        """All experts' fc1 or fc2 as one W3Weight of E * N rows (the checkpoint entry)."""
-        p, s, r = (self.planes13, self.scales13, self.row13) if fc1 else (self.planes2, self.scales2, self.row2)
-        n, k = self.shape13 if fc1 else self.shape2
-        book = (self.codebook, self.lut) if fc1 else (self.fc2_codebook, self.fc2_lut)
-        e = self.experts
-        return w3.W3Weight(None if p is None else p.reshape(e * n // 32, *p.shape[2:]), None if s is None else s.reshape(e * n // 32, *s.shape[2:]),
-                           r.reshape(-1), e * n, k, *book, tiled=self.tiled13 if fc1 else self.tiled2)
+        """All experts' fc1 or fc2 as one W3Weight of E * N rows (the checkpoint entry): the expert dim folds into the
+        32-row tile dim."""
+        planes, scales, rows, (n, k), book, lut, tiled = self._side(fc1)
+        fold = lambda t: None if t is None else t.flatten(0, 1)  # noqa: E731
+        return w3.W3Weight(fold(planes), fold(scales), rows.flatten(), self.experts * n, k, book, lut, tiled=tiled)
 
     @classmethod
     def from_stacked(cls, fc1: w3.W3Weight, fc2: w3.W3Weight, experts: int, base: int = 0) -> "W3Experts":
-        def split(m):
-            return (m.planes.reshape(experts, -1, *m.planes.shape[1:]), m.scales.reshape(experts, -1, *m.scales.shape[1:]),
-                    m.row_scale.reshape(experts, -1))
-        return cls(*split(fc1), *split(fc2), fc1.codebook, fc1.lut, fc2.codebook, fc2.lut, base)
+        """The inverse of `stacked`: two matrices of `experts` stacked experts each."""
+        fields = []
+        for m in (fc1, fc2):
+            if m.out_features % experts:
+                raise ValueError("a stack's rows must divide among its experts")
+            fields += [m.planes.unflatten(0, (experts, -1)), m.scales.unflatten(0, (experts, -1)), m.row_scale.unflatten(0, (experts, -1))]
+        return cls(*fields, fc1.codebook, fc1.lut, fc2.codebook, fc2.lut, base)
 
 
 def gated(experts: W3Experts) -> bool:
@@ -149,7 +154,8 @@ def w3_moe(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: torc
     ids32 = ids.to(torch.int32).contiguous()
     wt = weights.float().contiguous()
     mode |= MOE_E4M3 if e4m3 else 0
-    _lib.check(_lib.lib().hb_w3_moe(C.byref(st), _lib.ptr(x.contiguous()), _lib.ptr(ids32), _lib.ptr(wt), m, k, mode, _lib.ptr(out),
+    xc = x.contiguous()  # converted operands keep a name until the launch is enqueued
+    _lib.check(_lib.lib().hb_w3_moe(C.byref(st), _lib.ptr(xc), _lib.ptr(ids32), _lib.ptr(wt), m, k, mode, _lib.ptr(out),
                                     _lib.ptr(ws), need, _lib.stream()), "w3_moe")
     return out
 
@@ -173,7 +179,8 @@ def moe_layer(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: t
     wt = weights.float().contiguous()
     gv = None if gate_vec is None else gate_vec.float().contiguous()
     entry = _lib.lib().hb_w3_moe_layer_e4m3 if e4m3 else _lib.lib().hb_w3_moe_layer
-    _lib.check(entry(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(x.contiguous()),
+    xc = x.contiguous()
+    _lib.check(entry(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(xc),
                      _lib.ptr(ids32), _lib.ptr(wt), m, k, _lib.ptr(out), _lib.ptr(ws), need, _lib.stream()), "moe_layer")
     return out
 
@@ -201,8 +208,9 @@ def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, 
         ws = torch.empty(need, dtype=torch.uint8, device=x.device)
         gv = None if gate_vec is None else gate_vec.float().contiguous()
         entry = _lib.lib().hb_w3_moe_layer_logits_e4m3 if e4m3 else _lib.lib().hb_w3_moe_layer_logits
-        _lib.check(entry(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(x.contiguous()),
-                         _lib.ptr(logits.contiguous()), e_total, m, topk, _lib.ptr(ids), _lib.ptr(wt), _lib.ptr(out),
+        xc, lg = x.contiguous(), logits.contiguous()
+        _lib.check(entry(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(xc),
+                         _lib.ptr(lg), e_total, m, topk, _lib.ptr(ids), _lib.ptr(wt), _lib.ptr(out),
                          _lib.ptr(ws), need, _lib.stream()), "moe_layer_logits")
     return (out, ids, wt) if return_routing else out
 
@@ -211,86 +219,83 @@ def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, 
 
 @torch.no_grad()
 def fit_scales(weight: torch.Tensor, levels, ratios=RATIOS):
-    """float32 [N, K] -> (group scales float8_e4m3fn [N, K/32], row scales float32 [N]): per 32-group the stored scale,
-    among amax / max|level| * ratio on the ratio grid, with the smallest squared weight error at nearest-level codes;
-    the first of equal errors stays (hibana/weights/w3_calibration.py:17-37 with unit importance)."""
-    n, k = weight.shape
-    grouped = weight.float().reshape(n, k // w3.GROUP, w3.GROUP)
-    top = torch.tensor(max(abs(v) for v in levels), device=weight.device)
-    fp8_max = torch.tensor(w3.FP8_MAX, device=weight.device)
-    base = grouped.abs().amax(-1) / top
-    row_scale = (base.amax(-1) / fp8_max).clamp_min(1e-12)
-    lv = torch.tensor(levels, dtype=torch.float32, device=weight.device)
-    mids = (lv[1:] + lv[:-1]) / 2
-    best_loss = torch.full_like(base, float("inf"))
-    best = torch.zeros_like(base)
-    for ratio in ratios:
-        scale = (base * ratio / row_scale[:, None]).clamp(0, w3.FP8_MAX).to(torch.float8_e4m3fn).float()
-        effective = scale * row_scale[:, None]
-        q = torch.bucketize(grouped / effective.clamp_min(1e-30)[:, :, None], mids)
-        loss = (grouped - lv[q] * effective[:, :, None]).square().sum(-1)
-        improved = loss < best_loss
-        best_loss = torch.minimum(loss, best_loss)
-        best = torch.where(improved, scale, best)
-    return best.to(torch.float8_e4m3fn), row_scale
+    """float32 [N, K] -> (group scales float8_e4m3fn [N, K/32], row scales float32 [N]): per 32-group the STORED scale,
+    among e4m3(amax / max|level| * ratio / row scale) over the ratio grid, with the smallest squared weight error at
+    nearest-level codes; the first of equal errors stays (hibana/weights/w3_calibration.py:17-37 with unit importance).
+    Unlike `w3.pack(fit_scales=True)` the candidates are compared as they will be stored."""
+    book = w3._Levels(tuple(levels), weight.device)
+    groups = weight.float().unflatten(1, (weight.shape[1] // w3.GROUP, w3.GROUP))
+    base = groups.abs().amax(-1) / book.top
+    row = book.row_scale(base)
+
+    def candidates():
+        for ratio in ratios:
+            stored = book.stored(base * ratio, row).float()
+            yield book.loss(groups, stored * row.unsqueeze(1)), stored
+
+    return w3.first_best(candidates()).to(torch.float8_e4m3fn), row
 
 
 @torch.no_grad()
 def quantize(weight: torch.Tensor, codebook="lloyd", ratios=RATIOS):
-    """float32 [N, K] -> (codes int32 [N, K], group scales float8_e4m3fn [N, K/32], row scales [N]): the group scale
-    minimizing the weight error on the ratio grid, nearest level (hibana/kernels/w3_moe.py:113-124)."""
+    """float32 [N, K] -> (codes int32 [N, K], group scales float8_e4m3fn [N, K/32], row scales [N]): `fit_scales`, then
+    the nearest level under the fitted scale (hibana/kernels/w3_moe.py:113-124)."""
     levels = w3._codebook(codebook)
-    n, k = weight.shape
-    scales, row_scale = fit_scales(weight, levels, ratios)
-    effective = (scales.float() * row_scale[:, None]).clamp_min(1e-30)
-    lv = torch.tensor(levels, device=weight.device)
-    codes = torch.bucketize(weight.float().reshape(n, k // w3.GROUP, w3.GROUP) / effective[:, :, None], (lv[1:] + lv[:-1]) / 2, out_int32=True)
-    return codes.reshape(n, k), scales, row_scale
+    stored, row = fit_scales(weight, levels, ratios)
+    book = w3._Levels(levels, weight.device)
+    groups = weight.float().unflatten(1, (weight.shape[1] // w3.GROUP, w3.GROUP))
+    codes = book.nearest(groups, stored.float() * row.unsqueeze(1))
+    return codes.flatten(1).to(torch.int32), stored, row
+
+
+def nvfp4_dequant(packed: torch.Tensor, scales: torch.Tensor, scale2: torch.Tensor) -> torch.Tensor:
+    """NVFP4 experts (uint8 [E, R, K/2], float8_e4m3fn [E, R, K/16], FP32 [E]) -> float32 [E, R, K]: code value x block
+    scale, then x the expert's scale (hibana/kernels/w3_moe.py:105-110)."""
+    from hibana_amd.weights.modelopt import unpack_fp4
+    experts, rows, half = packed.shape
+    unscaled = unpack_fp4(packed.flatten(0, 1), scales.flatten(0, 1)).unflatten(0, (experts, rows))
+    return unscaled * scale2.float().view(experts, 1, 1)
+
+
+def _quantized_chunks(packed, scales, scale2, row_order, levels, ratios, chunk):
+    """A stack of NVFP4 experts, `chunk` experts at a time -> (their 3-bit W3Weight, squared error, squared norm)."""
+    rows = packed.shape[1]
+    for lo in range(0, packed.shape[0], chunk):
+        piece = slice(lo, lo + chunk)
+        source = nvfp4_dequant(packed[piece], scales[piece], scale2[piece])
+        if row_order is not None:
+            source = source.index_select(1, row_order)
+        source = source.flatten(0, 1)
+        copy = w3.pack_codes(*quantize(source, levels, ratios), levels, rows_per_chunk=rows)
+        delta = w3.dequantize(copy) - source
+        yield copy, float(delta.square().sum()), float(source.square().sum())
 
 
 @torch.no_grad()
 def calibrate(w13, s13, scale2_13, w2, s2, scale2_2, codebook="lloyd", ratios=RATIOS, chunk: int = 16):
     """A layer's NVFP4 experts (w13 uint8 [E, 2I, H/2] with rows [up; gate], unswizzled float8 block scales
-    [E, 2I, H/16], FP32 scales [E]; w2 likewise) -> (W3Experts with fc1 rows in fc1_order, report with the relative
-    weight error of fc1 and fc2 against the NVFP4 values) (hibana/kernels/w3_moe.py:127-155). Runs on the GPU the
-    tensors are on."""
+    [E, 2I, H/16], FP32 scales [E]; w2 likewise) -> (W3Experts with fc1 rows in fc1_order, report {"w13", "w2"}: the
+    relative weight error of each stack against the NVFP4 values) (hibana/kernels/w3_moe.py:127-155). Runs on the GPU
+    the tensors are on, `chunk` experts at a time."""
     levels = w3._codebook(codebook)
-    order = fc1_order(w13.shape[1] // 2, w13.device)
-    parts, report = {}, {}
-    for key, (packed, scales, scale2, perm) in {"w13": (w13, s13, scale2_13, order), "w2": (w2, s2, scale2_2, None)}.items():
-        e, r = packed.shape[:2]
-        out, num, den = [], 0.0, 0.0
-        for lo in range(0, e, chunk):
-            hi = min(e, lo + chunk)
-            w = nvfp4_dequant(packed[lo:hi], scales[lo:hi], scale2[lo:hi])
-            if perm is not None:
-                w = w[:, perm]
-            w = w.reshape((hi - lo) * r, -1)
-            codes, sc, rs = quantize(w, levels, ratios)
-            m = w3.pack_codes(codes, sc, rs, levels, rows_per_chunk=r)
-            num += (w3.dequantize(m) - w).square().sum().item()
-            den += w.square().sum().item()
-            out.append(m)
-            del w, codes, sc, rs
-        k = packed.shape[2] * 2
-        cat = lambda a: torch.cat([getattr(m, a).view(torch.int32) if a == "planes" else getattr(m, a) for m in out])  # noqa: E731
-        parts[key] = w3.W3Weight(cat("planes").view(torch.uint32), cat("scales"), cat("row_scale"), e * r, k, levels, w3.lut_of(levels))
-        report[key] = (num / den) ** 0.5 if den else 0.0
-    return W3Experts.from_stacked(parts["w13"], parts["w2"], w13.shape[0]), report
+    experts = w13.shape[0]
+    stacks = {"w13": (w13, s13, scale2_13, fc1_order(w13.shape[1] // 2, w13.device)), "w2": (w2, s2, scale2_2, None)}
+    built, report = {}, {}
+    for key, (packed, scales, scale2, row_order) in stacks.items():
+        copies, err, norm = [], 0.0, 0.0
+        for copy, e2, n2 in _quantized_chunks(packed, scales, scale2, row_order, levels, ratios, chunk):
+            copies.append(copy)
+            err += e2
+            norm += n2
+        report[key] = (err / norm) ** 0.5 if norm else 0.0
+        planes = torch.cat([c.planes.view(torch.int32) for c in copies]).view(torch.uint32)
+        built[key] = w3.W3Weight(planes, torch.cat([c.scales for c in copies]), torch.cat([c.row_scale for c in copies]),
+                                 experts * packed.shape[1], packed.shape[2] * 2, levels, w3.lut_of(levels))
+    return W3Experts.from_stacked(built["w13"], built["w2"], experts), report
 
 
 def unswizzle_batched(swizzled: torch.Tensor, rows: int, groups: int) -> torch.Tensor:
     """[E, ...] block scales in the 128x4 interleave -> float8_e4m3fn [E, rows, groups] (hibana/kernels/w3_moe.py:97-102)."""
     from hibana_amd.weights.modelopt import unswizzle_block_scales
-    e = swizzled.shape[0]
-    flat = swizzled.reshape(e, -1).view(torch.uint8)
-    return torch.stack([unswizzle_block_scales(flat[i], rows, groups) for i in range(e)]).view(torch.float8_e4m3fn)
-
-
-def nvfp4_dequant(packed: torch.Tensor, scales: torch.Tensor, scale2: torch.Tensor) -> torch.Tensor:
-    """NVFP4 experts (uint8 [E, R, K/2], float8_e4m3fn [E, R, K/16], FP32 [E]) -> float32 [E, R, K]
-    (hibana/kernels/w3_moe.py:105-110)."""
-    from hibana_amd.weights.modelopt import unpack_fp4
-    e, r, _ = packed.shape
-    w = unpack_fp4(packed.reshape(e * r, -1), scales.reshape(e * r, -1)).reshape(e, r, -1)
-    return w * scale2.float().reshape(e, 1, 1)
+    flat = swizzled.reshape(swizzled.shape[0], -1).view(torch.uint8)
+    return torch.stack([unswizzle_block_scales(one, rows, groups) for one in flat]).view(torch.float8_e4m3fn)

@@ -1,0 +1,97 @@
+"""The gated-MoE block of Flash-Next on MI355X behind the reference's `MoeLayer` surface
+(hibana/model/flashnext/moe.py:75-192): x [M, H] BF16 -> BF16 [M, H],
+
+    logits  = x router^T                                      BF16 [M, E] (one GEMM), read as FP32 by the routing
+    ids, w  = top-k of softmax(logits), renormalized          (padded rows of a graph: id E, weight 0)
+    routed  = sum_k w_k * down_e(silu(gate_e x) * up_e x)      3-bit experts
+    shared  = shared_down(silu(shared_gate x) * shared_up x)   3-bit, rides in the experts' launches as one more expert
+    out     = bf16(bf16(routed) + sigmoid(x . shared_gate_vec) * shared)
+
+The block is assembled from tensors already on the device (a loader's job ends there). The routed experts are a
+`W3Experts`; the shared expert is either a one-expert `W3Experts` or the pair of linears the reference holds
+(`shared_gate_up` with rows [gate; up], `shared_down`), whose 3-bit copies are re-stored once, at construction, in the
+experts' row order (`shared_from_linears`). Budgeted expert selection (HIBANA_MOE_KEEP / HIBANA_MOE_BUDGET of the
+reference) is not built: every call routes top-k.
+"""
+from __future__ import annotations
+
+import torch
+
+from hibana_amd.kernels import ops, w3, w3_moe
+
+
+def shared_from_linears(gate_up: w3.W3Weight, down: w3.W3Weight) -> w3_moe.W3Experts:
+    """A shared expert held as two 3-bit matrices - gate_up [2 I, H] with rows [gate; up], down [H, I] - as the
+    one-expert `W3Experts` the kernels take: fc1 = [up; gate] in `fc1_order` (sixteen up rows, then their sixteen gate
+    rows). Rows move in units of sixteen, half a 32-row tile of the fragment order, so the codes are unpacked, reordered
+    and packed again (exactly: no requantization)."""
+    inter = gate_up.out_features // 2
+    if down.in_features != inter or down.out_features != gate_up.in_features:
+        raise ValueError("gate_up [2 I, H] and down [H, I] do not describe one expert")
+    dev = gate_up.row_scale.device
+    rows = torch.cat((torch.arange(inter, 2 * inter), torch.arange(inter)))[w3_moe.fc1_order(inter)].to(dev)  # [up; gate] of [gate; up], then the order
+    fc1 = w3.pack_codes(w3.codes(gate_up).index_select(0, rows).to(torch.uint8), w3.scale_bytes(gate_up).view(torch.uint8).index_select(0, rows).view(torch.float8_e4m3fn),
+                        gate_up.row_scale.index_select(0, rows), gate_up.codebook)
+    if down.planes is None:  # only a tiled copy left: back through the codes
+        down = w3.pack_codes(w3.codes(down).to(torch.uint8), w3.scale_bytes(down), down.row_scale, down.codebook)
+    return w3_moe.tile(w3_moe.W3Experts.from_stacked(fc1, down, 1))
+
+
+class MoeLayer:
+    def __init__(self, router: torch.Tensor, shared_gate: torch.Tensor, experts: w3_moe.W3Experts, topk: int, shared: w3_moe.W3Experts | None = None,
+                 shared_gate_up=None, shared_down=None):
+        """router BF16 [E, H]; shared_gate [1, H] or [H] (the shared expert's sigmoid gate); `experts` this rank's 3-bit
+        experts (a range base .. base + experts - 1 of the E); the shared expert as `shared`, or as the two linears
+        `shared_gate_up` / `shared_down` with 3-bit copies attached (`.w3`)."""
+        self.router = router.contiguous()
+        self.experts, self.hidden = router.shape
+        self.topk = topk
+        self.shared_gate = shared_gate.float().reshape(1, -1).contiguous()
+        self.shared_gate_vec = self.shared_gate.reshape(-1)
+        self.w3 = w3_moe.tile(experts)
+        if experts.base + experts.experts > self.experts:
+            raise ValueError(f"3-bit experts {experts.base}..{experts.base + experts.experts - 1}: the model has {self.experts}")
+        if shared is None and shared_gate_up is not None:
+            if getattr(shared_gate_up, "w3", None) is None or getattr(shared_down, "w3", None) is None:
+                raise ValueError("the shared expert's linears need their 3-bit copies (w3.attach)")
+            shared = shared_from_linears(shared_gate_up.w3, shared_down.w3)
+        self.shared = None if shared is None else w3_moe.tile(shared)
+        self.shared_gate_up, self.shared_down = shared_gate_up, shared_down
+
+    @property
+    def expert_bytes(self) -> int:
+        return self.w3.bytes
+
+    @property
+    def bytes(self) -> int:
+        return self.expert_bytes + self.router.numel() * 2 + (self.shared.bytes if self.shared is not None else 0)
+
+    @staticmethod
+    def _padding(ctx):
+        """(slots, steps) of a decode / verify forward whose graph may hold padded requests, else (None, 1)."""
+        mode = getattr(ctx, "mode", None)
+        if mode == "decode":
+            return getattr(ctx, "slots", None), 1
+        if mode == "verify":
+            return getattr(ctx, "seq_slots", None), int(getattr(ctx, "verify_steps", 1))
+        return None, 1
+
+    def route(self, x: torch.Tensor, ctx=None):
+        """(ids int32 [M, k], weights FP32 [M, k]); padded rows of a decode / verify graph name no expert
+        (hibana/model/flashnext/moe.py:122-144; softmax -> top-k -> renormalize at every size)."""
+        logits = torch.mm(x, self.router.T)
+        slots, steps = self._padding(ctx)
+        return ops.route_topk(logits, self.topk, slots, steps, repeat=False)
+
+    def routed(self, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+        """The routed experts' weighted sum (this rank's part) for x [M, H] -> BF16 [M, H]."""
+        return w3_moe.w3_moe(self.w3, x, ids, weights)
+
+    def __call__(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+        x = x.contiguous()
+        slots, _ = self._padding(ctx)
+        if slots is None:  # routing, plan, both streams and the combine as one chain
+            logits = torch.mm(x, self.router.T).float()
+            return w3_moe.moe_layer_logits(self.w3, x, logits, self.topk, shared=self.shared, gate_vec=self.shared_gate_vec)
+        ids, weights = self.route(x, ctx)
+        return w3_moe.moe_layer(self.w3, x, ids, weights, shared=self.shared, gate_vec=self.shared_gate_vec)

@@ -36,7 +36,8 @@ def route_topk(fused: torch.Tensor, bias: torch.Tensor, k: int, latent: int, slo
     lat = torch.empty((m, latent), dtype=torch.bfloat16, device=dev)
     if m:
         sl = None if slots is None else slots.to(torch.int32).contiguous()
-        _lib.check(_lib.lib().hb_route_sigmoid_topk(_lib.ptr(fused), fused.stride(0), _lib.ptr(bias.float().contiguous()), m, e, k, latent,
+        bias32 = bias.float().contiguous()
+        _lib.check(_lib.lib().hb_route_sigmoid_topk(_lib.ptr(fused), fused.stride(0), _lib.ptr(bias32), m, e, k, latent,
                                                     _lib.ptr(sl), steps, int(repeat), _lib.ptr(ids), _lib.ptr(w), _lib.ptr(lat), _lib.stream()),
                    "route_topk")
     return ids, w, lat

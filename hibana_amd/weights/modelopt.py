@@ -65,6 +65,7 @@ class Nvfp4Linear:
     w3: object = None
     pairs: int = 0
     tiled: torch.Tensor | None = None  # the kernels' block layout (built by tile())
+    scale2: float | None = None  # alpha * input_scale_inv as a host float, read from the device ONCE (by tile())
 
     @property
     def bytes(self) -> int:
@@ -72,9 +73,15 @@ class Nvfp4Linear:
 
     @property
     def global_scale(self) -> float:
-        return float((self.alpha * self.input_scale_inv).float())
+        """The FP32 scale of the matrix as the kernels take it (an argument of the launch). Reading it from the device
+        is a synchronization, so it happens once, at load time (`tile()`), never on the call path; assigning new
+        `alpha` / `input_scale_inv` tensors needs `scale2 = None` to be read again."""
+        if self.scale2 is None:
+            self.scale2 = float((self.alpha.float() * self.input_scale_inv.float()).item())
+        return self.scale2
 
     def tile(self) -> "Nvfp4Linear":
+        _ = self.global_scale
         if self.tiled is None:
             _lib.need_gpu(self.weight, self.weight_scale_swizzled)
             n, k = self.out_features, self.in_features
@@ -83,7 +90,8 @@ class Nvfp4Linear:
                 raise ValueError("NVFP4 kernels need N a multiple of 64 and K a multiple of 128")
             tiled = torch.empty(size, dtype=torch.uint8, device=self.weight.device)
             scales = self.weight_scale_swizzled.contiguous().view(torch.uint8)
-            _lib.check(_lib.lib().hb_nvfp4_repack(_lib.ptr(self.weight.contiguous()), _lib.ptr(scales), 1, n, k, _lib.ptr(tiled), _lib.stream()),
+            codes = self.weight.contiguous()
+            _lib.check(_lib.lib().hb_nvfp4_repack(_lib.ptr(codes), _lib.ptr(scales), 1, n, k, _lib.ptr(tiled), _lib.stream()),
                        "nvfp4 repack")
             self.tiled = tiled
         return self
@@ -113,7 +121,8 @@ def unpack_fp4(packed: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
         raise ValueError("NVFP4 kernels need rows a multiple of 64 and K a multiple of 128")
     tiled = torch.empty(size, dtype=torch.uint8, device=packed.device)
     raw = scales.contiguous().view(torch.uint8) if scales.dtype == torch.float8_e4m3fn else scales.contiguous()
-    _lib.check(_lib.lib().hb_nvfp4_repack(_lib.ptr(packed.contiguous()), _lib.ptr(raw), 0, rows, k, _lib.ptr(tiled), _lib.stream()), "nvfp4 repack")
+    codes = packed.contiguous()
+    _lib.check(_lib.lib().hb_nvfp4_repack(_lib.ptr(codes), _lib.ptr(raw), 0, rows, k, _lib.ptr(tiled), _lib.stream()), "nvfp4 repack")
     out = torch.empty((rows, k), dtype=torch.float32, device=packed.device)
     _lib.check(_lib.lib().hb_nvfp4_dequant(_lib.ptr(tiled), 1.0, rows, k, _lib.ptr(out), _lib.stream()), "unpack_fp4")
     return out

@@ -7,18 +7,24 @@ Loading is where the gfx950 block layout is made: with `tile=True` (the default 
 repacked once by `w3.tile(..., release=True)` and the fragment-order tensors are dropped, so a served model holds one
 copy of each matrix.
 
+Reading goes through three small steps, each with one job: `ManifestEntry` (a manifest record, validated when it is
+parsed), `read_verified` (bytes of a file whose digest matches) and `FragmentTensors` (the three tensors of a file,
+checked against the shapes the record implies, then cut to a shard).
+
 Downloading published checkpoints (`fetch` in the reference) is not part of this module.
 """
 from __future__ import annotations
 
 import hashlib
 import json
+from dataclasses import dataclass
 from pathlib import Path
 
 import torch
 from safetensors.torch import load as load_bytes, save_file
 
 FORMAT_VERSION = 1
+_READ_BLOCK = 8 << 20
 
 
 class Shard:
@@ -50,58 +56,133 @@ class ExpertRange(Shard):
 
 
 def sha256(path: Path) -> str:
-    digest = hashlib.sha256()
-    with Path(path).open("rb") as handle:
-        for block in iter(lambda: handle.read(8 * 2 ** 20), b""):
-            digest.update(block)
-    return digest.hexdigest()
+    """Hex digest of a file, read in blocks."""
+    state = hashlib.sha256()
+    with open(path, "rb") as stream:
+        while True:
+            block = stream.read(_READ_BLOCK)
+            if not block:
+                return state.hexdigest()
+            state.update(block)
+
+
+def read_verified(path: Path, digest: str, what: str) -> bytes:
+    """The file's bytes, read once and refused before anything parses them unless their SHA-256 is `digest`."""
+    data = Path(path).read_bytes()
+    if hashlib.sha256(data).hexdigest() != digest:
+        raise ValueError(f"calibrated W3 checksum mismatch for {what}")
+    return data
+
+
+@dataclass(frozen=True)
+class ManifestEntry:
+    """One weight of the manifest: {"file", "sha256", "out_features", "in_features", "codebook"}."""
+    name: str
+    file: str
+    sha256: str
+    out_features: int
+    in_features: int
+    codebook: tuple[float, ...]
+
+    @classmethod
+    def parse(cls, name: str, record: dict) -> "ManifestEntry":
+        file = str(record["file"])
+        if Path(file).name != file:  # no directories, no "..": a manifest names files of its own folder only
+            raise ValueError("calibrated W3 files must be directly inside the checkpoint")
+        return cls(name, file, str(record["sha256"]), int(record["out_features"]), int(record["in_features"]),
+                   tuple(float(v) for v in record["codebook"]))
+
+    def record(self) -> dict:
+        return {"file": self.file, "sha256": self.sha256, "out_features": self.out_features, "in_features": self.in_features,
+                "codebook": list(self.codebook)}
+
+    def tensor_spec(self) -> dict[str, tuple[tuple[int, ...], torch.dtype]]:
+        """Name -> (shape, dtype) of the tensors the file must hold, and no others."""
+        tiles, chunks = self.out_features // 32, self.in_features // 128
+        return {"planes": ((tiles, chunks, 3, 32, 4), torch.uint32), "scales": ((tiles, chunks, 4, 32), torch.uint8),
+                "row_scale": ((self.out_features,), torch.float32)}
+
+
+@dataclass
+class FragmentTensors:
+    planes: torch.Tensor
+    scales: torch.Tensor
+    row_scale: torch.Tensor
+
+    @classmethod
+    def parse(cls, data: bytes, entry: ManifestEntry) -> "FragmentTensors":
+        tensors = load_bytes(data)
+        spec = entry.tensor_spec()
+        ok = set(tensors) == set(spec) and all(tuple(tensors[k].shape) == shape and tensors[k].dtype == dtype for k, (shape, dtype) in spec.items())
+        if not ok:
+            raise ValueError(f"invalid calibrated W3 tensors for {entry.name}")
+        return cls(tensors["planes"], tensors["scales"], tensors["row_scale"])
+
+    def cut(self, shard: Shard) -> "FragmentTensors":
+        """The shard's part: dim 0 of planes / scales counts 32-row tiles, dim 1 128-wide K chunks; row scales go with
+        the rows."""
+        return FragmentTensors(shard.cols(shard.rows(self.planes, 32), dim=1), shard.cols(shard.rows(self.scales, 32), dim=1),
+                               shard.rows(self.row_scale))
+
+    @property
+    def shape(self) -> tuple[int, int]:
+        return self.row_scale.shape[0], self.planes.shape[1] * 128
 
 
 def save_weight(path: Path, weight) -> dict:
     """Write one W3Weight (its fragment-order tensors) and return its manifest entry
-    (hibana/weights/w3_checkpoint.py:47-54)."""
+    (hibana/weights/w3_checkpoint.py:47-54). The file appears under its name only once it is complete."""
     if weight.planes is None or weight.scales is None:
         raise ValueError("the fragment-order tensors were released; a tiled-only weight cannot be saved")
     path = Path(path)
     path.parent.mkdir(parents=True, exist_ok=True)
-    temporary = path.with_suffix(".tmp")
-    save_file({"planes": weight.planes.cpu().contiguous(), "scales": weight.scales.cpu().contiguous(),
-               "row_scale": weight.row_scale.cpu().contiguous()}, str(temporary))
-    temporary.replace(path)
-    return {"file": path.name, "sha256": sha256(path), "out_features": weight.out_features, "in_features": weight.in_features,
-            "codebook": list(weight.codebook)}
+    staging = path.with_suffix(".tmp")
+    host = {key: getattr(weight, key).detach().cpu().contiguous() for key in ("planes", "scales", "row_scale")}
+    save_file(host, str(staging))
+    staging.replace(path)
+    return ManifestEntry(path.stem, path.name, sha256(path), weight.out_features, weight.in_features, tuple(weight.codebook)).record()
 
 
 class CalibratedWeights:
     def __init__(self, directory: str | Path, revision: str):
         """The calibrated copies in `directory` for the target at `revision` (hibana/weights/w3_checkpoint.py:57-65)."""
         self.directory = Path(directory)
-        self.manifest = json.loads((self.directory / "manifest.json").read_text())
-        if self.manifest.get("format") != FORMAT_VERSION or self.manifest.get("target_revision") != revision:
+        manifest_path = self.directory / "manifest.json"
+        self.manifest = json.loads(manifest_path.read_text())
+        found = (self.manifest.get("format"), self.manifest.get("target_revision"))
+        if found != (FORMAT_VERSION, revision):
             raise ValueError("calibrated W3 checkpoint format or target revision does not match")
         self.weights = self.manifest["weights"]
-        self.identity = sha256(self.directory / "manifest.json")
+        self.identity = sha256(manifest_path)
+
+    def entry(self, name: str) -> ManifestEntry:
+        return ManifestEntry.parse(name, self.weights[name])
 
     def paths(self, names) -> list[tuple[Path, str]]:
         """The files of `names` and their recorded checksums."""
-        return [(self.directory / self.weights[name]["file"], self.weights[name]["sha256"]) for name in names]
+        return [(self.directory / self.weights[n]["file"], self.weights[n]["sha256"]) for n in names]
 
     @staticmethod
     def expert_names(layer: int) -> list[str]:
-        return [f"layers.{layer}.experts.w13", f"layers.{layer}.experts.w2"]
+        return [f"layers.{layer}.experts.{part}" for part in ("w13", "w2")]
 
     def expert_layers(self) -> set[int]:
         """The layers whose routed experts the checkpoint carries."""
-        return {int(name.split(".")[1]) for name in self.weights if name.startswith("layers.") and ".experts." in name}
+        layers = set()
+        for name in self.weights:
+            parts = name.split(".")
+            if len(parts) >= 4 and parts[0] == "layers" and parts[2] == "experts":
+                layers.add(int(parts[1]))
+        return layers
 
     def load(self, name: str, linear, shard: Shard = REPLICATED, tile: bool | None = None):
         """`linear`'s copy (its `out_features` x `in_features`, on `linear.weight.device`), in `linear`'s row order: an
         MLP's gate|up interleaved in blocks of `linear.pairs` (hibana/weights/w3_checkpoint.py:80-88)."""
-        pairs = getattr(linear, "pairs", 0)
         weight = self._load(name, linear.out_features, linear.in_features, linear.weight.device, shard, tile=False)
-        if pairs:
+        block = getattr(linear, "pairs", 0)
+        if block:
             from hibana_amd.kernels.w3 import interleave_rows
-            weight = interleave_rows(weight, pairs)
+            weight = interleave_rows(weight, block)
         return self._finish(weight, tile)
 
     def load_many(self, items):
@@ -115,10 +196,11 @@ class CalibratedWeights:
         over the experts (hibana/weights/w3_checkpoint.py:104-113)."""
         from hibana_amd.kernels import w3_moe
         hi = experts if hi is None else hi
-        w13, w2 = self.expert_names(layer)
-        fc1 = self._load(w13, (hi - lo) * 2 * inter, hidden, device, ExpertRange(lo, hi, 2 * inter), tile=False)
-        fc2 = self._load(w2, (hi - lo) * hidden, inter, device, ExpertRange(lo, hi, hidden), tile=False)
-        ex = w3_moe.W3Experts.from_stacked(fc1, fc2, hi - lo, base=lo)
+        held = hi - lo
+        stacks = []
+        for name, rows, k in zip(self.expert_names(layer), (2 * inter, hidden), (hidden, inter)):
+            stacks.append(self._load(name, held * rows, k, device, ExpertRange(lo, hi, rows), tile=False))
+        ex = w3_moe.W3Experts.from_stacked(stacks[0], stacks[1], held, base=lo)
         if self._wants_tile(tile, torch.device(device)):
             w3_moe.tile(ex, release=True)
         return ex
@@ -134,27 +216,12 @@ class CalibratedWeights:
         return weight
 
     def _load(self, name: str, out_features: int, in_features: int, device, shard: Shard = REPLICATED, tile: bool | None = None):
-        from hibana_amd.kernels.w3 import W3Weight, _codebook, lut_of
-        entry = self.weights[name]
-        n, k = entry["out_features"], entry["in_features"]
-        filename = entry["file"]
-        if Path(filename).name != filename:
-            raise ValueError("calibrated W3 files must be directly inside the checkpoint")
-        data = (self.directory / filename).read_bytes()  # read once, checked before it is parsed
-        if hashlib.sha256(data).hexdigest() != entry["sha256"]:
-            raise ValueError(f"calibrated W3 checksum mismatch for {name}")
-        tensors = load_bytes(data)
-        expected = {"planes": ((n // 32, k // 128, 3, 32, 4), torch.uint32), "scales": ((n // 32, k // 128, 4, 32), torch.uint8),
-                    "row_scale": ((n,), torch.float32)}
-        if tensors.keys() != expected.keys() or any(tuple(tensors[key].shape) != shape or tensors[key].dtype != dtype
-                                                     for key, (shape, dtype) in expected.items()):
-            raise ValueError(f"invalid calibrated W3 tensors for {name}")
-        levels = _codebook(entry["codebook"])
-        # the fragment tensors index 32 rows by dim 0 and a 128-wide K chunk by dim 1; row scales follow the rows
-        planes, scales = (shard.cols(shard.rows(tensors[key], 32), dim=1) for key in ("planes", "scales"))
-        row_scale = shard.rows(tensors["row_scale"])
-        n, k = row_scale.shape[0], planes.shape[1] * 128
-        if (n, k) != (out_features, in_features):
+        from hibana_amd.kernels import w3
+        entry = self.entry(name)
+        data = read_verified(self.directory / entry.file, entry.sha256, name)
+        part = FragmentTensors.parse(data, entry).cut(shard)
+        if part.shape != (out_features, in_features):
             raise ValueError(f"calibrated W3 shape mismatch for {name}")
-        weight = W3Weight(*(t.contiguous().to(device) for t in (planes, scales, row_scale)), n, k, levels, lut_of(levels))
-        return self._finish(weight, tile)
+        levels = w3._codebook(entry.codebook)
+        on_device = [t.contiguous().to(device) for t in (part.planes, part.scales, part.row_scale)]
+        return self._finish(w3.W3Weight(*on_device, out_features, in_features, levels, w3.lut_of(levels)), tile)

@@ -102,6 +102,13 @@ int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, 
  * reciprocal, whose bits are NVIDIA's. */
 int hb_w3_quant_groups(const void* x, int64_t m, int k, void* q, float* scales, void* stream);
 
+/* The per-row form of the activation rounding: x BF16 [m, k] (k % 8 == 0) -> q E4M3 bytes [m, k], scales float32 [m]:
+ * s = max(amax of the row / 448, 1e-12), q = e4m3(clamp(x / s, -448, 448)), IEEE FP32 divisions. hb_w3_gemm_e4m3 takes
+ * the result with the row's scale repeated over its k / 32 groups.
+ * ref: w3.quant_rows, hibana/kernels/w3.py:326-330 (quant_rows_kernel, hibana/kernels/csrc/w3_gemm.cu:244-288, which
+ * multiplies by a reciprocal where this divides, as hb_w3_quant_groups does). */
+int hb_w3_quant_rows(const void* x, int64_t m, int k, void* q, float* scales, void* stream);
+
 /* hb_w3_gemm on rounded activations, the reference kernel's own arithmetic:
  * y[m, n] = bf16( row_scale[n] * sum_g (x_scale[m, g] * scale[n, g]) * sum_{k in g} xq[m, k] * level[code[n, k]] ),
  * FP8 x FP8 products summed in FP32 a group. xq E4M3 [m, k], x_scale float32 [m, k / 32] as hb_w3_quant_groups makes
@@ -185,10 +192,19 @@ int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int32_t* ids, 
                          const void* x, const float* gate_vec, int e_lo, int e_n, int m, int topk, int h, void* out,
                          void* stream);
 
+/* out BF16 [rows, half] = bf16( bf16(silu(gate)) * up ) from gate_up BF16 [rows, 2 * half]: columns [gate | up]
+ * (pairs == 0) or blocks of `pairs` gate columns alternating with their `pairs` up columns (half % pairs == 0; half and
+ * pairs even). The experts' fc1 epilogues do this inside their launches; this is the standalone op.
+ * ref: ops.silu_and_mul, hibana/kernels/ops.py:86-92. */
+int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int pairs, void* out, void* stream);
+
 /* Softmax top-k routing: logits float32 [m, e] -> ids int32 [m, k] (descending probability, ties to the lower id),
- * weights float32 [m, k] renormalized over the selection.
- * ref: route_topk, hibana/kernels/flashnext_fused.py:278-319 (plain form, no padded-slot table). */
-int hb_route_softmax_topk(const float* logits, int m, int e, int k, int32_t* ids, float* weights, void* stream);
+ * weights float32 [m, k] renormalized over the selection. slots (may be NULL: every row is real): row r is real iff
+ * slots[r / steps] != 0; a padded row gets weight 0 in every slot and the id e ("no expert", which the 3-bit experts
+ * skip) or, repeat != 0, row 0's first choice.
+ * ref: route_topk, hibana/kernels/flashnext_fused.py:278-319. */
+int hb_route_softmax_topk(const float* logits, int m, int e, int k, const int32_t* slots, int steps, int repeat, int32_t* ids,
+                          float* weights, void* stream);
 
 /* Sigmoid top-k routing of the latent MoE on the fused router|fc1_latent GEMM output: fused FP32 [m, stride], columns
  * 0..e-1 the router logits, e..e+latent-1 the latent projection. s = 1 / (1 + exp(-logit)); ids = the k largest of

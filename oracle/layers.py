@@ -25,6 +25,8 @@ points of the reference kept.
                          to follow; the CUDA quantizer of hibana/kernels/csrc/w3_gemm.cu:291-327 multiplies by an
                          approximate reciprocal instead of dividing, so its bits are PARITY UNPINNED here): per (row,
                          32-group) s = max(amax / 448, 1e-12) in FP32, q = e4m3(clamp(x / s, -448, 448))
+  quant_e4m3_rows        hibana/kernels/w3.py:326-330: the same rounding with one scale a row (pinned as quant_e4m3_groups:
+                         the brute-force nearest-value search, and a row of one group equals the group form)
   dense_a8_ref           hibana/kernels/w3.py:340-365 with quantized activations (the reference kernel's own math,
                          hibana/kernels/csrc/w3_gemm.cu:105-108,209-210): x is replaced by q * s
   `quant=` of the expert functions: hibana/kernels/w3_moe.py:193-214 with quant = quant_e4m3 (x and h both rounded)
@@ -70,6 +72,16 @@ def quant_e4m3_groups(t: torch.Tensor):
     s = (g.abs().amax(-1, keepdim=True) / 448.0).clamp_min(1e-12)
     q = (g / s).clamp(-448, 448).to(torch.float8_e4m3fn)
     return q.view(torch.uint8).reshape(m, k), s.reshape(m, k // 32)
+
+
+def quant_e4m3_rows(t: torch.Tensor):
+    """t [M, K] -> (E4M3 bytes uint8 [M, K], scales float32 [M]): one scale a row, s = max(amax of the row / 448, 1e-12),
+    q = e4m3(clamp(x / s, -448, 448)) (hibana/kernels/w3.py:326-330; the CUDA kernel, hibana/kernels/csrc/
+    w3_gemm.cu:244-288, multiplies by a reciprocal: the divisions here are exact, as in quant_e4m3_groups)."""
+    f = t.float()
+    s = (f.abs().amax(-1, keepdim=True) / 448.0).clamp_min(1e-12)
+    q = (f / s).clamp(-448, 448).to(torch.float8_e4m3fn)
+    return q.view(torch.uint8), s.reshape(-1)
 
 
 def dequant_e4m3_groups(q: torch.Tensor, s: torch.Tensor) -> torch.Tensor:

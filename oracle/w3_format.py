@@ -30,10 +30,13 @@ Pinned by (tests/test_oracle_w3.py):
   fit_scales_ratio     with ratios (1.0,) it must reproduce pack's stored scales and codes exactly; per group the fitted
                        loss is never above the ratio-1.0 loss and is the minimum over a brute-force loop on a tiny matrix;
                        the reference's bounds (tests/unit/test_w3_moe_pack.py:35-47: error < 0.25, fitted <= nearest)
-
-PARITY UNPINNED: pack(fit_scales=True) picks, per group, the first of FIT_SCALES whose float32 squared error is strictly
-the least; the error sum's summation order differs between numpy and torch, so an exact tie could resolve differently
-from the reference. Only the reference's error bounds for the fitted variant are held (test_w3_pack.py:57-76).
+  pack(fit_scales=True), fit_scales_ratio, quantize_groups
+                       bit for bit against what the reference's own functions returned on five seeded matrices, among
+                       them a coarse-grid one whose candidates' errors differ only in the last bits and one with groups
+                       built to tie (tests/golden/w3_fit_scales.npz, written by tests/golden/make_fit_fixtures.py). Both
+                       pick, per group, the FIRST candidate whose float32 squared error is strictly the least, and the
+                       error is summed in the order torch's CPU reduction takes over 32 contiguous floats (sum32 below):
+                       with numpy's pairwise order the coarse-grid fixture fails in one group.
 """
 from __future__ import annotations
 
@@ -167,6 +170,18 @@ def dequantize(w3) -> np.ndarray:
     return lv[codes(w3)] * np.repeat(group_scales(w3), GROUP, axis=1)
 
 
+def sum32(err: np.ndarray) -> np.ndarray:
+    """float32 sum over a last axis of 32 in the order the reference's `.sum(-1)` takes on the CPU: element i goes into
+    partial sum i % 8 (ascending i), then the eight partial sums are added in ascending order. Pinned by the fitted-scale
+    fixture: near a tie between two candidate scales the order decides which one wins."""
+    v = np.asarray(err, dtype=np.float32).reshape(*err.shape[:-1], 4, 8)
+    part = ((v[..., 0, :] + v[..., 1, :]) + v[..., 2, :]) + v[..., 3, :]
+    total = part[..., 0]
+    for j in range(1, 8):
+        total = total + part[..., j]
+    return total.astype(np.float32)
+
+
 def _bucketize(x: np.ndarray, mids: np.ndarray) -> np.ndarray:
     """torch.bucketize(x, mids) with right=False: the number of boundaries strictly below x (a value equal to a
     midpoint takes the lower code)."""
@@ -190,7 +205,7 @@ def pack(weight, codebook=None, fit_scales: bool = False):
         for m in FIT_SCALES:
             s = (scale * np.float32(m)).astype(np.float32)
             deq = lv[_bucketize(g / np.maximum(s, np.float32(1e-30))[:, :, None], mids)] * s[:, :, None]
-            err = ((deq - g) ** 2).astype(np.float32).sum(-1, dtype=np.float32)
+            err = sum32(((deq - g) ** 2).astype(np.float32))
             if best is None:
                 best, fitted = err, s
             else:
@@ -234,8 +249,8 @@ def fit_scales_ratio(weight, codebook=None, ratios=tuple(round(0.5 + 0.025 * i, 
     """float32 [N, K] -> (scale bytes uint8 [N, K/32], row scales float32 [N]): per 32-group the stored E4M3 scale among
     e4m3(amax / max|level| * ratio / row scale) over the ratio grid with the smallest squared error at nearest-level codes;
     the first of equal losses stays (hibana/weights/w3_calibration.py:17-37, unit importance; the routed experts'
-    quantizer, hibana/kernels/w3_moe.py:113-124). With ratios == (1.0,) this is `pack`'s scale rule. PARITY UNPINNED for
-    which of two ratios wins when their float32 losses differ in the last bits (summation order)."""
+    quantizer, hibana/kernels/w3_moe.py:113-124). With ratios == (1.0,) this is `pack`'s scale rule. The loss is
+    summed by sum32, the order that decides near-ties as the reference does (pinned by tests/golden/w3_fit_scales.npz)."""
     w = np.asarray(weight, dtype=np.float32)
     n, k = w.shape
     levels = check_codebook(codebook)
@@ -251,7 +266,7 @@ def fit_scales_ratio(weight, codebook=None, ratios=tuple(round(0.5 + 0.025 * i, 
         eff = (e4m3_floats(raw) * row_scale[:, None]).astype(np.float32)
         q = _bucketize(g / np.maximum(eff, np.float32(1e-30))[:, :, None], mids)
         err = (g - lv[q] * eff[:, :, None]).astype(np.float32)
-        loss = (err * err).sum(-1, dtype=np.float32)
+        loss = sum32(err * err)
         better = loss < best_loss
         best_loss = np.where(better, loss, best_loss)
         best = np.where(better, raw, best)

@@ -78,8 +78,10 @@ def test_host_logic_mirrors_the_reference_interface(monkeypatch):
     sw = modelopt.swizzle_block_scales(s)
     assert sw.shape == (256, 8) and (sw.numpy() == onv.swizzle_block_scales(s.numpy())).all()
     assert torch.equal(modelopt.unswizzle_block_scales(sw, 130, 6), s)
-    gu = torch.randn(3, 256)
-    assert torch.allclose(ops.silu_and_mul(gu), layers.silu_and_mul(gu)) and torch.allclose(ops.silu_and_mul(gu, 64), layers.silu_and_mul(gu, 64))
+    with pytest.raises(RuntimeError):
+        ops.silu_and_mul(torch.randn(3, 256).bfloat16())  # a kernel: no CPU path
+    with pytest.raises(ValueError):
+        ops.silu_and_mul(torch.randn(3, 256))  # not BF16
     monkeypatch.delenv("HIBANA_W3_DECODE", raising=False)
     assert not w3.enabled()
     monkeypatch.setenv("HIBANA_W3_DECODE", "1")
@@ -99,8 +101,10 @@ def test_host_logic_mirrors_the_reference_interface(monkeypatch):
         w3.pack_codes(torch.zeros(128, 128, dtype=torch.uint8), torch.zeros(128, 4).to(torch.float8_e4m3fn), torch.ones(128))
     with pytest.raises(ValueError):
         w3.pack_codes(torch.full((128, 128), 9, dtype=torch.uint8), torch.zeros(128, 4).to(torch.float8_e4m3fn), torch.ones(128))
-    with pytest.raises(NotImplementedError):
-        w3.quant_rows(torch.zeros(1, 32))
+    with pytest.raises(ValueError):
+        w3.quant_rows(torch.zeros(1, 32))  # not BF16
+    with pytest.raises(RuntimeError):
+        w3.quant_rows(torch.zeros(1, 32, dtype=torch.bfloat16))  # no CPU path
     with pytest.raises(ValueError):
         w3.quant_groups(torch.zeros(1, 32))  # not BF16
     with pytest.raises(RuntimeError):

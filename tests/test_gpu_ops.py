@@ -1,0 +1,161 @@
+"""The small ops either side of the experts on the GPU: per-row activation rounding, the standalone SiLU-gate, softmax
+routing with a graph's padded rows, the gated-MoE block (`MoeLayer`), attaching calibrated copies to a model."""
+import json
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import layers, w3_format as ow3
+from tests.util import MAX_REL, NORM_REL, errors, oracle_expert_getter, random_experts, random_w3, to_device_w3
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("m,k", [(1, 32), (3, 104), (17, 2048), (64, 5120)])
+def test_quant_rows_matches_the_oracle_bit_for_bit(m, k):
+    from hibana_amd.kernels import w3
+    g = torch.Generator().manual_seed(m + k)
+    x = torch.randn(m, k, generator=g) * torch.logspace(-4, 4, m)[:, None]
+    x[0] = 0 if m > 1 else x[0]  # an all-zero row
+    x[-1, -1] = 3.0e38
+    x = x.bfloat16()
+    want_q, want_s = layers.quant_e4m3_rows(x)
+    q, s = w3.quant_rows(x.cuda())
+    assert q.dtype == torch.float8_e4m3fn and q.shape == (m, k) and s.shape == (m,) and s.dtype == torch.float32
+    assert torch.equal(s.cpu(), want_s)
+    got = q.view(torch.uint8).cpu()
+    same = (got == want_q) | (((got | want_q) & 0x7f) == 0)  # a zero of either sign is a zero
+    assert bool(same.all()), int((~same).sum())
+
+
+def test_w3_linear_takes_per_row_scales():
+    """w3_linear on quant_rows' output is the oracle's product of the row-rounded activations."""
+    from hibana_amd.kernels import w3
+    packed, *_ = random_w3(256, 384, 3)
+    dev = to_device_w3(packed)
+    x = torch.randn(5, 384, generator=torch.Generator().manual_seed(1)).bfloat16()
+    q, s = w3.quant_rows(x.cuda())
+    got = w3.w3_linear(q, dev, s)
+    qo, so = layers.quant_e4m3_rows(x)
+    rounded = qo.view(torch.float8_e4m3fn).float() * so[:, None]
+    want = layers.dense_ref(rounded, ow3.dequantize(packed))
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+
+
+@pytest.mark.parametrize("shape,pairs", [((3, 256), 0), ((3, 256), 64), ((2, 5, 1024), 0), ((7, 1024), 16), ((1, 4), 2)])
+def test_silu_and_mul_matches_the_bf16_tensor_expression(shape, pairs):
+    from hibana_amd.kernels import ops
+    gu = (torch.randn(*shape, generator=torch.Generator().manual_seed(shape[-1] + pairs)) * 3).bfloat16()
+    want = layers.silu_and_mul(gu, pairs)
+    got = ops.silu_and_mul(gu.cuda(), pairs).cpu()
+    assert got.dtype == torch.bfloat16 and got.shape == want.shape
+    # the device exponential may differ from the host's in its last bit: one BF16 unit at most, and rarely
+    off = got.view(torch.int16).int() - want.view(torch.int16).int()
+    assert off.abs().max() <= 1 and (off != 0).float().mean() < 0.01
+    # closed form in FP64 on a few values: silu(g) * u with the two BF16 roundings
+    g64, u64 = (gu[..., :gu.shape[-1] // 2], gu[..., gu.shape[-1] // 2:]) if not pairs else (None, None)
+    if g64 is not None:
+        ref = ((g64.double() / (1 + torch.exp(-g64.double()))).bfloat16().double() * u64.double()).bfloat16()
+        assert (got.view(torch.int16).int() - ref.view(torch.int16).int()).abs().max() <= 1
+
+
+def test_softmax_routing_with_padded_rows():
+    from hibana_amd.kernels import ops
+    g = torch.Generator().manual_seed(4)
+    logits = torch.randn(6, 64, generator=g).cuda()
+    k = 5
+    plain_ids, plain_w = ops.route_topk(logits, k)
+    ref_w, ref_ids = torch.topk(torch.softmax(logits.float().cpu(), -1), k)
+    assert torch.equal(plain_ids.cpu().long(), ref_ids)
+    assert torch.allclose(plain_w.cpu(), ref_w / ref_w.sum(-1, keepdim=True), rtol=1e-5)
+    slots = torch.tensor([3, 0, 9], dtype=torch.int32).cuda()  # request 1 is a graph's padding: rows 2, 3 at two steps a request
+    ids, w = ops.route_topk(logits, k, slots, 2)
+    real = [0, 1, 4, 5]
+    assert torch.equal(ids[real], plain_ids[real]) and torch.equal(w[real], plain_w[real])
+    assert (ids[2:4] == 64).all() and (w[2:4] == 0).all()  # no expert
+    ids, w = ops.route_topk(logits, k, slots, 2, repeat=True)
+    assert (ids[2:4] == plain_ids[0, 0]).all() and (w[2:4] == 0).all()  # row 0's first choice at weight 0
+
+
+@pytest.mark.parametrize("m,mode", [(1, "decode"), (6, "verify"), (40, "prefill")])
+def test_moe_layer_block(m, mode):
+    """`MoeLayer.__call__(x, ctx)`: router GEMM, routing (padded rows of a decode / verify graph name no expert), routed
+    experts, the shared expert given as the reference holds it (two linears, rows [gate; up]), gated combine."""
+    from hibana_amd.kernels import w3
+    from hibana_amd.model.flashnext_moe import MoeLayer, shared_from_linears
+    e, hidden, inter, topk = 16, 256, 128, 4
+    ex, per = random_experts(e, hidden, inter, True, 61)
+    get = oracle_expert_getter(per, True, inter)
+    g = torch.Generator().manual_seed(62 + m)
+    router = (torch.randn(e, hidden, generator=g) * 0.3).bfloat16()
+    gate_vec = torch.randn(1, hidden, generator=g) * 0.05
+    gate_up, *_ = random_w3(2 * inter, hidden, 63)  # rows [gate; up]
+    down, *_ = random_w3(hidden, inter, 64)
+    lin_gu = SimpleNamespace(w3=to_device_w3(gate_up))
+    lin_d = SimpleNamespace(w3=to_device_w3(down))
+    layer = MoeLayer(router.cuda(), gate_vec.cuda(), ex, topk, shared_gate_up=lin_gu, shared_down=lin_d)
+    # the re-stored shared expert dequantizes to the same weights, rows moved
+    fc1 = w3.dequantize(layer.shared.matrix(0, True)).cpu().numpy()
+    gu = ow3.dequantize(gate_up)
+    inverse = np.argsort(layers.fc1_order(inter))
+    assert np.array_equal(fc1[inverse], np.concatenate([gu[inter:], gu[:inter]]))
+    x = torch.randn(m, hidden, generator=g).bfloat16()
+    steps = 2 if mode == "verify" else 1
+    slots = None
+    if mode != "prefill":
+        slots = torch.ones(m // steps, dtype=torch.int32)
+        if m > 1:
+            slots[-1] = 0  # the last request is padding
+    ctx = SimpleNamespace(mode=mode, slots=None if slots is None else slots.cuda(), seq_slots=None if slots is None else slots.cuda(), verify_steps=steps)
+    got = layer(x.cuda(), ctx)
+    ids, weights = layer.route(x.cuda(), ctx)
+    logits = torch.mm(x.cuda(), router.cuda().T).float().cpu()
+    ref_ids = torch.topk(torch.softmax(logits, -1), topk).indices
+    pad = torch.zeros(m, dtype=torch.bool) if slots is None else (slots.repeat_interleave(steps) == 0)
+    assert torch.equal(ids.cpu().long()[~pad], ref_ids[~pad]) and (ids.cpu()[pad] == e).all() and (weights.cpu()[pad] == 0).all()
+    shared_w13 = np.concatenate([gu[inter:], gu[:inter]])  # checkpoint order [up; gate]
+    want = layers.moe_layer_ref(x, ids.cpu().numpy(), weights.cpu(), get, True, shared=(shared_w13, ow3.dequantize(down)), gate_vec=gate_vec.reshape(-1), e_n=e)
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    assert torch.equal(layer(x.cuda(), None), layer(x.cuda(), SimpleNamespace(mode="prefill")))
+
+
+def test_attach_model_takes_calibrated_copies(tmp_path):
+    """attach_model with a W3 checkpoint: every projection gets the checkpoint's copy (tiled), the model's identity is
+    the manifest's digest; a checkpoint that does not cover the model is refused; without one, nearest-level copies."""
+    from hibana_amd.kernels import w3
+    from hibana_amd.weights.w3_checkpoint import CalibratedWeights, save_weight
+    names = ["layers.0.mlp.gate_up", "layers.0.mlp.down"]
+    shapes = [(256, 128), (128, 256)]
+    packed = [random_w3(n, k, 70 + i)[0] for i, (n, k) in enumerate(shapes)]
+    entries = {name: save_weight(tmp_path / f"{i}.safetensors", to_device_w3(p, "cpu")) for i, (name, p) in enumerate(zip(names, packed))}
+    (tmp_path / "manifest.json").write_text(json.dumps({"format": 1, "target_revision": "rev", "weights": entries}))
+
+    class Lin:
+        def __init__(self, n, k, deq):
+            self.out_features, self.in_features, self.w3, self.weight = n, k, None, torch.zeros(1, device="cuda")
+            self._deq = deq
+
+        def dequantize(self):
+            return torch.from_numpy(self._deq).cuda()
+
+    def model():
+        lins = [Lin(n, k, ow3.dequantize(p)) for (n, k), p in zip(shapes, packed)]
+        return SimpleNamespace(linears=lambda: list(zip(names, lins)), revision="rev"), lins
+
+    mdl, lins = model()
+    report = w3.attach_model(mdl, log=lambda *_: None, checkpoint=tmp_path)
+    assert report["matrices"] == 2 and mdl.w3_identity == CalibratedWeights(tmp_path, "rev").identity
+    for lin, p in zip(lins, packed):
+        assert lin.w3.tiled is not None
+        assert np.array_equal(w3.dequantize(lin.w3).cpu().numpy().view(np.uint32), ow3.dequantize(p).view(np.uint32))
+    mdl, lins = model()
+    mdl.linears = lambda: list(zip(names[:1], lins[:1]))
+    with pytest.raises(ValueError, match="every target layer projection"):
+        w3.attach_model(mdl, log=lambda *_: None, checkpoint=tmp_path)
+    mdl, lins = model()
+    report = w3.attach_model(mdl, log=lambda *_: None, codebook="uniform")
+    assert report["matrices"] == 2 and mdl.w3_identity == "nearest:uniform" and all(lin.w3.tiled is not None for lin in lins)

@@ -210,6 +210,28 @@ def test_quant_e4m3_groups_keeps_what_is_already_representable():
     assert torch.equal(L.rounded_e4m3(vals.bfloat16()), vals)
 
 
+def test_quant_e4m3_rows_is_the_same_rounding_with_one_scale_a_row():
+    table = _e4m3_table()
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(5, 96, generator=g) * torch.tensor([1e-3, 0.1, 1.0, 300.0, 1.0])[:, None]).bfloat16()
+    x[4] = 0  # an all-zero row: scale 1e-12, codes zero
+    q, s = L.quant_e4m3_rows(x)
+    assert q.dtype == torch.uint8 and q.shape == (5, 96) and s.shape == (5,) and s.dtype == torch.float32
+    xf = x.float().numpy()
+    for r in range(5):
+        scale = max(np.float32(np.float32(np.abs(xf[r]).max()) / np.float32(448.0)), np.float32(1e-12))
+        assert s[r].item() == scale
+        for i, v in enumerate(xf[r]):
+            want = _nearest_e4m3(min(max(float(np.float32(v) / scale), -448.0), 448.0), table)
+            got = int(q[r, i])
+            assert table[got] == table[want] and (got == want or table[got] == 0), (r, i, v, got, want)
+    # a row that is one 32-group: the per-row and the per-group forms are the same function
+    one = x[:, :32].contiguous()
+    qg, sg = L.quant_e4m3_groups(one)
+    qr, sr = L.quant_e4m3_rows(one)
+    assert torch.equal(qg, qr) and torch.equal(sg.reshape(-1), sr)
+
+
 def test_dense_a8_ref_is_the_dense_product_of_the_rounded_activations():
     g = torch.Generator().manual_seed(2)
     x = torch.randn(3, 64, generator=g).bfloat16()

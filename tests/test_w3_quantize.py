@@ -1,6 +1,8 @@
 """The routed experts' offline quantizer (ratio-grid group scales, nearest level): the oracle pinned against the
 nearest-level `pack` and a brute-force search on the CPU; the shipped `w3_moe.quantize` / `calibrate` against the oracle and
 the reference's own assertions (tests/unit/test_w3_moe_pack.py:35-47 of the reference) on the GPU."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -47,6 +49,96 @@ def test_fitted_scale_is_the_brute_force_minimum():
         return ((w.reshape(128, 4, 32) - levels[q].reshape(128, 4, 32) * eff[:, :, None]) ** 2).sum(-1)
 
     assert (loss(raw) <= loss(one) * (1 + 1e-5)).all()
+
+
+# ---- the fitted-scale searches against what the reference's own functions returned (tests/golden/w3_fit_scales.npz,
+# written in the build container by tests/golden/make_fit_fixtures.py): which candidate wins a near-tie is part of the bits
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "w3_fit_scales.npz")
+CASES = [(name, book) for name in ("gauss0", "gauss1", "grid", "ties") for book in ("lloyd", "uniform", "lloyd2")]
+
+
+@pytest.fixture(scope="module")
+def golden():
+    return np.load(GOLDEN)
+
+
+def _same_bits(a, b):
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    return a.shape == b.shape and a.dtype.itemsize == b.dtype.itemsize and np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+@pytest.mark.parametrize("name,book", CASES)
+def test_oracle_reproduces_the_reference_fitted_scales(golden, name, book):
+    w = golden[f"{name}.weight"]
+    packed = ow3.pack(w, book, fit_scales=True)
+    for part in ("planes", "scales", "row_scale"):
+        assert _same_bits(packed[part], golden[f"{name}.{book}.pack.{part}"]), part
+    raw, row = ow3.fit_scales_ratio(w, book)
+    assert _same_bits(raw, golden[f"{name}.{book}.fit.scales"]) and _same_bits(row, golden[f"{name}.{book}.fit.row_scale"])
+    assert np.array_equal(ow3.quantize_groups(w, raw, row, book), golden[f"{name}.{book}.quantize.codes"])
+
+
+def test_the_golden_cases_hold_near_ties_that_the_summation_order_decides(golden):
+    """With numpy's own (pairwise) float32 sum in place of sum32 at least one group of the coarse-grid case picks another
+    candidate: the fixture does pin the order."""
+    w = golden["grid.weight"]
+    levels = np.asarray(ow3.CODEBOOKS["uniform"], dtype=np.float32)
+    mids = ((levels[1:] + levels[:-1]) / np.float32(2)).astype(np.float32)
+    g = w.reshape(128, 8, 32)
+    scale = (np.abs(g).max(-1) / np.float32(3.5)).astype(np.float32)
+    differs = 0
+    for order in ("sum32", "pairwise"):
+        best = fitted = None
+        for m in ow3.FIT_SCALES:
+            s = (scale * np.float32(m)).astype(np.float32)
+            deq = levels[ow3._bucketize(g / np.maximum(s, np.float32(1e-30))[:, :, None], mids)] * s[:, :, None]
+            sq = ((deq - g) ** 2).astype(np.float32)
+            err = ow3.sum32(sq) if order == "sum32" else sq.sum(-1, dtype=np.float32)
+            if best is None:
+                best, fitted = err, s
+            else:
+                better = err < best
+                best, fitted = np.where(better, err, best), np.where(better, s, fitted)
+        if order == "sum32":
+            kept = fitted
+        else:
+            differs = int((fitted != kept).sum())
+    assert differs >= 1
+
+
+def _shipped_against_golden(golden, name, book, device):
+    from hibana_amd.kernels import w3, w3_moe
+    w = torch.from_numpy(golden[f"{name}.weight"]).to(device)
+    levels = w3._codebook(book)
+    q, stored, row = w3.quantize_rows(w, w3._Levels(levels, device), True)
+    want = ow3.pack(golden[f"{name}.weight"], book, fit_scales=True)  # equal to the golden planes (test above); gives the codes
+    assert np.array_equal(q.cpu().numpy(), ow3.codes(want)) and _same_bits(row.cpu().numpy(), golden[f"{name}.{book}.pack.row_scale"])
+    assert _same_bits(stored.view(torch.uint8).cpu().numpy(), ow3.scale_bytes(want))
+    sc, rs = w3_moe.fit_scales(w, levels)
+    assert _same_bits(sc.view(torch.uint8).cpu().numpy(), golden[f"{name}.{book}.fit.scales"]) and _same_bits(rs.cpu().numpy(), golden[f"{name}.{book}.fit.row_scale"])
+    codes, sc2, rs2 = w3_moe.quantize(w, book)
+    assert codes.dtype == torch.int32 and torch.equal(sc2.view(torch.uint8), sc.view(torch.uint8)) and torch.equal(rs2, rs)
+    assert np.array_equal(codes.cpu().numpy(), golden[f"{name}.{book}.quantize.codes"])
+    return w
+
+
+@pytest.mark.parametrize("name,book", CASES)
+def test_shipped_searches_reproduce_the_reference_on_the_host(golden, name, book):
+    """The searches are torch expressions with a fixed summation order, so they give the same bits on any device; here
+    on the CPU (the packing itself is a GPU kernel)."""
+    _shipped_against_golden(golden, name, book, "cpu")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,book", CASES)
+def test_shipped_pack_reproduces_the_reference_on_the_gpu(golden, name, book):
+    from hibana_amd.kernels import w3
+    w = _shipped_against_golden(golden, name, book, "cuda")
+    packed = w3.pack(w, book, fit_scales=True)
+    for part in ("planes", "scales", "row_scale"):
+        got = getattr(packed, part)
+        got = got.view(torch.int32) if got.dtype == torch.uint32 else got
+        assert _same_bits(got.cpu().numpy(), golden[f"{name}.{book}.pack.{part}"]), part
 
 
 def _nvfp4(e, rows, k, seed):
