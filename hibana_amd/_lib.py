@@ -9,7 +9,7 @@ import torch
 
 LIBRARY = Path(__file__).resolve().parent / "libhibana_hip.so"
 
-HB_OK, HB_EINVAL, HB_ENULL, HB_EWORKSPACE, HB_ELAUNCH = 0, -1, -2, -3, -4
+HB_OK, HB_EINVAL, HB_ENULL, HB_EWORKSPACE, HB_ELAUNCH, HB_ESCRATCH = 0, -1, -2, -3, -4, -5
 
 
 class HbW3Experts(C.Structure):
@@ -46,6 +46,7 @@ SIGNATURES = {
     "hb_w3_moe_workspace_bytes": (_Z, [_I, _I, _EX, _I]),
     "hb_w3_moe": (_I, [_EX, _P, _P, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "hb_w3_moe_layer": (_I, [_EX, _EX, _P, _P, _P, _P, _I, _I, _P, _P, _Z, _P]),
+    "hb_w3_moe_layer_static": (_I, [_EX, _EX, _P, _P, _P, _P, _I, _I, _P, _P]),
     "hb_w3_moe_layer_e4m3": (_I, [_EX, _EX, _P, _P, _P, _P, _I, _I, _P, _P, _Z, _P]),
     "hb_w3_moe_layer_logits": (_I, [_EX, _EX, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P]),
     "hb_w3_moe_layer_logits_e4m3": (_I, [_EX, _EX, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P]),
@@ -80,7 +81,7 @@ def check(code: int, what: str) -> None:
     if code == HB_OK:
         return
     text = lib().hb_error_string(code).decode()
-    if code == HB_EINVAL:
+    if code in (HB_EINVAL, HB_ESCRATCH):
         raise ValueError(f"{what}: {text}")
     raise RuntimeError(f"{what}: {text}")
 

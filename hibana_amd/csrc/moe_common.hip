@@ -812,6 +812,7 @@ extern "C" const char* hb_error_string(int code) {
     case HB_ENULL: return "a required pointer is null";
     case HB_EWORKSPACE: return "workspace too small";
     case HB_ELAUNCH: return "the HIP runtime refused a launch";
+    case HB_ESCRATCH: return "the call needs more scratch than the library's static buffer holds";
     default: return "unknown error";
   }
 }

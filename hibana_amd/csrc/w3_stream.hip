@@ -19,6 +19,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
 
 #include "ring.hpp"
 #include "stream_common.hpp"
@@ -912,6 +913,44 @@ extern "C" int hb_w3_moe_layer_e4m3(const hb_w3_experts* routed, const hb_w3_exp
                                     const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
                                     size_t workspace_bytes, void* stream) {
   return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, nullptr, true);
+}
+
+// ------------------------------------------------------------------------------- the entry point that allocates nothing
+// hb_w3_moe_layer with its workspace in a device array of this library instead of a caller's buffer, for callers that
+// cannot allocate. Every GPU the library runs on holds its own copy of the array at its own address; the array's name
+// is a host-side stand-in, so the address is asked for once a device (hipGetSymbolAddress, with that device current)
+// and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) uint8_t scratch[HB_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int SCRATCH_MAX_DEVICES = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_ptr[SCRATCH_MAX_DEVICES] = {};
+
+// The current device's copy of `scratch`, or null if the runtime will not say where it is.
+void* scratch_of_current_device() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= SCRATCH_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_ptr[device]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    g_scratch_ptr[device] = ptr;
+  }
+  return g_scratch_ptr[device];
+}
+}  // namespace
+
+extern "C" int hb_w3_moe_layer_static(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                                      const int32_t* ids, const float* weights, int m, int topk, void* out, void* stream) {
+  if (int e = check_experts(routed)) return e;
+  if (m <= 0 || topk <= 0) return HB_EINVAL;
+  // sized before anything is touched: the same carve as hb_w3_moe_workspace_bytes
+  if (moe_carve(nullptr, m, topk, routed->experts, routed->inter, routed->hidden_out, shared ? 1 : 0, routed->hidden).bytes > HB_STATIC_SCRATCH_BYTES)
+    return HB_ESCRATCH;
+  void* ptr = scratch_of_current_device();
+  if (!ptr) return HB_ELAUNCH;
+  return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, ptr, HB_STATIC_SCRATCH_BYTES, stream, nullptr);
 }
 
 extern "C" int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,

@@ -27,7 +27,8 @@ enum {
                          4-byte ones (any allocator's blocks do; the calls check) */
   HB_ENULL = -2,      /* a required pointer is NULL */
   HB_EWORKSPACE = -3, /* workspace smaller than hb_*_workspace_bytes() says */
-  HB_ELAUNCH = -4     /* the HIP runtime refused a launch (hipGetLastError is left set for the caller) */
+  HB_ELAUNCH = -4,    /* the HIP runtime refused a launch (hipGetLastError is left set for the caller) */
+  HB_ESCRATCH = -5    /* hb_w3_moe_layer_static: the call needs more scratch than HB_STATIC_SCRATCH_BYTES */
 };
 
 /* Library version (major * 1000 + minor). */
@@ -159,6 +160,21 @@ int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32_t* ids, co
 int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
                     const int32_t* ids, const float* weights, int m, int topk, void* out, void* workspace,
                     size_t workspace_bytes, void* stream);
+
+/* hb_w3_moe_layer for callers that cannot allocate device memory or carry a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same chain of launches and the same bits, with the plan, the
+ * sorted pair list, h and the pair outputs in a device array of HB_STATIC_SCRATCH_BYTES that the library itself holds
+ * (one copy on every GPU it runs on, until the process ends). A call whose hb_w3_moe_workspace_bytes(m, topk, routed,
+ * shared != NULL) exceeds that returns HB_ESCRATCH and enqueues nothing (the benchmark's verify step - 32 tokens, top-10,
+ * 512 experts of 2048 x 512 and a shared one - takes 3.7 MB). It calls no allocator. Nothing in the array has to start
+ * at zero (every launch of the chain writes what it later reads), so nothing is cleared. All calls on one GPU share
+ * the array: two calls that overlap on one GPU (different streams, or replays of graphs holding them) race; on one
+ * stream they are ordered like any other work.
+ * No counterpart in the reference (its op allocates its scratch from torch's caching allocator on every call,
+ * hibana/kernels/csrc/w3_gemm.cu:1234-1247); for the callers above. */
+#define HB_STATIC_SCRATCH_BYTES (8u << 20)
+int hb_w3_moe_layer_static(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                           const int32_t* ids, const float* weights, int m, int topk, void* out, void* stream);
 
 /* hb_w3_moe_layer in the reference kernel's own arithmetic: x and h of the routed experts and of the shared expert go
  * through the activation rounding (hb_w3_quant_groups' arithmetic) before their products, as with HB_MOE_E4M3 in
