@@ -1,6 +1,8 @@
 // Kernels and host helpers shared by every routed-expert call: the expert plan, the combine, softmax top-k routing.
 #include <string.h>
 
+#include <atomic>
+#include <mutex>
 #include <vector>
 
 #include "stream_common.hpp"
@@ -14,7 +16,7 @@ namespace hb {
 // registers as order-preserving 32-bit keys, so a selection round is a register scan, one wave-wide integer maximum
 // (DPP within rows of 16, four scalar reads across them) and a ballot: among equal scores the lowest lane, then the
 // lowest register, wins - the lowest expert id.
-constexpr int ROUTE_PER_LANE = 16;  // up to 1024 experts (instantiated for 8 and 16 registers a lane)
+constexpr int ROUTE_PER_LANE = 16;
 
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
   x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false));   // lane ^ 1
@@ -127,7 +129,7 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane)
       id = p.repeat ? __builtin_amdgcn_readfirstlane(mine_id) : e;
       w = 0.f;
     }
-    p.ids[(int64_t)r * p.k + lane] = id;
+    store_through(&p.ids[(int64_t)r * p.k + lane], id);  // the plan may read it in this very launch, from another workgroup
     p.weights[(int64_t)r * p.k + lane] = w;
   }
 }
@@ -213,7 +215,7 @@ __device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 
 __device__ __forceinline__ void plan_few_pairs(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows, int32_t* __restrict__ plan,
                                                int32_t* __restrict__ order, int slot_rows, int slot_cap) {
   const int lane = threadIdx.x & 63;
-  int e = lane < pairs ? ids[lane] - e_lo : -1;
+  int e = lane < pairs ? load_through(&ids[lane]) - e_lo : -1;
   if (e < 0 || e >= e_n) e = -1;
   int id_bits = 1;
   while ((1 << id_bits) < e_n) id_bits++;
@@ -267,6 +269,7 @@ __device__ __forceinline__ void plan_few_pairs(const int32_t* ids, int pairs, in
     int32_t* entry = plan + PLAN_HEADER + 4 * s;
     entry[0] = entry[1] = entry[2] = entry[3] = 0;
   }
+  for (int s = lane; s < slot_cap; s += 64) plan_done(plan, slot_cap)[s * DONE_PITCH] = 0;
   if (lane == 0) {
     plan[0] = slots;
     plan[1] = distinct;
@@ -274,37 +277,13 @@ __device__ __forceinline__ void plan_few_pairs(const int32_t* ids, int pairs, in
   }
 }
 
-// With `route.logits` set the workgroup first routes the route.m rows itself (softmax top-k, a row a wavefront at a
-// time) into route.ids / route.weights, which `ids` then names.
-//
-// With `job.lanes` set the launch has further workgroups, which round the job's activations to E4M3 and plan nothing.
-//
-// Many pairs (a prefill chunk) are shared among `groups` workgroups in three launches of this kernel, `wide` [groups, e_n]
-// between them: phase 1, each group counts its share of the pairs per expert; phase 2, one workgroup adds the groups'
-// counts, writes the slot table and turns `wide` into the first sorted position of each group's run of each expert;
-// phase 3, each group places its share. Phase 0 is all of it in one workgroup.
+// The plan itself, by one workgroup of PLAN_THREADS (`group` of `groups` when many pairs are shared): `lds` is the
+// launch's dynamic LDS.
 template <bool WIDE>  // false: one workgroup (phase 0) and nothing of the shared form compiled in
-__global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
-                                                                int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
-                                                                int route_rows, int slot_rows, int slot_cap, int32_t* __restrict__ wide, int groups_,
-                                                                int phase_, QuantJob job) {
+__device__ __forceinline__ void plan_work(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows, int32_t* __restrict__ plan,
+                                          int32_t* __restrict__ order, int slot_rows, int slot_cap, int32_t* __restrict__ wide, int groups_, int phase_,
+                                          int group_, int* lds) {
   const int groups = WIDE ? groups_ : 1, phase = WIDE ? phase_ : 0;
-  extern __shared__ int lds[];
-  if (!WIDE && blockIdx.x > 0) {  // the workgroups beside the plan's: the activation rounding, PLAN_THREADS lanes each
-    const int64_t i = (int64_t)(blockIdx.x - 1) * PLAN_THREADS + threadIdx.x;
-    if (i < job.lanes) quant_groups_lane(job.x, i, job.q, job.scales);  // whole groups: four lanes in or out together
-    return;
-  }
-  if (route.logits) {
-    for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
-      if (route.per <= 8) {
-        route_row<false, 8>(route, r, threadIdx.x & 63);
-      } else {
-        route_row<false, 16>(route, r, threadIdx.x & 63);
-      }
-    }
-    __syncthreads();
-  }
   if (!WIDE && pairs <= 64) {  // a decode step: one wavefront plans it
     if (threadIdx.x < 64) plan_few_pairs(ids, pairs, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap);
     return;
@@ -312,7 +291,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   int* seg_count = lds;                         // [PLAN_WAVES][e_n]: pairs of expert e in segment w, then running positions
   int* start = lds + PLAN_WAVES * e_n;          // [e_n]: first sorted position of expert e
   int* scratch = start + e_n;                   // [3 * (PLAN_WAVES + 1)]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, group = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, group = WIDE ? group_ : 0;
   // segment (group, w) = pairs [(group * PLAN_WAVES + w) * seg, ... + seg), seg a multiple of 64
   const int seg = (((pairs + groups - 1) / groups + PLAN_WAVES - 1) / PLAN_WAVES + 63) / 64 * 64;
   const int lo = min(pairs, (group * PLAN_WAVES + wave) * seg), hi = min(pairs, lo + seg);
@@ -326,7 +305,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   int only = -1;  // seg == 64: the local expert of this lane's one pair, kept for the placement (no second read of the ids)
   for (int i0 = lo + lane; phase != 2 && i0 < hi; i0 += 64 * batch) {
     if (batch == 1) {
-      const int e = ids[i0] - e_lo;
+      const int e = load_through(&ids[i0]) - e_lo;
       if (e >= 0 && e < e_n) {
         atomicAdd(&seg_count[wave * e_n + e], 1);
         only = e;
@@ -335,7 +314,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
     }
     int e[PLAN_BATCH];
 #pragma unroll
-    for (int j = 0; j < PLAN_BATCH; j++) e[j] = i0 + 64 * j < hi ? ids[i0 + 64 * j] - e_lo : -1;
+    for (int j = 0; j < PLAN_BATCH; j++) e[j] = i0 + 64 * j < hi ? load_through(&ids[i0 + 64 * j]) - e_lo : -1;
 #pragma unroll
     for (int j = 0; j < PLAN_BATCH; j++)
       if (e[j] >= 0 && e[j] < e_n) atomicAdd(&seg_count[wave * e_n + e[j]], 1);
@@ -424,6 +403,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
     int32_t* entry = plan + PLAN_HEADER + 4 * s;
     entry[0] = entry[1] = entry[2] = entry[3] = 0;
   }
+  for (int s = threadIdx.x; s < slot_cap; s += PLAN_THREADS) plan_done(plan, slot_cap)[s * DONE_PITCH] = 0;
   if (threadIdx.x == 0) {
     plan[0] = slots;
     plan[1] = distinct;
@@ -444,7 +424,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
       if (seg == 64) {  // uniform: one tile a wavefront, read when it was counted
         e = j == 0 ? only : -1;
       } else {
-        e = j < batch && i < hi ? ids[i] - e_lo : -1;
+        e = j < batch && i < hi ? load_through(&ids[i]) - e_lo : -1;
         if (e < 0 || e >= e_n) e = -1;
       }
       eb[j] = e;
@@ -470,6 +450,81 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
     // the read of `base` above and the update by `last` are in the same wavefront; LDS operations of one wavefront
     // execute in program order, and the next tile's reads come after this write
   }
+}
+
+// With `route.logits` set the workgroup first routes the route_rows rows itself (softmax top-k, a row a wavefront at a
+// time) into route.ids / route.weights, which `ids` then names.
+//
+// With `job.lanes` set the launch has further workgroups, which round the job's activations to E4M3 and plan nothing.
+//
+// Many pairs (a prefill chunk) are shared among `groups` workgroups in three launches of this kernel, `wide` [groups, e_n]
+// between them: phase 1, each group counts its share of the pairs per expert; phase 2, one workgroup adds the groups'
+// counts, writes the slot table and turns `wide` into the first sorted position of each group's run of each expert;
+// phase 3, each group places its share. Phase 0 is all of it in one workgroup.
+template <bool WIDE>
+__global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
+                                                                int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
+                                                                int route_rows, int slot_rows, int slot_cap, int32_t* __restrict__ wide, int groups,
+                                                                int phase, QuantJob job) {
+  extern __shared__ int lds[];
+  if (!WIDE && blockIdx.x > 0) {  // the workgroups beside the plan's: the activation rounding
+    quant_job_share(job, blockIdx.x - 1, reinterpret_cast<float*>(lds));
+    return;
+  }
+  if (route.logits) {
+    for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
+      if (route.per <= 8) {
+        route_row<false, 8>(route, r, threadIdx.x & 63);
+      } else {
+        route_row<false, 16>(route, r, threadIdx.x & 63);
+      }
+    }
+    __syncthreads();
+  }
+  plan_work<WIDE>(ids, pairs, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, wide, groups, phase, blockIdx.x, lds);
+}
+
+// Routing and plan of a verify-sized call in ONE launch: `route_groups` workgroups route ROUTE_GROUP_ROWS rows each (a
+// row a wavefront, spread over the device, as the routing launch does), and the one that finishes last plans - it
+// learns that it is the last from a ticket counter of the library (`route_tickets`, zero when the library is loaded and
+// put back to zero by every last arriver, as the split-K counters of the reference's dense kernel are,
+// hibana/kernels/csrc/w3_gemm.cu:230-240). A workgroup's ids are written through to memory and waited for before its
+// ticket is drawn, and the plan reads ids past its own L2 (store_through / load_through): no cache write-back, no
+// invalidate. Launches in flight together draw from different counters
+// (`ticket`: the host hands them out round-robin, ROUTE_TICKETS of them). Workgroups past the routing ones round the
+// job's activations, as in moe_plan_kernel.
+constexpr int ROUTE_TICKETS = 1024;
+constexpr int ROUTE_GROUP_ROWS = 1;
+static __device__ unsigned int route_tickets[ROUTE_TICKETS];
+
+__global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
+                                                                      int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
+                                                                      int route_rows, int route_groups, int ticket, int slot_rows, int slot_cap,
+                                                                      QuantJob job) {
+  extern __shared__ int lds[];
+  __shared__ int last;
+  if ((int)blockIdx.x >= route_groups) {
+    quant_job_share(job, blockIdx.x - route_groups, reinterpret_cast<float*>(lds));
+    return;
+  }
+  const int wave = threadIdx.x >> 6, r = blockIdx.x * ROUTE_GROUP_ROWS + wave;
+  if (wave < ROUTE_GROUP_ROWS && r < route_rows) {
+    if (route.per <= 8) {
+      route_row<false, 8>(route, r, threadIdx.x & 63);
+    } else {
+      route_row<false, 16>(route, r, threadIdx.x & 63);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this row's ids (write-through stores) have reached memory before the ticket is drawn
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned drawn = atomicAdd(&route_tickets[ticket], 1u);
+    last = drawn == (unsigned)route_groups - 1u;
+    if (last) route_tickets[ticket] = 0u;  // every other workgroup of this launch has drawn: the counter is free again
+  }
+  __syncthreads();
+  if (!last) return;  // the last arriver: every row's ids are in memory, and the plan reads them from there (load_through)
+  plan_work<false>(ids, pairs, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, nullptr, 1, 0, 0, lds);
 }
 
 // ---------------------------------------------------------------------------------------------------- combine
@@ -539,9 +594,15 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------- host side
+// The measurement hook's state: `g_events_armed` is all a launch reads while no events are armed (one relaxed load); the
+// list itself is only touched under its lock.
+static std::atomic<bool> g_events_armed{false};
+static std::mutex g_events_lock;
 static std::vector<hipEvent_t> g_events;
 static size_t g_event_next = 0;
 bool moe_next_events(hipEvent_t* start, hipEvent_t* stop) {
+  if (!g_events_armed.load(std::memory_order_relaxed)) return false;
+  std::lock_guard<std::mutex> hold(g_events_lock);
   if (g_event_next + 1 >= g_events.size()) return false;
   *start = g_events[g_event_next];
   *stop = g_events[g_event_next + 1];
@@ -574,7 +635,7 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
     off += align256(bytes);
     return ptr;
   };
-  w.plan = static_cast<int32_t*>(take((PLAN_HEADER + 4 * moe_max_slots(pairs, experts, shared ? m : 0, ROWS_PER_SLOT)) * sizeof(int32_t)));
+  w.plan = static_cast<int32_t*>(take((PLAN_HEADER + (4 + DONE_PITCH) * moe_max_slots(pairs, experts, shared ? m : 0, ROWS_PER_SLOT) + 32) * sizeof(int32_t)));  // entries, then plan_done
   w.plan_wide = static_cast<int32_t*>(take((size_t)PLAN_WIDE_GROUPS * experts * sizeof(int32_t)));
   w.order = static_cast<int32_t*>(take(rows * sizeof(int32_t)));
   w.h = static_cast<uint16_t*>(take((size_t)rows * inter * sizeof(uint16_t)));
@@ -584,14 +645,16 @@ MoeWorkspace moe_carve(void* base, int m, int topk, int experts, int inter, int 
     w.xs = static_cast<float*>(take((size_t)m * (hidden / 32) * sizeof(float)));
     w.hq = static_cast<uint8_t*>(take((size_t)rows * inter));
     w.hs = static_cast<float*>(take((size_t)rows * (inter / 32) * sizeof(float)));
+    w.x2 = static_cast<uint8_t*>(take((size_t)m * 2 * hidden));
+    w.x2s = static_cast<float*>(take((size_t)m * sizeof(float)));
   }
   w.bytes = off;
   return w;
 }
 
 __global__ __launch_bounds__(256) void quant_groups_kernel(QuantJob job) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < job.lanes) quant_groups_lane(job.x, i, job.q, job.scales);
+  __shared__ float red[4];
+  quant_job_share(job, blockIdx.x, red);
 }
 
 // BF16 [m, k] (k % 8 == 0) -> E4M3 codes [m, k] and ONE FP32 scale a row: s = max(amax / 448, 1e-12),
@@ -640,10 +703,22 @@ void moe_launch_quant_rows(const uint16_t* x, int64_t m, int k, uint8_t* q, floa
 }
 
 void moe_launch_quant_groups(const QuantJob& job, hipStream_t stream) {
-  HB_LAUNCH(quant_groups_kernel, dim3((unsigned)((job.lanes + 255) / 256)), dim3(256), 0, stream, job);
+  const unsigned groups = job.split_rows ? (unsigned)job.split_rows : (unsigned)((job.lanes + 255) / 256);
+  HB_LAUNCH(quant_groups_kernel, dim3(groups), dim3(256), 0, stream, job);
 }
 
-static unsigned plan_groups(const QuantJob* job) { return 1u + (job ? (unsigned)((job->lanes + PLAN_THREADS - 1) / PLAN_THREADS) : 0u); }
+static std::atomic<unsigned> g_route_ticket_next{0};
+static std::atomic<int> g_route_plan_fused{0};  // hb_tune("route_plan", 2): routing and plan as two launches
+int moe_tune(const char* key, int value) {
+  if (strcmp(key, "route_plan") || value < 0 || value > 2) return HB_EINVAL;
+  g_route_plan_fused.store(value, std::memory_order_relaxed);
+  return HB_OK;
+}
+
+static unsigned plan_groups(const QuantJob* job) {
+  if (!job) return 1u;
+  return 1u + (job->split_rows ? (unsigned)job->split_rows : (unsigned)((job->lanes + PLAN_THREADS - 1) / PLAN_THREADS));
+}
 
 int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream, int slot_rows,
                     const QuantJob* job) {
@@ -678,12 +753,21 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   rp.ids = ids;
   rp.weights = weights;
   const int64_t pairs = (int64_t)m * topk;
-  if (m > ROUTE_FUSED_ROWS) {  // many rows: a wavefront a row over the whole device, then the plan
+  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
+  if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
+  if (m > ROUTE_FUSED_ROWS && pairs < PLAN_WIDE_PAIRS && g_route_plan_fused.load(std::memory_order_relaxed) != 2) {
+    // a verify-sized call: the routing spread over the device, the plan by the workgroup that finishes last
+    const int groups = (m + ROUTE_GROUP_ROWS - 1) / ROUTE_GROUP_ROWS;
+    const int ticket = (int)(g_route_ticket_next.fetch_add(1u, std::memory_order_relaxed) % ROUTE_TICKETS);
+    HB_LAUNCH(moe_route_plan_kernel, dim3((unsigned)groups + plan_groups(job) - 1u), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n,
+              shared_rows, ws.plan, ws.order, rp, m, groups, ticket, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows),
+              job ? *job : QuantJob{});
+    return HB_OK;
+  }
+  if (m > ROUTE_FUSED_ROWS) {  // a prefill-sized call: a wavefront a row over the whole device, then the plan's launches
     launch_route<false>(rp, m, stream);
     return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, slot_rows, job);
   }
-  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
-  if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
   HB_LAUNCH(moe_plan_kernel<false>, dim3(plan_groups(job)), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order,
             rp, m, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows), ws.plan_wide, 1, 0, job ? *job : QuantJob{});
   return HB_OK;
@@ -796,10 +880,19 @@ extern "C" int hb_route_sigmoid_topk(const float* fused, int64_t stride, const f
   return launch_status();
 }
 
+static std::atomic<int64_t*> g_trace{nullptr};
+int64_t* hb::moe_trace_buffer() { return g_trace.load(std::memory_order_relaxed); }
+extern "C" int hb_debug_trace(void* buffer) {
+  g_trace.store(static_cast<int64_t*>(buffer), std::memory_order_relaxed);
+  return HB_OK;
+}
+
 extern "C" int hb_debug_events(void* const* events, int count) {
   if (count < 0 || (count > 0 && !events)) return HB_EINVAL;
+  std::lock_guard<std::mutex> hold(g_events_lock);
   g_events.assign(reinterpret_cast<hipEvent_t const*>(events), reinterpret_cast<hipEvent_t const*>(events) + count);
   g_event_next = 0;
+  g_events_armed.store(count > 0, std::memory_order_relaxed);
   return HB_OK;
 }
 

@@ -11,6 +11,8 @@
 // Codes expand with v_cvt_scalef32_pk_bf16_fp4 (two weights per instruction, exact).
 #include <string.h>
 
+#include <atomic>
+
 #include "ring.hpp"
 #include "stream_common.hpp"
 #include "tile_kernel.hpp"
@@ -337,14 +339,14 @@ __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
 }
 
 // experiments (hb_tune): the stream's workgroup shape ("nvfp4_ksplit", "nvfp4_nbw"); "nvfp4_tile": 1 forces the tile kernel, 2 the stream
-static int g_nvfp4_ksplit = 0, g_nvfp4_nbw = 0, g_nvfp4_tile = 0, g_nvfp4_few = 0;  // "nvfp4_few": 2 switches off the body for slots of at most eight rows
+static std::atomic<int> g_nvfp4_ksplit{0}, g_nvfp4_nbw{0}, g_nvfp4_tile{0}, g_nvfp4_few{0};  // "nvfp4_few": 2 switches off the body for slots of at most eight rows
 
 template <int EPI>
 static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipStream_t stream) {
   pick_shape(p.n_blocks, p.chunks, busy_slots, 4096, &p.ks, &p.nbw);
   if (g_nvfp4_ksplit) {
     p.ks = g_nvfp4_ksplit;
-    p.nbw = g_nvfp4_nbw ? g_nvfp4_nbw : 1;
+    p.nbw = g_nvfp4_nbw ? g_nvfp4_nbw.load() : 1;
   }
   if (p.ks * p.nbw > 16 || p.ks > p.chunks || (p.ks & (p.ks - 1))) return HB_EINVAL;
   set_split(p);
@@ -519,7 +521,7 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
 }  // namespace
 
 int hb::nvfp4_tune(const char* key, int value) {
-  int* slot = !strcmp(key, "nvfp4_tile") ? &g_nvfp4_tile : !strcmp(key, "nvfp4_ksplit") ? &g_nvfp4_ksplit : !strcmp(key, "nvfp4_nbw") ? &g_nvfp4_nbw
+  std::atomic<int>* slot = !strcmp(key, "nvfp4_tile") ? &g_nvfp4_tile : !strcmp(key, "nvfp4_ksplit") ? &g_nvfp4_ksplit : !strcmp(key, "nvfp4_nbw") ? &g_nvfp4_nbw
               : !strcmp(key, "nvfp4_few") ? &g_nvfp4_few : nullptr;
   if (!slot || value < 0 || value > 16) return HB_EINVAL;
   *slot = value;

@@ -27,7 +27,6 @@ namespace hb {
 constexpr int RING_CHUNKS = 2;
 template <class Ring>
 constexpr int ring_bytes() { return RING_CHUNKS * Ring::BLOCK_BYTES; }
-
 typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
 
 struct RingSource {
@@ -42,9 +41,10 @@ struct RingSource {
 
 // Chunks c0 .. c1 - 1 (at least one) of block row `nb`, through the wavefront's ring, for the slot's rows from row0 (the
 // four-row bodies: row0 .. row0 + 3; the sixteen-row body: all, row0 = 0).
+// `acts`: the body's state (the caller's object when the body keeps results of its own beside the four accumulators).
 template <int EPI, class Acts, class Ring>
 __device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& sl, int row0, int nb, int c0, int c1, int lane, uint8_t* ring,
-                                             f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) {
+                                             f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, Acts& acts) {
   constexpr int BEHIND = Ring::LOADS + Acts::LOADS;
   const int r16 = lane & 15, n = c1 - c0;
   RingSource src;
@@ -53,7 +53,6 @@ __device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& 
   const lds_ptr_t slot0 = (lds_ptr_t)ring, slot1 = (lds_ptr_t)(ring + Ring::BLOCK_BYTES);
   uint32_t codes, scales;  // LDS byte addresses of what the lane reads back from slot 0; the reads select the slot by their offset
   Ring::lanes(src, lane, r16, (uint32_t)(uintptr_t)slot0, codes, scales);
-  Acts acts;
   typename Ring::Chunk ch;
   Ring::request(src, c0, slot0);
   asm volatile("" ::: "memory");  // whatever else the prologue asks for stands behind the first block
@@ -87,6 +86,13 @@ __device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& 
       acts.template step<1, false, false>(ch, i + 1, acc0, acc1, acc2, acc3, sl);
     }
   }
+}
+
+template <int EPI, class Acts, class Ring>
+__device__ __forceinline__ void stream_block(const StreamParams& p, const Slot& sl, int row0, int nb, int c0, int c1, int lane, uint8_t* ring,
+                                             f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) {
+  Acts acts;
+  stream_block<EPI, Acts, Ring>(p, sl, row0, nb, c0, c1, lane, ring, acc0, acc1, acc2, acc3, acts);
 }
 
 }  // namespace hb

@@ -31,6 +31,8 @@ struct StreamParams {
   int64_t a_stride;       // elements between rows
   const uint8_t* aq;      // E4M3 activation mode: codes [rows, a_stride] ...
   const float* aq_scale;  // ... and their scales [rows, a_stride / 32]
+  const uint8_t* a2;      // two-plane form of the BF16 activations (split_row below): [rows, a_stride / 128, 2, 128] E4M3 bytes ...
+  const float* a2_scale;  // ... and one FP32 scale a row; slots of at most four rows read these instead of `a`
   const int32_t* plan;    // grouped calls: slot table
   const int32_t* order;   // grouped calls: sorted position -> pair index
   int m;                  // dense calls: rows
@@ -44,7 +46,35 @@ struct StreamParams {
   int ks, nbw;            // wavefronts per workgroup = ks (K splits) * nbw (64-row blocks)
   int ks_inv, chunks_base, chunks_rem;  // set_split(): ceil(65536 / ks), chunks / ks, chunks % ks
   int no_few;             // W3 stream: slots of at most four rows take the sixteen-row body too
+  int64_t* trace;         // measurement hook (hb_debug_trace): a record a workgroup, else null
+  int32_t* done;          // fc1 and fc2 in one launch: the slots' arrival counters (plan_done), else null
+  int done_need;          // ... and the fc1 workgroups a slot has
 };
+
+// Device-scope accesses that do not rest in the compute die's own L2: a store that is written through to memory, a
+// load that is served from there. A workgroup that has waited for its write-through stores (vmcnt) and then draws a
+// ticket has published them to whichever workgroup draws a later ticket and reads with load_through, on any compute
+// die, without a cache write-back or invalidate of its own.
+__device__ __forceinline__ void store_through(int32_t* at, int32_t v) { __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ int32_t load_through(const int32_t* at) { return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }  // up to 1024 experts (instantiated for 8 and 16 registers a lane)
+
+__device__ __forceinline__ void store_through(uint16_t* at, uint16_t v) { __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// One arrival counter a slot, behind the plan's slot table (`slot_cap`: the table's entries, the launch's upper bound
+// on the slots); the plan leaves them zero. A launch that runs fc1 and fc2 together counts there the fc1 workgroups of
+// a slot that have finished, and the slot's fc2 workgroups wait for all of them.
+// Each counter has a 128-byte line of its own (DONE_PITCH ints apart): the workgroups that poll one slot's counter do
+// not stand in the way of another slot's arrivals.
+constexpr int DONE_PITCH = 32;
+__host__ __device__ inline int32_t* plan_done(int32_t* plan, int64_t slot_cap) { return plan + (PLAN_HEADER + 4 * slot_cap + 31) / 32 * 32; }
+
+// Waits (every lane of the wavefront together) until the counter has reached `need`. The spin is bounded: a count that
+// never comes - it cannot, short of a fault elsewhere - ends the wait after about a second and the results are wrong,
+// but every wavefront still leaves.
+__device__ __forceinline__ void await_count(const int32_t* at, int need) {
+  for (int spins = 0; load_through(at) < need && spins < (1 << 20); spins++) __builtin_amdgcn_s_sleep(8);
+  asm volatile("" ::: "memory");  // what the count guards is read after it
+}
 
 // The epilogue's roundings use the hardware FP32 -> BF16 conversion (round to nearest even).
 __device__ __forceinline__ uint16_t bf16_of(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
@@ -55,6 +85,7 @@ __device__ __forceinline__ float silu(float g) { return __fdividef(g, 1.0f + __e
 
 // What a workgroup needs to know about its slot (up to 16 activation rows of one expert, or of the dense matrix).
 struct Slot {
+  int index;           // which slot of the table (or of the dense call)
   int p0, rows;        // first row (sorted position) and number of rows
   const uint8_t* w;    // the expert's tile-layout matrix
   const float* rs;     // its row scales (formats that have them)
@@ -90,11 +121,14 @@ __device__ __forceinline__ float fc1_value(float y0, float y1) {
 template <int EPI>
 __device__ __forceinline__ void store_out(const StreamParams& p, const Slot& sl, int nb, int t, int i, int r16, float y0, float y1) {
   const int64_t pos = sl.p0 + i;
+  // h goes through to memory: its readers may be workgroups of the same launch on another compute die
   if (EPI == EPI_FC1_GATED) {
-    reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16] = bf16_of(fc1_value<EPI>(y0, y1));
+    store_through(&reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * t + r16], bf16_of(fc1_value<EPI>(y0, y1)));
   } else {
     const int n = nb * 64 + 16 * t + r16;
-    if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
+    if (EPI == EPI_FC1_RELU2) {
+      store_through(&reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n], bf16_of(fc1_value<EPI_FC1_RELU2>(y0, 0.f)));
+    } else if (EPI == EPI_DENSE_RELU2) {
       reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(fc1_value<EPI_FC1_RELU2>(y0, 0.f));
     } else if (EPI == EPI_DENSE) {
       reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + n] = bf16_of(y0);
@@ -174,6 +208,7 @@ __device__ __forceinline__ void quant_emit(const StreamParams& p, const Slot& sl
 template <int EPI>
 __device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
   Slot s;
+  s.index = slot;
   int expert = 0;
   if (epi_dense(EPI)) {
     const int per = p.slot_rows ? p.slot_rows : ROWS_PER_SLOT;
@@ -238,10 +273,11 @@ __device__ __forceinline__ const uint16_t* activation_row(const StreamParams& p,
 // of slot rows r, r + 4, ...), since a group's maximum needs two tiles.
 template <int EPI, bool PER_ROW, int STRIDE = 1024, bool QUANT = false>
 __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& sl, const RowScales& rs, int nb, bool active, int ks, int nbi, float* partial,
-                                             const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2, const f32x4_t& acc3) {
+                                             const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2, const f32x4_t& acc3, int stride_floats = 0) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q = lane >> 4, r16 = lane & 15;
   const int rows = sl.rows;
+  const int stride = stride_floats ? stride_floats : STRIDE;  // floats between the wavefronts' exchange areas (the launch's ring size when it varies)
   if (p.ks == 1) {
     if (!active) return;
     if (QUANT) {
@@ -270,7 +306,7 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
     }
     return;
   }
-  float* mine = partial + (int64_t)wave * STRIDE;
+  float* mine = partial + (int64_t)wave * stride;
   {
     const f32x4_t all[4] = {acc0, acc1, acc2, acc3};
 #pragma unroll
@@ -283,14 +319,14 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
   }
   __syncthreads();
   if (!active) return;
-  const float* first = partial + (int64_t)nbi * p.ks * STRIDE;
+  const float* first = partial + (int64_t)nbi * p.ks * stride;
   if (QUANT) {
     for (int r = ks; r < 4; r += p.ks) {
       if (r >= rows) continue;
       float v[4] = {0.f, 0.f, 0.f, 0.f};
       for (int s = 0; s < p.ks; s++) {
 #pragma unroll
-        for (int t = 0; t < 4; t++) v[t] += first[s * STRIDE + (t * 4 + r) * 64 + lane];
+        for (int t = 0; t < 4; t++) v[t] += first[s * stride + (t * 4 + r) * 64 + lane];
       }
       quant_emit<EPI>(p, sl, rs, nb, r, q, r16, v[0], v[1], v[2], v[3]);
     }
@@ -300,8 +336,8 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
       if (r >= rows) continue;
       float up = 0.f, gate = 0.f;
       for (int s = 0; s < p.ks; s++) {
-        up += first[s * STRIDE + ((2 * t) * 4 + r) * 64 + lane];
-        gate += first[s * STRIDE + ((2 * t + 1) * 4 + r) * 64 + lane];
+        up += first[s * stride + ((2 * t) * 4 + r) * 64 + lane];
+        gate += first[s * stride + ((2 * t + 1) * 4 + r) * 64 + lane];
       }
       emit<EPI, PER_ROW>(p, sl, rs, nb, t, r, q, r16, up, gate);
     }
@@ -310,7 +346,7 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, const Slot& 
       const int t = idx >> 2, r = idx & 3;
       if (r >= rows) continue;
       float v = 0.f;
-      for (int s = 0; s < p.ks; s++) v += first[s * STRIDE + (t * 4 + r) * 64 + lane];
+      for (int s = 0; s < p.ks; s++) v += first[s * stride + (t * 4 + r) * 64 + lane];
       emit<EPI, PER_ROW>(p, sl, rs, nb, t, r, q, r16, v, 0.f);
     }
   }
@@ -350,13 +386,89 @@ __device__ __forceinline__ void quant_groups_lane(const uint16_t* __restrict__ x
   if ((i & 3) == 0) scales[i >> 2] = s;
 }
 
-// A rounding to run beside a plan: `lanes` = values / 8 (0: none).
+// A rounding to run beside a plan: `lanes` = values / 8 (0: none) through quant_groups_lane, or, with split_rows set,
+// the rows of x [split_rows, split_k] through split_row (q: the two planes, scales: one a row).
 struct QuantJob {
   const uint16_t* x;
   int64_t lanes;
   uint8_t* q;
   float* scales;
+  int split_rows, split_k;
 };
+
+// BF16 activations as the sum of two E4M3 values under one FP32 scale a row, for the FP8 matrix cores:
+//   s = amax of the row / 448 rounded up to a power of two, hi = e4m3(x / s), lo = e4m3(x / s - hi),  x = (hi + lo) * s.
+// x / s is exact and has BF16's eight significant bits; hi takes the upper four (rounded to nearest), and what is left is
+// a multiple of x's last place below half a step of hi: four significant bits again, so lo holds it EXACTLY as long as
+// that last place is not below E4M3's smallest step, 2^-9 - true of every element within a factor 1792 of the row's
+// largest; smaller ones are off by at most 2^-10 s, 2^-19 of the largest. Both planes share the scale, so their
+// products add in one accumulator, and the sums are those of the BF16 activations up to the order of the additions. Layout: [row][chunk of 128 k]{ 128 hi bytes, 128 lo bytes }. One workgroup (any number of whole
+// wavefronts) a row; `red`: LDS, one float a wavefront.
+__device__ __forceinline__ void split_row(const uint16_t* __restrict__ x, int k, int64_t row, uint8_t* __restrict__ planes, float* __restrict__ scales,
+                                          float* red) {
+  const uint16_t* xr = x + row * k;
+  const int waves = blockDim.x >> 6;
+  float amax = 0.f;
+  for (int c = 8 * threadIdx.x; c < k; c += 8 * blockDim.x) {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(xr + c);
+#pragma unroll
+    for (int j = 0; j < 4; j++) amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(raw[j] << 16)), fabsf(__uint_as_float(raw[j] & 0xffff0000u))));
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  amax = 0.f;
+  for (int w = 0; w < waves; w++) amax = fmaxf(amax, red[w]);
+  // up to the next power of two (a zero row: the smallest normal), so that every division below is exact
+  const float s = __uint_as_float(max((__float_as_uint(amax / 448.0f) + 0x007fffffu) & 0x7f800000u, 0x00800000u));
+  if (threadIdx.x == 0) scales[row] = s;
+  uint8_t* out = planes + row * 2 * k;
+  for (int c = 8 * threadIdx.x; c < k; c += 8 * blockDim.x) {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(xr + c);
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      v[2 * j] = __uint_as_float(raw[j] << 16);
+      v[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = fminf(fmaxf(v[j] / s, -448.0f), 448.0f);
+    int h0 = 0, h1 = 0;
+    h0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], h0, false);
+    h0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], h0, true);
+    h1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], h1, false);
+    h1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], h1, true);
+    float r[8];
+    r[0] = v[0] - __builtin_amdgcn_cvt_f32_fp8(h0, 0);
+    r[1] = v[1] - __builtin_amdgcn_cvt_f32_fp8(h0, 1);
+    r[2] = v[2] - __builtin_amdgcn_cvt_f32_fp8(h0, 2);
+    r[3] = v[3] - __builtin_amdgcn_cvt_f32_fp8(h0, 3);
+    r[4] = v[4] - __builtin_amdgcn_cvt_f32_fp8(h1, 0);
+    r[5] = v[5] - __builtin_amdgcn_cvt_f32_fp8(h1, 1);
+    r[6] = v[6] - __builtin_amdgcn_cvt_f32_fp8(h1, 2);
+    r[7] = v[7] - __builtin_amdgcn_cvt_f32_fp8(h1, 3);
+    int l0 = 0, l1 = 0;
+    l0 = __builtin_amdgcn_cvt_pk_fp8_f32(r[0], r[1], l0, false);
+    l0 = __builtin_amdgcn_cvt_pk_fp8_f32(r[2], r[3], l0, true);
+    l1 = __builtin_amdgcn_cvt_pk_fp8_f32(r[4], r[5], l1, false);
+    l1 = __builtin_amdgcn_cvt_pk_fp8_f32(r[6], r[7], l1, true);
+    typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+    uint8_t* at = out + (c >> 7) * 256 + (c & 127);
+    *reinterpret_cast<i32x2_t*>(at) = i32x2_t{h0, h1};
+    *reinterpret_cast<i32x2_t*>(at + 128) = i32x2_t{l0, l1};
+  }
+}
+
+// One workgroup's share of a QuantJob: `index` counts the job's workgroups from zero.
+__device__ __forceinline__ void quant_job_share(const QuantJob& job, int index, float* red) {
+  if (job.split_rows) {
+    if (index < job.split_rows) split_row(job.x, job.split_k, index, job.q, job.scales, red);
+    return;
+  }
+  const int64_t i = (int64_t)index * blockDim.x + threadIdx.x;
+  if (i < job.lanes) quant_groups_lane(job.x, i, job.q, job.scales);  // whole groups: four lanes in or out together
+}
 
 // ---------------------------------------------------------------------------------------------------- host side
 // Workspace of a routed call, carved from one caller-owned buffer.
@@ -370,6 +482,8 @@ struct MoeWorkspace {
   float* xs;     // ... and their scales [m, hidden / 32]
   uint8_t* hq;   // the same for h: [(pairs + shared rows), inter], [.., inter / 32]
   float* hs;
+  uint8_t* x2;   // the two-plane form of x (split_row): [m, 2 * hidden] ...
+  float* x2s;    // ... and its scales [m]
   size_t bytes;
 };
 
@@ -423,6 +537,7 @@ __device__ __forceinline__ float combine_shared(float routed, float g, float sha
 // Measurement hook: the caller's next (start, stop) event pair, if any is armed. A kernel launched through HB_LAUNCH
 // then carries the pair: the runtime stamps the two events with that kernel's own begin and end.
 bool moe_next_events(hipEvent_t* start, hipEvent_t* stop);
+int64_t* moe_trace_buffer();  // hb_debug_trace's buffer, or null
 
 #define HB_LAUNCH(kernel, grid, block, lds, stream, ...)                                            \
   do {                                                                                              \
@@ -440,5 +555,7 @@ void pick_shape(int n_blocks, int chunks, int64_t slots, int want, int* ks, int*
 
 // hb_tune keys of the NVFP4 kernels ("nvfp4_tile": 1 forces the tile kernel, 2 the stream, 0 the built-in choice).
 int nvfp4_tune(const char* key, int value);
+// hb_tune keys of the kernels shared by the routed calls ("route_plan": 2 keeps routing and plan in separate launches).
+int moe_tune(const char* key, int value);
 
 }  // namespace hb

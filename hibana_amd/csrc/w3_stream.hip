@@ -19,6 +19,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 
 #include "ring.hpp"
@@ -283,6 +284,91 @@ struct FewActs8 {  // E4M3 activations: eight codes a lane and chunk, and the sc
   }
 };
 
+// The four-row body on the two-plane form of the activations (split_row): E4M3 activations times the codebook's E4M3
+// bytes as v_perm_b32 delivers them, on v_mfma_f32_16x16x32_fp8_fp8 - no conversion of the weights at all. The sixteen
+// MFMA rows carry (32-group parity g) x (plane hi / lo) x (slot row i): A row 8 g + 4 hl + i holds plane hl of slot
+// row i over the k of groups g and g + 2 only. The MFMAs of groups 0 and 1 chain into one accumulator, those of groups
+// 2 and 3 into a second one; lane (q, r16) then holds, for its four slot rows, group q / 2 (second accumulator: 2 + q / 2),
+// plane q % 2, and folds that group's scale. Both planes are in the same units, so everything a lane and its three
+// neighbours in q hold for a slot row adds up: the second accumulator is added to the first after the last chunk and
+// the exchange of finish_few does the rest; the row's activation scale multiplies the result there.
+struct FewSplitActs {
+  typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+  static constexpr int LOADS = 2;
+  u32x2_t held[2][2];   // [chunk parity][the lane's lower / upper group]: eight E4M3 bytes each
+  f32x4_t more[4];      // the second accumulator of each 16-row tile
+  bool upper;           // this lane's A row belongs to groups 1 and 3
+  uint32_t s8;          // where the lane's OUTPUT rows find their group's scale in a tile's scale dword
+  const uint8_t* at;    // the lane's bytes of its lower group in the wavefront's first chunk
+  __device__ __forceinline__ void load(int slot, int i) {
+    held[slot][0] = *reinterpret_cast<const u32x2_t*>(at + (int64_t)i * 256);
+    held[slot][1] = *reinterpret_cast<const u32x2_t*>(at + (int64_t)i * 256 + 64);
+  }
+  template <int EPI>
+  __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int row0, int c0, int n, int lane) {
+    const int q = lane >> 4, r16 = lane & 15;
+    upper = r16 >= 8;
+    s8 = 8 * (q >> 1);
+    at = p.a2 + activation_row_index<EPI>(p, sl, row0 + (r16 & 3)) * (2 * p.a_stride) + (int64_t)c0 * 256 + ((r16 >> 2) & 1) * 128 + (upper ? 32 : 0) + 8 * q;
+#pragma unroll
+    for (int t = 0; t < 4; t++) more[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    load(0, 0);
+    if (n > 1) load(1, 1);
+  }
+  __device__ __forceinline__ void tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const long (&a)[4], f32x4_t& acc, f32x4_t& acc2,
+                                       uint32_t lut_lo, uint32_t lut_hi) const {
+    uint32_t sel[8];
+    w3_selectors(q0, q1, q2, sel);
+    long b[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) b[j] = fp8x8(__builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j]), __builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j + 1]));
+    f32x4_t lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
+    lo = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[0], b[0], lo, 0, 0, 0);
+    hi = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[2], b[2], hi, 0, 0, 0);
+    lo = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[1], b[1], lo, 0, 0, 0);
+    hi = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[3], b[3], hi, 0, 0, 0);
+    const uint32_t mine = scales >> s8;
+    const float s_lo = __builtin_amdgcn_cvt_f32_fp8(mine, 0), s_hi = __builtin_amdgcn_cvt_f32_fp8(mine, 2);
+    acc.x = fmaf(lo.x, s_lo, acc.x);
+    acc.y = fmaf(lo.y, s_lo, acc.y);
+    acc.z = fmaf(lo.z, s_lo, acc.z);
+    acc.w = fmaf(lo.w, s_lo, acc.w);
+    acc2.x = fmaf(hi.x, s_hi, acc2.x);
+    acc2.y = fmaf(hi.y, s_hi, acc2.y);
+    acc2.z = fmaf(hi.z, s_hi, acc2.z);
+    acc2.w = fmaf(hi.w, s_hi, acc2.w);
+  }
+  template <int ODD, bool MORE2, bool MORE1>
+  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+    const long mine_lo = fp8x8(held[ODD][0].x, held[ODD][0].y), mine_hi = fp8x8(held[ODD][1].x, held[ODD][1].y);
+    // MFMA j (group j): the lane's bytes when its A row belongs to that group's parity, zero otherwise
+    const long a[4] = {upper ? 0L : mine_lo, upper ? mine_lo : 0L, upper ? 0L : mine_hi, upper ? mine_hi : 0L};
+    tile(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, a, acc0, more[0], sl.lut_lo, sl.lut_hi);
+    tile(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, a, acc1, more[1], sl.lut_lo, sl.lut_hi);
+    tile(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, a, acc2, more[2], sl.lut_lo, sl.lut_hi);
+    tile(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, a, acc3, more[3], sl.lut_lo, sl.lut_hi);
+    if (MORE2) load(ODD, i + 2);
+  }
+  // after the last chunk: the two accumulators of a tile hold parts of the same sums
+  __device__ __forceinline__ void fold(f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) const {
+    acc0 += more[0];
+    acc1 += more[1];
+    acc2 += more[2];
+    acc3 += more[3];
+  }
+};
+
+// The activation scales of a slot's (up to) four rows, asked for ahead of the weights like the pair indices.
+struct FewScales {
+  float s[FEW_ROWS];
+  template <int EPI>
+  __device__ __forceinline__ void ask(const StreamParams& p, const Slot& sl, int row0) {
+#pragma unroll
+    for (int r = 0; r < FEW_ROWS; r++) s[r] = p.a2_scale[activation_row_index<EPI>(p, sl, row0 + r)];
+  }
+  __device__ __forceinline__ float of(int r) const { return r == 0 ? s[0] : r == 1 ? s[1] : r == 2 ? s[2] : s[3]; }
+};
+
 struct FullActs {  // up to sixteen rows: lane (q, r16) feeds row r16, k 8 q .. 8 q + 7 of every group
   static constexpr int LOADS = 4;
   Rows held;           // one chunk's fragments; each half is asked for again as soon as its groups are done
@@ -385,10 +471,10 @@ struct FullActs8 {
 // multiplies by its tile's row scale (`scale`, asked for before the first chunk); a gated pair's gate comes from the
 // neighbouring tile's lane. Every wavefront of the workgroup must call it when K is split (one workgroup barrier).
 // QUANT (fc1 in the E4M3 activation mode): h leaves as codes and scales; a 32-group is two of the wavefront's DPP rows.
-template <int EPI, bool QUANT = false>
+template <int EPI, bool QUANT = false, bool SCALED = false>  // SCALED: the sums are of the two-plane activations and take their row's scale
 __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl, int row0, float scale, int nb, bool active, int wave, int ks,
                                            int nbi, float* partial, const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2,
-                                           const f32x4_t& acc3, const FewPairs& pairs = FewPairs{}) {
+                                           const f32x4_t& acc3, const FewPairs& pairs = FewPairs{}, const FewScales& xs = FewScales{}) {
   constexpr int STRIDE = RING_BYTES / 4;
   const int lane = threadIdx.x & 63, q = lane >> 4, r16 = lane & 15;
   float* mine = partial + wave * STRIDE;
@@ -415,7 +501,7 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
       v += (at[0] + at[16]) + (at[32] + at[48]);
       at += STRIDE;
     }
-    const float y = v * scale;
+    const float y = SCALED ? v * scale * xs.of(r) : v * scale;
     if (EPI == EPI_FC1_GATED) {
       const float gate = __shfl_xor(y, 16);  // tiles 2 t and 2 t + 1 are a pair's up and gate rows
       if (QUANT) {  // the pairs are in tiles 0 and 2: their two rows of lanes are the group
@@ -443,14 +529,13 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
 // General kernel, any K: one workgroup per (run of p.nbw 64-row blocks, slot), K split p.ks ways across its wavefronts.
 // A8: E4M3 activations (p.aq, p.aq_scale), with the two bodies' FP8 forms; fc1 then writes h as E4M3 codes and
 // scales (p.oq, p.oq_scale), the activation rounding done in its epilogue.
-template <int EPI, bool A8>
-__global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
-  extern __shared__ __align__(16) uint8_t rings[];
-  const Slot sl = slot_of<EPI>(p, blockIdx.y);
-  if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
+// SPLIT: slots of at most four rows read the two-plane form of the activations (p.a2) and run on the FP8 matrix cores.
+// One workgroup's work: slot `sl` (with rows), the run `bx` of p.nbw 64-row blocks; `rings`: the launch's dynamic LDS.
+template <int EPI, bool A8, bool SPLIT>
+__device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Slot& sl, int bx, uint8_t* rings) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: kept in scalars
   const WaveShare share = wave_share(p, wave);
-  const int ks = share.ks, nbi = share.nbi, nb = blockIdx.x * p.nbw + nbi;
+  const int ks = share.ks, nbi = share.nbi, nb = bx * p.nbw + nbi;
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
   uint8_t* ring = rings + wave * RING_BYTES;
@@ -473,6 +558,19 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
       }
       finish_block<EPI, true, RING_BYTES / 4, QUANT>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
     }
+  } else if (SPLIT && sl.rows <= FEW_ROWS) {  // uniform over the workgroup
+    float scale = 0.f;
+    FewPairs pairs{};
+    FewScales xs{};
+    if (active) {
+      scale = sl.rs[nb * 64 + lane];
+      if (EPI == EPI_FC2) pairs.ask(p, sl, 0);
+      xs.ask<EPI>(p, sl, 0);
+      FewSplitActs acts;
+      stream_block<EPI, FewSplitActs, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3, acts);
+      acts.fold(acc0, acc1, acc2, acc3);
+    }
+    finish_few<EPI, false, true>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs, xs);
   } else if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
     float scale = 0.f;
     FewPairs pairs{};
@@ -489,6 +587,84 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
       rs = row_scales<true>(sl, nb, lane & 15);
     }
     finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
+  }
+}
+
+template <int EPI, bool A8, bool SPLIT = false>
+__global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
+  extern __shared__ __align__(16) uint8_t rings[];
+  const Slot sl = slot_of<EPI>(p, blockIdx.y);
+  if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
+  stream_workgroup<EPI, A8, SPLIT>(p, sl, blockIdx.x, rings);
+}
+
+// fc1 and fc2 of a routed call in ONE launch, so that fc2's workgroups fill the compute units that fc1's last, partly
+// empty round of workgroups leaves idle (and no launch boundary lies between the two). The grid is one-dimensional:
+// first every fc1 workgroup (slot-major, the slot table's order), then every fc2 workgroup. A slot's fc2 needs all of
+// the slot's h, that is all `groups1` fc1 workgroups of the slot: each of those, once its h is in memory (write-through
+// stores, waited for), adds one to the slot's arrival counter (plan_done: zero from the plan), and the slot's fc2
+// workgroups ask for their first weight blocks, then wait for the counter before they touch h (await_count, in the
+// bodies' start). fc2 workgroups cannot starve fc1: the hardware starts a grid's workgroups in index order, so when an
+// fc2 workgroup waits, every fc1 workgroup has started, and an fc1 workgroup waits for nothing; should that order ever
+// fail to hold, await_count's bound ends the wait. Same sums in the same order as the two launches: the same bits.
+//
+// Order of the grid: slot-major, fc2 of a slot `lag` slots behind its fc1 - fc1(0) .. fc1(lag - 1), then fc1(s), fc2(s -
+// lag) for s = lag .., then the last `lag` slots' fc2. With `lag` about the slots whose workgroups fill the device once,
+// a slot's fc2 workgroups are started when its fc1 workgroups have had a workgroup's lifetime to finish: they rarely
+// wait, and fc1 and fc2 workgroups of different lengths run side by side instead of in rounds that start and end
+// together. The slots a call does not fill (the table's upper bound is far above them: every pair could name another
+// expert) come last in this order, fc1 and fc2 alike, so their workgroups, short as they are, hold nobody back.
+template <int EPI1, bool SPLIT>
+__global__ __launch_bounds__(1024) void w3_fc12_kernel(StreamParams p1, StreamParams p2, int groups1, int groups2, int slots, int lag) {
+  extern __shared__ __align__(16) uint8_t rings[];
+  int id = blockIdx.x, slot;
+  bool is_fc1;
+  const int head = lag * groups1, both = groups1 + groups2, middle = (slots - lag) * both;
+  if (id < head) {  // the first slots' fc1
+    slot = id / groups1;
+    id -= slot * groups1;
+    is_fc1 = true;
+  } else if (id < head + middle) {  // fc1(s) then fc2(s - lag)
+    id -= head;
+    const int step = id / both;
+    id -= step * both;
+    is_fc1 = id < groups1;
+    slot = is_fc1 ? lag + step : step;
+    if (!is_fc1) id -= groups1;
+  } else {  // the last slots' fc2
+    id -= head + middle;
+    const int step = id / groups2;
+    id -= step * groups2;
+    slot = slots - lag + step;
+    is_fc1 = false;
+  }
+  const int64_t t0 = p1.trace ? (int64_t)wall_clock64() : 0;
+  int64_t t1 = 0;
+  int rows = 0;
+  if (is_fc1) {
+    const Slot sl = slot_of<EPI1>(p1, slot);
+    if (sl.rows <= 0) return;
+    rows = sl.rows;
+    stream_workgroup<EPI1, false, SPLIT>(p1, sl, id, rings);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of h has reached memory
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(&p1.done[slot * DONE_PITCH], 1);
+  } else {
+    const Slot sl = slot_of<EPI_FC2>(p2, slot);
+    if (sl.rows <= 0) return;
+    rows = sl.rows;
+    // one wavefront polls for the workgroup; the others wait at the barrier
+    if (threadIdx.x < 64) await_count(p2.done + slot * DONE_PITCH, p2.done_need);
+    __syncthreads();
+    if (p1.trace) t1 = (int64_t)wall_clock64();
+    stream_workgroup<EPI_FC2, false, false>(p2, sl, id, rings);
+  }
+  if (p1.trace && threadIdx.x == 0) {  // measurement hook: start, end of the wait, end (100 MHz ticks), rows
+    int64_t* rec = p1.trace + 4 * (int64_t)blockIdx.x;
+    rec[0] = t0;
+    rec[1] = t1;
+    rec[2] = (int64_t)wall_clock64();
+    rec[3] = rows | (is_fc1 ? 1 << 16 : 0);
   }
 }
 
@@ -595,8 +771,8 @@ struct TileW3 {
 };
 
 // ---------------------------------------------------------------------------------------------------- host side
-struct Tuning {
-  int w3_tile = 0, w3_few = 0, w3_ksplit = 0, w3_nbw = 0, moe_fc1_ksplit = 0, moe_fc1_nbw = 0, moe_fc2_ksplit = 0, moe_fc2_nbw = 0, moe_one = 0;
+struct Tuning {  // hb_tune's knobs: relaxed atomics, so a knob set from one thread while another launches is a plain race-free read
+  std::atomic<int> w3_tile{0}, w3_few{0}, w3_ksplit{0}, w3_nbw{0}, moe_fc1_ksplit{0}, moe_fc1_nbw{0}, moe_fc2_ksplit{0}, moe_fc2_nbw{0}, moe_one{0}, moe_split{0}, moe_fused{0}, moe_lag{0};
 };
 static Tuning g_tune;
 
@@ -606,8 +782,8 @@ struct Launch {
   int ks, nbw;  // 0: chosen here
 };
 
-template <int EPI>
-static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Launch want, hipStream_t stream) {
+// Chooses the workgroup shape of a launch (p.ks, p.nbw and what follows from them).
+static int shape_stream(StreamParams& p, int64_t busy_slots, Launch want) {
   pick_shape(p.n_blocks, p.chunks, busy_slots, 8192, &p.ks, &p.nbw);
   if (want.ks) {
     p.ks = want.ks;
@@ -617,12 +793,21 @@ static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Lau
   if (p.ks * p.nbw > 16 || p.ks > p.chunks) return HB_EINVAL;
   set_split(p);
   p.no_few = g_tune.w3_few == 2;  // every slot takes the sixteen-row body
+  return HB_OK;
+}
+
+template <int EPI>
+static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Launch want, hipStream_t stream) {
+  if (int e = shape_stream(p, busy_slots, want)) return e;
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
+  const size_t lds = (size_t)waves * RING_BYTES;
   if (p.aq) {
-    HB_LAUNCH((w3_stream_kernel<EPI, true>), grid, dim3(64 * waves), (size_t)waves * RING_BYTES, stream, p);
+    HB_LAUNCH((w3_stream_kernel<EPI, true>), grid, dim3(64 * waves), lds, stream, p);
+  } else if (p.a2 && !p.no_few) {
+    HB_LAUNCH((w3_stream_kernel<EPI, false, true>), grid, dim3(64 * waves), lds, stream, p);
   } else {
-    HB_LAUNCH((w3_stream_kernel<EPI, false>), grid, dim3(64 * waves), (size_t)waves * RING_BYTES, stream, p);
+    HB_LAUNCH((w3_stream_kernel<EPI, false>), grid, dim3(64 * waves), lds, stream, p);
   }
   return HB_OK;
 }
@@ -635,16 +820,17 @@ extern "C" int hb_tune(const char* key, int value) {
   if (!key) return HB_ENULL;
   struct {
     const char* name;
-    int* slot;
+    std::atomic<int>* slot;
   } table[] = {{"w3_tile", &g_tune.w3_tile}, {"w3_few", &g_tune.w3_few}, {"w3_ksplit", &g_tune.w3_ksplit},           {"w3_nbw", &g_tune.w3_nbw},
                {"moe_fc1_ksplit", &g_tune.moe_fc1_ksplit}, {"moe_fc1_nbw", &g_tune.moe_fc1_nbw},
-               {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}, {"moe_one", &g_tune.moe_one}};
+               {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}, {"moe_one", &g_tune.moe_one}, {"moe_split", &g_tune.moe_split}, {"moe_fused", &g_tune.moe_fused}, {"moe_lag", &g_tune.moe_lag}};
   for (auto& t : table)
     if (!strcmp(t.name, key)) {
       if (value < 0 || value > 16) return HB_EINVAL;
       *t.slot = value;
       return HB_OK;
     }
+  if (moe_tune(key, value) == HB_OK) return HB_OK;
   return nvfp4_tune(key, value);
 }
 
@@ -664,7 +850,7 @@ extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* 
   p.m = m;
   p.out = y;
   p.out_stride = n;
-  if (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && tile_serves_dense(m, p.n_blocks))) {
+  if (tile_takes(m, k) && (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && tile_serves_dense(m, p.n_blocks)))) {
     if (int e = launch_tile<TileW3, EPI_DENSE>(p, (m + TILE_ROWS - 1) / TILE_ROWS, m, as_stream(stream))) return e;
     return launch_status();
   }
@@ -678,7 +864,7 @@ extern "C" int hb_w3_quant_groups(const void* x, int64_t m, int k, void* q, floa
   if (!x || !q || !scales) return HB_ENULL;
   if (m <= 0 || k <= 0 || k % 32) return HB_EINVAL;
   if (!aligned(x, 16) || !aligned(q, 8) || !aligned(scales, 4)) return HB_EINVAL;
-  moe_launch_quant_groups(QuantJob{static_cast<const uint16_t*>(x), m * k / 8, static_cast<uint8_t*>(q), scales}, as_stream(stream));
+  moe_launch_quant_groups(QuantJob{static_cast<const uint16_t*>(x), m * k / 8, static_cast<uint8_t*>(q), scales, 0, 0}, as_stream(stream));
   return launch_status();
 }
 
@@ -749,12 +935,16 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows, slot_rows);
   if (slots > 65535) return HB_EINVAL;
   // E4M3 activations: x is rounded by further workgroups of the plan's launch, h in fc1's epilogue
-  const QuantJob xjob{static_cast<const uint16_t*>(x), (int64_t)m * ex->hidden / 8, ws.xq, ws.xs};
+  // weight-only on the stream: x also in its two-plane form, for the slots of at most four rows (fc1 on the FP8 matrix cores)
+  const bool split = !e4m3 && !dense && g_tune.moe_split == 1 && g_tune.w3_few != 2;
+  const QuantJob xjob = split ? QuantJob{static_cast<const uint16_t*>(x), 0, ws.x2, ws.x2s, m, ex->hidden}
+                              : QuantJob{static_cast<const uint16_t*>(x), (int64_t)m * ex->hidden / 8, ws.xq, ws.xs, 0, 0};
+  const QuantJob* job = e4m3 || split ? &xjob : nullptr;
   if (route) {
     if (int e = moe_launch_route_plan(route->logits, m, route->e, topk, route->ids, route->weights, ex->base, ex->experts, shared_rows, ws, stream,
-                                      slot_rows, e4m3 ? &xjob : nullptr))
+                                      slot_rows, job))
       return e;
-  } else if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, shared_rows, ws, stream, slot_rows, e4m3 ? &xjob : nullptr)) {
+  } else if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, shared_rows, ws, stream, slot_rows, job)) {
     return e;
   }
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
@@ -817,12 +1007,43 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
     f2.aq = ws.hq;
     f2.aq_scale = ws.hs;
   }
+  if (split) {
+    p.a2 = ws.x2;
+    p.a2_scale = ws.x2s;
+  }
+  // more than one token, weight-only: fc1 and fc2 as one launch when their workgroups have the same shape
+  if (!e4m3 && m > 1 && g_tune.moe_fused != 2) {
+    StreamParams q1 = p, q2 = f2;
+    if (shape_stream(q1, est, l1) == HB_OK && shape_stream(q2, est, l2) == HB_OK && q1.ks * q1.nbw == q2.ks * q2.nbw) {
+      const int groups1 = (q1.n_blocks + q1.nbw - 1) / q1.nbw, groups2 = (q2.n_blocks + q2.nbw - 1) / q2.nbw;
+      const int64_t total = slots * (groups1 + groups2);
+      if (total <= 0x7fffffff) {
+        q1.done = q2.done = plan_done(ws.plan, slots);
+        q1.trace = moe_trace_buffer();
+        q1.done_need = q2.done_need = groups1;
+        const int waves = q1.ks * q1.nbw;
+        // about the slots whose workgroups fill the device once (four workgroups of four wavefronts a compute unit)
+        const int lag_tuned = g_tune.moe_lag.load();
+        const int lag = (int)std::min<int64_t>(slots, lag_tuned ? 8 * lag_tuned : std::max(8, 2304 / (groups1 + groups2)));
+        const bool use_split = q1.a2 && !q1.no_few;
+        auto launch = [&](auto kernel) { HB_LAUNCH(kernel, dim3((unsigned)total), dim3(64 * waves), (size_t)waves * RING_BYTES, stream, q1, q2, groups1, groups2, (int)slots, lag); };
+        if (ex->gated) {
+          use_split ? launch(w3_fc12_kernel<EPI_FC1_GATED, true>) : launch(w3_fc12_kernel<EPI_FC1_GATED, false>);
+        } else {
+          use_split ? launch(w3_fc12_kernel<EPI_FC1_RELU2, true>) : launch(w3_fc12_kernel<EPI_FC1_RELU2, false>);
+        }
+        if (combine) moe_launch_combine(*combine, stream);
+        return launch_status();
+      }
+    }
+  }
   if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) return e;
   int fc2_ks = l2.ks, fc2_nbw;
   if (!fc2_ks) pick_shape(f2.n_blocks, f2.chunks, est, 8192, &fc2_ks, &fc2_nbw);
   // one token, and a separate fc2 would not split K either: the fused launch makes the same sums
   const int one_waves = (int)slots + (combine && combine->gate_vec && combine->shared ? ONE_GATE_WAVES : 0);
-  if (combine && m == 1 && !e4m3 && one_waves <= ONE_MAX_WAVES && fc2_ks == 1 && g_tune.moe_one != 2) {
+  // (its chain hands the selections' weights from lane to lane: at most 64 of them)
+  if (combine && m == 1 && topk <= 64 && !e4m3 && one_waves <= ONE_MAX_WAVES && fc2_ks == 1 && g_tune.moe_one != 2) {
     f2.ks = 1;
     f2.nbw = 1;
     set_split(f2);

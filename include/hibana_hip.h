@@ -50,6 +50,11 @@ int hb_tune(const char* key, int value);
  * has more than 16 rows. count = 0 switches the hook off. Not for captured graphs. */
 int hb_debug_events(void* const* events, int count);
 
+/* Measurement hook (no counterpart in the reference): `buffer` (device, int64, four values a workgroup of the launch
+ * that runs a routed call's fc1 and fc2 together; NULL switches it off) receives, per workgroup that had rows, its start,
+ * the end of its wait for fc1 (fc2 workgroups; else 0) and its end, in ticks of the 100 MHz device clock, and its rows. */
+int hb_debug_trace(void* buffer);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * W3 format: 3-bit (or 2-bit) codes into an 8-entry E4M3 codebook, one E4M3 scale per 32 weights along K, one FP32
  * multiplier per output row.

@@ -12,17 +12,21 @@ from tests.util import MAX_REL, NORM_REL, errors, oracle_expert_getter, random_e
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["auto", "tile", "stream", "stream16"], autouse=True)
+@pytest.fixture(params=["auto", "tile", "stream", "stream16", "apart", "planes"], autouse=True)
 def kernel_choice(request):
     """Every case runs with the library's own choice between the 128-row MFMA tile kernel and the 16-row weight stream,
-    with each of them forced, and with the stream's body for slots of at most four rows switched off (so those slots
-    take the sixteen-row body, as they do when the activation matrix is too large for a buffer descriptor)."""
+    with each of them forced, with the stream's body for slots of at most four rows switched off (so those slots
+    take the sixteen-row body, as they do when the activation matrix is too large for a buffer descriptor), with fc1
+    and fc2 of a call in launches of their own instead of one ("apart"), and with fc1's slots of at most four rows on the
+    two-plane E4M3 form of the activations and the FP8 matrix cores ("planes")."""
     from hibana_amd import _lib
-    tile, few = {"auto": (0, 0), "tile": (1, 0), "stream": (2, 0), "stream16": (2, 2)}[request.param]
-    assert _lib.lib().hb_tune(b'w3_tile', tile) == 0 and _lib.lib().hb_tune(b'w3_few', few) == 0
+    knobs = {"auto": {}, "tile": {"w3_tile": 1}, "stream": {"w3_tile": 2}, "stream16": {"w3_tile": 2, "w3_few": 2},
+             "apart": {"w3_tile": 2, "moe_fused": 2}, "planes": {"w3_tile": 2, "moe_split": 1}}[request.param]
+    for key, value in knobs.items():
+        assert _lib.lib().hb_tune(key.encode(), value) == 0
     yield request.param
-    _lib.lib().hb_tune(b'w3_tile', 0)
-    _lib.lib().hb_tune(b'w3_few', 0)
+    for key in knobs:
+        _lib.lib().hb_tune(key.encode(), 0)
 
 E, H, I, TOPK = 16, 256, 128, 10
 
@@ -274,6 +278,28 @@ def test_graph_replay_gives_the_eager_bits(gated, m):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(captured, eager)
+
+
+@pytest.mark.parametrize("m", [2, 5, 17, 32, 100])
+def test_one_launch_for_fc1_and_fc2_gives_the_bits_of_two(gated, m):
+    """fc1 and fc2 in one launch (fc2's workgroups wait for their slot's fc1 workgroups) against the two launches: the
+    same sums in the same order."""
+    from hibana_amd import _lib
+    from hibana_amd.kernels import w3_moe
+    ex, _ = gated
+    shared_ex, _ = random_experts(1, H, I, True, 77)
+    x, ids, weights = _inputs(m, TOPK, 40 + m)
+    call = lambda: w3_moe.moe_layer(ex, x.cuda(), ids.cuda(), weights.cuda(), shared=shared_ex)  # noqa: E731
+    _lib.lib().hb_tune(b"moe_fused", 0)
+    one = call()
+    for lag in (1, 16):  # fc2 of a slot right behind its fc1's successor, or far behind
+        _lib.lib().hb_tune(b"moe_lag", lag)
+        assert torch.equal(call(), one)
+    _lib.lib().hb_tune(b"moe_lag", 0)
+    _lib.lib().hb_tune(b"moe_fused", 2)
+    two = call()
+    _lib.lib().hb_tune(b"moe_fused", 0)
+    assert torch.equal(one, two)
 
 
 @pytest.mark.parametrize("m", [819, 820, 2000])
