@@ -7,8 +7,11 @@ expert) on one batch of 32 tokens. Steps cycle through LAYERS distinct layers (e
 its own routing), so every step streams its experts from HBM, not from the 256 MB Infinity Cache. The K timed steps
 are one HIP-graph replay (the way a serving engine issues them), bracketed by synchronizations.
 
-Prints one JSON line: tokens/s, the HBM roofline of the dominant kernel (the fc1 stream) measured live with HIP events,
-and the CPU oracle timed on this host's cores on a bounded sample of the same workload.
+Prints one JSON line: tokens/s (the median of repeated replays of one HIP graph of all steps, with their minimum and
+maximum), the HBM roofline of the dominant kernel (the weight stream: fc1 and fc2 in one launch) measured live with HIP
+events, against the vendor peak and against a plain streaming read measured in the same run, the same layer at one token
+(config 2) as a sub-record `m1`, and the CPU oracle timed on this host's cores on a bounded sample of the same workload
+(whole calls, and the same without the time spent unpacking weights).
 
 The other BASELINE configs are `--config 2` (the same layer at M = 1), `--config 0` / `--config 1` (the w3 / NVFP4 dense
 decode projection, `--rows` for M) and `--config 4` (the NVFP4 latent-MoE layer on a 2048-token prefill chunk, MFMA
@@ -33,7 +36,6 @@ def w3_bytes(n: int, k: int) -> int:
 
 FC1_BYTES, FC2_BYTES = w3_bytes(2 * INTER, HIDDEN), w3_bytes(HIDDEN, INTER)
 EXPERT_BYTES = FC1_BYTES + FC2_BYTES  # 1 290 240
-FC1_TRAFFIC_RATIO = 1.017  # measured HBM bytes / algorithmic bytes of the fc1 launch (counter runs, see the roofline entry)
 
 
 class Hip:
@@ -78,13 +80,17 @@ def cpu_baseline(layer, x, ids, weights, budget_s: float = 15.0):
     xb = x.view(torch.int16).cpu().numpy().view(np.uint16)
     idn, wn = ids.cpu().numpy(), weights.cpu().numpy()
     out, distinct = c_port.moe_layer(routed, xb, idn, wn, sh)  # warm-up, and the result the GPU is compared with below
-    calls, spent = 0, 0.0
+    calls, spent, unpacking = 0, 0.0, 0.0
     while spent < budget_s and calls < 50:
         t0 = time.perf_counter()
         c_port.moe_layer(routed, xb, idn, wn, sh)
         spent += time.perf_counter() - t0
+        unpacking += c_port.last_unpack_seconds()
         calls += 1
     info = {"value": x.shape[0] * calls / spent, "unit": "tokens/s", "cores": c_port.threads(), "kind": "port",
+            "matmul_only": {"value": x.shape[0] * calls / max(spent - unpacking, 1e-9), "unit": "tokens/s",
+                            "what": "the same calls without the time spent unpacking weights (weights as if pre-dequantized)"},
+            "unpack_share": unpacking / spent,
             "sample": f"{calls} whole layer calls of {x.shape[0]} tokens on layer 0 ({distinct} distinct experts + shared): C/OpenMP oracle, "
                       f"unpack from the checkpoint layout + FP32 matmul"}
     return info, torch.from_numpy(out.view(np.int16).copy()).view(torch.bfloat16)
@@ -107,7 +113,7 @@ def latent_prefill(args) -> int:
     torch.cuda.set_device(dev)
     tokens, hidden, latent, inter, experts, topk = 2048, 4096, 1024, 2688, 512, 22
     g = torch.Generator(device=dev).manual_seed(5)
-    ex = synthetic.nvfp4_experts(experts, latent, inter, 11, dev)
+    ex = synthetic.nvfp4_experts(experts, latent, inter, 11, dev, keep=not args.no_cpu)
     router = torch.randn(experts, hidden, device=dev, generator=g) * (1.0 / hidden ** 0.5)  # logits ~ N(0, 1) for x ~ N(0, 1)
     fc1 = torch.randn(latent, hidden, device=dev, generator=g) * 0.02
     fc2 = (torch.randn(hidden, latent, device=dev, generator=g) * 0.02).bfloat16()
@@ -133,30 +139,68 @@ def latent_prefill(args) -> int:
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         outs = [block(x) for _ in range(steps)]
-    graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    graph.replay()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    times = replay_times(graph, steps)
+    elapsed = median(times) * 1e-3 * steps
     del outs
     gemm_flops = tokens * topk * 2 * inter * latent  # one expert GEMM (fc1 or fc2), useful flops
     fc1_ms = mean(per_kernel["fc1"])
+    cpu, check = None, None
+    if not args.no_cpu:
+        cpu, check = latent_cpu_leg(block, ex, fc1.bfloat16().cpu(), fc2.cpu(), x, latent, inter)
     line = {
         "metric": "NVFP4 latent-MoE layer tokens/s on a 2048-token prefill chunk, with achieved MFMA TFLOP/s",
         "value": tokens * steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
-        "ms_per_step": elapsed / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "ms_per_step": elapsed / steps * 1e3, "ms_per_step_min": times[0], "ms_per_step_max": times[-1], "replays": len(times),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "BASELINE config 4: NVFP4 latent-MoE layer, 2048 tokens, hidden 4096 -> latent 1024, 512 experts x inter 2688, "
-                               "ReLU^2, top-22 sigmoid routing of N(0,1) logits, no shared expert", "timed_as": "one HIP-graph replay of all steps"},
+                               "ReLU^2, top-22 sigmoid routing of N(0,1) logits, no shared expert",
+                   "timed_as": "replays of one HIP graph of all steps; value and ms_per_step are the median replay"},
         "roofline": {"bound": "mfma", "kernel": "tile_kernel<TileNvfp4, fc1 relu2>", "achieved": gemm_flops / (fc1_ms * 1e-3) / 1e12,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": None, "launch_flops": gemm_flops, "launch_ms": fc1_ms},
         "layer_chain": {"kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
-        "cpu_baseline": None,
+        "cpu_baseline": cpu,
+        "parity": check,
     }
     print(json.dumps(line))
     return 0
+
+
+def latent_cpu_leg(block, ex, fc1, fc2, x, latent: int, inter: int, rows: int = 12):
+    """The CPU oracle of the latent-MoE block (oracle/layers.py: per distinct expert, unpack the NVFP4 matrices, BF16
+    linears with FP32 accumulation, ReLU^2, weighted FP32 sum, then the latent projection back) on a seeded sample of
+    `rows` token rows - a row's output depends on its own experts only - timed on this host's cores, and the GPU's rows
+    against it."""
+    import numpy as np
+    import torch
+
+    from oracle import layers, nvfp4_format as onv
+    dev = x.device
+    sample = torch.randperm(x.shape[0], generator=torch.Generator().manual_seed(1))[:rows].sort().values
+    fused = torch.mm(x, block.gate_fc1.T, out_dtype=torch.float32)
+    ids, w, _ = block.route(fused)
+    got = block(x)[sample.to(dev)].cpu()
+    host = {}  # the experts the sample names, as the checkpoint holds them, copied before the clock starts
+    for i in torch.unique(ids[sample.to(dev)]).tolist():
+        host[i] = (ex.w1[i].cpu().numpy(), ex.s1[i].view(torch.uint8).cpu().numpy(), float(ex.alpha1[i]), ex.w2[i].cpu().numpy(),
+                   ex.s2[i].view(torch.uint8).cpu().numpy(), float(ex.alpha2[i]))
+
+    def get(i):
+        w1, s1, a1, w2, s2, a2 = host[i]
+        return (onv.unpack_fp4(w1, onv.unswizzle_block_scales(s1, inter, latent // 16)), np.float32(a1),
+                onv.unpack_fp4(w2, onv.unswizzle_block_scales(s2, latent, inter // 16)), np.float32(a2))
+
+    xs, ids_s, w_s = x[sample.to(dev)].cpu(), ids[sample.to(dev)].cpu().numpy(), w[sample.to(dev)].cpu()
+    t0 = time.perf_counter()
+    want = layers.latent_moe_ref(xs, fc1, fc2, ids_s, w_s, get)
+    spent = time.perf_counter() - t0
+    cpu = {"value": rows / spent, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"{rows} seeded token rows of the 2048 ({len(host)} distinct experts): numpy / torch oracle, unpack from the checkpoint layout + "
+                     f"matmuls, one call of {spent:.1f} s"}
+    a, e = got.double(), want.double()
+    check = {"rows_checked": rows, "max_rel_vs_cpu_oracle": float((a - e).abs().max() / e.abs().max()), "norm_rel_vs_cpu_oracle": float((a - e).norm() / e.norm())}
+    return cpu, check
 
 
 def dense_decode(args) -> int:
@@ -175,8 +219,9 @@ def dense_decode(args) -> int:
     m = args.rows
     if args.config == 0:
         n = k = 5120
-        mats = [w3.tile(synthetic.w3_matrix(n, k, 40 + i, dev, "uniform"), release=True) for i in range(args.layers)]
         nbytes = w3_bytes(n, k)
+        args.layers = max(args.layers, -(-320_000_000 // nbytes))  # more than the 256 MB Infinity Cache holds, so that every step streams from HBM
+        mats = [w3.tile(synthetic.w3_matrix(n, k, 40 + i, dev, "uniform"), release=True) for i in range(args.layers)]
         x = torch.randn(m, k, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
 
         def step(i: int):
@@ -218,25 +263,118 @@ def dense_decode(args) -> int:
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         outs = [step(i) for i in range(args.steps)]
-    graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    graph.replay()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    times = replay_times(graph, args.steps)
+    elapsed = median(times) * 1e-3 * args.steps
     del outs
     achieved = nbytes / (kernel_ms * 1e-3) / 1e9
     line = {
         "metric": "dense decode projection tokens/s, with achieved HBM GB/s", "value": m * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "ms_per_step_min": times[0], "ms_per_step_max": times[-1],
+        "replays": len(times), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": what, "matrices_cycled": args.layers, "timed_as": "one HIP-graph replay of all steps"},
+        "config": {"workload": what, "matrices_cycled": args.layers, "timed_as": "replays of one HIP graph of all steps; median replay"},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": None, "launch_bytes": nbytes, "launch_ms": kernel_ms},
         "cpu_baseline": None,
     }
     print(json.dumps(line))
     return 0
+
+
+def replay_times(graph, steps: int, floor_s: float = 0.2, least: int = 5):
+    """Per-step milliseconds of repeated replays of a graph of `steps` steps: at least `least` replays and at least
+    `floor_s` seconds of them, each bracketed by synchronizations."""
+    import torch
+    graph.replay()  # untimed: the first replay uploads the graph
+    torch.cuda.synchronize()
+    out, total = [], 0.0
+    while len(out) < least or total < floor_s:
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        out.append(dt / steps * 1e3)
+        total += dt
+    return sorted(out)
+
+
+def median(values):
+    v = sorted(values)
+    return v[len(v) // 2] if len(v) % 2 else 0.5 * (v[len(v) // 2 - 1] + v[len(v) // 2])
+
+
+def stream_read_gbs(dev, mib: int = 1024) -> float:
+    """What a kernel that only reads gets from this device's memory: a plain 128-bit-load streaming read of `mib` MiB
+    (hb_debug_stream_read), median of seven runs timed with events on the stream it runs on."""
+    import torch
+
+    from hibana_amd import _lib
+    src = torch.empty(mib << 20, dtype=torch.uint8, device=dev).random_()
+    sink = torch.zeros((mib << 20) // 65536 + 1, dtype=torch.int32, device=dev)
+    times = []
+    for i in range(9):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _lib.check(_lib.lib().hb_debug_stream_read(_lib.ptr(src), src.numel(), _lib.ptr(sink), _lib.stream()), "stream read")
+        e1.record()
+        torch.cuda.synchronize()
+        if i >= 2:
+            times.append(e0.elapsed_time(e1))
+    return src.numel() / (median(times) * 1e-3) / 1e9
+
+
+def traffic_ratio():
+    """HBM bytes a launch / algorithmic bytes of the fc1 + fc2 launch, from the committed counter summary (two rocprofv3
+    --pmc runs scaled by a plain copy of known size); None when the summary does not state it."""
+    import os
+    import re
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "w3_moe_layer_config3_hbm_traffic.md")
+    try:
+        found = re.search(r"^traffic_ratio_fc1_fc2\s*=\s*([0-9.]+)", open(path).read(), re.M)
+    except OSError:
+        return None
+    return float(found.group(1)) if found else None
+
+
+def measure_layer(args, layers, x, logits, m: int, hip, with_kernels: bool = True):
+    """Replays and per-kernel times of the w3 MoE layer on `m` tokens (x, per-layer logits)."""
+    import torch
+
+    from hibana_amd import _lib
+    from hibana_amd.kernels import w3_moe
+
+    def step(i: int):
+        return w3_moe.moe_layer_logits(layers[i % args.layers][0], x, logits[i % args.layers], TOPK, shared=layers[i % args.layers][1], e4m3=args.e4m3)
+
+    for i in range(max(args.warmup, args.layers)):  # untimed: also builds every layer's tiled weights and warms the allocator
+        step(i)
+    torch.cuda.synchronize()
+    # live kernel timing: each kernel of the chain is launched with its own (start, stop) HIP event pair, which the
+    # runtime stamps with that kernel's begin and end on the stream it runs on
+    if m == 1:
+        names = ["route + plan", "fc1", "fc2 + combine"]  # up to 4 rows are routed by the plan's workgroup; one token's fc2 and combine are one launch
+    elif args.e4m3:
+        names = ["route + plan", "fc1", "fc2", "combine"]
+    else:
+        names = ["route + plan", "fc1 + fc2", "combine"]  # the last routing workgroup plans; fc2's workgroups wait for their slot's fc1 inside one launch
+    per_kernel = {n: [] for n in names}
+    for rep in range(5):
+        for i in range(args.layers):
+            evs = hip.events(2 * len(names))
+            _lib.check(_lib.lib().hb_debug_events(evs, len(evs)), "events")
+            step(i)
+            _lib.lib().hb_debug_events(None, 0)
+            torch.cuda.synchronize()
+            ms = [hip.elapsed_ms(evs[2 * j], evs[2 * j + 1]) for j in range(len(names))]
+            if rep:  # the first sweep is untimed
+                for n, v in zip(names, ms):
+                    per_kernel[n].append(v)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = [step(i) for i in range(args.steps)]
+    times = replay_times(graph, args.steps)
+    del outs, graph
+    return times, {n: sum(v) / len(v) for n, v in per_kernel.items()}
 
 
 def main() -> int:
@@ -247,8 +385,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=6, help="distinct layers the steps cycle through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--config", type=int, default=3, choices=(0, 1, 2, 3, 4),
-                    help="3: the headline w3 verify-batch layer; 2: the same layer at M = 1 with N(0,1) logits; 0 / 1: the w3 / NVFP4 dense decode "
-                         "projection; 4: the NVFP4 prefill layer")
+                    help="3: the headline w3 verify-batch layer (with the M = 1 layer as a sub-record); 2: the same layer at M = 1 alone; 0 / 1: the "
+                         "w3 / NVFP4 dense decode projection; 4: the NVFP4 prefill layer")
     ap.add_argument("--rows", type=int, default=1, help="configs 0 and 1: activation rows M")
     ap.add_argument("--e4m3", action="store_true", help="configs 2 and 3: the reference kernel's own arithmetic (activations rounded to E4M3 per "
                     "32-group, FP8 MFMA) instead of the weight-only form; no CPU leg")
@@ -260,7 +398,7 @@ def main() -> int:
         return 2
     import torch
 
-    from hibana_amd import _lib, synthetic
+    from hibana_amd import synthetic
     from hibana_amd.kernels import ops, w3_moe
 
     if not torch.cuda.is_available():
@@ -281,57 +419,39 @@ def main() -> int:
         keep = i == 0 and not args.no_cpu  # the CPU leg reads layer 0 in the checkpoint layout
         layers.append((synthetic.w3_experts(EXPERTS, HIDDEN, INTER, True, 100 + i, dev, release=not keep),
                        synthetic.w3_experts(1, HIDDEN, INTER, True, 900 + i, dev, release=not keep)))
-    if decode:
-        logits = [torch.randn(m, EXPERTS, generator=torch.Generator().manual_seed(3000 + i)).to(dev) for i in range(args.layers)]
-    else:
-        logits = [synthetic.zipf_logits(m, EXPERTS, ZIPF, 3000 + i, dev) for i in range(args.layers)]
+    one_logits = [torch.randn(1, EXPERTS, generator=torch.Generator().manual_seed(3000 + i)).to(dev) for i in range(args.layers)]
+    logits = one_logits if decode else [synthetic.zipf_logits(m, EXPERTS, ZIPF, 3000 + i, dev) for i in range(args.layers)]
     x = torch.randn(m, HIDDEN, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
     torch.cuda.synchronize()
-
-    def step(i: int):
-        return w3_moe.moe_layer_logits(layers[i % args.layers][0], x, logits[i % args.layers], TOPK, shared=layers[i % args.layers][1], e4m3=args.e4m3)
-
-    distinct = [int(torch.unique(ops.route_topk(lg, TOPK)[0]).numel()) for lg in logits]
-    for i in range(max(args.warmup, args.layers)):  # untimed: also builds every layer's tiled weights and warms the allocator
-        step(i)
-    torch.cuda.synchronize()
-
-    # live kernel timing: each kernel of the chain is launched with its own (start, stop) HIP event pair, which the
-    # runtime stamps with that kernel's begin and end on the stream it runs on
     hip = Hip()
-    names = (["route + plan", "fc1", "fc2 + combine"] if decode else ["route", "plan", "fc1", "fc2", "combine"])  # up to 4 rows are routed by the plan's workgroup; one token's fc2 and combine are one launch
-    per_kernel = {n: [] for n in names}
-    reps = 5
-    for rep in range(reps):
-        for i in range(args.layers):
-            evs = hip.events(2 * len(names))
-            _lib.check(_lib.lib().hb_debug_events(evs, len(evs)), "events")
-            step(i)
-            _lib.lib().hb_debug_events(None, 0)
-            torch.cuda.synchronize()
-            ms = [hip.elapsed_ms(evs[2 * j], evs[2 * j + 1]) for j in range(len(names))]
-            if rep:  # the first sweep is untimed
-                for n, v in zip(names, ms):
-                    per_kernel[n].append(v)
+    distinct = [int(torch.unique(ops.route_topk(lg, TOPK)[0]).numel()) for lg in logits]
     mean = lambda v: sum(v) / len(v)  # noqa: E731
-    fc1_ms = mean(per_kernel["fc1"])
-    fc1_launch_bytes = mean([(d + 1) * FC1_BYTES for d in distinct])
-    achieved = fc1_launch_bytes / (fc1_ms * 1e-3) / 1e9
 
-    # the timed region: K steps as one graph replay
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        outs = [step(i) for i in range(args.steps)]
-    graph.replay()  # untimed: the first replay uploads the graph
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    graph.replay()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    del outs
-    ms_per_step = elapsed / args.steps * 1e3
+    times, kernel_ms = measure_layer(args, layers, x, logits, m, hip)
+    ms_per_step = median(times)
     step_bytes = mean([(distinct[i % args.layers] + 1) * EXPERT_BYTES + 2 * m * HIDDEN * 2 for i in range(args.steps)])
     chain_gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
+    # the dominant kernel: the weight stream - one launch for fc1 and fc2 (every distinct expert's and the shared expert's
+    # two matrices, read once), or, at one token and in the E4M3 mode, fc1's launch
+    fused = "fc1 + fc2" in kernel_ms
+    dominant = "fc1 + fc2" if fused else "fc1"
+    launch_bytes = mean([(d + 1) * (EXPERT_BYTES if fused else FC1_BYTES) for d in distinct])
+    launch_ms = kernel_ms[dominant]
+    achieved = launch_bytes / (launch_ms * 1e-3) / 1e9
+    kernel_name = ("w3_fc12_kernel<fc1 gated + fc2>" if fused else "w3_stream_kernel<fc1 gated, E4M3>" if args.e4m3 else "w3_stream_kernel<fc1 gated>")
+    read_gbs = stream_read_gbs(dev)
+
+    m1 = None
+    if not decode:  # the other half of the metric, in the same run: the layer at one token
+        x1 = x[:1].contiguous()
+        d1 = [int(torch.unique(ops.route_topk(lg, TOPK)[0]).numel()) for lg in one_logits]
+        t1, k1 = measure_layer(args, layers, x1, one_logits, 1, hip)
+        b1 = mean([(d + 1) * EXPERT_BYTES + 2 * HIDDEN * 2 for d in d1])
+        ms1 = median(t1)
+        m1 = {"workload": "BASELINE config 2: the same layer at 1 token, top-10 of N(0,1) logits", "value": 1.0 / (ms1 * 1e-3), "unit": "tokens/s",
+              "ms_per_step": ms1, "ms_per_step_min": t1[0], "ms_per_step_max": t1[-1], "replays": len(t1), "distinct_experts_per_step": mean(d1),
+              "algorithmic_bytes_per_step": b1, "achieved_GBs": b1 / (ms1 * 1e-3) / 1e9, "frac_of_hbm_peak": b1 / (ms1 * 1e-3) / 1e9 / HBM_PEAK_GBS,
+              "kernel_ms": k1}
 
     if args.copy_mib:
         src = torch.empty(args.copy_mib << 20, dtype=torch.uint8, device=dev).random_()
@@ -345,24 +465,30 @@ def main() -> int:
         got = w3_moe.moe_layer(layers[0][0], x, ids0, w0, shared=layers[0][1]).float().cpu()
         check = {"max_rel_vs_cpu_oracle": float((got - want.float()).abs().max() / want.float().abs().max()),
                  "norm_rel_vs_cpu_oracle": float((got - want.float()).norm() / want.float().norm())}
+    ratio = None if decode or args.e4m3 or not fused else traffic_ratio()
     line = {
         "metric": ("w3 MoE layer tokens/s at decode (M=1), with achieved HBM GB/s" if decode else
                    "w3 MoE layer tokens/s at the verify batch (M=32), with achieved HBM GB/s") + (" [E4M3 activation mode]" if args.e4m3 else ""),
-        "value": m * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8" if args.e4m3 else "bf16",
+        "value": m / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "ms_per_step_min": times[0], "ms_per_step_max": times[-1], "replays": len(times),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8" if args.e4m3 else "bf16",
         "data": "synthetic",
         "config": {"workload": ("BASELINE config 2: w3 MoE layer, 1 token, hidden 2048, 512 experts x inter 512 + 1 shared, top-10 of N(0,1) logits, "
                                 "SiLU-gated, codebook lloyd") if decode else
                                ("BASELINE config 3: w3 MoE layer, 32 tokens (4 seq x 8 draft), hidden 2048, 512 experts x inter 512 + 1 shared, "
                                 "top-10 Zipf(1.1) routing, SiLU-gated, codebook lloyd"),
-                   "layers_cycled": args.layers, "distinct_experts_per_step": mean(distinct), "timed_as": "one HIP-graph replay of all steps"},
-        "roofline": {"bound": "hbm", "kernel": "w3_stream_kernel<fc1 gated, E4M3>" if args.e4m3 else "w3_stream_kernel<fc1 gated>", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                   "layers_cycled": args.layers, "distinct_experts_per_step": mean(distinct),
+                   "timed_as": "replays of one HIP graph of all steps; value and ms_per_step are the median replay"},
+        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      # HBM bytes a launch: the ratio of scaled FETCH_SIZE + WRITE_SIZE to the algorithmic bytes measured with
-                     # rocprofv3 --pmc on this workload (summary kept under profiles/), applied to this run's bytes
-                     "traffic": None if decode or args.e4m3 else FC1_TRAFFIC_RATIO * fc1_launch_bytes, "launch_bytes": fc1_launch_bytes, "launch_ms": fc1_ms},
+                     # rocprofv3 --pmc on this workload (the summary under profiles/ states it), applied to this run's bytes
+                     "traffic": None if ratio is None else ratio * launch_bytes, "launch_bytes": launch_bytes, "launch_ms": launch_ms,
+                     "peak_measured": read_gbs, "frac_of_measured": achieved / read_gbs,
+                     "peak_measured_how": "plain streaming read of 1 GiB in this run (hb_debug_stream_read)"},
         "layer_chain": {"algorithmic_bytes_per_step": step_bytes, "achieved_GBs": chain_gbs, "frac_of_hbm_peak": chain_gbs / HBM_PEAK_GBS,
-                        "kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
+                        "kernel_ms": kernel_ms},
+        "m1": m1,
         "cpu_baseline": cpu,
         "parity": check,
     }

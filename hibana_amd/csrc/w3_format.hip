@@ -242,3 +242,30 @@ extern "C" int hb_w3_dequant(const void* tiled, const float* row_scale, int64_t 
                      row_scale, (uint64_t)lut, blocks, chunks, out);
   return launch_status();
 }
+
+// Measurement hook: a plain streaming read of `bytes` (a multiple of 16 KB), the yardstick a weight stream is held
+// against. Each wavefront reads 16 KB in sixteen 128-bit loads a lane, all in flight together, and folds them into
+// one word a workgroup (so that nothing is optimized away).
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t* __restrict__ src, int64_t pieces, uint32_t* __restrict__ sink) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // one 16 KB piece a wavefront
+  uint32_t fold = 0;
+  if (wave < pieces) {
+    const u32x4_t* at = src + wave * 1024 + lane;
+    u32x4_t v[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) v[j] = __builtin_nontemporal_load(at + 64 * j);
+#pragma unroll
+    for (int j = 0; j < 16; j++) fold ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+  }
+  if (fold == 0x9e3779b9u) sink[blockIdx.x] = fold;  // (practically never: the loads stay, the store does not cost)
+}
+
+extern "C" int hb_debug_stream_read(const void* src, size_t bytes, void* sink, void* stream) {
+  if (!src || !sink) return HB_ENULL;
+  if (bytes == 0 || bytes % 16384 || !aligned(src, 16) || !aligned(sink, 4)) return HB_EINVAL;
+  const int64_t pieces = (int64_t)(bytes / 16384);
+  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)((pieces + 3) / 4)), dim3(256), 0, as_stream(stream), static_cast<const u32x4_t*>(src), pieces,
+                     static_cast<uint32_t*>(sink));
+  return launch_status();
+}

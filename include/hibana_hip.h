@@ -55,6 +55,11 @@ int hb_debug_events(void* const* events, int count);
  * the end of its wait for fc1 (fc2 workgroups; else 0) and its end, in ticks of the 100 MHz device clock, and its rows. */
 int hb_debug_trace(void* buffer);
 
+/* Measurement hook (no counterpart in the reference): one plain streaming read of `bytes` (a multiple of 16 KB) from
+ * `src`, 128-bit loads, sixteen in flight a lane - the read rate this device gives a kernel that does nothing else, to
+ * hold a weight stream's rate against. `sink`: at least bytes / 65536 + 1 uint32 (practically never written). */
+int hb_debug_stream_read(const void* src, size_t bytes, void* sink, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * W3 format: 3-bit (or 2-bit) codes into an 8-entry E4M3 codebook, one E4M3 scale per 32 weights along K, one FP32
  * multiplier per output row.

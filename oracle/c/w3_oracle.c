@@ -17,6 +17,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 static float e4m3_to_float(uint8_t b) {
   const int sign = b >> 7, e = (b >> 3) & 15, m = b & 7;
@@ -112,13 +113,25 @@ typedef struct {
   int experts, base, hidden, inter, gated;
 } w3o_experts;
 
+/* Seconds the last w3o_moe_layer call spent unpacking weights (w3o_dequantize), so that a caller that times the whole
+ * call also has the matmul-and-the-rest part: total minus this. */
+static double unpack_seconds = 0.0;
+double w3o_last_unpack_seconds(void) { return unpack_seconds; }
+static double now_seconds(void) {
+  struct timespec t;
+  clock_gettime(CLOCK_MONOTONIC, &t);
+  return (double)t.tv_sec + 1e-9 * (double)t.tv_nsec;
+}
+
 /* one expert on `rows` gathered activation rows xs [rows, hidden] (float) -> y [rows, hidden] (float) */
 static void one_expert(const w3o_experts* ex, int e, const float* xs, int rows, float* y, float* w13, float* w2, float* h1, float* h) {
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter, hd = ex->hidden, it = ex->inter;
+  const double t0 = now_seconds();
   w3o_dequantize(ex->planes13 + (size_t)e * n1 / 32 * (hd / 128) * 3 * 128, ex->scales13 + (size_t)e * n1 / 32 * (hd / 128) * 128,
                  ex->row13 + (size_t)e * n1, ex->levels13, n1, hd, 3, w13);
   w3o_dequantize(ex->planes2 + (size_t)e * hd / 32 * (it / 128) * 3 * 128, ex->scales2 + (size_t)e * hd / 32 * (it / 128) * 128,
                  ex->row2 + (size_t)e * hd, ex->levels2, hd, it, 3, w2);
+  unpack_seconds += now_seconds() - t0;
   rows_times_matrix(xs, rows, w13, n1, hd, h1);
   for (int r = 0; r < rows; r++)
     for (int c = 0; c < it; c++) {
@@ -141,6 +154,7 @@ static void one_expert(const w3o_experts* ex, int e, const float* xs, int rows, 
 int w3o_moe_layer(const w3o_experts* ex, const w3o_experts* shared, const float* gate_vec, const uint16_t* x, const int32_t* ids,
                   const float* weights, int m, int topk, uint16_t* out) {
   const int hd = ex->hidden, it = ex->inter, n1 = ex->gated ? 2 * it : it;
+  unpack_seconds = 0.0;
   float* xf = (float*)malloc((size_t)m * hd * 4);
   for (size_t i = 0; i < (size_t)m * hd; i++) xf[i] = bf16_bits_to_float(x[i]);
   float* pairs = (float*)calloc((size_t)m * topk * hd, 4);

@@ -30,6 +30,7 @@ def lib() -> C.CDLL:
         build()
     h = C.CDLL(str(LIBRARY))
     h.w3o_moe_layer.restype = C.c_int
+    h.w3o_last_unpack_seconds.restype = C.c_double
     return h
 
 
@@ -82,6 +83,11 @@ def moe_layer(experts: HostExperts, x_bits: np.ndarray, ids: np.ndarray, weights
     d = lib().w3o_moe_layer(C.byref(experts.struct), C.byref(shared.struct) if shared else None, _p(gv) if gv is not None else None, _p(x_bits),
                             _p(ids), _p(weights), m, topk, _p(out))
     return out, d
+
+
+def last_unpack_seconds() -> float:
+    """Seconds the last moe_layer call spent unpacking weights (the rest is matmuls, activation and combine)."""
+    return float(lib().w3o_last_unpack_seconds())
 
 
 def linear(w3: dict, x_bits: np.ndarray) -> np.ndarray:
