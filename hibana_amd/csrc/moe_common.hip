@@ -47,17 +47,20 @@ struct RouteParams {
   const int32_t* slots;  // row r is real iff slots[r / steps] != 0 (null: every row)
   int steps, repeat;
   int e, k, per, latent;
+  int pad_id;            // the id of a padded row's slots without `repeat` (the callers' default: e, "no expert")
   int32_t* ids;
   float* weights;
   uint16_t* lat;         // sigmoid: BF16 [m, latent], the row's latent columns
 };
 
-template <bool SIGMOID, int PER>
+// THROUGH: the logits were written by other workgroups of the same launch and are read past the compute die's L2.
+template <bool SIGMOID, int PER, bool THROUGH = false>
 __device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane) {
   const int e = p.e, per = p.per, first = lane * per;
+  auto logit = [](const float* at) -> float { if constexpr (THROUGH) return load_through(at); else return *at; };
   if (SIGMOID) {
     const float* src = p.logits + (int64_t)r * p.stride + e;
-    for (int c = lane; c < p.latent; c += 64) p.lat[(int64_t)r * p.latent + c] = __builtin_bit_cast(uint16_t, (__bf16)src[c]);
+    for (int c = lane; c < p.latent; c += 64) p.lat[(int64_t)r * p.latent + c] = __builtin_bit_cast(uint16_t, (__bf16)logit(src + c));
   }
   const bool padded = p.slots && p.slots[r / p.steps] == 0;
   const float* row = p.logits + (int64_t)(padded ? 0 : r) * p.stride;  // a padded row repeats row 0's first choice
@@ -68,7 +71,7 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane)
     for (int j = 0; j < PER; j++) {
       const int i = first + j;
       const bool real = j < per && i < e;
-      val[j] = real ? 1.0f / (1.0f + expf(-row[i])) : 0.f;
+      val[j] = real ? 1.0f / (1.0f + expf(-logit(row + i))) : 0.f;
       key[j] = real ? score_key(val[j] + p.bias[i]) : 0u;
     }
   } else {
@@ -76,7 +79,7 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane)
 #pragma unroll
     for (int j = 0; j < PER; j++) {
       const int i = first + j;
-      val[j] = j < per && i < e ? row[i] : -INFINITY;
+      val[j] = j < per && i < e ? logit(row + i) : -INFINITY;
       mx = fmaxf(mx, val[j]);
     }
 #pragma unroll
@@ -126,7 +129,7 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane)
     int id = mine_id;
     float w = SIGMOID ? mine / (total + 1e-20f) : mine / total;
     if (padded) {
-      id = p.repeat ? __builtin_amdgcn_readfirstlane(mine_id) : e;
+      id = p.repeat ? __builtin_amdgcn_readfirstlane(mine_id) : p.pad_id;
       w = 0.f;
     }
     store_through(&p.ids[(int64_t)r * p.k + lane], id);  // the plan may read it in this very launch, from another workgroup
@@ -750,6 +753,7 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   rp.k = topk;
   rp.per = (e + 63) / 64;
   rp.steps = 1;
+  rp.pad_id = e;
   rp.ids = ids;
   rp.weights = weights;
   const int64_t pairs = (int64_t)m * topk;
@@ -851,6 +855,7 @@ extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, c
   p.e = e;
   p.k = k;
   p.per = (e + 63) / 64;
+  p.pad_id = e;
   p.ids = ids;
   p.weights = weights;
   launch_route<false>(p, m, as_stream(stream));
@@ -872,6 +877,7 @@ extern "C" int hb_route_sigmoid_topk(const float* fused, int64_t stride, const f
   p.e = e;
   p.k = k;
   p.per = (e + 63) / 64;
+  p.pad_id = e;
   p.latent = latent;
   p.ids = ids;
   p.weights = weights;

@@ -543,10 +543,14 @@ extern "C" int hb_nvfp4_moe(const hb_nvfp4_experts* routed, const void* x, const
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
   const bool sum = mode == HB_MOE_SUM;
   void* pairs_out = sum ? static_cast<void*>(ws.y) : out;
-  if (int e = run_experts(routed, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16, as_stream(stream))) return e;
+  // a summed prefill-sized call keeps its pair outputs in BF16: half the traffic of its widest tensor, as the reference's
+  // layer does from the same size (hibana/model/flashnext/moe.py:186)
+  const bool narrow = sum && m >= MOE_WIDE_ROWS;
+  if (int e = run_experts(routed, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16 || narrow, as_stream(stream))) return e;
   if (sum) {
     CombineParams c{};
     c.pairs = ws.y;
+    c.pairs_bf16 = narrow;
     c.ids = ids;
     c.weights = weights;
     c.e_lo = routed->base;

@@ -13,6 +13,7 @@ enum { EPI_DENSE = 0, EPI_FC1_GATED = 1, EPI_FC1_RELU2 = 2, EPI_FC2 = 3, EPI_DEN
 constexpr bool epi_dense(int epi) { return epi == EPI_DENSE || epi == EPI_DENSE_RELU2; }
 constexpr bool epi_gathers(int epi) { return epi == EPI_FC1_GATED || epi == EPI_FC1_RELU2; }  // activation rows found through `order`
 constexpr int ROWS_PER_SLOT = 16;
+constexpr int MOE_WIDE_ROWS = 1024;  // rows from which a routed sum keeps its pair outputs in BF16 (the reference's WIDE_ROWS)
 constexpr int PLAN_HEADER = 16;  // plan[0] = slots, plan[1] = distinct experts, plan[2] = routed pairs kept
 
 struct StreamParams {
@@ -56,7 +57,10 @@ struct StreamParams {
 // ticket has published them to whichever workgroup draws a later ticket and reads with load_through, on any compute
 // die, without a cache write-back or invalidate of its own.
 __device__ __forceinline__ void store_through(int32_t* at, int32_t v) { __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ int32_t load_through(const int32_t* at) { return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }  // up to 1024 experts (instantiated for 8 and 16 registers a lane)
+__device__ __forceinline__ int32_t load_through(const int32_t* at) { return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_through(float* at, float v) { __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float load_through(const float* at) { return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ uint16_t load_through(const uint16_t* at) { return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 __device__ __forceinline__ void store_through(uint16_t* at, uint16_t v) { __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 

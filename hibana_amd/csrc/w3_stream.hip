@@ -1074,8 +1074,10 @@ extern "C" int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
   void* pairs_out = mode == HB_MOE_SUM ? static_cast<void*>(ws.y) : out;
+  const bool narrow = mode == HB_MOE_SUM && m >= MOE_WIDE_ROWS;  // a summed prefill-sized call: BF16 pair outputs (hibana/model/flashnext/moe.py:186)
   CombineParams c{};
   c.pairs = ws.y;
+  c.pairs_bf16 = narrow;
   c.ids = ids;
   c.weights = weights;
   c.e_lo = routed->base;
@@ -1084,7 +1086,7 @@ extern "C" int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32
   c.topk = topk;
   c.h = routed->hidden_out;
   c.out = static_cast<uint16_t*>(out);
-  return run_experts(routed, nullptr, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16, as_stream(stream), nullptr, e4m3,
+  return run_experts(routed, nullptr, x, ids, m, topk, ws, pairs_out, mode == HB_MOE_PAIRS_BF16 || narrow, as_stream(stream), nullptr, e4m3,
                      mode == HB_MOE_SUM ? &c : nullptr);
 }
 
@@ -1103,13 +1105,18 @@ static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, c
   if (!aligned(x, 16) || !aligned(ids, 4) || !aligned(weights, 4) || !aligned(out, 4) || !aligned(workspace, 16) || !aligned(gate_vec, 4)) return HB_EINVAL;
   const MoeWorkspace ws = moe_carve(workspace, m, topk, routed->experts, routed->inter, routed->hidden_out, shared ? 1 : 0, routed->hidden);
   if (workspace_bytes < ws.bytes) return HB_EWORKSPACE;
+  // a prefill-sized call keeps its pair outputs (and the shared expert's rows behind them) in BF16, as the reference's
+  // layer does from the same size (hibana/model/flashnext/moe.py:186); the shared rows are rounded to BF16 by the combine anyway
+  const bool narrow = m >= MOE_WIDE_ROWS;
   CombineParams c{};
   c.pairs = ws.y;
+  c.pairs_bf16 = narrow;
   c.ids = ids;
   c.weights = weights;
   if (shared) {
-    c.shared = ws.y + (int64_t)m * topk * routed->hidden_out;
-    c.shared_f32 = 1;
+    c.shared = narrow ? static_cast<const void*>(reinterpret_cast<const uint16_t*>(ws.y) + (int64_t)m * topk * routed->hidden_out)
+                      : static_cast<const void*>(ws.y + (int64_t)m * topk * routed->hidden_out);
+    c.shared_f32 = narrow ? 0 : 1;
     c.shared_stride = routed->hidden_out;
     c.x = static_cast<const uint16_t*>(x);
     c.gate_vec = gate_vec;
@@ -1121,7 +1128,7 @@ static int moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, c
   c.topk = topk;
   c.h = routed->hidden_out;
   c.out = static_cast<uint16_t*>(out);
-  return run_experts(routed, shared, x, ids, m, topk, ws, ws.y, 0, as_stream(stream), route, e4m3, &c);
+  return run_experts(routed, shared, x, ids, m, topk, ws, ws.y, narrow, as_stream(stream), route, e4m3, &c);
 }
 
 extern "C" int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
