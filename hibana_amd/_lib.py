@@ -24,7 +24,14 @@ class HbNvfp4Experts(C.Structure):
                 ("hidden_out", C.c_int), ("gated", C.c_int)]
 
 
+class HbLatentWeights(C.Structure):
+    _fields_ = [("gate_fc1", C.c_void_p), ("bias", C.c_void_p), ("fc2", C.c_void_p), ("routed", C.POINTER(HbNvfp4Experts)),
+                ("shared_up", C.c_void_p), ("shared_down", C.c_void_p), ("shared_up_scale", C.c_float), ("shared_down_scale", C.c_float),
+                ("experts_total", C.c_int), ("latent", C.c_int), ("hidden", C.c_int), ("shared_inter", C.c_int)]
+
+
 _P, _I, _L, _Z, _F = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
+_LW = C.POINTER(HbLatentWeights)
 _EX = C.POINTER(HbW3Experts)
 _EX4 = C.POINTER(HbNvfp4Experts)
 # name -> (restype, argtypes): every symbol include/hibana_hip.h declares
@@ -62,6 +69,11 @@ SIGNATURES = {
     "hb_nvfp4_gemm": (_I, [_P, _I, _P, _F, _I, _I, _I, _P, _P]),
     "hb_nvfp4_moe_workspace_bytes": (_Z, [_I, _I, _EX4]),
     "hb_nvfp4_moe": (_I, [_EX4, _P, _P, _P, _I, _I, _I, _P, _P, _Z, _P]),
+    "hb_latent_workspace_bytes": (_Z, [_LW, _I, _I]),
+    "hb_latent_router": (_I, [_LW, _P, _I, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _Z, _P]),
+    "hb_latent_block": (_I, [_LW, _P, _P, _P, _P, _I, _I, _I, _P, _P, _Z, _P]),
+    "hb_latent_shared_up": (_I, [_LW, _P, _I, _I, _P, _Z, _P]),
+    "hb_latent_out": (_I, [_LW, _P, _I, _I, _P, _P, _Z, _P]),
 }
 
 

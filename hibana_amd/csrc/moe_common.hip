@@ -537,18 +537,10 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int3
 // shared expert is given; with one, its fused form (hibana/kernels/flashnext_fused.py:530-571).
 constexpr int COMBINE_SPAN = 512;  // columns per workgroup (two per thread)
 
-__global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
-  __shared__ float red[4];
-  const int r = blockIdx.x;
-  float g = 1.0f;
-  if (p.gate_vec && p.shared) {
-    combine_gate_partial(p.x, p.gate_vec, p.hx, r, threadIdx.x, red);
-    __syncthreads();
-    g = combine_gate_value(red);
-  }
-  const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
-  if (c >= p.h) return;
-  float v0 = 0.f, v1 = 0.f;
+// A row's weighted sum of its pairs at columns c, c + 1, in selection order (FP32 fma chain).
+__device__ __forceinline__ void combine_pairs_sum(const CombineParams& p, int r, int c, float& v0, float& v1) {
+  v0 = 0.f;
+  v1 = 0.f;
   // every slot's pair is read (so the loads are all in flight together) and a dropped slot contributes fma(0, 0, v)
   for (int s0 = 0; s0 < p.topk; s0 += 8) {
     float y0[8], y1[8], w[8];
@@ -578,6 +570,21 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
       v1 = fmaf(w[j], y1[j], v1);
     }
   }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  float g = 1.0f;
+  if (p.gate_vec && p.shared) {
+    combine_gate_partial(p.x, p.gate_vec, p.hx, r, threadIdx.x, red);
+    __syncthreads();
+    g = combine_gate_value(red);
+  }
+  const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
+  if (c >= p.h) return;
+  float v0, v1;
+  combine_pairs_sum(p, r, c, v0, v1);
   if (p.shared) {
     const int64_t at = (int64_t)r * p.shared_stride + c;
     float s0, s1;
@@ -594,6 +601,160 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
     v1 = combine_shared(v1, g, s1);
   }
   *reinterpret_cast<uint32_t*>(p.out + (int64_t)r * p.h + c) = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
+}
+
+// ------------------------------------------------------------------ the latent block's BF16 projections (M <= 16)
+//
+// y[i, n] = sum_k x[i, k] w[n, k] for at most sixteen rows of x, on the BF16 matrix cores with nothing staged: a
+// wavefront takes sixteen weight rows over `steps` K steps of 32 from k0; lane (q, r16) holds k = 32 s + 8 q .. + 7 of
+// weight row n0 + r16 (the B operand) and of activation row r16 (A; rows past m read row m - 1 and are never stored).
+// Register i of lane (q, r16) of the result is y[4 q + i][n0 + r16]. Up to eight steps are in flight at a time.
+struct GemvFrags {
+  u32x4_t v[8];
+};
+__device__ __forceinline__ void gemv16_load(GemvFrags& f, const uint16_t* __restrict__ base, int64_t ld, int row, int k0, int steps, int lane) {
+  const uint16_t* at = base + row * ld + k0 + 8 * (lane >> 4);
+#pragma unroll
+  for (int j = 0; j < 8; j++)
+    if (j < steps) f.v[j] = *reinterpret_cast<const u32x4_t*>(at + 32 * j);
+}
+__device__ __forceinline__ void gemv16_mfma(f32x4_t& acc, const GemvFrags& a, const GemvFrags& b, int steps) {
+#pragma unroll
+  for (int j = 0; j < 8; j++)
+    if (j < steps) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a.v[j]), __builtin_bit_cast(bf16x8_t, b.v[j]), acc, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4_t gemv16_wave(const uint16_t* __restrict__ w, int64_t ldw, int n0, int n, const uint16_t* __restrict__ x, int64_t ldx, int m,
+                                               int k0, int steps, int lane) {
+  const int r16 = lane & 15, wrow = min(n0 + r16, n - 1), xrow = min(r16, m - 1);
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0; s0 < steps; s0 += 8) {
+    GemvFrags a, b;
+    gemv16_load(b, w, ldw, wrow, k0 + 32 * s0, steps - s0, lane);
+    gemv16_load(a, x, ldx, xrow, k0 + 32 * s0, steps - s0, lane);
+    gemv16_mfma(acc, a, b, steps - s0);
+  }
+  return acc;
+}
+// The K splits' partial tiles, one per wavefront, added in wavefront order: thread t < 256 returns y[t / 16][n0 + t % 16].
+__device__ __forceinline__ float gemv16_reduce(const f32x4_t& acc, float* part, int waves) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  *reinterpret_cast<f32x4_t*>(part + wave * 256 + lane * 4) = acc;
+  __syncthreads();
+  float sum = 0.f;
+  if (threadIdx.x < 256) {
+    const int row = threadIdx.x >> 4, at = ((row >> 2) * 16 + (threadIdx.x & 15)) * 4 + (row & 3);
+    for (int w = 0; w < waves; w++) sum += part[w * 256 + at];
+  }
+  return sum;
+}
+
+// The router's launch of a small latent block (hibana/kernels/csrc/nemotron_moe.cu:496-558 of the reference):
+// fused[m, n] = x [router; fc1_latent]^T in FP32, sixteen output columns a workgroup, K split over its sixteen
+// wavefronts; then the workgroup that finishes last (ticket, as in moe_route_plan_kernel) rounds the latent columns to
+// BF16 and, with `do_route`, routes the rows - a wavefront a row, the logits read past its L2 - and, given a plan to
+// fill, plans the call.
+struct RouterGemv {
+  const uint16_t* w;  // BF16 [n, k]
+  const uint16_t* x;  // BF16 [m, k]
+  float* fused;       // FP32 [m, n]
+  int n, k, m;
+};
+__global__ __launch_bounds__(PLAN_THREADS) void latent_router_kernel(RouterGemv g, RouteParams route, int do_route, int ticket, int pairs, int e_lo, int e_n,
+                                                                     int32_t* __restrict__ plan, int32_t* __restrict__ order, int slot_rows, int slot_cap) {
+  extern __shared__ int lds[];
+  __shared__ int last;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n0 = blockIdx.x * 16, per_wave = g.k / PLAN_WAVES;
+  const f32x4_t acc = gemv16_wave(g.w, g.k, n0, g.n, g.x, g.k, g.m, wave * per_wave, per_wave / 32, lane);
+  const float sum = gemv16_reduce(acc, reinterpret_cast<float*>(lds), PLAN_WAVES);
+  if (threadIdx.x < 256) {
+    const int row = threadIdx.x >> 4, n = n0 + (threadIdx.x & 15);
+    if (row < g.m && n < g.n) store_through(&g.fused[(int64_t)row * g.n + n], sum);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // in memory before the ticket is drawn
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned drawn = atomicAdd(&route_tickets[ticket], 1u);
+    last = drawn == gridDim.x - 1u;
+    if (last) route_tickets[ticket] = 0u;
+  }
+  __syncthreads();
+  if (!last) return;
+  if (!do_route) {  // the caller routes from `fused` itself: the BF16 latent rows only
+    for (int i = threadIdx.x; i < g.m * route.latent; i += PLAN_THREADS) {
+      const int row = i / route.latent, col = i - row * route.latent;
+      route.lat[i] = bf16_of(load_through(&g.fused[(int64_t)row * g.n + route.e + col]));
+    }
+    return;
+  }
+  if (wave < g.m) {
+    if (route.per <= 8) {
+      route_row<true, 8, true>(route, wave, lane);
+    } else {
+      route_row<true, 16, true>(route, wave, lane);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  if (!plan) return;
+  __syncthreads();
+  plan_work<false>(route.ids, pairs, e_lo, e_n, 0, plan, order, slot_rows, slot_cap, nullptr, 1, 0, 0, lds);
+}
+
+// The last launch of a small latent block (nemotron_moe.cu's out kernel): out = bf16(shared + routed fc2^T) with
+// routed BF16 [m, latent]. When the routed experts' pair outputs are still to be summed, the launch's first `combines`
+// workgroups do that (the combine's FMA chain, a row and a 512-column span each, stored through to memory, then one
+// count on a ticket); the projection's workgroups - sixteen output columns each, K split over their wavefronts - load
+// their weights, wait for that count, and only then read routed. The last of them to finish clears both tickets.
+struct OutGemv {
+  const uint16_t* w;       // fc2 BF16 [n, k]
+  const uint16_t* routed;  // BF16 [m, k]
+  const uint16_t* shared;  // BF16 [m, n] or null
+  uint16_t* out;           // BF16 [m, n]
+  int n, k, m, waves;
+};
+__global__ __launch_bounds__(1024) void latent_out_kernel(OutGemv g, CombineParams c, int combines, int spans, int ticket, int ticket_done) {
+  __shared__ __align__(16) float part[16 * 256];
+  if ((int)blockIdx.x < combines) {
+    const int r = blockIdx.x / spans, col = (blockIdx.x - r * spans) * COMBINE_SPAN + 2 * threadIdx.x;
+    if (threadIdx.x < 256 && col < c.h) {
+      float v0, v1;
+      combine_pairs_sum(c, r, col, v0, v1);
+      __hip_atomic_store(reinterpret_cast<uint32_t*>(c.out + (int64_t)r * c.h + col), (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(&route_tickets[ticket], 1u);
+    return;
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n0 = ((int)blockIdx.x - combines) * 16;
+  const int per_wave = g.k / g.waves, steps = per_wave / 32, k0 = wave * per_wave, r16 = lane & 15;  // at most eight steps a wavefront
+  const bool live = wave < g.waves;  // a workgroup has at least the 256 threads of the epilogue
+  GemvFrags a, b;
+  if (live) gemv16_load(b, g.w, g.k, min(n0 + r16, g.n - 1), k0, steps, lane);
+  if (combines) {
+    if (wave == 0) await_count(reinterpret_cast<const int32_t*>(&route_tickets[ticket]), combines);
+    __syncthreads();
+  }
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  if (live) {
+    gemv16_load(a, g.routed, g.k, min(r16, g.m - 1), k0, steps, lane);
+    gemv16_mfma(acc, a, b, steps);
+  }
+  const float sum = gemv16_reduce(acc, part, g.waves);
+  if (threadIdx.x < 256) {
+    const int row = threadIdx.x >> 4, n = n0 + (threadIdx.x & 15);
+    if (row < g.m && n < g.n) {
+      const float base = g.shared ? bf16_bits_to_f32(g.shared[(int64_t)row * g.n + n]) : 0.f;
+      g.out[(int64_t)row * g.n + n] = f32_to_bf16_bits(base + sum);
+    }
+  }
+  if (combines && threadIdx.x == 0) {  // every projection workgroup is past its wait once all of them have counted here
+    const unsigned drawn = atomicAdd(&route_tickets[ticket_done], 1u);
+    if (drawn == gridDim.x - (unsigned)combines - 1u) {
+      route_tickets[ticket] = 0u;
+      route_tickets[ticket_done] = 0u;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------- host side
@@ -774,6 +935,63 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   }
   HB_LAUNCH(moe_plan_kernel<false>, dim3(plan_groups(job)), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order,
             rp, m, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows), ws.plan_wide, 1, 0, job ? *job : QuantJob{});
+  return HB_OK;
+}
+
+int latent_launch_router(const LatentRouter& r, hipStream_t stream) {
+  const int n = r.experts + r.latent;
+  if (r.m <= 0 || r.m > LATENT_MAX_ROWS || r.hidden <= 0 || r.hidden % (32 * PLAN_WAVES) || r.latent < 0 || r.steps <= 0) return HB_EINVAL;
+  if (int err = moe_check_route(r.m, r.experts, r.topk)) return err;
+  RouterGemv g{r.w, r.x, r.fused, n, r.hidden, r.m};
+  RouteParams rp{};
+  rp.logits = r.fused;
+  rp.stride = n;
+  rp.bias = r.bias;
+  rp.slots = r.slots;
+  rp.steps = r.steps;
+  rp.repeat = r.pad_id < 0;
+  rp.pad_id = r.pad_id;
+  rp.e = r.experts;
+  rp.k = r.topk;
+  rp.per = (r.experts + 63) / 64;
+  rp.latent = r.latent;
+  rp.ids = r.ids;
+  rp.weights = r.weights;
+  rp.lat = r.lat;
+  const int64_t pairs = (int64_t)r.m * r.topk;
+  size_t lds = (size_t)PLAN_WAVES * 256 * sizeof(float);
+  int slot_cap = 0;
+  if (r.route && r.plan) {
+    const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * r.e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
+    if (plan_lds > 64 * 1024 || r.e_n > PLAN_THREADS) return HB_EINVAL;
+    lds = std::max(lds, plan_lds);
+    slot_cap = (int)moe_max_slots(pairs, r.e_n, 0, ROWS_PER_SLOT);
+  }
+  const int ticket = (int)(g_route_ticket_next.fetch_add(1u, std::memory_order_relaxed) % ROUTE_TICKETS);
+  HB_LAUNCH(latent_router_kernel, dim3((unsigned)((n + 15) / 16)), dim3(PLAN_THREADS), lds, stream, g, rp, r.route, ticket, (int)pairs, r.e_lo, r.e_n,
+            r.route ? r.plan : nullptr, r.order, ROWS_PER_SLOT, slot_cap);
+  return HB_OK;
+}
+
+int latent_launch_out(const uint16_t* fc2, const uint16_t* routed, const uint16_t* shared, uint16_t* out, int m, int hidden, int latent,
+                      const CombineParams* pairs, hipStream_t stream) {
+  if (m <= 0 || m > LATENT_MAX_ROWS || hidden <= 0 || latent <= 0 || latent % 32) return HB_EINVAL;
+  const int steps = latent / 32;
+  int waves = 1;
+  while (waves < 16 && (steps % waves || steps / waves > 8)) waves *= 2;
+  if (steps % waves || steps / waves > 8) return HB_EINVAL;
+  OutGemv g{fc2, routed, shared, out, hidden, latent, m, waves};
+  CombineParams c{};
+  int combines = 0, spans = 1;
+  if (pairs) {
+    c = *pairs;
+    if (c.h != latent || c.m != m || c.h % 2) return HB_EINVAL;
+    spans = (c.h + COMBINE_SPAN - 1) / COMBINE_SPAN;
+    combines = m * spans;
+  }
+  const unsigned first = g_route_ticket_next.fetch_add(2u, std::memory_order_relaxed);
+  HB_LAUNCH(latent_out_kernel, dim3((unsigned)(combines + (hidden + 15) / 16)), dim3((unsigned)std::max(256, 64 * waves)), 0, stream, g, c, combines, spans,
+            (int)(first % ROUTE_TICKETS), (int)((first + 1u) % ROUTE_TICKETS));
   return HB_OK;
 }
 

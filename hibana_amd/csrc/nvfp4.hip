@@ -314,13 +314,13 @@ __device__ __forceinline__ void add_parities(f32x4_t& acc) {
 // y = x Wq^T, dense or grouped by the expert plan: one wavefront per (64-row block, K range, slot of 16 activation rows),
 // the same launch shape, slot table, weight ring, K-split exchange and epilogues as the W3 stream.
 template <int EPI>
-__global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
-  extern __shared__ __align__(16) uint8_t rings[];
-  const Slot sl = slot_of<EPI>(p, blockIdx.y);
+__device__ __forceinline__ void nvfp4_workgroup(const StreamParams& p, int slot, int bx, uint8_t* rings) {
+  const Slot sl = slot_of<EPI>(p, slot);
   if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: kept in scalars
+  if (wave >= p.ks * p.nbw) return;  // a launch shared with a matrix that takes more wavefronts a workgroup
   const WaveShare share = wave_share(p, wave);
-  const int ks = share.ks, nbi = share.nbi, nb = blockIdx.x * p.nbw + nbi;
+  const int ks = share.ks, nbi = share.nbi, nb = bx * p.nbw + nbi;
   const bool active = nb < p.n_blocks;
   f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
   if (active) {  // at least one chunk: the launch keeps ks <= chunks
@@ -338,11 +338,33 @@ __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
   finish_block<EPI, false, FP4_RING_BYTES / 4>(p, sl, RowScales{}, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
 }
 
+template <int EPI>
+__global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
+  extern __shared__ __align__(16) uint8_t rings[];
+  nvfp4_workgroup<EPI>(p, blockIdx.y, blockIdx.x, rings);
+}
+
+// Two matrices of different geometry in one launch (the routed experts' layer beside the shared expert's, which reads
+// other activations): the first `first` workgroups are (slot, block group) of `a`, slot-major, the rest of `b`. The
+// workgroup size is the larger of the two shapes'; the other matrix's workgroups retire the wavefronts they do not use.
+template <int EPI_A, int EPI_B>
+__global__ __launch_bounds__(1024) void nvfp4_twin_kernel(StreamParams a, StreamParams b, int groups_a, int groups_b, int first) {
+  extern __shared__ __align__(16) uint8_t rings[];
+  int id = blockIdx.x;
+  if (id < first) {
+    const int slot = id / groups_a;
+    nvfp4_workgroup<EPI_A>(a, slot, id - slot * groups_a, rings);
+  } else {
+    id -= first;
+    const int slot = id / groups_b;
+    nvfp4_workgroup<EPI_B>(b, slot, id - slot * groups_b, rings);
+  }
+}
+
 // experiments (hb_tune): the stream's workgroup shape ("nvfp4_ksplit", "nvfp4_nbw"); "nvfp4_tile": 1 forces the tile kernel, 2 the stream
 static std::atomic<int> g_nvfp4_ksplit{0}, g_nvfp4_nbw{0}, g_nvfp4_tile{0}, g_nvfp4_few{0};  // "nvfp4_few": 2 switches off the body for slots of at most eight rows
 
-template <int EPI>
-static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipStream_t stream) {
+static int shape_nvfp4(StreamParams& p, int64_t busy_slots) {
   pick_shape(p.n_blocks, p.chunks, busy_slots, 4096, &p.ks, &p.nbw);
   if (g_nvfp4_ksplit) {
     p.ks = g_nvfp4_ksplit;
@@ -351,9 +373,28 @@ static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipS
   if (p.ks * p.nbw > 16 || p.ks > p.chunks || (p.ks & (p.ks - 1))) return HB_EINVAL;
   set_split(p);
   p.no_few = g_nvfp4_few == 2;
+  return HB_OK;
+}
+
+template <int EPI>
+static int launch_nvfp4(StreamParams& p, int64_t slots, int64_t busy_slots, hipStream_t stream) {
+  if (int e = shape_nvfp4(p, busy_slots)) return e;
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
   HB_LAUNCH(nvfp4_stream_kernel<EPI>, grid, dim3(64 * waves), (size_t)waves * FP4_RING_BYTES, stream, p);
+  return HB_OK;
+}
+
+// `a` over its plan's slots beside the dense `b` in one launch (nvfp4_twin_kernel).
+template <int EPI_A, int EPI_B>
+static int launch_twin(StreamParams& a, int64_t slots_a, int64_t busy_a, StreamParams& b, int64_t slots_b, hipStream_t stream) {
+  if (int e = shape_nvfp4(a, busy_a)) return e;
+  if (int e = shape_nvfp4(b, slots_b)) return e;
+  const int groups_a = (a.n_blocks + a.nbw - 1) / a.nbw, groups_b = (b.n_blocks + b.nbw - 1) / b.nbw;
+  const int64_t first = slots_a * groups_a, all = first + slots_b * groups_b;
+  if (all > 0x7fffffff) return HB_EINVAL;
+  const int waves = std::max(a.ks * a.nbw, b.ks * b.nbw);
+  HB_LAUNCH((nvfp4_twin_kernel<EPI_A, EPI_B>), dim3((unsigned)all), dim3(64 * waves), (size_t)waves * FP4_RING_BYTES, stream, a, b, groups_a, groups_b, (int)first);
   return HB_OK;
 }
 
@@ -469,21 +510,12 @@ int check_experts(const hb_nvfp4_experts* ex) {
   return HB_OK;
 }
 
-// plan -> fc1 -> fc2: `out_pairs` receives fc2's per-pair outputs.
-int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, int m, int topk, const MoeWorkspace& ws, void* out_pairs,
-                int pairs_bf16, hipStream_t stream) {
+// The two launches' parameters of a routed call over a filled plan: fc1 from x into ws.h, fc2 from there into `out_pairs`.
+void expert_params(const hb_nvfp4_experts* ex, const void* x, int m, int topk, const MoeWorkspace& ws, void* out_pairs, int pairs_bf16, StreamParams& p,
+                   StreamParams& f2) {
   const int64_t pairs = (int64_t)m * topk;
-  // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel; below that the
-  // 16-row slots of the weight stream
-  const bool dense = tile_takes(m, ex->hidden) && tile_takes(pairs, ex->inter) &&
-                     (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && pairs >= (int64_t)ex->experts * TILE_DENSE_ROWS));
-  const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
-  const int64_t slots = moe_max_slots(pairs, ex->experts, 0, slot_rows);
-  if (slots > 65535) return HB_EINVAL;
-  if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, 0, ws, stream, slot_rows)) return e;
   const int n1 = ex->gated ? 2 * ex->inter : ex->inter;
-  const int64_t est = pairs < 2 * ex->experts ? (pairs + 1) / 2 : slots;
-  StreamParams p{};
+  p = StreamParams{};
   p.w = static_cast<const uint8_t*>(ex->fc1);
   p.expert_bytes = (int64_t)hb_nvfp4_tiled_bytes(n1, ex->hidden);
   p.scalars = ex->fc1_scale2;
@@ -497,7 +529,7 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
   p.pairs = (int)pairs;
   p.out = ws.h;
   p.out_stride = ex->inter;
-  StreamParams f2 = p;
+  f2 = p;
   f2.w = static_cast<const uint8_t*>(ex->fc2);
   f2.expert_bytes = (int64_t)hb_nvfp4_tiled_bytes(ex->hidden_out, ex->inter);
   f2.scalars = ex->fc2_scale2;
@@ -508,6 +540,26 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
   f2.out = out_pairs;
   f2.out_stride = ex->hidden_out;
   f2.out_bf16 = pairs_bf16;
+}
+
+// the slots the stream's shape is chosen for: a call of few pairs fills about one slot a distinct expert
+int64_t busy_slots(int64_t pairs, int experts, int64_t slots) { return pairs < 2 * experts ? (pairs + 1) / 2 : slots; }
+
+// plan -> fc1 -> fc2: `out_pairs` receives fc2's per-pair outputs.
+int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, int m, int topk, const MoeWorkspace& ws, void* out_pairs,
+                int pairs_bf16, hipStream_t stream) {
+  const int64_t pairs = (int64_t)m * topk;
+  // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel; below that the
+  // 16-row slots of the weight stream
+  const bool dense = tile_takes(m, ex->hidden) && tile_takes(pairs, ex->inter) &&
+                     (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && pairs >= (int64_t)ex->experts * TILE_DENSE_ROWS));
+  const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
+  const int64_t slots = moe_max_slots(pairs, ex->experts, 0, slot_rows);
+  if (slots > 65535) return HB_EINVAL;
+  if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, 0, ws, stream, slot_rows)) return e;
+  const int64_t est = busy_slots(pairs, ex->experts, slots);
+  StreamParams p, f2;
+  expert_params(ex, x, m, topk, ws, out_pairs, pairs_bf16, p, f2);
   if (dense) {
     if (int e = ex->gated ? launch_tile<TileNvfp4, EPI_FC1_GATED>(p, slots, m, stream) : launch_tile<TileNvfp4, EPI_FC1_RELU2>(p, slots, m, stream)) return e;
     if (int e = launch_tile<TileNvfp4, EPI_FC2>(f2, slots, pairs, stream)) return e;
@@ -516,6 +568,64 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
   if (int e = ex->gated ? launch_nvfp4<EPI_FC1_GATED>(p, slots, est, stream) : launch_nvfp4<EPI_FC1_RELU2>(p, slots, est, stream)) return e;
   if (int e = launch_nvfp4<EPI_FC2>(f2, slots, est, stream)) return e;
   return launch_status();
+}
+
+StreamParams dense_params(const void* tiled, float scale, int n, int k, const void* x, int m, void* y) {
+  StreamParams p{};
+  p.w = static_cast<const uint8_t*>(tiled);
+  p.scalar = scale;
+  p.n_blocks = n / 64;
+  p.chunks = k / 128;
+  p.a = static_cast<const uint16_t*>(x);
+  p.a_stride = k;
+  p.m = m;
+  p.out = y;
+  p.out_stride = n;
+  return p;
+}
+
+// ------------------------------------------------------------------------------------- the small latent block
+struct LatentWorkspace {
+  MoeWorkspace moe;    // the routed experts' (absent without NVFP4 experts)
+  uint16_t* routed;    // BF16 [m, latent]: the routed sum
+  uint16_t* shared_h;  // BF16 [m, shared_inter]
+  uint16_t* shared_y;  // BF16 [m, hidden]
+  size_t bytes;
+};
+
+LatentWorkspace latent_carve(const hb_latent_weights* w, void* base, int m, int topk) {
+  LatentWorkspace l{};
+  size_t off = 0;
+  if (w->routed) {
+    l.moe = moe_carve(base, m, topk, w->routed->experts, w->routed->inter, w->routed->hidden_out, 0);
+    off = l.moe.bytes;
+  }
+  auto take = [&](size_t bytes) {
+    void* ptr = base ? static_cast<char*>(base) + off : nullptr;
+    off += (bytes + 255) & ~(size_t)255;
+    return static_cast<uint16_t*>(ptr);
+  };
+  l.routed = take((size_t)m * w->latent * 2);
+  l.shared_h = take((size_t)m * w->shared_inter * 2);
+  l.shared_y = take((size_t)m * w->hidden * 2);
+  l.bytes = off;
+  return l;
+}
+
+int check_latent(const hb_latent_weights* w, int m, int topk) {
+  if (!w) return HB_ENULL;
+  if (!w->gate_fc1 || !w->bias || !w->fc2) return HB_ENULL;
+  if (m <= 0 || m > LATENT_MAX_ROWS || topk <= 0) return HB_EINVAL;
+  if (w->experts_total <= 0 || w->latent <= 0 || w->hidden <= 0 || w->latent % 128 || w->hidden % 512) return HB_EINVAL;
+  if (!aligned(w->gate_fc1, 16) || !aligned(w->fc2, 16) || !aligned(w->bias, 4)) return HB_EINVAL;
+  if (w->routed) {
+    if (int e = check_experts(w->routed)) return e;
+    if (w->routed->hidden != w->latent || w->routed->hidden_out != w->latent || w->routed->base + w->routed->experts > w->experts_total) return HB_EINVAL;
+  }
+  if ((w->shared_up != nullptr) != (w->shared_down != nullptr)) return HB_ENULL;
+  if (w->shared_up && (w->shared_inter <= 0 || w->shared_inter % 128 || w->hidden % 128 || !aligned(w->shared_up, 16) || !aligned(w->shared_down, 16)))
+    return HB_EINVAL;
+  return HB_OK;
 }
 
 }  // namespace
@@ -561,5 +671,115 @@ extern "C" int hb_nvfp4_moe(const hb_nvfp4_experts* routed, const void* x, const
     c.out = static_cast<uint16_t*>(out);
     moe_launch_combine(c, as_stream(stream));
   }
+  return launch_status();
+}
+
+extern "C" size_t hb_latent_workspace_bytes(const hb_latent_weights* w, int m, int topk) {
+  if (check_latent(w, m, topk) != HB_OK) return 0;
+  return latent_carve(w, nullptr, m, topk).bytes;
+}
+
+extern "C" int hb_latent_router(const hb_latent_weights* w, const void* x, int m, int topk, const int32_t* slots, int steps, int route, int pad_id,
+                                float* fused, int32_t* ids, float* weights, void* lat, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int e = check_latent(w, m, topk)) return e;
+  if (!x || !fused || !lat || !workspace || (route && (!ids || !weights))) return HB_ENULL;
+  if (!aligned(x, 16) || !aligned(fused, 4) || !aligned(ids, 4) || !aligned(weights, 4) || !aligned(lat, 2) || !aligned(slots, 4) || !aligned(workspace, 16))
+    return HB_EINVAL;
+  if (pad_id > w->experts_total) return HB_EINVAL;
+  const LatentWorkspace l = latent_carve(w, workspace, m, topk);
+  if (workspace_bytes < l.bytes) return HB_EWORKSPACE;
+  LatentRouter r{};
+  r.w = static_cast<const uint16_t*>(w->gate_fc1);
+  r.bias = w->bias;
+  r.x = static_cast<const uint16_t*>(x);
+  r.slots = slots;
+  r.m = m;
+  r.experts = w->experts_total;
+  r.latent = w->latent;
+  r.hidden = w->hidden;
+  r.topk = topk;
+  r.steps = steps;
+  r.route = route != 0;
+  r.pad_id = pad_id;
+  r.fused = fused;
+  r.ids = ids;
+  r.weights = weights;
+  r.lat = static_cast<uint16_t*>(lat);
+  if (w->routed) {
+    r.e_lo = w->routed->base;
+    r.e_n = w->routed->experts;
+    r.plan = l.moe.plan;
+    r.order = l.moe.order;
+  }
+  if (int e = latent_launch_router(r, as_stream(stream))) return e;
+  return launch_status();
+}
+
+extern "C" int hb_latent_shared_up(const hb_latent_weights* w, const void* x, int m, int topk, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int e = check_latent(w, m, topk)) return e;
+  if (!x || !workspace || !w->shared_up) return HB_ENULL;
+  if (!aligned(x, 16) || !aligned(workspace, 16)) return HB_EINVAL;
+  const LatentWorkspace l = latent_carve(w, workspace, m, topk);
+  if (workspace_bytes < l.bytes) return HB_EWORKSPACE;
+  StreamParams up = dense_params(w->shared_up, w->shared_up_scale, w->shared_inter, w->hidden, x, m, l.shared_h);
+  if (int e = launch_nvfp4<EPI_DENSE_RELU2>(up, 1, 1, as_stream(stream))) return e;
+  return launch_status();
+}
+
+extern "C" int hb_latent_out(const hb_latent_weights* w, const void* routed, int m, int topk, void* out, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+  if (int e = check_latent(w, m, topk)) return e;
+  if (!routed || !out || !workspace) return HB_ENULL;
+  if (!aligned(routed, 16) || !aligned(out, 2) || !aligned(workspace, 16)) return HB_EINVAL;
+  const LatentWorkspace l = latent_carve(w, workspace, m, topk);
+  if (workspace_bytes < l.bytes) return HB_EWORKSPACE;
+  if (w->shared_up) {  // the shared expert's down projection of what hb_latent_shared_up left
+    StreamParams down = dense_params(w->shared_down, w->shared_down_scale, w->hidden, w->shared_inter, l.shared_h, m, l.shared_y);
+    if (int e = launch_nvfp4<EPI_DENSE>(down, 1, 1, as_stream(stream))) return e;
+  }
+  if (int e = latent_launch_out(static_cast<const uint16_t*>(w->fc2), static_cast<const uint16_t*>(routed), w->shared_up ? l.shared_y : nullptr,
+                                static_cast<uint16_t*>(out), m, w->hidden, w->latent, nullptr, as_stream(stream)))
+    return e;
+  return launch_status();
+}
+
+extern "C" int hb_latent_block(const hb_latent_weights* w, const void* x, const void* lat, const int32_t* ids, const float* weights, int m, int topk,
+                               int plan, void* out, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int e = check_latent(w, m, topk)) return e;
+  if (!w->routed) return HB_ENULL;
+  if (!x || !lat || !ids || !weights || !out || !workspace) return HB_ENULL;
+  if (!aligned(x, 16) || !aligned(lat, 16) || !aligned(ids, 4) || !aligned(weights, 4) || !aligned(out, 2) || !aligned(workspace, 16)) return HB_EINVAL;
+  const LatentWorkspace l = latent_carve(w, workspace, m, topk);
+  if (workspace_bytes < l.bytes) return HB_EWORKSPACE;
+  const hb_nvfp4_experts* ex = w->routed;
+  hipStream_t s = as_stream(stream);
+  const int64_t pairs = (int64_t)m * topk, slots = moe_max_slots(pairs, ex->experts, 0, ROWS_PER_SLOT), est = busy_slots(pairs, ex->experts, slots);
+  if (plan)
+    if (int e = moe_launch_plan(ids, pairs, ex->base, ex->experts, 0, l.moe, s)) return e;
+  StreamParams fc1, fc2;
+  expert_params(ex, lat, m, topk, l.moe, l.moe.y, 0, fc1, fc2);
+  if (w->shared_up) {
+    StreamParams up = dense_params(w->shared_up, w->shared_up_scale, w->shared_inter, w->hidden, x, m, l.shared_h);
+    StreamParams down = dense_params(w->shared_down, w->shared_down_scale, w->hidden, w->shared_inter, l.shared_h, m, l.shared_y);
+    if (int e = ex->gated ? launch_twin<EPI_FC1_GATED, EPI_DENSE_RELU2>(fc1, slots, est, up, 1, s) : launch_twin<EPI_FC1_RELU2, EPI_DENSE_RELU2>(fc1, slots, est, up, 1, s))
+      return e;
+    if (int e = launch_twin<EPI_FC2, EPI_DENSE>(fc2, slots, est, down, 1, s)) return e;
+  } else {
+    if (int e = ex->gated ? launch_nvfp4<EPI_FC1_GATED>(fc1, slots, est, s) : launch_nvfp4<EPI_FC1_RELU2>(fc1, slots, est, s)) return e;
+    if (int e = launch_nvfp4<EPI_FC2>(fc2, slots, est, s)) return e;
+  }
+  CombineParams c{};
+  c.pairs = l.moe.y;
+  c.ids = ids;
+  c.weights = weights;
+  c.e_lo = ex->base;
+  c.e_n = ex->experts;
+  c.m = m;
+  c.topk = topk;
+  c.h = w->latent;
+  c.out = l.routed;
+  if (int e = latent_launch_out(static_cast<const uint16_t*>(w->fc2), l.routed, w->shared_up ? l.shared_y : nullptr, static_cast<uint16_t*>(out), m, w->hidden,
+                                w->latent, &c, s))
+    return e;
   return launch_status();
 }

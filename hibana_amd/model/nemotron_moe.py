@@ -7,16 +7,19 @@
     routed  = sum_k w_k * down_e(relu(up_e latent)^2)  BF16 [M, L]      (NVFP4 or 3-bit experts, scaling in fc2's scale)
     out     = shared_down(relu(shared_up x)^2) + routed fc2_latent^T
 
-Routing and the experts run on this package's kernels for any number of rows (the reference switches to a separate
-small-call block at 16 rows; here the same chain serves both); the two dense BF16 projections are torch GEMMs
-(rocBLAS / hipBLASLt), as they are cuBLAS GEMMs in the reference (`forward`, :508-517).
+Up to sixteen rows (decode, verify) the block runs through the small-call kernels of `kernels/nemotron_moe.py`, four
+launches with the two BF16 projections inside them (`small`, :484-502 of the reference). Past that, routing and the
+experts run on this package's kernels and the two dense BF16 projections are torch GEMMs (rocBLAS / hipBLASLt), as
+they are cuBLAS GEMMs in the reference (`forward`, :508-517).
 """
 from __future__ import annotations
 
 import torch
 
 from hibana_amd import _lib
-from hibana_amd.kernels import ops
+from hibana_amd.kernels import nemotron_moe as small_block, ops
+from hibana_amd.kernels.b12x_moe import B12xExperts
+from hibana_amd.kernels.w3_moe import W3Experts, w3_moe
 
 
 def route_topk(fused: torch.Tensor, bias: torch.Tensor, k: int, latent: int, slots: torch.Tensor | None = None, steps: int = 1,
@@ -47,20 +50,44 @@ class NemotronMoe:
     """One block's weights, assembled from tensors already on the device.
 
     gate_fc1 BF16 [E + L, H] = [router; fc1_latent], bias FP32 [E], fc2 BF16 [H, L], shared_up / shared_down
-    `Nvfp4Linear` (or None for a block without a shared expert), `experts` a callable
-    (latent BF16 [M, L], ids, weights) -> BF16 [M, L] carrying the routed scaling factor: `B12xExperts` for NVFP4
-    experts or `lambda l, i, w: w3_moe(w3_experts, l, i, w)` for 3-bit ones."""
+    `Nvfp4Linear` (or None for a block without a shared expert), `experts` the routed experts carrying the routed
+    scaling factor: a `B12xExperts` (NVFP4), a `W3Experts` (3-bit), or any callable
+    (latent BF16 [M, L], ids, weights) -> BF16 [M, L]."""
+
+    SMALL_ROWS = small_block.MAX_ROWS
 
     def __init__(self, gate_fc1: torch.Tensor, bias: torch.Tensor, fc2: torch.Tensor, experts, topk: int, shared_up=None, shared_down=None):
         self.gate_fc1, self.bias, self.fc2 = gate_fc1.contiguous(), bias.float().contiguous(), fc2.contiguous()
-        self.experts_op, self.topk = experts, topk
+        self.topk = topk
         self.shared_up, self.shared_down = shared_up, shared_down
         self.experts = bias.numel()
         self.latent = gate_fc1.shape[0] - self.experts
         self.hidden = gate_fc1.shape[1]
+        self.w3 = experts if isinstance(experts, W3Experts) else None
+        self.b12x = experts if isinstance(experts, B12xExperts) else None
+        self.experts_op = (lambda lat, ids, w: w3_moe(self.w3, lat, ids, w)) if self.w3 is not None else experts
+        self._small = None
 
-    def route(self, fused: torch.Tensor, slots=None, steps: int = 1, repeat: bool = True):
-        return route_topk(fused, self.bias, self.topk, self.latent, slots, steps, repeat)
+    def small_weights(self) -> small_block.SmallWeights:
+        """What the small-call kernels read (hibana/model/nemotron/moe.py's small_weights), assembled once."""
+        if self._small is None:
+            self._small = small_block.SmallWeights(self.gate_fc1, self.bias, self.fc2, self.b12x, self.shared_up, self.shared_down)
+        return self._small
+
+    @staticmethod
+    def _padding(ctx):
+        """(slots, steps) of a decode / verify forward whose graph may hold padded requests, else (None, 1)."""
+        mode = getattr(ctx, "mode", None)
+        if mode == "decode":
+            return getattr(ctx, "slots", None), 1
+        if mode == "verify":
+            return getattr(ctx, "seq_slots", None), int(getattr(ctx, "verify_steps", 1))
+        return None, 1
+
+    def route(self, fused: torch.Tensor, slots=None, steps: int = 1, repeat: bool | None = None):
+        """FP32 router|fc1 rows -> (ids, renormalized weights, BF16 latent). Padded rows take row 0's first choice at
+        weight 0; around 3-bit experts, id E (no expert), which their kernel skips (hibana/model/nemotron/moe.py:448-462)."""
+        return route_topk(fused, self.bias, self.topk, self.latent, slots, steps, self.w3 is None if repeat is None else repeat)
 
     def routed(self, latent: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
         return self.experts_op(latent, ids, weights)
@@ -69,10 +96,24 @@ class NemotronMoe:
         """shared_down(relu(shared_up x)^2), the square in FP32 with one rounding (fused into the up projection's epilogue)."""
         return ops.nvfp4_linear(ops.nvfp4_linear(x, self.shared_up, relu2=True), self.shared_down)
 
-    def forward(self, x: torch.Tensor, slots=None, steps: int = 1) -> torch.Tensor:
+    def small(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+        """The block through `kernels/nemotron_moe.py` (at most SMALL_ROWS rows): the router's launch also routes and
+        plans as `route` would (hibana/model/nemotron/moe.py:484-502)."""
+        w = self.small_weights()
+        slots, steps = self._padding(ctx)
+        if self.w3 is not None:  # padded rows name no expert (id E), which w3_moe skips
+            _, ids, weights, ws, lat = small_block.router(x, w, None, self.topk, slots, steps, pad_id=self.experts, latent=True)
+            return small_block.w3_block(x, ws, lat, ids, weights, w, self.w3)
+        _, ids, weights, ws = small_block.router(x, w, None, self.topk, slots, steps)
+        return small_block.block(x, ws, ids, weights, w)
+
+    def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+        """Post-norm rows x [M, H] BF16 -> the block's mixer output [M, H] BF16 (hibana/model/nemotron/moe.py:508-517)."""
         x = x.contiguous()
+        if 0 < x.shape[0] <= self.SMALL_ROWS and (self.b12x is not None or self.w3 is not None):
+            return self.small(x, ctx)
         fused = torch.mm(x, self.gate_fc1.T, out_dtype=torch.float32)  # [M, E + L]
-        ids, weights, latent = self.route(fused, slots, steps)
+        ids, weights, latent = self.route(fused, *self._padding(ctx))
         routed = self.routed(latent, ids, weights)
         if self.shared_up is None:
             return torch.mm(routed, self.fc2.T)

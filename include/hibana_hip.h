@@ -290,6 +290,63 @@ size_t hb_nvfp4_moe_workspace_bytes(int m, int topk, const hb_nvfp4_experts* rou
 int hb_nvfp4_moe(const hb_nvfp4_experts* routed, const void* x, const int32_t* ids, const float* weights, int m,
                  int topk, int mode, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------------------------------------------------
+ * The latent-MoE block of a decode / verify call (at most HB_LATENT_MAX_ROWS rows), the native surface of the
+ * reference's hibana/kernels/nemotron_moe.py:45-68 (`router`, `block`, `shared_up`, `out`; kernels in
+ * hibana/kernels/csrc/nemotron_moe.cu):
+ *
+ *   fused  = x [router; fc1_latent]^T                    FP32 [m, experts_total + latent]
+ *   ids, w = top-k of sigmoid(logits) + bias, w = the plain sigmoids renormalized; lat = bf16(fused[:, experts_total:])
+ *   routed = sum_k w_k * down_e(relu(up_e lat)^2)         BF16 [m, latent]
+ *   out    = bf16(shared_down(relu(shared_up x)^2) + routed fc2^T)
+ *
+ * Weight-only arithmetic: activations stay BF16 (the reference's small-call kernels round x, lat and h to NVFP4 for its
+ * FP4 tensor cores; its own FP32 statement of the block, NemotronMoe.reference, hibana/model/nemotron/moe.py:521-566,
+ * is what these entry points follow). hb_latent_router followed by hb_latent_block is four launches.
+ * ---------------------------------------------------------------------------------------------------------------- */
+#define HB_LATENT_MAX_ROWS 16
+
+typedef struct hb_latent_weights {
+  const void* gate_fc1;            /* BF16 [experts_total + latent, hidden]: the router's rows, then fc1_latent's */
+  const float* bias;               /* [experts_total]: added to the scores for the choice only */
+  const void* fc2;                 /* BF16 [hidden, latent] */
+  const hb_nvfp4_experts* routed;  /* NVFP4 experts with hidden = hidden_out = latent; NULL when the routed experts
+                                      are not NVFP4 (then hb_latent_block is not available) */
+  const void* shared_up;           /* tile layout of [shared_inter, hidden], or NULL: no shared expert */
+  const void* shared_down;         /* tile layout of [hidden, shared_inter] */
+  float shared_up_scale, shared_down_scale;  /* their FP32 scales (weight_scale_2) */
+  int experts_total, latent, hidden, shared_inter;
+} hb_latent_weights;
+
+/* One workspace serves the four calls of a block; its size depends on (weights, m, topk) only. 0 on invalid input. */
+size_t hb_latent_workspace_bytes(const hb_latent_weights* w, int m, int topk);
+
+/* ref: `router`, hibana/kernels/nemotron_moe.py:45-55 (router_kernel, nemotron_moe.cu:496-558). x BF16 [m, hidden] ->
+ * fused FP32 [m, experts_total + latent] and lat BF16 [m, latent]; with `route`, ids int32 [m, topk] / weights FP32
+ * [m, topk] as hb_route_sigmoid_topk gives them from `fused`, bit for bit (slots / steps: its padded rows; a padded
+ * row takes row 0's first choice at weight 0, or `pad_id` when that is >= 0), and the call's plan is left in the
+ * workspace for hb_latent_block. Without `route`, ids / weights are not written (and may be NULL). One launch. */
+int hb_latent_router(const hb_latent_weights* w, const void* x, int m, int topk, const int32_t* slots, int steps,
+                     int route, int pad_id, float* fused, int32_t* ids, float* weights, void* lat, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
+/* ref: `block`, hibana/kernels/nemotron_moe.py:58-60: the rest of the block after hb_latent_router -> out BF16
+ * [m, hidden]. `plan` != 0 when ids are not the router's (the caller routed): the plan is then made here, one more
+ * launch. Three launches otherwise: routed fc1 beside the shared expert's up, routed fc2 beside its down, then the
+ * combine and fc2_latent. */
+int hb_latent_block(const hb_latent_weights* w, const void* x, const void* lat, const int32_t* ids,
+                    const float* weights, int m, int topk, int plan, void* out, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* ref: `shared_up` / `out` as `w3_block` uses them around other routed experts, hibana/kernels/nemotron_moe.py:63-68:
+ * hb_latent_shared_up leaves relu(shared_up x)^2 in the workspace; hb_latent_out, given the routed sum BF16
+ * [m, latent], writes out = bf16(shared_down(...) + routed fc2^T). Without a shared expert hb_latent_shared_up
+ * returns HB_ENULL and hb_latent_out adds nothing. */
+int hb_latent_shared_up(const hb_latent_weights* w, const void* x, int m, int topk, void* workspace,
+                        size_t workspace_bytes, void* stream);
+int hb_latent_out(const hb_latent_weights* w, const void* routed, int m, int topk, void* out, void* workspace,
+                  size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
