@@ -48,6 +48,7 @@ struct RouteParams {
   int steps, repeat;
   int e, k, per, latent;
   int pad_id;            // the id of a padded row's slots without `repeat` (the callers' default: e, "no expert")
+  int sigmoid;           // the rule a kernel that serves both applies (route_any)
   int32_t* ids;
   float* weights;
   uint16_t* lat;         // sigmoid: BF16 [m, latent], the row's latent columns
@@ -58,9 +59,25 @@ template <bool SIGMOID, int PER, bool THROUGH = false>
 __device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane) {
   const int e = p.e, per = p.per, first = lane * per;
   auto logit = [](const float* at) -> float { if constexpr (THROUGH) return load_through(at); else return *at; };
-  if (SIGMOID) {
+  if (SIGMOID && p.lat) {  // the row's latent columns, rounded: four a lane and sixteen loads in flight where the row allows
     const float* src = p.logits + (int64_t)r * p.stride + e;
-    for (int c = lane; c < p.latent; c += 64) p.lat[(int64_t)r * p.latent + c] = __builtin_bit_cast(uint16_t, (__bf16)logit(src + c));
+    uint16_t* dst = p.lat + (int64_t)r * p.latent;
+    if (!THROUGH && !((p.stride | e | p.latent) & 3)) {
+      for (int c0 = 4 * lane; c0 < p.latent; c0 += 1024) {
+        f32x4_t v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (c0 + 256 * j < p.latent) v[j] = *reinterpret_cast<const f32x4_t*>(src + c0 + 256 * j);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (c0 + 256 * j < p.latent) {
+            const uint32_t lo = (uint32_t)bf16_of(v[j].x) | ((uint32_t)bf16_of(v[j].y) << 16), hi = (uint32_t)bf16_of(v[j].z) | ((uint32_t)bf16_of(v[j].w) << 16);
+            *reinterpret_cast<uint2*>(dst + c0 + 256 * j) = make_uint2(lo, hi);
+          }
+      }
+    } else {
+      for (int c = lane; c < p.latent; c += 64) dst[c] = bf16_of(logit(src + c));
+    }
   }
   const bool padded = p.slots && p.slots[r / p.steps] == 0;
   const float* row = p.logits + (int64_t)(padded ? 0 : r) * p.stride;  // a padded row repeats row 0's first choice
@@ -134,6 +151,21 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int r, int lane)
     }
     store_through(&p.ids[(int64_t)r * p.k + lane], id);  // the plan may read it in this very launch, from another workgroup
     p.weights[(int64_t)r * p.k + lane] = w;
+  }
+}
+
+// Row r by the rule and the register count the parameters name.
+__device__ __forceinline__ void route_any(const RouteParams& p, int r, int lane) {
+  if (p.sigmoid) {
+    if (p.per <= 8) {
+      route_row<true, 8>(p, r, lane);
+    } else {
+      route_row<true, 16>(p, r, lane);
+    }
+  } else if (p.per <= 8) {
+    route_row<false, 8>(p, r, lane);
+  } else {
+    route_row<false, 16>(p, r, lane);
   }
 }
 
@@ -476,11 +508,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
   }
   if (route.logits) {
     for (int r = threadIdx.x >> 6; r < route_rows; r += PLAN_WAVES) {
-      if (route.per <= 8) {
-        route_row<false, 8>(route, r, threadIdx.x & 63);
-      } else {
-        route_row<false, 16>(route, r, threadIdx.x & 63);
-      }
+      route_any(route, r, threadIdx.x & 63);
     }
     __syncthreads();
   }
@@ -512,11 +540,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int3
   }
   const int wave = threadIdx.x >> 6, r = blockIdx.x * ROUTE_GROUP_ROWS + wave;
   if (wave < ROUTE_GROUP_ROWS && r < route_rows) {
-    if (route.per <= 8) {
-      route_row<false, 8>(route, r, threadIdx.x & 63);
-    } else {
-      route_row<false, 16>(route, r, threadIdx.x & 63);
-    }
+    route_any(route, r, threadIdx.x & 63);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this row's ids (write-through stores) have reached memory before the ticket is drawn
   }
   __syncthreads();
@@ -537,15 +561,14 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int3
 // shared expert is given; with one, its fused form (hibana/kernels/flashnext_fused.py:530-571).
 constexpr int COMBINE_SPAN = 512;  // columns per workgroup (two per thread)
 
-// A row's weighted sum of its pairs at columns c, c + 1, in selection order (FP32 fma chain).
-__device__ __forceinline__ void combine_pairs_sum(const CombineParams& p, int r, int c, float& v0, float& v1) {
-  v0 = 0.f;
-  v1 = 0.f;
-  // every slot's pair is read (so the loads are all in flight together) and a dropped slot contributes fma(0, 0, v)
-  for (int s0 = 0; s0 < p.topk; s0 += 8) {
-    float y0[8], y1[8], w[8];
+// A row's weighted sum of its pairs at columns c, c + 1, in selection order (FP32 fma chain). The pairs of B slots are
+// read together (so the loads are all in flight at once) and a dropped slot contributes fma(0, 0, v).
+template <int B>
+__device__ __forceinline__ void combine_pairs_batches(const CombineParams& p, int r, int c, float& v0, float& v1) {
+  for (int s0 = 0; s0 < p.topk; s0 += B) {
+    float y0[B], y1[B], w[B];
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
+    for (int j = 0; j < B; j++) {
       const int s = min(s0 + j, p.topk - 1);
       const int e = p.ids[r * p.topk + s] - p.e_lo;
       const bool keep = s0 + j < p.topk && e >= 0 && e < p.e_n;
@@ -565,10 +588,21 @@ __device__ __forceinline__ void combine_pairs_sum(const CombineParams& p, int r,
       w[j] = keep ? p.weights[r * p.topk + s] : 0.f;
     }
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
+    for (int j = 0; j < B; j++) {
       v0 = fmaf(w[j], y0[j], v0);
       v1 = fmaf(w[j], y1[j], v1);
     }
+  }
+}
+__device__ __forceinline__ void combine_pairs_sum(const CombineParams& p, int r, int c, float& v0, float& v1) {
+  v0 = 0.f;
+  v1 = 0.f;
+  if (p.topk <= 8) {
+    combine_pairs_batches<8>(p, r, c, v0, v1);
+  } else if (p.topk <= 12) {
+    combine_pairs_batches<12>(p, r, c, v0, v1);
+  } else {
+    combine_pairs_batches<24>(p, r, c, v0, v1);
   }
 }
 
@@ -648,62 +682,32 @@ __device__ __forceinline__ float gemv16_reduce(const f32x4_t& acc, float* part, 
   return sum;
 }
 
-// The router's launch of a small latent block (hibana/kernels/csrc/nemotron_moe.cu:496-558 of the reference):
+// The router's product of a small latent block (hibana/kernels/csrc/nemotron_moe.cu:496-558 of the reference):
 // fused[m, n] = x [router; fc1_latent]^T in FP32, sixteen output columns a workgroup, K split over its sixteen
-// wavefronts; then the workgroup that finishes last (ticket, as in moe_route_plan_kernel) rounds the latent columns to
-// BF16 and, with `do_route`, routes the rows - a wavefront a row, the logits read past its L2 - and, given a plan to
-// fill, plans the call.
+// wavefronts; the latent columns (e .. n - 1) are also left rounded to BF16.
 struct RouterGemv {
   const uint16_t* w;  // BF16 [n, k]
   const uint16_t* x;  // BF16 [m, k]
   float* fused;       // FP32 [m, n]
-  int n, k, m;
+  uint16_t* lat;      // BF16 [m, n - e]
+  int n, k, m, e;
 };
-__global__ __launch_bounds__(PLAN_THREADS) void latent_router_kernel(RouterGemv g, RouteParams route, int do_route, int ticket, int pairs, int e_lo, int e_n,
-                                                                     int32_t* __restrict__ plan, int32_t* __restrict__ order, int slot_rows, int slot_cap) {
-  extern __shared__ int lds[];
-  __shared__ int last;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n0 = blockIdx.x * 16, per_wave = g.k / PLAN_WAVES;
+__global__ __launch_bounds__(1024) void latent_router_kernel(RouterGemv g) {
+  __shared__ __align__(16) float part[16 * 256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n0 = blockIdx.x * 16, per_wave = g.k / 16;
   const f32x4_t acc = gemv16_wave(g.w, g.k, n0, g.n, g.x, g.k, g.m, wave * per_wave, per_wave / 32, lane);
-  const float sum = gemv16_reduce(acc, reinterpret_cast<float*>(lds), PLAN_WAVES);
+  const float sum = gemv16_reduce(acc, part, 16);
   if (threadIdx.x < 256) {
     const int row = threadIdx.x >> 4, n = n0 + (threadIdx.x & 15);
-    if (row < g.m && n < g.n) store_through(&g.fused[(int64_t)row * g.n + n], sum);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // in memory before the ticket is drawn
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const unsigned drawn = atomicAdd(&route_tickets[ticket], 1u);
-    last = drawn == gridDim.x - 1u;
-    if (last) route_tickets[ticket] = 0u;
-  }
-  __syncthreads();
-  if (!last) return;
-  if (!do_route) {  // the caller routes from `fused` itself: the BF16 latent rows only
-    for (int i = threadIdx.x; i < g.m * route.latent; i += PLAN_THREADS) {
-      const int row = i / route.latent, col = i - row * route.latent;
-      route.lat[i] = bf16_of(load_through(&g.fused[(int64_t)row * g.n + route.e + col]));
+    if (row < g.m && n < g.n) {
+      g.fused[(int64_t)row * g.n + n] = sum;
+      if (n >= g.e) g.lat[(int64_t)row * (g.n - g.e) + n - g.e] = bf16_of(sum);
     }
-    return;
   }
-  if (wave < g.m) {
-    if (route.per <= 8) {
-      route_row<true, 8, true>(route, wave, lane);
-    } else {
-      route_row<true, 16, true>(route, wave, lane);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  }
-  if (!plan) return;
-  __syncthreads();
-  plan_work<false>(route.ids, pairs, e_lo, e_n, 0, plan, order, slot_rows, slot_cap, nullptr, 1, 0, 0, lds);
 }
 
 // The last launch of a small latent block (nemotron_moe.cu's out kernel): out = bf16(shared + routed fc2^T) with
-// routed BF16 [m, latent]. When the routed experts' pair outputs are still to be summed, the launch's first `combines`
-// workgroups do that (the combine's FMA chain, a row and a 512-column span each, stored through to memory, then one
-// count on a ticket); the projection's workgroups - sixteen output columns each, K split over their wavefronts - load
-// their weights, wait for that count, and only then read routed. The last of them to finish clears both tickets.
+// routed BF16 [m, latent]; sixteen output columns a workgroup, K split over its wavefronts (at most eight steps each).
 struct OutGemv {
   const uint16_t* w;       // fc2 BF16 [n, k]
   const uint16_t* routed;  // BF16 [m, k]
@@ -711,50 +715,17 @@ struct OutGemv {
   uint16_t* out;           // BF16 [m, n]
   int n, k, m, waves;
 };
-__global__ __launch_bounds__(1024) void latent_out_kernel(OutGemv g, CombineParams c, int combines, int spans, int ticket, int ticket_done) {
+__global__ __launch_bounds__(1024) void latent_out_kernel(OutGemv g) {
   __shared__ __align__(16) float part[16 * 256];
-  if ((int)blockIdx.x < combines) {
-    const int r = blockIdx.x / spans, col = (blockIdx.x - r * spans) * COMBINE_SPAN + 2 * threadIdx.x;
-    if (threadIdx.x < 256 && col < c.h) {
-      float v0, v1;
-      combine_pairs_sum(c, r, col, v0, v1);
-      __hip_atomic_store(reinterpret_cast<uint32_t*>(c.out + (int64_t)r * c.h + col), (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16),
-                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) atomicAdd(&route_tickets[ticket], 1u);
-    return;
-  }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n0 = ((int)blockIdx.x - combines) * 16;
-  const int per_wave = g.k / g.waves, steps = per_wave / 32, k0 = wave * per_wave, r16 = lane & 15;  // at most eight steps a wavefront
-  const bool live = wave < g.waves;  // a workgroup has at least the 256 threads of the epilogue
-  GemvFrags a, b;
-  if (live) gemv16_load(b, g.w, g.k, min(n0 + r16, g.n - 1), k0, steps, lane);
-  if (combines) {
-    if (wave == 0) await_count(reinterpret_cast<const int32_t*>(&route_tickets[ticket]), combines);
-    __syncthreads();
-  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n0 = blockIdx.x * 16;
+  const int per_wave = g.k / g.waves;
+  const int out_row = threadIdx.x >> 4, out_n = n0 + (threadIdx.x & 15);
+  const bool stores = threadIdx.x < 256 && out_row < g.m && out_n < g.n;  // a workgroup has at least these 256 threads
+  const float base = stores && g.shared ? bf16_bits_to_f32(g.shared[(int64_t)out_row * g.n + out_n]) : 0.f;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-  if (live) {
-    gemv16_load(a, g.routed, g.k, min(r16, g.m - 1), k0, steps, lane);
-    gemv16_mfma(acc, a, b, steps);
-  }
+  if (wave < g.waves) acc = gemv16_wave(g.w, g.k, n0, g.n, g.routed, g.k, g.m, wave * per_wave, per_wave / 32, lane);
   const float sum = gemv16_reduce(acc, part, g.waves);
-  if (threadIdx.x < 256) {
-    const int row = threadIdx.x >> 4, n = n0 + (threadIdx.x & 15);
-    if (row < g.m && n < g.n) {
-      const float base = g.shared ? bf16_bits_to_f32(g.shared[(int64_t)row * g.n + n]) : 0.f;
-      g.out[(int64_t)row * g.n + n] = f32_to_bf16_bits(base + sum);
-    }
-  }
-  if (combines && threadIdx.x == 0) {  // every projection workgroup is past its wait once all of them have counted here
-    const unsigned drawn = atomicAdd(&route_tickets[ticket_done], 1u);
-    if (drawn == gridDim.x - (unsigned)combines - 1u) {
-      route_tickets[ticket] = 0u;
-      route_tickets[ticket_done] = 0u;
-    }
-  }
+  if (stores) g.out[(int64_t)out_row * g.n + out_n] = f32_to_bf16_bits(base + sum);
 }
 
 // ---------------------------------------------------------------------------------------------------- host side
@@ -904,6 +875,34 @@ int moe_launch_plan(const int32_t* ids, int64_t pairs, int e_lo, int e_n, int sh
 
 int moe_check_route(int m, int e, int k) { return m <= 0 || e <= 0 || k <= 0 || k > e || k > 64 || e > 64 * ROUTE_PER_LANE ? HB_EINVAL : HB_OK; }
 
+// Routing by `rp` (either rule) and the plan of its ids, in as few launches as the size allows.
+static int launch_route_plan(const RouteParams& rp, int m, int e_lo, int e_n, int shared_rows, const MoeWorkspace& ws, hipStream_t stream, int slot_rows,
+                             const QuantJob* job) {
+  const int64_t pairs = (int64_t)m * rp.k;
+  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
+  if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
+  if (m > ROUTE_FUSED_ROWS && pairs < PLAN_WIDE_PAIRS && g_route_plan_fused.load(std::memory_order_relaxed) != 2) {
+    // a verify-sized call: the routing spread over the device, the plan by the workgroup that finishes last
+    const int groups = (m + ROUTE_GROUP_ROWS - 1) / ROUTE_GROUP_ROWS;
+    const int ticket = (int)(g_route_ticket_next.fetch_add(1u, std::memory_order_relaxed) % ROUTE_TICKETS);
+    HB_LAUNCH(moe_route_plan_kernel, dim3((unsigned)groups + plan_groups(job) - 1u), dim3(PLAN_THREADS), plan_lds, stream, rp.ids, (int)pairs, e_lo, e_n,
+              shared_rows, ws.plan, ws.order, rp, m, groups, ticket, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows),
+              job ? *job : QuantJob{});
+    return HB_OK;
+  }
+  if (m > ROUTE_FUSED_ROWS) {  // a prefill-sized call: a wavefront a row over the whole device, then the plan's launches
+    if (rp.sigmoid) {
+      launch_route<true>(rp, m, stream);
+    } else {
+      launch_route<false>(rp, m, stream);
+    }
+    return moe_launch_plan(rp.ids, pairs, e_lo, e_n, shared_rows, ws, stream, slot_rows, job);
+  }
+  HB_LAUNCH(moe_plan_kernel<false>, dim3(plan_groups(job)), dim3(PLAN_THREADS), plan_lds, stream, rp.ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order,
+            rp, m, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows), ws.plan_wide, 1, 0, job ? *job : QuantJob{});
+  return HB_OK;
+}
+
 int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
                           const MoeWorkspace& ws, hipStream_t stream, int slot_rows, const QuantJob* job) {
   if (int err = moe_check_route(m, e, topk)) return err;
@@ -917,33 +916,18 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   rp.pad_id = e;
   rp.ids = ids;
   rp.weights = weights;
-  const int64_t pairs = (int64_t)m * topk;
-  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
-  if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
-  if (m > ROUTE_FUSED_ROWS && pairs < PLAN_WIDE_PAIRS && g_route_plan_fused.load(std::memory_order_relaxed) != 2) {
-    // a verify-sized call: the routing spread over the device, the plan by the workgroup that finishes last
-    const int groups = (m + ROUTE_GROUP_ROWS - 1) / ROUTE_GROUP_ROWS;
-    const int ticket = (int)(g_route_ticket_next.fetch_add(1u, std::memory_order_relaxed) % ROUTE_TICKETS);
-    HB_LAUNCH(moe_route_plan_kernel, dim3((unsigned)groups + plan_groups(job) - 1u), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n,
-              shared_rows, ws.plan, ws.order, rp, m, groups, ticket, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows),
-              job ? *job : QuantJob{});
-    return HB_OK;
-  }
-  if (m > ROUTE_FUSED_ROWS) {  // a prefill-sized call: a wavefront a row over the whole device, then the plan's launches
-    launch_route<false>(rp, m, stream);
-    return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, slot_rows, job);
-  }
-  HB_LAUNCH(moe_plan_kernel<false>, dim3(plan_groups(job)), dim3(PLAN_THREADS), plan_lds, stream, ids, (int)pairs, e_lo, e_n, shared_rows, ws.plan, ws.order,
-            rp, m, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows), ws.plan_wide, 1, 0, job ? *job : QuantJob{});
-  return HB_OK;
+  return launch_route_plan(rp, m, e_lo, e_n, shared_rows, ws, stream, slot_rows, job);
 }
 
 int latent_launch_router(const LatentRouter& r, hipStream_t stream) {
   const int n = r.experts + r.latent;
-  if (r.m <= 0 || r.m > LATENT_MAX_ROWS || r.hidden <= 0 || r.hidden % (32 * PLAN_WAVES) || r.latent < 0 || r.steps <= 0) return HB_EINVAL;
+  if (r.m <= 0 || r.m > LATENT_MAX_ROWS || r.hidden <= 0 || r.hidden % 512 || r.latent < 0 || r.steps <= 0) return HB_EINVAL;
   if (int err = moe_check_route(r.m, r.experts, r.topk)) return err;
-  RouterGemv g{r.w, r.x, r.fused, n, r.hidden, r.m};
+  RouterGemv g{r.w, r.x, r.fused, r.lat, n, r.hidden, r.m, r.experts};
+  HB_LAUNCH(latent_router_kernel, dim3((unsigned)((n + 15) / 16)), dim3(1024), 0, stream, g);
+  if (!r.route) return HB_OK;
   RouteParams rp{};
+  rp.sigmoid = 1;
   rp.logits = r.fused;
   rp.stride = n;
   rp.bias = r.bias;
@@ -957,41 +941,22 @@ int latent_launch_router(const LatentRouter& r, hipStream_t stream) {
   rp.latent = r.latent;
   rp.ids = r.ids;
   rp.weights = r.weights;
-  rp.lat = r.lat;
-  const int64_t pairs = (int64_t)r.m * r.topk;
-  size_t lds = (size_t)PLAN_WAVES * 256 * sizeof(float);
-  int slot_cap = 0;
-  if (r.route && r.plan) {
-    const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * r.e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
-    if (plan_lds > 64 * 1024 || r.e_n > PLAN_THREADS) return HB_EINVAL;
-    lds = std::max(lds, plan_lds);
-    slot_cap = (int)moe_max_slots(pairs, r.e_n, 0, ROWS_PER_SLOT);
+  rp.lat = nullptr;  // the product's epilogue has written them
+  if (!r.ws) {  // no plan to fill: the routing alone
+    launch_route<true>(rp, r.m, stream);
+    return HB_OK;
   }
-  const int ticket = (int)(g_route_ticket_next.fetch_add(1u, std::memory_order_relaxed) % ROUTE_TICKETS);
-  HB_LAUNCH(latent_router_kernel, dim3((unsigned)((n + 15) / 16)), dim3(PLAN_THREADS), lds, stream, g, rp, r.route, ticket, (int)pairs, r.e_lo, r.e_n,
-            r.route ? r.plan : nullptr, r.order, ROWS_PER_SLOT, slot_cap);
-  return HB_OK;
+  return launch_route_plan(rp, r.m, r.e_lo, r.e_n, 0, *r.ws, stream, ROWS_PER_SLOT, nullptr);
 }
 
-int latent_launch_out(const uint16_t* fc2, const uint16_t* routed, const uint16_t* shared, uint16_t* out, int m, int hidden, int latent,
-                      const CombineParams* pairs, hipStream_t stream) {
+int latent_launch_out(const uint16_t* fc2, const uint16_t* routed, const uint16_t* shared, uint16_t* out, int m, int hidden, int latent, hipStream_t stream) {
   if (m <= 0 || m > LATENT_MAX_ROWS || hidden <= 0 || latent <= 0 || latent % 32) return HB_EINVAL;
   const int steps = latent / 32;
   int waves = 1;
   while (waves < 16 && (steps % waves || steps / waves > 8)) waves *= 2;
   if (steps % waves || steps / waves > 8) return HB_EINVAL;
   OutGemv g{fc2, routed, shared, out, hidden, latent, m, waves};
-  CombineParams c{};
-  int combines = 0, spans = 1;
-  if (pairs) {
-    c = *pairs;
-    if (c.h != latent || c.m != m || c.h % 2) return HB_EINVAL;
-    spans = (c.h + COMBINE_SPAN - 1) / COMBINE_SPAN;
-    combines = m * spans;
-  }
-  const unsigned first = g_route_ticket_next.fetch_add(2u, std::memory_order_relaxed);
-  HB_LAUNCH(latent_out_kernel, dim3((unsigned)(combines + (hidden + 15) / 16)), dim3((unsigned)std::max(256, 64 * waves)), 0, stream, g, c, combines, spans,
-            (int)(first % ROUTE_TICKETS), (int)((first + 1u) % ROUTE_TICKETS));
+  HB_LAUNCH(latent_out_kernel, dim3((unsigned)((hidden + 15) / 16)), dim3((unsigned)std::max(256, 64 * waves)), 0, stream, g);
   return HB_OK;
 }
 

@@ -345,19 +345,20 @@ __global__ __launch_bounds__(1024) void nvfp4_stream_kernel(StreamParams p) {
 }
 
 // Two matrices of different geometry in one launch (the routed experts' layer beside the shared expert's, which reads
-// other activations): the first `first` workgroups are (slot, block group) of `a`, slot-major, the rest of `b`. The
-// workgroup size is the larger of the two shapes'; the other matrix's workgroups retire the wavefronts they do not use.
+// other activations): the first `first` workgroups are (slot, block group) of the dense `b`, slot-major - every one of
+// them has a whole K range to stream, so they start first - the rest of the planned `a`. Should the two shapes differ
+// in wavefronts a workgroup, the smaller one's workgroups retire the wavefronts they do not use.
 template <int EPI_A, int EPI_B>
 __global__ __launch_bounds__(1024) void nvfp4_twin_kernel(StreamParams a, StreamParams b, int groups_a, int groups_b, int first) {
   extern __shared__ __align__(16) uint8_t rings[];
   int id = blockIdx.x;
   if (id < first) {
-    const int slot = id / groups_a;
-    nvfp4_workgroup<EPI_A>(a, slot, id - slot * groups_a, rings);
-  } else {
-    id -= first;
     const int slot = id / groups_b;
     nvfp4_workgroup<EPI_B>(b, slot, id - slot * groups_b, rings);
+  } else {
+    id -= first;
+    const int slot = id / groups_a;
+    nvfp4_workgroup<EPI_A>(a, slot, id - slot * groups_a, rings);
   }
 }
 
@@ -390,8 +391,14 @@ template <int EPI_A, int EPI_B>
 static int launch_twin(StreamParams& a, int64_t slots_a, int64_t busy_a, StreamParams& b, int64_t slots_b, hipStream_t stream) {
   if (int e = shape_nvfp4(a, busy_a)) return e;
   if (int e = shape_nvfp4(b, slots_b)) return e;
+  if (b.ks * b.nbw != a.ks * a.nbw) {  // one workgroup size (and LDS a workgroup) for both: the plan's matrix sets it
+    const int waves = a.ks * a.nbw;
+    b.ks = std::min(b.ks, waves);
+    b.nbw = waves / b.ks;
+    set_split(b);
+  }
   const int groups_a = (a.n_blocks + a.nbw - 1) / a.nbw, groups_b = (b.n_blocks + b.nbw - 1) / b.nbw;
-  const int64_t first = slots_a * groups_a, all = first + slots_b * groups_b;
+  const int64_t first = slots_b * groups_b, all = first + slots_a * groups_a;
   if (all > 0x7fffffff) return HB_EINVAL;
   const int waves = std::max(a.ks * a.nbw, b.ks * b.nbw);
   HB_LAUNCH((nvfp4_twin_kernel<EPI_A, EPI_B>), dim3((unsigned)all), dim3(64 * waves), (size_t)waves * FP4_RING_BYTES, stream, a, b, groups_a, groups_b, (int)first);
@@ -708,8 +715,7 @@ extern "C" int hb_latent_router(const hb_latent_weights* w, const void* x, int m
   if (w->routed) {
     r.e_lo = w->routed->base;
     r.e_n = w->routed->experts;
-    r.plan = l.moe.plan;
-    r.order = l.moe.order;
+    r.ws = &l.moe;
   }
   if (int e = latent_launch_router(r, as_stream(stream))) return e;
   return launch_status();
@@ -738,7 +744,7 @@ extern "C" int hb_latent_out(const hb_latent_weights* w, const void* routed, int
     if (int e = launch_nvfp4<EPI_DENSE>(down, 1, 1, as_stream(stream))) return e;
   }
   if (int e = latent_launch_out(static_cast<const uint16_t*>(w->fc2), static_cast<const uint16_t*>(routed), w->shared_up ? l.shared_y : nullptr,
-                                static_cast<uint16_t*>(out), m, w->hidden, w->latent, nullptr, as_stream(stream)))
+                                static_cast<uint16_t*>(out), m, w->hidden, w->latent, as_stream(stream)))
     return e;
   return launch_status();
 }
@@ -778,8 +784,9 @@ extern "C" int hb_latent_block(const hb_latent_weights* w, const void* x, const 
   c.topk = topk;
   c.h = w->latent;
   c.out = l.routed;
+  moe_launch_combine(c, s);
   if (int e = latent_launch_out(static_cast<const uint16_t*>(w->fc2), l.routed, w->shared_up ? l.shared_y : nullptr, static_cast<uint16_t*>(out), m, w->hidden,
-                                w->latent, &c, s))
+                                w->latent, s))
     return e;
   return launch_status();
 }

@@ -522,9 +522,9 @@ struct CombineParams {
 void moe_launch_combine(const CombineParams& c, hipStream_t stream);
 
 // The dense ends of a latent block of at most LATENT_MAX_ROWS rows (hibana/kernels/csrc/nemotron_moe.cu of the reference).
-// Router: fused FP32 [m, experts + latent] = x [router; fc1_latent]^T; with `route`, sigmoid + bias top-k routing of the
-// rows (ids, weights, BF16 latent; padded rows take `pad_id`, or row 0's first choice when it is negative) and, with
-// `plan`, the expert plan of experts e_lo .. e_lo + e_n - 1 - all in one launch.
+// Router: fused FP32 [m, experts + latent] = x [router; fc1_latent]^T and its latent columns as BF16 (one launch);
+// with `route`, a second launch: sigmoid + bias top-k routing of the rows (ids, weights; padded rows take `pad_id`, or
+// row 0's first choice when it is negative) and, given a workspace, the expert plan of experts e_lo .. e_lo + e_n - 1.
 constexpr int LATENT_MAX_ROWS = HB_LATENT_MAX_ROWS;
 struct LatentRouter {
   const uint16_t* w;     // BF16 [experts + latent, hidden]
@@ -537,14 +537,11 @@ struct LatentRouter {
   float* weights;
   uint16_t* lat;
   int e_lo, e_n;
-  int32_t* plan;   // or null: routing only
-  int32_t* order;
+  const MoeWorkspace* ws;  // the plan's home, or null: routing only
 };
 int latent_launch_router(const LatentRouter& r, hipStream_t stream);
-// Out: out = bf16(shared + routed fc2^T), routed BF16 [m, latent]. With `pairs`, the same launch first sums the routed
-// experts' pair outputs into `routed` (pairs->out; pairs->h = latent).
-int latent_launch_out(const uint16_t* fc2, const uint16_t* routed, const uint16_t* shared, uint16_t* out, int m, int hidden, int latent,
-                      const CombineParams* pairs, hipStream_t stream);
+// Out: out = bf16(shared + routed fc2^T), routed BF16 [m, latent].
+int latent_launch_out(const uint16_t* fc2, const uint16_t* routed, const uint16_t* shared, uint16_t* out, int m, int hidden, int latent, hipStream_t stream);
 
 // The pieces of the combine that every kernel doing it shares, so that each gives the other's bits.
 // g = sigmoid(x[r] . gate_vec): 256 threads (t = 0 .. 255, four whole wavefronts) each add their share and leave four

@@ -302,7 +302,8 @@ int hb_nvfp4_moe(const hb_nvfp4_experts* routed, const void* x, const int32_t* i
  *
  * Weight-only arithmetic: activations stay BF16 (the reference's small-call kernels round x, lat and h to NVFP4 for its
  * FP4 tensor cores; its own FP32 statement of the block, NemotronMoe.reference, hibana/model/nemotron/moe.py:521-566,
- * is what these entry points follow). hb_latent_router followed by hb_latent_block is four launches.
+ * is what these entry points follow). hb_latent_router (two launches: the product; routing and plan) followed by
+ * hb_latent_block (four) is six launches where the block through separate operators is nine.
  * ---------------------------------------------------------------------------------------------------------------- */
 #define HB_LATENT_MAX_ROWS 16
 
@@ -325,15 +326,15 @@ size_t hb_latent_workspace_bytes(const hb_latent_weights* w, int m, int topk);
  * fused FP32 [m, experts_total + latent] and lat BF16 [m, latent]; with `route`, ids int32 [m, topk] / weights FP32
  * [m, topk] as hb_route_sigmoid_topk gives them from `fused`, bit for bit (slots / steps: its padded rows; a padded
  * row takes row 0's first choice at weight 0, or `pad_id` when that is >= 0), and the call's plan is left in the
- * workspace for hb_latent_block. Without `route`, ids / weights are not written (and may be NULL). One launch. */
+ * workspace for hb_latent_block. Without `route`, ids / weights are not written (and may be NULL). */
 int hb_latent_router(const hb_latent_weights* w, const void* x, int m, int topk, const int32_t* slots, int steps,
                      int route, int pad_id, float* fused, int32_t* ids, float* weights, void* lat, void* workspace,
                      size_t workspace_bytes, void* stream);
 
 /* ref: `block`, hibana/kernels/nemotron_moe.py:58-60: the rest of the block after hb_latent_router -> out BF16
  * [m, hidden]. `plan` != 0 when ids are not the router's (the caller routed): the plan is then made here, one more
- * launch. Three launches otherwise: routed fc1 beside the shared expert's up, routed fc2 beside its down, then the
- * combine and fc2_latent. */
+ * launch. Four launches otherwise: routed fc1 beside the shared expert's up, routed fc2 beside its down, the combine,
+ * fc2_latent. */
 int hb_latent_block(const hb_latent_weights* w, const void* x, const void* lat, const int32_t* ids,
                     const float* weights, int m, int topk, int plan, void* out, void* workspace,
                     size_t workspace_bytes, void* stream);
