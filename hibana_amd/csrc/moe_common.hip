@@ -601,6 +601,8 @@ __device__ __forceinline__ void combine_pairs_sum(const CombineParams& p, int r,
     combine_pairs_batches<8>(p, r, c, v0, v1);
   } else if (p.topk <= 12) {
     combine_pairs_batches<12>(p, r, c, v0, v1);
+  } else if (p.m > 64) {  // a long call is bound by its traffic: fewer registers, more wavefronts
+    combine_pairs_batches<8>(p, r, c, v0, v1);
   } else {
     combine_pairs_batches<24>(p, r, c, v0, v1);
   }

@@ -490,7 +490,7 @@ extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float glob
   p.m = m;
   p.out = y;
   p.out_stride = n;
-  if (tile_takes(m, k) && (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && tile_serves_dense(m, p.n_blocks)))) {
+  if (tile_takes(m, k) && tile_writes(y, false) && (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && tile_serves_dense(m, p.n_blocks)))) {
     const int64_t tile_slots = (m + TILE_ROWS - 1) / TILE_ROWS;
     if (int e = relu2 ? launch_tile<TileNvfp4, EPI_DENSE_RELU2>(p, tile_slots, m, as_stream(stream)) : launch_tile<TileNvfp4, EPI_DENSE>(p, tile_slots, m, as_stream(stream)))
       return e;
@@ -558,7 +558,7 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
   const int64_t pairs = (int64_t)m * topk;
   // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel; below that the
   // 16-row slots of the weight stream
-  const bool dense = tile_takes(m, ex->hidden) && tile_takes(pairs, ex->inter) &&
+  const bool dense = tile_takes(m, ex->hidden) && tile_takes(pairs, ex->inter) && tile_writes(out_pairs, !pairs_bf16) &&
                      (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && pairs >= (int64_t)ex->experts * TILE_DENSE_ROWS));
   const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
   const int64_t slots = moe_max_slots(pairs, ex->experts, 0, slot_rows);

@@ -114,7 +114,7 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
           }
           const bf16x8_t af = __builtin_bit_cast(bf16x8_t, a);
 #pragma unroll
-          for (int nt = 0; nt < 4; nt++) acc[t][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, b[nt], acc[t][nt], 0, 0, 0);
+          for (int nt = 0; nt < 4; nt++) acc[t][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[nt], af, acc[t][nt], 0, 0, 0);
         }
       }
     }
@@ -123,37 +123,48 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
     __syncthreads();                                   // the next buffer is complete and this one is free to refill
   }
   if (!active) return;
-  // accumulator register r of lane (q, r16) of tile (t, nt): slot row 16 t + 4 q + r, weight row nb * 64 + 16 nt + r16
-  float scale[4];
-#pragma unroll
-  for (int nt = 0; nt < 4; nt++) scale[nt] = Fmt::PER_ROW ? sl.rs[nb * 64 + 16 * nt + r16] : sl.scalar;
+  // The weights are the MFMA's A operand and the activations its B: accumulator register r of lane (q, r16) of tile
+  // (t, nt) is slot row 16 t + r16, weight row nb * 64 + 16 nt + 4 q + r - four neighbouring output columns a lane, one
+  // store of 8 (BF16) or 16 bytes (FP32) for them.
+  const int i16 = r16;
 #pragma unroll
   for (int t = 0; t < MT; t++) {
     if (FULL || t < tiles) {
+      const int i = 16 * t + i16;
+      if (i < sl.rows) {
+        const int64_t pos = sl.p0 + i;
+        if (EPI == EPI_FC1_GATED) {
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int i = 16 * t + 4 * q + r;
-        if (i < sl.rows) {
-          const int64_t pos = sl.p0 + i;
-          if (EPI == EPI_FC1_GATED) {
+          for (int g = 0; g < 2; g++) {
+            uint16_t h[4];
 #pragma unroll
-            for (int g = 0; g < 2; g++) {
-              const float up = through_bf16(acc[t][2 * g][r] * scale[2 * g]), gate = through_bf16(acc[t][2 * g + 1][r] * scale[2 * g + 1]);
-              reinterpret_cast<uint16_t*>(p.out)[pos * p.out_stride + nb * 32 + 16 * g + r16] = bf16_of(silu(gate) * up);
+            for (int r = 0; r < 4; r++) {
+              const float su = Fmt::PER_ROW ? sl.rs[nb * 64 + 32 * g + 4 * q + r] : sl.scalar, sg = Fmt::PER_ROW ? sl.rs[nb * 64 + 32 * g + 16 + 4 * q + r] : sl.scalar;
+              const float up = through_bf16(acc[t][2 * g][r] * su), gate = through_bf16(acc[t][2 * g + 1][r] * sg);
+              h[r] = bf16_of(silu(gate) * up);
             }
-          } else {
-            const int64_t at = (EPI == EPI_FC2 ? (int64_t)p.order[pos] : pos) * p.out_stride + nb * 64 + r16;
+            *reinterpret_cast<tile_u32x2_t*>(reinterpret_cast<uint16_t*>(p.out) + pos * p.out_stride + nb * 32 + 16 * g + 4 * q) =
+                tile_u32x2_t{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+          }
+        } else {
+          const int64_t at = (EPI == EPI_FC2 ? (int64_t)p.order[pos] : pos) * p.out_stride + nb * 64 + 4 * q;
 #pragma unroll
-            for (int nt = 0; nt < 4; nt++) {
-              const float y = acc[t][nt][r] * scale[nt];
-              if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
-                const float h = fmaxf(through_bf16(y), 0.f);
-                reinterpret_cast<uint16_t*>(p.out)[at + 16 * nt] = bf16_of(h * h);
-              } else if (EPI == EPI_DENSE || p.out_bf16) {
-                reinterpret_cast<uint16_t*>(p.out)[at + 16 * nt] = bf16_of(y);
-              } else {
-                reinterpret_cast<float*>(p.out)[at + 16 * nt] = y;
+          for (int nt = 0; nt < 4; nt++) {
+            float y[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) y[r] = acc[t][nt][r] * (Fmt::PER_ROW ? sl.rs[nb * 64 + 16 * nt + 4 * q + r] : sl.scalar);
+            if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
+#pragma unroll
+              for (int r = 0; r < 4; r++) {
+                const float h = fmaxf(through_bf16(y[r]), 0.f);
+                y[r] = h * h;
               }
+            }
+            if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2 || EPI == EPI_DENSE || p.out_bf16) {
+              *reinterpret_cast<tile_u32x2_t*>(reinterpret_cast<uint16_t*>(p.out) + at + 16 * nt) =
+                  tile_u32x2_t{(uint32_t)bf16_of(y[0]) | ((uint32_t)bf16_of(y[1]) << 16), (uint32_t)bf16_of(y[2]) | ((uint32_t)bf16_of(y[3]) << 16)};
+            } else {
+              *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(p.out) + at + 16 * nt) = f32x4_t{y[0], y[1], y[2], y[3]};
             }
           }
         }
@@ -186,8 +197,10 @@ inline bool tile_serves_dense(int m, int n_blocks) {
 }
 
 // Whether an activation matrix of `rows` rows is one the tile kernel takes: it addresses the matrix with 32-bit byte
-// offsets.
+// offsets ...
 inline bool tile_takes(int64_t rows, int64_t a_stride) { return rows * a_stride * 2 <= 0xffffffffll; }
+// ... and writes four neighbouring output columns with one store: 8 bytes of BF16, 16 of FP32.
+inline bool tile_writes(const void* out, bool f32) { return aligned(out, f32 ? 16 : 8); }
 
 // `slots`: the grid's second dimension (routed: the plan's upper bound; dense: ceil(m / TILE_ROWS)); `a_rows`: rows of
 // the activation matrix.

@@ -850,7 +850,7 @@ extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* 
   p.m = m;
   p.out = y;
   p.out_stride = n;
-  if (tile_takes(m, k) && (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && tile_serves_dense(m, p.n_blocks)))) {
+  if (tile_takes(m, k) && tile_writes(y, false) && (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && tile_serves_dense(m, p.n_blocks)))) {
     if (int e = launch_tile<TileW3, EPI_DENSE>(p, (m + TILE_ROWS - 1) / TILE_ROWS, m, as_stream(stream))) return e;
     return launch_status();
   }
@@ -929,7 +929,7 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   const int shared_rows = shared ? m : 0;
   // a dense contraction once an expert sees a few dozen rows: slots of 128 rows on the MFMA tile kernel
   // (E4M3 activations: the stream only)
-  const bool dense = !e4m3 && tile_takes(m, ex->hidden) && tile_takes(pairs + shared_rows, ex->inter) &&
+  const bool dense = !e4m3 && tile_takes(m, ex->hidden) && tile_takes(pairs + shared_rows, ex->inter) && tile_writes(out_pairs, !pairs_bf16) &&
                      (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && pairs >= (int64_t)ex->experts * 2 * TILE_DENSE_ROWS));  // the pre-scaled expansion costs more here than the stream's
   const int slot_rows = dense ? TILE_ROWS : ROWS_PER_SLOT;
   const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows, slot_rows);

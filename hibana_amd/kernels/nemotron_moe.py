@@ -1,8 +1,8 @@
 """The latent-MoE block of a decode / verify call (at most MAX_ROWS rows) behind the reference's small-call surface
-(hibana/kernels/nemotron_moe.py:45-68): `router` (the router|fc1_latent product, the routing of every row as
-`model.nemotron_moe.route_topk` does it from the same FP32 rows, bit for bit, and the call's plan - one launch), then
-`block` (routed up beside the shared expert's up, routed down beside its down, combine + fc2_latent: three launches),
-or `w3_block` around 3-bit routed experts.
+(hibana/kernels/nemotron_moe.py:45-68): `router` (the router|fc1_latent product on the matrix cores, then the routing
+of every row as `model.nemotron_moe.route_topk` does it from the same FP32 rows, bit for bit, with the call's plan: two
+launches), then `block` (routed up beside the shared expert's up, routed down beside its down, the combine,
+fc2_latent: four launches), or `w3_block` around 3-bit routed experts.
 
 `weights` is a `SmallWeights` (what the kernels read, the reference's `NemotronMoe.small_weights()` list): assembled
 once a block, it holds the device pointers' owners. Activations stay BF16 throughout (weight-only arithmetic: the
