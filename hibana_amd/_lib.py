@@ -67,6 +67,8 @@ SIGNATURES = {
     "hb_nvfp4_repack": (_I, [_P, _P, _I, _L, _I, _P, _P]),
     "hb_nvfp4_dequant": (_I, [_P, _F, _L, _I, _P, _P]),
     "hb_nvfp4_gemm": (_I, [_P, _I, _P, _F, _I, _I, _I, _P, _P]),
+    "hb_nvfp4_gemm_workspace_bytes": (_Z, [_I, _I, _I]),
+    "hb_nvfp4_gemm_ws": (_I, [_P, _I, _P, _F, _I, _I, _I, _P, _P, _Z, _P]),
     "hb_nvfp4_moe_workspace_bytes": (_Z, [_I, _I, _EX4]),
     "hb_nvfp4_moe": (_I, [_EX4, _P, _P, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "hb_latent_workspace_bytes": (_Z, [_LW, _I, _I]),

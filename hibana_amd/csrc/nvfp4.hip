@@ -363,7 +363,7 @@ __global__ __launch_bounds__(1024) void nvfp4_twin_kernel(StreamParams a, Stream
 }
 
 // experiments (hb_tune): the stream's workgroup shape ("nvfp4_ksplit", "nvfp4_nbw"); "nvfp4_tile": 1 forces the tile kernel, 2 the stream
-static std::atomic<int> g_nvfp4_ksplit{0}, g_nvfp4_nbw{0}, g_nvfp4_tile{0}, g_nvfp4_few{0};  // "nvfp4_few": 2 switches off the body for slots of at most eight rows
+static std::atomic<int> g_nvfp4_ksplit{0}, g_nvfp4_nbw{0}, g_nvfp4_tile{0}, g_nvfp4_few{0}, g_nvfp4_tile_ks{0};  // "nvfp4_few": 2 switches off the body for slots of at most eight rows; "nvfp4_tile_ks": the workgroups that share a tile's K
 
 static int shape_nvfp4(StreamParams& p, int64_t busy_slots) {
   pick_shape(p.n_blocks, p.chunks, busy_slots, 4096, &p.ks, &p.nbw);
@@ -449,6 +449,20 @@ static inline unsigned grid_for(int64_t threads) { return (unsigned)((threads + 
 
 using namespace hb;
 
+static StreamParams dense_params(const void* tiled, float scale, int n, int k, const void* x, int m, void* y) {
+  StreamParams p{};
+  p.w = static_cast<const uint8_t*>(tiled);
+  p.scalar = scale;
+  p.n_blocks = n / 64;
+  p.chunks = k / 128;
+  p.a = static_cast<const uint16_t*>(x);
+  p.a_stride = k;
+  p.m = m;
+  p.out = y;
+  p.out_stride = n;
+  return p;
+}
+
 extern "C" size_t hb_nvfp4_tiled_bytes(int64_t rows, int k) {
   if (rows <= 0 || k <= 0 || rows % 64 || k % 128) return 0;
   return (size_t)(rows / 64) * (size_t)(k / 128) * NVFP4_BLOCK_BYTES;
@@ -476,31 +490,47 @@ extern "C" int hb_nvfp4_dequant(const void* tiled, float global_scale, int64_t r
   return launch_status();
 }
 
-extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y, void* stream) {
+// `workspace`: room for partial tiles (hb_nvfp4_gemm_workspace_bytes), or null: no call shares K among workgroups.
+static int nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y, void* workspace, size_t workspace_bytes,
+                      hipStream_t stream) {
   if (!x || !tiled || !y) return HB_ENULL;
   if (m <= 0 || n <= 0 || k <= 0 || n % 64 || k % 128) return HB_EINVAL;
-  if (!aligned(x, 16) || !aligned(tiled, 16) || !aligned(y, 2)) return HB_EINVAL;
-  StreamParams p{};
-  p.w = static_cast<const uint8_t*>(tiled);
-  p.scalar = global_scale;
-  p.n_blocks = n / 64;
-  p.chunks = k / 128;
-  p.a = static_cast<const uint16_t*>(x);
-  p.a_stride = k;
-  p.m = m;
-  p.out = y;
-  p.out_stride = n;
-  if (tile_takes(m, k) && tile_writes(y, false) && (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && tile_serves_dense(m, p.n_blocks)))) {
+  if (!aligned(x, 16) || !aligned(tiled, 16) || !aligned(y, 2) || !aligned(workspace, 16)) return HB_EINVAL;
+  StreamParams p = dense_params(tiled, global_scale, n, k, x, m, y);
+  // between the weight stream's sixteen rows a pass and a call that fills the device with 128-row tiles: tiles whose K
+  // is shared among workgroups
+  int ks = workspace && m > TILE_SPLIT_ROWS ? tile_split(m, p.n_blocks, p.chunks) : 1;
+  if (g_nvfp4_tile_ks && workspace) ks = std::min(g_nvfp4_tile_ks.load(), p.chunks);
+  if (tile_partial_bytes(m, p.n_blocks, ks) > workspace_bytes) ks = 1;
+  if (tile_takes(m, k) && tile_writes(y, false) && (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && (ks > 1 || tile_serves_dense(m, p.n_blocks))))) {
     const int64_t tile_slots = (m + TILE_ROWS - 1) / TILE_ROWS;
-    if (int e = relu2 ? launch_tile<TileNvfp4, EPI_DENSE_RELU2>(p, tile_slots, m, as_stream(stream)) : launch_tile<TileNvfp4, EPI_DENSE>(p, tile_slots, m, as_stream(stream)))
-      return e;
+    if (ks > 1) {
+      p.tile_ks = ks;
+      p.tile_mt = tile_partial_mt(m);
+      p.partial = static_cast<float*>(workspace);
+    }
+    if (int e = relu2 ? launch_tile<TileNvfp4, EPI_DENSE_RELU2>(p, tile_slots, m, stream) : launch_tile<TileNvfp4, EPI_DENSE>(p, tile_slots, m, stream)) return e;
     return launch_status();
   }
   const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
   if (slots > 65535) return HB_EINVAL;
-  if (int e = relu2 ? launch_nvfp4<EPI_DENSE_RELU2>(p, slots, slots, as_stream(stream)) : launch_nvfp4<EPI_DENSE>(p, slots, slots, as_stream(stream)))
-    return e;
+  if (int e = relu2 ? launch_nvfp4<EPI_DENSE_RELU2>(p, slots, slots, stream) : launch_nvfp4<EPI_DENSE>(p, slots, slots, stream)) return e;
   return launch_status();
+}
+
+extern "C" int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y, void* stream) {
+  return nvfp4_gemm(x, m, tiled, global_scale, n, k, relu2, y, nullptr, 0, as_stream(stream));
+}
+
+extern "C" size_t hb_nvfp4_gemm_workspace_bytes(int m, int n, int k) {
+  if (m <= TILE_SPLIT_ROWS || n <= 0 || k <= 0 || n % 64 || k % 128) return 0;
+  const int want = g_nvfp4_tile_ks ? std::min(g_nvfp4_tile_ks.load(), k / 128) : tile_split(m, n / 64, k / 128);
+  return tile_partial_bytes(m, n / 64, want);
+}
+
+extern "C" int hb_nvfp4_gemm_ws(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  return nvfp4_gemm(x, m, tiled, global_scale, n, k, relu2, y, workspace_bytes ? workspace : nullptr, workspace_bytes, as_stream(stream));
 }
 
 // ------------------------------------------------------------------------------------------------ routed experts
@@ -577,20 +607,6 @@ int run_experts(const hb_nvfp4_experts* ex, const void* x, const int32_t* ids, i
   return launch_status();
 }
 
-StreamParams dense_params(const void* tiled, float scale, int n, int k, const void* x, int m, void* y) {
-  StreamParams p{};
-  p.w = static_cast<const uint8_t*>(tiled);
-  p.scalar = scale;
-  p.n_blocks = n / 64;
-  p.chunks = k / 128;
-  p.a = static_cast<const uint16_t*>(x);
-  p.a_stride = k;
-  p.m = m;
-  p.out = y;
-  p.out_stride = n;
-  return p;
-}
-
 // ------------------------------------------------------------------------------------- the small latent block
 struct LatentWorkspace {
   MoeWorkspace moe;    // the routed experts' (absent without NVFP4 experts)
@@ -639,7 +655,7 @@ int check_latent(const hb_latent_weights* w, int m, int topk) {
 
 int hb::nvfp4_tune(const char* key, int value) {
   std::atomic<int>* slot = !strcmp(key, "nvfp4_tile") ? &g_nvfp4_tile : !strcmp(key, "nvfp4_ksplit") ? &g_nvfp4_ksplit : !strcmp(key, "nvfp4_nbw") ? &g_nvfp4_nbw
-              : !strcmp(key, "nvfp4_few") ? &g_nvfp4_few : nullptr;
+              : !strcmp(key, "nvfp4_few") ? &g_nvfp4_few : !strcmp(key, "nvfp4_tile_ks") ? &g_nvfp4_tile_ks : nullptr;
   if (!slot || value < 0 || value > 16) return HB_EINVAL;
   *slot = value;
   return HB_OK;

@@ -47,6 +47,9 @@ struct StreamParams {
   int ks, nbw;            // wavefronts per workgroup = ks (K splits) * nbw (64-row blocks)
   int ks_inv, chunks_base, chunks_rem;  // set_split(): ceil(65536 / ks), chunks / ks, chunks % ks
   int no_few;             // W3 stream: slots of at most four rows take the sixteen-row body too
+  float* partial;         // tile kernel with K shared among workgroups: their partial tiles (see tile_kernel.hpp)
+  int tile_ks, tile_mt;   // ... the workgroups a tile (1: none), the 16-row tiles a partial region holds
+  int tile_ticket;        // ... and the first of the launch's arrival counters
   int64_t* trace;         // measurement hook (hb_debug_trace): a record a workgroup, else null
   int32_t* done;          // fc1 and fc2 in one launch: the slots' arrival counters (plan_done), else null
   int done_need;          // ... and the fc1 workgroups a slot has

@@ -16,6 +16,9 @@
 // and PER_ROW (FP32 scale per output row, else one per matrix).
 #pragma once
 
+#include <algorithm>
+#include <atomic>
+
 #include "stream_common.hpp"
 
 namespace hb {
@@ -49,16 +52,35 @@ __device__ __forceinline__ void stage_tile(const StreamParams& p, const uint32_t
 
 // ST: the slot's number of 16-row tiles when it is a compile-time constant (no test around a tile's MFMAs, so every
 // accumulator stays in place from chunk to chunk), or 0 for any count.
+//
+// K shared among workgroups (p.tile_ks > 1, dense calls of a few dozen rows, which alone would fill too few compute
+// units): workgroup z of a tile takes chunks c0 .. c1 - 1, leaves its unscaled FP32 accumulators in `p.partial`
+// (stores written through to memory and waited for: a release at device scope, which writes back the whole L2, costs
+// each workgroup tens of microseconds here), counts itself on the tile's arrival counter, and the one that arrives
+// last (an acquire, then ordinary loads) adds all the partial tiles in the order of z - the same sum whichever it is -
+// and runs the epilogue. The counters are the
+// library's (tile_tickets: zero between launches, put back by every last arriver; a launch takes a range of them).
+constexpr int TILE_TICKETS = 1 << 16;
+static __device__ unsigned int tile_tickets[TILE_TICKETS];
+
+__device__ __forceinline__ void store_through16(f32x4_t* at, const f32x4_t& v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(at), "v"(v) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_but(void) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
 template <class Fmt, int EPI, int ST>
-__device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl, uint8_t* tile_lds) {
+__device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl, uint8_t* tile_lds, int c0, int c1, int z) {
   constexpr bool FULL = ST > 0;
   constexpr int MT = FULL ? ST : TILE_MT;
+  constexpr int BUFS = 2, BUF = TILE_BUF;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: kept in scalars
   const int q = lane >> 4, r16 = lane & 15;
   const int nb = blockIdx.x * 4 + wave;
   const bool active = nb < p.n_blocks;
   const int tiles = FULL ? ST : (sl.rows + 15) >> 4;
-  int32_t* rowtab = reinterpret_cast<int32_t*>(tile_lds + 2 * TILE_BUF);
+  int32_t* rowtab = reinterpret_cast<int32_t*>(tile_lds + BUFS * BUF);
   if (threadIdx.x < TILE_ROWS) {  // the source row of each slot row (rows past the last repeat it)
     int64_t arow = sl.p0 + min((int)threadIdx.x, sl.rows - 1);
     if (epi_gathers(EPI)) {
@@ -80,22 +102,13 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) acc[t][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const uint8_t* blk = sl.w + (int64_t)(active ? nb : 0) * p.chunks * Fmt::BLOCK_BYTES;
-  typename Fmt::Chunk cur, nxt;
-  Fmt::load(cur, blk, lane, r16);
-  stage_tile(p, piece, tile_lds, 0, tiles, wave);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  for (int c = 0; c < p.chunks; c++) {
-    uint8_t* buf = tile_lds + (c & 1) * TILE_BUF;
-    if (c + 1 < p.chunks) {
-      Fmt::load(nxt, blk + (int64_t)(c + 1) * Fmt::BLOCK_BYTES, lane, r16);
-      stage_tile(p, piece, tile_lds + ((c + 1) & 1) * TILE_BUF, c + 1, tiles, wave);
-    }
+  // One chunk: the products of the chunk's four 32-k steps from its weights `w` and its activation buffer.
+  auto multiply = [&](const typename Fmt::Chunk& w, const uint8_t* buf) {
 #pragma unroll
     for (int s = 0; s < 4; s++) {  // 32-k steps of the chunk
       bf16x8_t b[4];
 #pragma unroll
-      for (int nt = 0; nt < 4; nt++) b[nt] = Fmt::fragment(cur, nt, s, sl);
+      for (int nt = 0; nt < 4; nt++) b[nt] = Fmt::fragment(w, nt, s, sl);
       // lane (q, r16) of tile t: row 16 t + r16; its eight k of the step as the format's tile layout owns them
       const int half = (q & 1) << 3;
       const int slot_lo = ((4 * s + (q >> 1)) ^ r16) << 4, slot_hi = ((4 * s + 2 + (q >> 1)) ^ r16) << 4;
@@ -118,9 +131,56 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
         }
       }
     }
+  };
+  auto request = [&](typename Fmt::Chunk& w, uint8_t* buf, int c) {  // a chunk's weights and this wavefront's share of its activation rows
+    Fmt::load(w, blk + (int64_t)c * Fmt::BLOCK_BYTES, lane, r16);
+    stage_tile(p, piece, buf, c, tiles, wave);
+  };
+  typename Fmt::Chunk cur, nxt;
+  request(cur, tile_lds, c0);
+  wait_but<0>();
+  __syncthreads();
+  for (int c = c0; c < c1; c++) {
+    uint8_t* buf = tile_lds + ((c - c0) & 1) * BUF;
+    if (c + 1 < c1) request(nxt, tile_lds + ((c - c0 + 1) & 1) * BUF, c + 1);
+    multiply(cur, buf);
     cur = nxt;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's LDS-direct loads have landed before it signals
-    __syncthreads();                                   // the next buffer is complete and this one is free to refill
+    wait_but<0>();    // this wavefront's LDS-direct loads have landed before it signals
+    __syncthreads();  // the next buffer is complete and this one is free to refill
+  }
+  if (p.tile_ks > 1) {
+    const int64_t region = (int64_t)p.tile_mt * 4 * 64;  // f32x4 a wavefront
+    const int64_t tile = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+    f32x4_t* mine = reinterpret_cast<f32x4_t*>(p.partial) + ((tile * p.tile_ks + z) * 4 + wave) * region + lane;
+    if (active) {
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+        if (FULL || t < tiles)
+#pragma unroll
+          for (int nt = 0; nt < 4; nt++) store_through16(mine + (t * 4 + nt) * 64, acc[t][nt]);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the partial tile is in memory before the count
+    __syncthreads();
+    int* last = reinterpret_cast<int*>(rowtab);  // the row table has served
+    if (threadIdx.x == 0) {
+      unsigned int* ticket = &tile_tickets[(p.tile_ticket + tile) & (TILE_TICKETS - 1)];
+      const unsigned drawn = atomicAdd(ticket, 1u);
+      *last = drawn == (unsigned)p.tile_ks - 1u;
+      if (*last) *ticket = 0u;
+    }
+    __syncthreads();
+    if (!*last || !active) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // drop what this compute die's L2 holds of the others' regions
+    const f32x4_t* all = reinterpret_cast<const f32x4_t*>(p.partial) + (tile * p.tile_ks * 4 + wave) * region + lane;
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+      if (FULL || t < tiles)
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+          f32x4_t sum = all[(t * 4 + nt) * 64];
+          for (int k = 1; k < p.tile_ks; k++) sum += all[(int64_t)k * 4 * region + (t * 4 + nt) * 64];
+          acc[t][nt] = sum;
+        }
   }
   if (!active) return;
   // The weights are the MFMA's A operand and the activations its B: accumulator register r of lane (q, r16) of tile
@@ -180,10 +240,13 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(StreamParams p) {
   if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
   // uniform over the workgroup; more compile-time counts than the full slot were tried: with a third body the
   // compiler spills and every one of them gets slower
+  // blockIdx.z shares K: the first chunks % tile_ks of them take one chunk more
+  const int ks = p.tile_ks > 1 ? p.tile_ks : 1, z = blockIdx.z, base = p.chunks / ks, rem = p.chunks - base * ks;
+  const int c0 = z * base + min(z, rem), c1 = c0 + base + (z < rem ? 1 : 0);
   if (sl.rows > TILE_ROWS - 16) {
-    tile_slot<Fmt, EPI, TILE_MT>(p, sl, tile_lds);
+    tile_slot<Fmt, EPI, TILE_MT>(p, sl, tile_lds, c0, c1, z);
   } else {
-    tile_slot<Fmt, EPI, 0>(p, sl, tile_lds);
+    tile_slot<Fmt, EPI, 0>(p, sl, tile_lds, c0, c1, z);
   }
 }
 
@@ -204,11 +267,34 @@ inline bool tile_writes(const void* out, bool f32) { return aligned(out, f32 ? 1
 
 // `slots`: the grid's second dimension (routed: the plan's upper bound; dense: ceil(m / TILE_ROWS)); `a_rows`: rows of
 // the activation matrix.
+static std::atomic<unsigned> g_tile_ticket_next{0};
+
+// Workgroups a tile for a dense call of m rows (K shared among them), given room for their partial tiles: about four
+// hundred workgroups in all (measured at 25600 x 5120: the best count from 24 to 128 rows), each with at least four
+// chunks. 1: the call has two hundred tiles or more and fills the device alone.
+inline int tile_split(int m, int n_blocks, int chunks) {
+  const int64_t tiles = (int64_t)((n_blocks + 3) / 4) * ((m + TILE_ROWS - 1) / TILE_ROWS);
+  if (tiles >= 200) return 1;
+  return (int)std::max<int64_t>(1, std::min<int64_t>(chunks / 4, 400 / tiles));
+}
+constexpr int TILE_SPLIT_ROWS = 20;  // up to here two passes of the weight stream are the faster
+inline int tile_partial_mt(int m) { return (std::min(m, TILE_ROWS) + 15) / 16; }
+inline size_t tile_partial_bytes(int m, int n_blocks, int ks) {
+  const int64_t tiles = (int64_t)((n_blocks + 3) / 4) * ((m + TILE_ROWS - 1) / TILE_ROWS);
+  return ks > 1 ? (size_t)tiles * ks * 4 * tile_partial_mt(m) * 4 * 64 * sizeof(f32x4_t) : 0;
+}
+
 template <class Fmt, int EPI>
 static int launch_tile(StreamParams& p, int64_t slots, int64_t a_rows, hipStream_t stream) {
   if (!tile_takes(a_rows, p.a_stride)) return HB_EINVAL;
   p.slot_rows = TILE_ROWS;
-  const dim3 grid((unsigned)((p.n_blocks + 3) / 4), (unsigned)slots);
+  const unsigned groups = (unsigned)((p.n_blocks + 3) / 4);
+  const int ks = p.tile_ks > 1 ? p.tile_ks : 1;
+  if (ks > 1) {
+    if (!p.partial || ks > p.chunks || (int64_t)groups * slots > TILE_TICKETS) return HB_EINVAL;
+    p.tile_ticket = (int)(g_tile_ticket_next.fetch_add(groups * (unsigned)slots, std::memory_order_relaxed) & (TILE_TICKETS - 1));
+  }
+  const dim3 grid(groups, (unsigned)slots, (unsigned)ks);
   HB_LAUNCH((tile_kernel<Fmt, EPI>), grid, dim3(256), 2 * TILE_BUF + TILE_ROWS * sizeof(int32_t), stream, p);
   return HB_OK;
 }

@@ -266,6 +266,16 @@ int hb_nvfp4_dequant(const void* tiled, float global_scale, int64_t rows, int k,
 int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y,
                   void* stream);
 
+/* The same product with room for partial sums: calls of a few dozen rows (17 .. about 250), too many for the weight
+ * stream's sixteen rows a pass over the matrix and too few to fill the device with 128-row tiles, share K among the
+ * workgroups of a tile; their partial tiles meet in `workspace` and whichever workgroup of a tile finishes last adds them
+ * in one fixed order: the result does not depend on the schedule. hb_nvfp4_gemm_workspace_bytes: what a call of this
+ * shape uses (0: none, the call is hb_nvfp4_gemm's). No counterpart in the reference (cuBLASLt / FlashInfer own their
+ * workspaces there). */
+size_t hb_nvfp4_gemm_workspace_bytes(int m, int n, int k);
+int hb_nvfp4_gemm_ws(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * Routed experts on NVFP4 weights (ReLU^2 when fc1 has inter rows per expert, gated SiLU when it has 2*inter rows in
  * the W3 path's fc1_order).

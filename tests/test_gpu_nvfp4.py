@@ -97,6 +97,31 @@ def test_weight_only_linear_matches_the_oracle(m, relu2, n, k):
     assert torch.equal(lin(x.cuda()), ops.nvfp4_linear(x.cuda(), lin))
 
 
+@pytest.mark.parametrize("m", [17, 21, 40, 64, 100, 128, 200])
+@pytest.mark.parametrize("ks", [0, 2, 3, 5])
+def test_tiles_whose_k_is_shared_among_workgroups(m, ks):
+    """A few dozen rows: the workgroups of a tile split K, leave their partial tiles in the workspace and the last one
+    to arrive adds them in a fixed order: the oracle's product, the same bits on every call, and (an order of FP32 sums
+    aside) the bits of the undivided tile."""
+    from hibana_amd import _lib
+    from hibana_amd.kernels import ops
+    n, k = 320, 2688
+    packed, scales = _matrix(n, k, 13, hi=8.0)
+    lin = _linear(packed, scales, alpha=0.3, inv=1.0)
+    x = torch.randn(m, k, generator=torch.Generator().manual_seed(m)).bfloat16()
+    want = layers.nvfp4_dense_ref(x, onv.unpack_fp4(packed, scales), np.float32(0.3), relu2=bool(ks & 1))
+    lib = _lib.lib()
+    assert lib.hb_tune(b"nvfp4_tile_ks", ks) == 0
+    try:
+        assert (lib.hb_nvfp4_gemm_workspace_bytes(m, n, k) > 0) == (m > 20)  # up to twenty rows the weight stream serves
+        got = [ops.nvfp4_linear(x.cuda(), lin, relu2=bool(ks & 1)) for _ in range(3)]
+    finally:
+        lib.hb_tune(b"nvfp4_tile_ks", 0)
+    assert torch.equal(got[0], got[1]) and torch.equal(got[0], got[2])
+    mx, nr = errors(got[0], want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+
+
 def test_up_projection_shape_against_the_dequantized_product():
     """BASELINE config 1 (K = 5120, N = 25600, global scale 1/448), M = 1 and 8: the kernel against
     (x @ unpack^T) * s2 in FP32 on the GPU; the unpack itself is pinned bit-exact on the smaller shapes."""
