@@ -99,7 +99,7 @@ def cpu_baseline(layer, x, ids, weights, budget_s: float = 15.0):
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
-def latent_prefill(args) -> int:
+def latent_prefill(args) -> dict:
     """BASELINE config 4 (not the headline line; `--config 4`): the NVFP4 latent-MoE layer on a prefill chunk of 2048
     tokens - hidden 4096 projected to latent 1024, 512 ReLU^2 experts of intermediate 2688, top-22 by sigmoid scores.
     A step is the whole block (fused router|fc1_latent GEMM, routing, plan, the two expert GEMMs on the MFMA tile kernel,
@@ -147,6 +147,7 @@ def latent_prefill(args) -> int:
     cpu, check = None, None
     if not args.no_cpu:
         cpu, check = latent_cpu_leg(block, ex, fc1.bfloat16().cpu(), fc2.cpu(), x, latent, inter)
+    small = latent_small_calls(block, ex, hidden, dev, g)
     line = {
         "metric": "NVFP4 latent-MoE layer tokens/s on a 2048-token prefill chunk, with achieved MFMA TFLOP/s",
         "value": tokens * steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
@@ -160,11 +161,46 @@ def latent_prefill(args) -> int:
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": None, "launch_flops": gemm_flops, "launch_ms": fc1_ms},
         "layer_chain": {"kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
+        "decode_calls": small,
         "cpu_baseline": cpu,
         "parity": check,
     }
-    print(json.dumps(line))
-    return 0
+    return line
+
+
+def latent_small_calls(block, ex, hidden: int, dev, g, shared_inter: int = 5376):
+    """The same block with a shared expert of intermediate 5376 at 1, 4 and 16 rows (decode and verify calls):
+    microseconds a call through the small-call kernels (router, block: six launches) and through the operators a
+    longer call uses (two GEMMs, routing, plan, two expert layers, combine, the shared expert's two linears: nine), each
+    as replays of a graph of 32 calls over 8 inputs."""
+    import torch
+
+    from hibana_amd import synthetic
+    from hibana_amd.model import nemotron_moe
+
+    up, down = synthetic.nvfp4_linear(shared_inter, hidden, 61, dev), synthetic.nvfp4_linear(hidden, shared_inter, 62, dev)
+    both = nemotron_moe.NemotronMoe(block.gate_fc1, block.bias, block.fc2, ex, block.topk, up, down)
+
+    def operators(x):
+        fused = torch.mm(x, both.gate_fc1.T, out_dtype=torch.float32)
+        ids, w, lat = both.route(fused)
+        return torch.addmm(both.shared(x), both.routed(lat, ids, w), both.fc2.T)
+
+    out = {"workload": f"config 4's block with a shared expert of intermediate {shared_inter}, M = 1 / 4 / 16 rows of N(0,1)"}
+    for m in (1, 4, 16):
+        xs = [torch.randn(m, hidden, device=dev, generator=g).bfloat16() for _ in range(8)]
+        row = {}
+        for name, fn in (("small_call_kernels_us", both.small), ("operators_us", operators)):
+            for x in xs:
+                fn(x)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                outs = [fn(x) for x in xs for _ in range(4)]
+            row[name] = median(replay_times(graph, 32)) * 1e3
+            del outs, graph
+        out[str(m)] = row
+    return out
 
 
 def latent_cpu_leg(block, ex, fc1, fc2, x, latent: int, inter: int, rows: int = 12):
@@ -203,7 +239,7 @@ def latent_cpu_leg(block, ex, fc1, fc2, x, latent: int, inter: int, rows: int = 
     return cpu, check
 
 
-def dense_decode(args) -> int:
+def dense_decode(args) -> dict:
     """BASELINE configs 0 and 1 (not the headline line): one dense decode projection a step - config 0 the w3 linear
     5120 x 5120 at M = 1, config 1 the NVFP4 up-projection 25600 x 5120 at M = --rows (1, 8 or 64) - cycling through six
     copies of the matrix so that every step streams its weights from HBM. The roofline entry is that one kernel against
@@ -237,14 +273,24 @@ def dense_decode(args) -> int:
             blocks = t.view(-1, 4608)[:, 4096:]
             blocks.copy_(blocks % 120 + 1)
         nbytes = n * k // 2 + n * k // 16
-        x = torch.randn(m, k, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
-        y = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
 
-        def step(i: int):
-            _lib.check(lib.hb_nvfp4_gemm(_lib.ptr(x), m, _lib.ptr(mats[i % args.layers]), 1.0 / 448.0, n, k, 0, _lib.ptr(y), _lib.stream()), "nvfp4 gemm")
-            return y
+        def call(rows: int):
+            """(step, kernel name) of the projection at `rows` activation rows, its workspace (the partial tiles of a
+            call whose tiles share K among workgroups) allocated once."""
+            xr = torch.randn(rows, k, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
+            yr = torch.empty(rows, n, dtype=torch.bfloat16, device=dev)
+            need = lib.hb_nvfp4_gemm_workspace_bytes(rows, n, k)
+            ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
 
-        kernel, what = "nvfp4_stream_kernel<dense>", f"BASELINE config 1: NVFP4 dense linear {n} x {k}, M = {m} (codes and block scales random, global scale 1/448)"
+            def run(i: int):
+                _lib.check(lib.hb_nvfp4_gemm_ws(_lib.ptr(xr), rows, _lib.ptr(mats[i % args.layers]), 1.0 / 448.0, n, k, 0, _lib.ptr(yr), _lib.ptr(ws), need,
+                                                _lib.stream()), "nvfp4 gemm")
+                return yr
+
+            return run, "tile_kernel<TileNvfp4, dense>, K shared among workgroups" if need else "nvfp4_stream_kernel<dense>"
+
+        step, kernel = call(m)
+        what = f"BASELINE config 1: NVFP4 dense linear {n} x {k}, M = {m} (codes and block scales random, global scale 1/448)"
     for i in range(max(args.warmup, args.layers)):
         step(i)
     torch.cuda.synchronize()
@@ -267,6 +313,19 @@ def dense_decode(args) -> int:
     elapsed = median(times) * 1e-3 * args.steps
     del outs
     achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+    by_rows = None
+    if args.config == 1:  # the same projection at the configuration's other row counts: microseconds a call, graph-replayed
+        by_rows = {}
+        for rows in (1, 8, 64):
+            run, name = call(rows)
+            for i in range(args.layers):
+                run(i)
+            torch.cuda.synchronize()
+            g2 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g2):
+                outs = [run(i) for i in range(args.steps)]
+            by_rows[str(rows)] = {"us_per_call": median(replay_times(g2, args.steps)) * 1e3, "kernel": name}
+            del outs, g2
     line = {
         "metric": "dense decode projection tokens/s, with achieved HBM GB/s", "value": m * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "ms_per_step_min": times[0], "ms_per_step_max": times[-1],
@@ -277,8 +336,9 @@ def dense_decode(args) -> int:
                      "traffic": None, "launch_bytes": nbytes, "launch_ms": kernel_ms},
         "cpu_baseline": None,
     }
-    print(json.dumps(line))
-    return 0
+    if by_rows:
+        line["by_rows"] = by_rows
+    return line
 
 
 def replay_times(graph, steps: int, floor_s: float = 0.2, least: int = 5):
@@ -388,6 +448,7 @@ def main() -> int:
                     help="3: the headline w3 verify-batch layer (with the M = 1 layer as a sub-record); 2: the same layer at M = 1 alone; 0 / 1: the "
                          "w3 / NVFP4 dense decode projection; 4: the NVFP4 prefill layer")
     ap.add_argument("--rows", type=int, default=1, help="configs 0 and 1: activation rows M")
+    ap.add_argument("--headline-only", action="store_true", help="config 3 without the other configurations' lines (profiling runs)")
     ap.add_argument("--e4m3", action="store_true", help="configs 2 and 3: the reference kernel's own arithmetic (activations rounded to E4M3 per "
                     "32-group, FP8 MFMA) instead of the weight-only form; no CPU leg")
     ap.add_argument("--copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (a known-size "
@@ -405,9 +466,11 @@ def main() -> int:
         print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
         return 2
     if args.config == 4:
-        return latent_prefill(args)
+        print(json.dumps(latent_prefill(args)))
+        return 0
     if args.config in (0, 1):
-        return dense_decode(args)
+        print(json.dumps(dense_decode(args)))
+        return 0
     if args.e4m3:
         args.no_cpu = True  # the C oracle states the weight-only form
     decode = args.config == 2  # the layer at batch 1: logits from N(0, 1), ten experts and the shared one a step
@@ -492,6 +555,19 @@ def main() -> int:
         "cpu_baseline": cpu,
         "parity": check,
     }
+    if not decode and not args.e4m3 and not args.headline_only:
+        # the other configurations' lines in the same run, each as its own mode would print it (their CPU legs kept short)
+        del layers, x, logits, one_logits
+        torch.cuda.empty_cache()
+        others = {}
+        for name, mode, overrides in (("config1", dense_decode, {"config": 1, "rows": 1}), ("config4", latent_prefill, {"config": 4})):
+            sub = argparse.Namespace(**{**vars(args), **overrides})
+            try:
+                others[name] = mode(sub)
+            except Exception as err:  # the headline line stands on its own
+                others[name] = {"error": f"{type(err).__name__}: {err}"}
+            torch.cuda.empty_cache()
+        line["other_configs"] = others
     print(json.dumps(line))
     return 0
 

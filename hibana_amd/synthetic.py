@@ -68,3 +68,13 @@ def nvfp4_experts(experts: int, hidden: int, inter: int, seed: int, device="cuda
     w1, s1, g1 = stack(inter, hidden)
     w2, s2, g2 = stack(hidden, inter)
     return b12x_moe.B12xExperts(w1, s1, g1, 1.0, w2, s2, g2, 1.0, routed_scaling=routed_scaling, release=not keep)
+
+
+def nvfp4_linear(out_features: int, in_features: int, seed: int, device="cuda", global_scale: float = 1.0 / 448.0):
+    """A random NVFP4 linear as `nvfp4_experts` draws its matrices, tiled: an `Nvfp4Linear` a loader would hand over."""
+    from hibana_amd.weights import modelopt
+    g = torch.Generator(device=device).manual_seed(seed)
+    w = torch.randint(0, 256, (out_features, in_features // 2), dtype=torch.uint8, device=device, generator=g)
+    sc = torch.randn(out_features, in_features // 16, device=device, generator=g).abs().clamp(2.0 ** -6, 448.0).to(torch.float8_e4m3fn)
+    return modelopt.Nvfp4Linear(w, modelopt.swizzle_block_scales(sc), torch.tensor(global_scale, device=device), torch.tensor(1.0, device=device),
+                                out_features, in_features).tile()
