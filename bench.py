@@ -168,6 +168,36 @@ def latent_prefill(args) -> dict:
     return line
 
 
+def latent_small_only(args) -> dict:
+    """`--config 4 --small-rows M`: config 4's block with the shared expert at M rows through the small-call kernels
+    alone (a profiling mode: its kernel trace shows the six launches of a decode or verify call)."""
+    import torch
+
+    from hibana_amd import synthetic
+    from hibana_amd.model import nemotron_moe
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    hidden, latent, inter, experts, topk, shared_inter, m = 4096, 1024, 2688, 512, 22, 5376, args.small_rows
+    g = torch.Generator(device=dev).manual_seed(5)
+    ex = synthetic.nvfp4_experts(experts, latent, inter, 11, dev)
+    gate_fc1 = torch.cat([torch.randn(experts, hidden, device=dev, generator=g) * (1.0 / hidden ** 0.5), torch.randn(latent, hidden, device=dev, generator=g) * 0.02])
+    fc2 = (torch.randn(hidden, latent, device=dev, generator=g) * 0.02).bfloat16()
+    block = nemotron_moe.NemotronMoe(gate_fc1.bfloat16(), torch.zeros(experts, device=dev), fc2, ex, topk, synthetic.nvfp4_linear(shared_inter, hidden, 61, dev),
+                                     synthetic.nvfp4_linear(hidden, shared_inter, 62, dev))
+    xs = [torch.randn(m, hidden, device=dev, generator=g).bfloat16() for _ in range(8)]
+    for x in xs:
+        block.small(x)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = [block.small(xs[i % 8]) for i in range(args.steps)]
+    times = replay_times(graph, args.steps)
+    del outs
+    return {"metric": "NVFP4 latent-MoE block microseconds a call through the small-call kernels", "rows": m, "us_per_call": median(times) * 1e3,
+            "us_per_call_min": times[0] * 1e3, "us_per_call_max": times[-1] * 1e3, "steps": args.steps, "replays": len(times)}
+
+
 def latent_small_calls(block, ex, hidden: int, dev, g, shared_inter: int = 5376):
     """The same block with a shared expert of intermediate 5376 at 1, 4 and 16 rows (decode and verify calls):
     microseconds a call through the small-call kernels (router, block: six launches) and through the operators a
@@ -448,6 +478,8 @@ def main() -> int:
                     help="3: the headline w3 verify-batch layer (with the M = 1 layer as a sub-record); 2: the same layer at M = 1 alone; 0 / 1: the "
                          "w3 / NVFP4 dense decode projection; 4: the NVFP4 prefill layer")
     ap.add_argument("--rows", type=int, default=1, help="configs 0 and 1: activation rows M")
+    ap.add_argument("--small-rows", type=int, default=0, help="config 4: only its block (with a shared expert) at this many rows (1 .. 16) through the "
+                    "small-call kernels")
     ap.add_argument("--headline-only", action="store_true", help="config 3 without the other configurations' lines (profiling runs)")
     ap.add_argument("--e4m3", action="store_true", help="configs 2 and 3: the reference kernel's own arithmetic (activations rounded to E4M3 per "
                     "32-group, FP8 MFMA) instead of the weight-only form; no CPU leg")
@@ -466,7 +498,7 @@ def main() -> int:
         print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
         return 2
     if args.config == 4:
-        print(json.dumps(latent_prefill(args)))
+        print(json.dumps(latent_small_only(args) if args.small_rows else latent_prefill(args)))
         return 0
     if args.config in (0, 1):
         print(json.dumps(dense_decode(args)))

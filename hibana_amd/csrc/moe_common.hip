@@ -594,20 +594,9 @@ __device__ __forceinline__ void combine_pairs_batches(const CombineParams& p, in
     }
   }
 }
-__device__ __forceinline__ void combine_pairs_sum(const CombineParams& p, int r, int c, float& v0, float& v1) {
-  v0 = 0.f;
-  v1 = 0.f;
-  if (p.topk <= 8) {
-    combine_pairs_batches<8>(p, r, c, v0, v1);
-  } else if (p.topk <= 12) {
-    combine_pairs_batches<12>(p, r, c, v0, v1);
-  } else if (p.m > 64) {  // a long call is bound by its traffic: fewer registers, more wavefronts
-    combine_pairs_batches<8>(p, r, c, v0, v1);
-  } else {
-    combine_pairs_batches<24>(p, r, c, v0, v1);
-  }
-}
-
+// B: the slots read together - 8 or 12 where the call is long or top-k small, 24 for a short call of many slots
+// (one wait on memory instead of three); a kernel of its own each, so that the longer batches' registers are theirs alone.
+template <int B>
 __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
   __shared__ float red[4];
   const int r = blockIdx.x;
@@ -619,8 +608,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
   }
   const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
   if (c >= p.h) return;
-  float v0, v1;
-  combine_pairs_sum(p, r, c, v0, v1);
+  float v0 = 0.f, v1 = 0.f;
+  combine_pairs_batches<B>(p, r, c, v0, v1);
   if (p.shared) {
     const int64_t at = (int64_t)r * p.shared_stride + c;
     float s0, s1;
@@ -963,7 +952,14 @@ int latent_launch_out(const uint16_t* fc2, const uint16_t* routed, const uint16_
 }
 
 void moe_launch_combine(const CombineParams& c, hipStream_t stream) {
-  HB_LAUNCH(moe_combine_kernel, dim3((unsigned)c.m, (unsigned)((c.h + COMBINE_SPAN - 1) / COMBINE_SPAN)), dim3(256), 0, stream, c);
+  const dim3 grid((unsigned)c.m, (unsigned)((c.h + COMBINE_SPAN - 1) / COMBINE_SPAN));
+  if (c.topk <= 8 || (c.topk > 12 && c.m > 64)) {  // a long call is bound by its traffic: fewer registers, more wavefronts
+    HB_LAUNCH(moe_combine_kernel<8>, grid, dim3(256), 0, stream, c);
+  } else if (c.topk <= 12) {
+    HB_LAUNCH(moe_combine_kernel<12>, grid, dim3(256), 0, stream, c);
+  } else {
+    HB_LAUNCH(moe_combine_kernel<24>, grid, dim3(256), 0, stream, c);
+  }
 }
 
 }  // namespace hb
