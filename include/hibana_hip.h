@@ -39,15 +39,21 @@ const char* hb_error_string(int code);
  * "moe_fc1_ksplit" / "moe_fc1_nbw", "moe_fc2_ksplit" / "moe_fc2_nbw", "nvfp4_ksplit" / "nvfp4_nbw": K splits and 64-row
  * blocks per workgroup (their product at most 16); "w3_tile" / "nvfp4_tile": 1 forces the MFMA tile kernel, 2 the weight
  * stream; "w3_few" / "nvfp4_few": 2 switches off the stream's body for slots of few rows (W3: at most four, NVFP4: at
- * most eight); "moe_one": 2 switches off the single launch that does one token's fc2 and combine. Returns HB_EINVAL for
- * an unknown key or a value out of range. Not thread-safe against concurrent launches. */
+ * most eight); "moe_one": 2 switches off the single launch that does one token's fc2 and combine; "moe_fused": 2 runs a
+ * routed call's fc1 and fc2 as two launches; "moe_lag": the slots fc2 lags fc1 by in their common launch; "moe_split":
+ * 1 gives fc1's few-row body a two-plane E4M3 form of x (FP8 matrix cores; 3e-4 of the norm); "route_plan": 2 keeps
+ * routing and plan in separate launches; "nvfp4_tile_ks": the workgroups that share a tile's K in hb_nvfp4_gemm_ws.
+ * Returns HB_EINVAL for an unknown key or a value out of range. The knobs are process-wide relaxed atomics: setting one
+ * while another thread launches is a race-free read of either value, not a per-call setting. */
 int hb_tune(const char* key, int value);
 
 /* Measurement hook (no counterpart in the reference): `events` are hipEvent_t handles the caller created, taken in
  * (start, stop) pairs: each kernel the next calls launch carries the next pair, and the runtime stamps the two events
  * with that kernel's own begin and end (hipEventElapsedTime(start, stop) is the kernel's duration). A routed call
- * launches plan, fc1, fc2 and, when it sums, combine; hb_w3_moe_layer_logits launches the routing kernel first when it
- * has more than 16 rows. count = 0 switches the hook off. Not for captured graphs. */
+ * launches plan, fc1 and fc2 (one launch for both when it has more than one row, weight-only) and, when it sums,
+ * combine; hb_w3_moe_layer_logits routes inside the plan's launch (up to 4 rows: its workgroup routes them first; up
+ * to 8191 pairs: a workgroup a row routes and the last to finish plans) or, beyond that, in a launch of its own ahead
+ * of the plan's three. count = 0 switches the hook off. Not for captured graphs. */
 int hb_debug_events(void* const* events, int count);
 
 /* Measurement hook (no counterpart in the reference): `buffer` (device, int64, four values a workgroup of the launch
@@ -197,7 +203,8 @@ int hb_w3_moe_layer_e4m3(const hb_w3_experts* routed, const hb_w3_experts* share
 
 /* The same layer from the router's logits (float32 [m, experts_total]): softmax top-k routing as
  * hb_route_softmax_topk, written to ids int32 [m, topk] and weights float32 [m, topk] (caller's buffers), then the
- * chain of hb_w3_moe_layer. Up to 16 rows the routing runs inside the planning workgroup (one launch fewer).
+ * chain of hb_w3_moe_layer. Routing and plan are one launch up to 8191 pairs (up to 4 rows the planning workgroup
+ * routes them itself; beyond, a workgroup a row routes and the last one to finish plans).
  * ref: MoeLayer.__call__ with its route step, hibana/model/flashnext/moe.py:122-144,177-192. */
 int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec,
                            const void* x, const float* logits, int experts_total, int m, int topk, int32_t* ids,
