@@ -1022,6 +1022,28 @@ extern "C" int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int 
   return launch_status();
 }
 
+// x[r, c] = bf16(relu(x[r, c])^2) in place for BF16 rows `stride` elements apart: the square in FP32, one rounding
+// (torch's relu(x) ** 2; relu2_, hibana/model/nemotron/moe.py:316-321 of the reference). Two columns a thread.
+__global__ __launch_bounds__(256) void relu2_kernel(uint16_t* __restrict__ x, int64_t rows, int n, int64_t stride) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int per_row = n >> 1;
+  if (i >= rows * per_row) return;
+  const int64_t r = i / per_row;
+  uint32_t* at = reinterpret_cast<uint32_t*>(x + r * stride + 2 * (i - r * per_row));
+  const uint32_t two = *at;
+  const float a = fmaxf(__uint_as_float(two << 16), 0.f), b = fmaxf(__uint_as_float(two & 0xffff0000u), 0.f);
+  *at = (uint32_t)f32_to_bf16_bits(a * a) | ((uint32_t)f32_to_bf16_bits(b * b) << 16);
+}
+
+extern "C" int hb_relu2(void* x, int64_t rows, int n, int64_t stride, void* stream) {
+  if (!x) return HB_ENULL;
+  if (rows <= 0 || n <= 0 || n % 2 || stride < n || stride % 2) return HB_EINVAL;
+  if (!aligned(x, 4)) return HB_EINVAL;
+  const int64_t threads = rows * (n / 2);
+  hipLaunchKernelGGL(relu2_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, as_stream(stream), static_cast<uint16_t*>(x), rows, n, stride);
+  return launch_status();
+}
+
 extern "C" int hb_route_softmax_topk(const float* logits, int m, int e, int k, const int32_t* slots, int steps, int repeat, int32_t* ids,
                                      float* weights, void* stream) {
   if (!logits || !ids || !weights) return HB_ENULL;

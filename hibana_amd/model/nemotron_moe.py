@@ -46,6 +46,18 @@ def route_topk(fused: torch.Tensor, bias: torch.Tensor, k: int, latent: int, slo
     return ids, w, lat
 
 
+def relu2_(x: torch.Tensor) -> torch.Tensor:
+    """relu(x)^2 in place for BF16 [M, N] (FP32 square, one rounding: torch's relu(x) ** 2)
+    (hibana/model/nemotron/moe.py:316-321). The expert kernels and `NemotronMoe.shared` do it in their epilogues; this
+    is the standalone form."""
+    if x.dtype != torch.bfloat16 or x.ndim != 2 or x.stride(1) != 1 or x.shape[1] % 2 or x.stride(0) % 2:
+        raise ValueError("relu2_: BF16 [M, N] with contiguous rows, N and the row stride even")
+    _lib.need_gpu(x)
+    if x.numel():
+        _lib.check(_lib.lib().hb_relu2(_lib.ptr(x), x.shape[0], x.shape[1], x.stride(0), _lib.stream()), "relu2_")
+    return x
+
+
 class NemotronMoe:
     """One block's weights, assembled from tensors already on the device.
 

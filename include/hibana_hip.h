@@ -231,6 +231,10 @@ int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int32_t* ids, 
  * ref: ops.silu_and_mul, hibana/kernels/ops.py:86-92. */
 int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int pairs, void* out, void* stream);
 
+/* x = bf16(relu(x)^2) in place, BF16 [rows, n] with rows `stride` elements apart (n and stride even): the square in FP32
+ * with one rounding. ref: relu2_, hibana/model/nemotron/moe.py:316-321 (the expert kernels do it in their epilogues). */
+int hb_relu2(void* x, int64_t rows, int n, int64_t stride, void* stream);
+
 /* Softmax top-k routing: logits float32 [m, e] -> ids int32 [m, k] (descending probability, ties to the lower id),
  * weights float32 [m, k] renormalized over the selection. slots (may be NULL: every row is real): row r is real iff
  * slots[r / steps] != 0; a padded row gets weight 0 in every slot and the id e ("no expert", which the 3-bit experts

@@ -62,6 +62,23 @@ def test_silu_and_mul_matches_the_bf16_tensor_expression(shape, pairs):
         assert (got.view(torch.int16).int() - ref.view(torch.int16).int()).abs().max() <= 1
 
 
+def test_relu2_in_place():
+    from hibana_amd.model import nemotron_moe
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(37, 130, generator=g) * 3).bfloat16()
+    x[0, :4] = torch.tensor([0.0, -0.0, float("inf"), -float("inf")]).bfloat16()
+    want = (torch.relu(x).float() ** 2).bfloat16()
+    y = x.cuda()
+    assert nemotron_moe.relu2_(y) is y and torch.equal(y.cpu().view(torch.int16), want.view(torch.int16))
+    wide = (torch.randn(5, 64, generator=g)).bfloat16().cuda()
+    before = wide.cpu()
+    nemotron_moe.relu2_(wide[:, :32])  # rows of a wider tensor: the columns beside them stay
+    assert torch.equal(wide[:, 32:].cpu(), before[:, 32:])
+    assert torch.equal(wide[:, :32].cpu(), (torch.relu(before[:, :32]).float() ** 2).bfloat16())
+    with pytest.raises(ValueError):
+        nemotron_moe.relu2_(torch.zeros(2, 3, dtype=torch.bfloat16).cuda())
+
+
 def test_softmax_routing_with_padded_rows():
     from hibana_amd.kernels import ops
     g = torch.Generator().manual_seed(4)
