@@ -53,6 +53,27 @@ def test_validation_without_a_gpu():
     assert lib.hb_w3_gemm(258, 1, 256, 256, 0, 128, 128, 256, None) == _lib.HB_EINVAL  # x on a 2-byte boundary
     assert lib.hb_w3_moe(C.byref(ex), 256, 256, 256, 1, 1, 0, 256, 264, 1 << 30, None) == _lib.HB_EINVAL  # workspace on 8
     assert lib.hb_nvfp4_gemm(256, 1, 260, 1.0, 128, 128, 0, 256, None) == _lib.HB_EINVAL  # tile layout on 4
+    # the dense product with a workspace: sizes only (no launch without a GPU)
+    assert lib.hb_nvfp4_gemm_workspace_bytes(8, 25600, 5120) == 0 and lib.hb_nvfp4_gemm_workspace_bytes(2048, 25600, 5120) == 0
+    assert lib.hb_nvfp4_gemm_workspace_bytes(64, 25600, 5120) == 100 * 4 * 4 * 4 * 4 * 64 * 16  # 100 tiles x 4 shares of K x 4 wavefronts x 4 row tiles x 4 x 64 lanes x 16 B
+    assert lib.hb_nvfp4_gemm_workspace_bytes(64, 100, 5120) == 0
+    assert lib.hb_nvfp4_gemm_ws(None, 64, None, 1.0, 128, 128, 0, None, None, 0, None) == _lib.HB_ENULL
+    assert lib.hb_relu2(None, 1, 2, 2, None) == _lib.HB_ENULL and lib.hb_relu2(256, 1, 3, 4, None) == _lib.HB_EINVAL
+    # the small latent block: shapes and pointers are checked before anything is launched
+    nv = _lib.HbNvfp4Experts(256, 256, 256, 256, 8, 0, 256, 128, 256, 0)
+    lw = _lib.HbLatentWeights(256, 256, 256, C.pointer(nv), 256, 256, 1.0, 1.0, 8, 256, 512, 640)
+    need = lib.hb_latent_workspace_bytes(C.byref(lw), 4, 2)
+    assert need >= 4 * (256 + 640 + 512) * 2 and lib.hb_latent_workspace_bytes(C.byref(lw), 17, 2) == 0  # at most sixteen rows
+    assert lib.hb_latent_workspace_bytes(None, 4, 2) == 0
+    assert lib.hb_latent_router(None, 256, 4, 2, None, 1, 1, -1, 256, 256, 256, 256, 256, need, None) == _lib.HB_ENULL
+    assert lib.hb_latent_router(C.byref(lw), 256, 4, 2, None, 1, 1, -1, 256, 256, 256, 256, 256, need - 1, None) == _lib.HB_EWORKSPACE
+    assert lib.hb_latent_router(C.byref(lw), 256, 4, 2, None, 1, 1, 9, 256, 256, 256, 256, 256, need, None) == _lib.HB_EINVAL  # pad_id past "no expert"
+    assert lib.hb_latent_block(C.byref(lw), 256, 256, 256, 256, 17, 2, 0, 256, 256, need, None) == _lib.HB_EINVAL
+    bare = _lib.HbLatentWeights(256, 256, 256, None, None, None, 0.0, 0.0, 8, 256, 512, 0)  # 3-bit experts, no shared expert
+    assert lib.hb_latent_block(C.byref(bare), 256, 256, 256, 256, 4, 2, 0, 256, 256, 1 << 20, None) == _lib.HB_ENULL
+    assert lib.hb_latent_shared_up(C.byref(bare), 256, 4, 2, 256, 1 << 20, None) == _lib.HB_ENULL
+    lopsided = _lib.HbLatentWeights(256, 256, 256, None, 256, None, 1.0, 0.0, 8, 256, 512, 640)  # an up projection without its down
+    assert lib.hb_latent_workspace_bytes(C.byref(lopsided), 4, 2) == 0
     with pytest.raises(ValueError):
         _lib.check(_lib.HB_EINVAL, "x")
     with pytest.raises(RuntimeError):
