@@ -1,0 +1,172 @@
+// Top-k routing of one row by one wavefront (device code shared by the routing launches and by kernels that route for
+// themselves).
+#pragma once
+
+#include "stream_common.hpp"
+
+namespace hb {
+
+// Top-k routing, one wavefront per row: softmax over all experts, top-k, renormalized
+// (hibana/kernels/flashnext_fused.py:278-319 of the reference), or sigmoid scores chosen by score + bias with the plain
+// scores as weights (hibana/model/nemotron/moe.py:57-121). Lane l holds experts l * per .. l * per + per - 1 in
+// registers as order-preserving 32-bit keys, so a selection round is a register scan, one wave-wide integer maximum
+// (DPP within rows of 16, four scalar reads across them) and a ballot: among equal scores the lowest lane, then the
+// lowest register, wins - the lowest expert id.
+constexpr int ROUTE_PER_LANE = 16;
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false));   // lane ^ 1
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false));   // lane ^ 2
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, false));  // mirror within 8
+  x = max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x140, 0xF, 0xF, false));  // mirror within 16
+  const uint32_t a = __builtin_amdgcn_readlane((int)x, 0), b = __builtin_amdgcn_readlane((int)x, 16);
+  const uint32_t c = __builtin_amdgcn_readlane((int)x, 32), d = __builtin_amdgcn_readlane((int)x, 48);
+  return max(max(a, b), max(c, d));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+  return v;
+}
+
+// Key of a score: larger score <=> larger key, every real key above 0 (the key of an empty register).
+__device__ __forceinline__ uint32_t score_key(float v) {
+  const int32_t bits = __builtin_bit_cast(int32_t, v);
+  return (uint32_t)(bits ^ ((bits >> 31) & 0x7fffffff)) ^ 0x80000000u;
+}
+
+struct RouteParams {
+  const float* logits;   // [m, stride]: e logits a row (sigmoid: followed by `latent` FP32 columns)
+  int64_t stride;
+  const float* bias;     // sigmoid: [e] added to the scores for the choice only
+  const int32_t* slots;  // row r is real iff slots[r / steps] != 0 (null: every row)
+  int steps, repeat;
+  int e, k, per, latent;
+  int pad_id;            // the id of a padded row's slots without `repeat` (the callers' default: e, "no expert")
+  int sigmoid;           // the rule a kernel that serves both applies (route_any)
+  int32_t* ids;
+  float* weights;
+  uint16_t* lat;         // sigmoid: BF16 [m, latent], the row's latent columns
+};
+
+// THROUGH: the logits were written by other workgroups of the same launch and are read past the compute die's L2.
+// Returns, in lane s < k, the id of the row's selection s. `write` = false keeps the row's results in registers only (a
+// workgroup that routes for itself a row some other workgroup writes).
+template <bool SIGMOID, int PER, bool THROUGH = false>
+__device__ __forceinline__ int route_row(const RouteParams& p, int r, int lane, bool write = true, float* weight = nullptr) {
+  const int e = p.e, per = p.per, first = lane * per;
+  auto logit = [](const float* at) -> float { if constexpr (THROUGH) return load_through(at); else return *at; };
+  if (SIGMOID && p.lat && write) {  // the row's latent columns, rounded: four a lane and sixteen loads in flight where the row allows
+    const float* src = p.logits + (int64_t)r * p.stride + e;
+    uint16_t* dst = p.lat + (int64_t)r * p.latent;
+    if (!THROUGH && !((p.stride | e | p.latent) & 3)) {
+      for (int c0 = 4 * lane; c0 < p.latent; c0 += 1024) {
+        f32x4_t v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (c0 + 256 * j < p.latent) v[j] = *reinterpret_cast<const f32x4_t*>(src + c0 + 256 * j);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (c0 + 256 * j < p.latent) {
+            const uint32_t lo = (uint32_t)bf16_of(v[j].x) | ((uint32_t)bf16_of(v[j].y) << 16), hi = (uint32_t)bf16_of(v[j].z) | ((uint32_t)bf16_of(v[j].w) << 16);
+            *reinterpret_cast<uint2*>(dst + c0 + 256 * j) = make_uint2(lo, hi);
+          }
+      }
+    } else {
+      for (int c = lane; c < p.latent; c += 64) dst[c] = bf16_of(logit(src + c));
+    }
+  }
+  const bool padded = p.slots && p.slots[r / p.steps] == 0;
+  const float* row = p.logits + (int64_t)(padded ? 0 : r) * p.stride;  // a padded row repeats row 0's first choice
+  float val[PER];   // the weight an expert would get before renormalization
+  uint32_t key[PER];
+  if (SIGMOID) {
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      const int i = first + j;
+      const bool real = j < per && i < e;
+      val[j] = real ? 1.0f / (1.0f + expf(-logit(row + i))) : 0.f;
+      key[j] = real ? score_key(val[j] + p.bias[i]) : 0u;
+    }
+  } else {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      const int i = first + j;
+      val[j] = j < per && i < e ? logit(row + i) : -INFINITY;
+      mx = fmaxf(mx, val[j]);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      val[j] = j < per && first + j < e ? expf(val[j] - mx) : 0.f;
+      sum += val[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      val[j] = val[j] / sum;
+      key[j] = j < per && first + j < e ? score_key(val[j]) : 0u;
+    }
+  }
+  float total = 0.f, mine = 0.f;
+  int mine_id = 0;
+  for (int s = 0; s < p.k; s++) {
+    uint32_t best = 0;
+    int at = 0;
+    float bv = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++)
+      if (key[j] > best) {  // ascending index within the lane: the first of equals stays
+        best = key[j];
+        at = j;
+        bv = val[j];
+      }
+    const uint32_t top = wave_max_u32(best);
+    const int winner = __builtin_ctzll(__ballot(best == top));
+    const int wj = __builtin_amdgcn_readlane(at, winner);
+    const float wv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv), winner));
+    total += wv;
+    if (lane == s) {
+      mine = wv;
+      mine_id = winner * per + wj;
+    }
+    if (lane == winner) {
+#pragma unroll
+      for (int j = 0; j < PER; j++)
+        if (j == wj) key[j] = 0u;
+    }
+  }
+  int id = mine_id;
+  float w = SIGMOID ? mine / (total + 1e-20f) : mine / total;
+  if (padded) {
+    id = p.repeat ? __builtin_amdgcn_readfirstlane(mine_id) : p.pad_id;
+    w = 0.f;
+  }
+  if (lane < p.k && write) {
+    store_through(&p.ids[(int64_t)r * p.k + lane], id);  // the plan may read it in this very launch, from another workgroup
+    p.weights[(int64_t)r * p.k + lane] = w;
+  }
+  if (weight) *weight = w;
+  return id;
+}
+
+// Row r by the rule and the register count the parameters name.
+__device__ __forceinline__ void route_any(const RouteParams& p, int r, int lane) {
+  if (p.sigmoid) {
+    if (p.per <= 8) {
+      route_row<true, 8>(p, r, lane);
+    } else {
+      route_row<true, 16>(p, r, lane);
+    }
+  } else if (p.per <= 8) {
+    route_row<false, 8>(p, r, lane);
+  } else {
+    route_row<false, 16>(p, r, lane);
+  }
+}
+
+}  // namespace hb

@@ -212,20 +212,12 @@ __device__ __forceinline__ void quant_emit(const StreamParams& p, const Slot& sl
   }
 }
 
-template <int EPI>
-__device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
+// The slot of rows p0 .. p0 + rows - 1 of `expert` (negative: the shared expert).
+__device__ __forceinline__ Slot make_slot(const StreamParams& p, int index, int expert, int p0, int rows) {
   Slot s;
-  s.index = slot;
-  int expert = 0;
-  if (epi_dense(EPI)) {
-    const int per = p.slot_rows ? p.slot_rows : ROWS_PER_SLOT;
-    s.p0 = slot * per;
-    s.rows = min(per, p.m - s.p0);
-  } else {
-    expert = p.plan[PLAN_HEADER + 4 * slot];
-    s.p0 = p.plan[PLAN_HEADER + 4 * slot + 1];
-    s.rows = p.plan[PLAN_HEADER + 4 * slot + 2];
-  }
+  s.index = index;
+  s.p0 = p0;
+  s.rows = rows;
   s.w = expert < 0 ? p.w_shared : p.w + (int64_t)expert * p.expert_bytes;
   s.rs = expert < 0 ? p.rows_shared : p.rows + (int64_t)expert * p.expert_rows;
   // an entry without rows names no expert: nothing indexed by it is read
@@ -233,6 +225,16 @@ __device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
   s.lut_lo = expert < 0 ? p.lut_lo_shared : p.lut_lo;
   s.lut_hi = expert < 0 ? p.lut_hi_shared : p.lut_hi;
   return s;
+}
+
+template <int EPI>
+__device__ __forceinline__ Slot slot_of(const StreamParams& p, int slot) {
+  if (epi_dense(EPI)) {
+    const int per = p.slot_rows ? p.slot_rows : ROWS_PER_SLOT, p0 = slot * per;
+    return make_slot(p, slot, 0, p0, min(per, p.m - p0));
+  }
+  const int32_t* entry = p.plan + PLAN_HEADER + 4 * slot;
+  return make_slot(p, slot, entry[0], entry[1], entry[2]);
 }
 
 // Which K split (`ks`) and which of the workgroup's blocks (`nbi`) a wavefront is, and the chunks c0 .. c1 - 1 of its
@@ -505,6 +507,7 @@ void moe_launch_quant_rows(const uint16_t* x, int64_t m, int k, uint8_t* q, floa
 
 // Softmax top-k routing of `m` rows of `e` logits into ids / weights [m, topk], then the plan of those ids: one launch
 // for up to a few dozen rows, two beyond.
+int moe_check_route(int m, int e, int k);  // HB_EINVAL for a row the routing wavefront cannot hold
 int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
                           const MoeWorkspace& ws, hipStream_t stream, int slot_rows = ROWS_PER_SLOT, const QuantJob* job = nullptr);
 

@@ -23,6 +23,7 @@
 #include <mutex>
 
 #include "ring.hpp"
+#include "route.hpp"
 #include "stream_common.hpp"
 #include "tile_kernel.hpp"
 #include "w3_layout.hpp"
@@ -598,6 +599,46 @@ __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   stream_workgroup<EPI, A8, SPLIT>(p, sl, blockIdx.x, rings);
 }
 
+// One token from its router logits: fc1 with the routing inside it, so that the call has no launch for routing and plan.
+// Every wavefront of the launch routes the row for itself (about three microseconds in which it could not have known
+// its expert anyway; the logits are 2 KB): lane s then holds selection s, slot s is that expert with the token's one
+// row, and the slot after the last selection is the shared expert's. The first wavefront of the first workgroup also
+// writes what the caller and the next launch read: ids, weights, and the slot table and pair list in the plan's format
+// (in selection order: every slot has one row, so no order is better). The activation row is row 0 whatever a slot's
+// pair index says: the launch passes a row stride of 0.
+template <int EPI>
+__global__ __launch_bounds__(1024) void w3_fc1_route_one_kernel(StreamParams p, RouteParams route, int e_lo, int e_n, int shared_slot, int32_t* plan,
+                                                                int32_t* order) {
+  extern __shared__ __align__(16) uint8_t rings[];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && wave == 0;
+  const int id = route.per <= 8 ? route_row<false, 8>(route, 0, lane, writer) : route_row<false, 16>(route, 0, lane, writer);
+  const int local = id - e_lo;
+  const bool here = lane < route.k && local >= 0 && local < e_n;  // an expert of another rank's range has no slot
+  if (writer) {
+    const int kept = __popcll(__ballot(here));
+    if (lane < route.k || lane == shared_slot) {
+      int32_t* entry = plan + PLAN_HEADER + 4 * lane;
+      entry[0] = lane == shared_slot ? -1 : here ? local : 0;
+      entry[1] = lane;
+      entry[2] = lane == shared_slot || here ? 1 : 0;
+      entry[3] = 0;
+      order[lane] = lane;  // a selection's pair index is its own; the shared expert's row follows the pairs
+    }
+    if (lane == 0) {
+      plan[0] = route.k + (shared_slot >= 0 ? 1 : 0);
+      plan[1] = plan[2] = kept;
+    }
+  }
+  const int slot = blockIdx.y;
+  int expert = -1;
+  if (slot != shared_slot) {
+    if (!__builtin_amdgcn_readlane((int)here, slot)) return;  // uniform over the workgroup
+    expert = __builtin_amdgcn_readlane(local, slot);
+  }
+  stream_workgroup<EPI, false, false>(p, make_slot(p, slot, expert, slot, 1), blockIdx.x, rings);
+}
+
 // fc1 and fc2 of a routed call in ONE launch, so that fc2's workgroups fill the compute units that fc1's last, partly
 // empty round of workgroups leaves idle (and no launch boundary lies between the two). The grid is one-dimensional:
 // first every fc1 workgroup (slot-major, the slot table's order), then every fc2 workgroup. A slot's fc2 needs all of
@@ -940,7 +981,13 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   const QuantJob xjob = split ? QuantJob{static_cast<const uint16_t*>(x), 0, ws.x2, ws.x2s, m, ex->hidden}
                               : QuantJob{static_cast<const uint16_t*>(x), (int64_t)m * ex->hidden / 8, ws.xq, ws.xs, 0, 0};
   const QuantJob* job = e4m3 || split ? &xjob : nullptr;
-  if (route) {
+  // one token from its logits, a slot a selection, and fc2 + combine as one launch after it: fc1 routes for itself
+  const bool route_in_fc1 = route && m == 1 && combine && !e4m3 && !split && !dense && topk <= 63 && slots == topk + shared_rows &&
+                            slots + (combine->gate_vec && combine->shared ? ONE_GATE_WAVES : 0) <= ONE_MAX_WAVES && g_tune.moe_one == 0 &&
+                            moe_check_route(m, route->e, topk) == HB_OK;
+  if (route_in_fc1) {
+    // (nothing to launch here)
+  } else if (route) {
     if (int e = moe_launch_route_plan(route->logits, m, route->e, topk, route->ids, route->weights, ex->base, ex->experts, shared_rows, ws, stream,
                                       slot_rows, job))
       return e;
@@ -1037,7 +1084,29 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
       }
     }
   }
-  if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) return e;
+  if (route_in_fc1) {
+    StreamParams q = p;
+    if (int e = shape_stream(q, est, l1)) return e;
+    q.a_stride = 0;  // every slot's row is the token's
+    RouteParams rp{};
+    rp.logits = route->logits;
+    rp.stride = route->e;
+    rp.e = route->e;
+    rp.k = topk;
+    rp.per = (route->e + 63) / 64;
+    rp.steps = 1;
+    rp.pad_id = route->e;
+    rp.ids = route->ids;
+    rp.weights = route->weights;
+    const dim3 grid((unsigned)((q.n_blocks + q.nbw - 1) / q.nbw), (unsigned)slots);
+    const int waves = q.ks * q.nbw;
+    auto launch = [&](auto kernel) {
+      HB_LAUNCH(kernel, grid, dim3(64 * waves), (size_t)waves * RING_BYTES, stream, q, rp, ex->base, ex->experts, shared ? topk : -1, ws.plan, ws.order);
+    };
+    ex->gated ? launch(w3_fc1_route_one_kernel<EPI_FC1_GATED>) : launch(w3_fc1_route_one_kernel<EPI_FC1_RELU2>);
+  } else if (int e = ex->gated ? launch_stream<EPI_FC1_GATED>(p, slots, est, l1, stream) : launch_stream<EPI_FC1_RELU2>(p, slots, est, l1, stream)) {
+    return e;
+  }
   int fc2_ks = l2.ks, fc2_nbw;
   if (!fc2_ks) pick_shape(f2.n_blocks, f2.chunks, est, 8192, &fc2_ks, &fc2_nbw);
   // one token, and a separate fc2 would not split K either: the fused launch makes the same sums

@@ -204,7 +204,8 @@ int hb_w3_moe_layer_e4m3(const hb_w3_experts* routed, const hb_w3_experts* share
 /* The same layer from the router's logits (float32 [m, experts_total]): softmax top-k routing as
  * hb_route_softmax_topk, written to ids int32 [m, topk] and weights float32 [m, topk] (caller's buffers), then the
  * chain of hb_w3_moe_layer. Routing and plan are one launch up to 8191 pairs (up to 4 rows the planning workgroup
- * routes them itself; beyond, a workgroup a row routes and the last one to finish plans).
+ * routes them itself; beyond, a workgroup a row routes and the last one to finish plans); one token has no such launch
+ * at all: fc1's wavefronts route the row themselves.
  * ref: MoeLayer.__call__ with its route step, hibana/model/flashnext/moe.py:122-144,177-192. */
 int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec,
                            const void* x, const float* logits, int experts_total, int m, int topk, int32_t* ids,
