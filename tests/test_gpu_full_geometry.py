@@ -145,6 +145,36 @@ def test_nvfp4_dense_at_the_benchmark_geometry(nvfp4_dense, m, kernel):
     assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
 
 
+def test_nvfp4_dense_partial_tiles_do_not_depend_on_what_the_workspace_held(nvfp4_dense):
+    """64 rows at config 1's size share K among four workgroups a tile: whichever finishes last must find the others'
+    partial tiles in memory. The workspace is filled with NaN before every call; every call gives the first one's bits,
+    which are the stream's result to the summation order."""
+    from hibana_amd import _lib
+    from hibana_amd.kernels import ops
+    lin, _ = nvfp4_dense
+    n, k, m = 25600, 5120, 64
+    lib = _lib.lib()
+    x = torch.randn(m, k, generator=torch.Generator().manual_seed(m)).bfloat16().cuda()
+    need = lib.hb_nvfp4_gemm_workspace_bytes(m, n, k)
+    assert need > 0
+    ws = torch.empty(need // 4, dtype=torch.float32, device="cuda")
+    y = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    first = None
+    for _ in range(12):
+        ws.fill_(float("nan"))
+        _lib.check(lib.hb_nvfp4_gemm_ws(_lib.ptr(x), m, _lib.ptr(lin.tiled), lin.global_scale, n, k, 0, _lib.ptr(y), _lib.ptr(ws), need, _lib.stream()), "gemm")
+        if first is None:
+            first = y.clone()
+        assert torch.equal(y, first)
+    assert lib.hb_tune(b"nvfp4_tile", 2) == 0
+    try:
+        stream = ops.nvfp4_linear(x, lin)
+    finally:
+        lib.hb_tune(b"nvfp4_tile", 0)
+    mx, nr = errors(first, stream)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+
+
 @pytest.fixture(scope="module")
 def latent_block():
     from hibana_amd import synthetic
