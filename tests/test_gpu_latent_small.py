@@ -198,3 +198,29 @@ def test_small_block_at_the_benchmark_geometry():
         assert mx < MAX_REL and nr < 2 * NORM_REL, (m, mx, nr)
     del block, ex
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("m", [1, 7])
+def test_small_block_on_an_expert_range(m):
+    """Expert parallelism: a rank holds experts lo .. hi - 1 of the E the router scores; pairs of other ranks' experts
+    are dropped by its plan and its combine. Without a shared expert the ranks' outputs add up to the whole block's."""
+    from hibana_amd.kernels import b12x_moe, nemotron_moe as small
+    from hibana_amd.model import nemotron_moe
+    e, hidden, latent, inter, topk = 16, 512, 256, 384, 4
+    whole, ref = _block(e, hidden, latent, inter, topk, 0, 44)
+    w1, s1, g1, w2, s2, g2 = ref.host
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    x = torch.randn(m, hidden, generator=torch.Generator().manual_seed(m)).bfloat16().cuda()
+    want = whole(x).float()
+    total = torch.zeros_like(want)
+    ids_seen = None
+    for lo, hi in ((0, 6), (6, 16)):
+        part = b12x_moe.B12xExperts(dev(w1[lo:hi]), dev(onv.swizzle_batched(s1[lo:hi])), dev(g1[lo:hi]), 1.0, dev(w2[lo:hi]), dev(onv.swizzle_batched(s2[lo:hi])),
+                                    dev(g2[lo:hi]), 1.0, routed_scaling=2.0, base=lo)
+        rank = nemotron_moe.NemotronMoe(whole.gate_fc1, whole.bias, whole.fc2, part, topk)
+        _, ids, w, ws = small.router(x, rank.small_weights(), None, topk)
+        assert ids_seen is None or torch.equal(ids, ids_seen)  # every rank routes over all E experts
+        ids_seen = ids
+        total += small.block(x, ws, ids, w, rank.small_weights()).float()
+    mx, nr = errors(total.bfloat16(), want.bfloat16())
+    assert mx < MAX_REL and nr < 2 * NORM_REL, (mx, nr)
