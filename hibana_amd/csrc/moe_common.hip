@@ -865,6 +865,58 @@ extern "C" int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int 
   return launch_status();
 }
 
+// (q, scales) = the per-(row, 32-group) E4M3 rounding of silu(gate) * up in one launch: BF16 [rows, 2 half] with the
+// gate | up columns as in silu_and_mul_kernel -> E4M3 [rows, half], FP32 scales [rows, half / 32]. The product is
+// rounded to BF16 as that kernel does it (`torch_chain`: silu to BF16 first, then the BF16 product) or from the FP32
+// product with one rounding; the rounding to E4M3 is quant_groups_lane's, value for value (silu_mul_quant_groups,
+// hibana/kernels/flashnext_fused.py:814-853 of the reference, with the exact divisions of its torch statement). A lane
+// takes eight consecutive output columns, four lanes a group.
+__global__ __launch_bounds__(256) void silu_mul_quant_groups_kernel(const uint16_t* __restrict__ x, int64_t rows, int half, int pairs, int torch_chain,
+                                                                    uint8_t* __restrict__ q, float* __restrict__ scales) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // eight columns from 8 (i % (half / 8)) of row i / (half / 8)
+  const int per_row = half >> 3;
+  if (i >= rows * per_row) return;  // whole groups leave together: rows * per_row is a multiple of four
+  const int64_t r = i / per_row;
+  const int c = 8 * (int)(i - r * per_row);
+  const int gate_at = pairs ? (c / pairs) * 2 * pairs + c % pairs : c, up_at = pairs ? gate_at + pairs : half + c;
+  const uint16_t* row = x + r * 2 * half;
+  const u32x4_t g4 = *reinterpret_cast<const u32x4_t*>(row + gate_at), u4 = *reinterpret_cast<const u32x4_t*>(row + up_at);
+  float v[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const float g = __uint_as_float((j & 1) ? g4[j >> 1] & 0xffff0000u : g4[j >> 1] << 16);
+    const float u = __uint_as_float((j & 1) ? u4[j >> 1] & 0xffff0000u : u4[j >> 1] << 16);
+    const float silu = g / (1.0f + expf(-g));
+    v[j] = round_bf16(torch_chain ? round_bf16(silu) * u : silu * u);
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(v[j]));
+  amax = fmaxf(amax, __shfl_xor(amax, 1));
+  amax = fmaxf(amax, __shfl_xor(amax, 2));
+  const float s = fmaxf(amax / 448.0f, 1e-12f);
+#pragma unroll
+  for (int j = 0; j < 8; j++) v[j] = fminf(fmaxf(v[j] / s, -448.0f), 448.0f);
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], hi, true);
+  typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+  *reinterpret_cast<i32x2_t*>(q + r * half + c) = i32x2_t{lo, hi};
+  if ((c & 31) == 0) scales[r * (half >> 5) + (c >> 5)] = s;
+}
+
+extern "C" int hb_silu_mul_quant_groups(const void* gate_up, int64_t rows, int half, int pairs, int torch_chain, void* q, float* scales, void* stream) {
+  if (!gate_up || !q || !scales) return HB_ENULL;
+  if (rows <= 0 || half <= 0 || half % 32 || pairs < 0 || (pairs && (pairs % 32 || half % pairs))) return HB_EINVAL;
+  if (!aligned(gate_up, 16) || !aligned(q, 8) || !aligned(scales, 4)) return HB_EINVAL;
+  const int64_t threads = rows * (half / 8);
+  hipLaunchKernelGGL(silu_mul_quant_groups_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint16_t*>(gate_up), rows, half, pairs, torch_chain, static_cast<uint8_t*>(q), scales);
+  return launch_status();
+}
+
 // x[r, c] = bf16(relu(x[r, c])^2) in place for BF16 rows `stride` elements apart: the square in FP32, one rounding
 // (torch's relu(x) ** 2; relu2_, hibana/model/nemotron/moe.py:316-321 of the reference). Two columns a thread.
 __global__ __launch_bounds__(256) void relu2_kernel(uint16_t* __restrict__ x, int64_t rows, int n, int64_t stride) {

@@ -51,6 +51,27 @@ def silu_and_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:
     return out.reshape(*gate_up.shape[:-1], half)
 
 
+def silu_mul_quant_groups(gate_up: torch.Tensor, pairs: int = 0, torch_chain: bool = False):
+    """`w3.quant_groups(silu_mul(gate_up))` in one launch, bit for bit: BF16 [M, 2I] -> (E4M3 [M, I], FP32 scales
+    [M, I/32]); `pairs`: gate and up interleaved in blocks of that many columns; `torch_chain`: the product as
+    `silu_and_mul` rounds it (hibana/kernels/flashnext_fused.py:841-853), the dense MLP's 3-bit decode input
+    (hibana/model/mlp.py:36-42)."""
+    if gate_up.dtype != torch.bfloat16 or gate_up.ndim != 2 or gate_up.stride(1) != 1 or gate_up.shape[1] % 64:
+        raise ValueError("silu_mul_quant_groups: BF16 [M, 2 I] with I a multiple of 32")
+    half = gate_up.shape[1] // 2
+    if pairs and (pairs % 32 or half % pairs):
+        raise ValueError("silu_mul_quant_groups: pairs must be a multiple of 32 dividing I")
+    _lib.need_gpu(gate_up)
+    gu = gate_up.contiguous()
+    m = gu.shape[0]
+    q = torch.empty((m, half), dtype=torch.float8_e4m3fn, device=gu.device)
+    scales = torch.empty((m, half // 32), dtype=torch.float32, device=gu.device)
+    if m:
+        _lib.check(_lib.lib().hb_silu_mul_quant_groups(_lib.ptr(gu), m, half, pairs, int(torch_chain), _lib.ptr(q), _lib.ptr(scales), _lib.stream()),
+                   "silu_mul_quant_groups")
+    return q, scales
+
+
 def route_topk(logits: torch.Tensor, k: int, slots: torch.Tensor | None = None, steps: int = 1, repeat: bool = False):
     """[M, E] FP32 logits -> (int32 ids [M, k], FP32 renormalized softmax weights [M, k]), largest first. With `slots`,
     row r is real iff slots[r // steps] != 0; a padded row takes expert E at weight 0 (the 3-bit experts skip it) or,

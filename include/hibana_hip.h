@@ -236,6 +236,15 @@ int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int pairs, void
  * with one rounding. ref: relu2_, hibana/model/nemotron/moe.py:316-321 (the expert kernels do it in their epilogues). */
 int hb_relu2(void* x, int64_t rows, int n, int64_t stride, void* stream);
 
+/* silu(gate) * up of BF16 [rows, 2 half] (columns as in hb_silu_and_mul) rounded to E4M3 per (row, 32-group) in one
+ * launch: q E4M3 [rows, half], scales FP32 [rows, half / 32], bit for bit hb_w3_quant_groups of hb_silu_and_mul's
+ * result when `torch_chain` != 0 (silu rounded to BF16, then the BF16 product), else of bf16(silu(gate) * up) from the
+ * FP32 product. half % 32 == 0, pairs % 32 == 0.
+ * ref: silu_mul_quant_groups, hibana/kernels/flashnext_fused.py:814-853 (caller Mlp.__call__, hibana/model/mlp.py:36-42),
+ * with the exact divisions of the quantizer's torch statement. */
+int hb_silu_mul_quant_groups(const void* gate_up, int64_t rows, int half, int pairs, int torch_chain, void* q,
+                             float* scales, void* stream);
+
 /* Softmax top-k routing: logits float32 [m, e] -> ids int32 [m, k] (descending probability, ties to the lower id),
  * weights float32 [m, k] renormalized over the selection. slots (may be NULL: every row is real): row r is real iff
  * slots[r / steps] != 0; a padded row gets weight 0 in every slot and the id e ("no expert", which the 3-bit experts

@@ -163,6 +163,44 @@ def test_w3_copy_serves_the_call_when_enabled():
         w3.set_enabled(None)
 
 
+@pytest.mark.parametrize("m,pairs", [(3, 0), (40, 0), (5, 64)])
+def test_dense_mlp_on_both_paths(m, pairs):
+    """`Mlp.__call__` (hibana/model/mlp.py:26-48): NVFP4 gate|up and down against the oracle's dense products around
+    silu_and_mul; with 3-bit copies enabled, the decode path - the 3-bit gate|up product, its SiLU product rounded to
+    E4M3 per 32-group in one launch, the 3-bit down product on those codes - against the same ops called one by one
+    (bit for bit) and against the oracle's rounding of the device's own SiLU product."""
+    from hibana_amd.kernels import ops, w3
+    from hibana_amd.model.mlp import Mlp
+    hidden, inter = 256, 384
+    gp, gs = _matrix(2 * inter, hidden, 21, hi=2.0)
+    dp, ds = _matrix(hidden, inter, 22, hi=2.0)
+    gate_up, down = _linear(gp, gs, alpha=0.05, inv=1.0), _linear(dp, ds, alpha=0.03, inv=1.0)
+    gate_up.pairs = pairs
+    mlp = Mlp(gate_up, down)
+    x = torch.randn(m, hidden, generator=torch.Generator().manual_seed(m)).bfloat16()
+    got = mlp(x.cuda())
+    h = layers.silu_and_mul(layers.nvfp4_dense_ref(x, onv.unpack_fp4(gp, gs), np.float32(0.05)), pairs)
+    want = layers.nvfp4_dense_ref(h, onv.unpack_fp4(dp, ds), np.float32(0.03))
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < 2 * NORM_REL, (mx, nr)  # two products and a BF16 SiLU between them
+    with pytest.raises(ValueError):
+        mlp(None, prequantized=(x, x))
+    if m > w3.MAX_ROWS:
+        return
+    w3.attach([("gate_up", gate_up), ("down", down)], "lloyd")
+    try:
+        w3.set_enabled(True)
+        three = mlp(x.cuda())
+        gu3 = w3.w3_linear(x.cuda(), gate_up.w3)
+        q, s = ops.silu_mul_quant_groups(gu3, pairs, torch_chain=True)
+        assert torch.equal(three, w3.w3_linear(q, down.w3, s))
+        want3 = layers.dense_a8_ref(ops.silu_and_mul(gu3, pairs).cpu(), w3.dequantize(down.w3).cpu().numpy())  # (the unpacking is pinned bit for bit elsewhere)
+        mx, nr = errors(three, want3)
+        assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    finally:
+        w3.set_enabled(None)
+
+
 def test_bad_calls_raise():
     from hibana_amd.kernels import ops
     from hibana_amd.weights import modelopt

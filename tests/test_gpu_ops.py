@@ -62,6 +62,27 @@ def test_silu_and_mul_matches_the_bf16_tensor_expression(shape, pairs):
         assert (got.view(torch.int16).int() - ref.view(torch.int16).int()).abs().max() <= 1
 
 
+@pytest.mark.parametrize("m,inter,pairs", [(1, 64, 0), (5, 256, 0), (7, 512, 64), (33, 17408 // 8, 32)])
+def test_silu_mul_quant_groups_is_the_two_ops_in_one_launch(m, inter, pairs):
+    """Bit for bit `quant_groups(silu_and_mul(gu, pairs))` with `torch_chain` (the reference's statement of the fused
+    kernel, hibana/kernels/flashnext_fused.py:842); the single-rounding product against the oracle's rounding of it."""
+    from hibana_amd.kernels import ops, w3
+    gu = (torch.randn(m, 2 * inter, generator=torch.Generator().manual_seed(m + inter)) * 2).bfloat16().cuda()
+    q, s = ops.silu_mul_quant_groups(gu, pairs, torch_chain=True)
+    q2, s2 = w3.quant_groups(ops.silu_and_mul(gu, pairs))
+    assert q.dtype == torch.float8_e4m3fn and q.shape == (m, inter) and s.shape == (m, inter // 32)
+    assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
+    # one rounding of the FP32 product: the oracle's quantizer on the device's own BF16 product (within one unit of the
+    # host's, as for silu_and_mul), then the same bytes and scales
+    q1, s1 = ops.silu_mul_quant_groups(gu, pairs)
+    g = layers.silu_and_mul(gu.cpu().float(), pairs).bfloat16()  # FP32 product, one rounding
+    wq, ws = layers.quant_e4m3_groups(g)
+    same = (q1.view(torch.uint8).cpu() == wq).float().mean()
+    assert same > 0.98 and torch.allclose(s1.cpu(), ws, rtol=1e-2)  # a last-bit exponential moves a code here and there
+    with pytest.raises(ValueError):
+        ops.silu_mul_quant_groups(gu[:, :-2], pairs)
+
+
 def test_relu2_in_place():
     from hibana_amd.model import nemotron_moe
     g = torch.Generator().manual_seed(9)
