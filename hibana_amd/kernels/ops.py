@@ -101,6 +101,10 @@ def moe_combine_pairs(y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
         return out
     if y.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("moe_combine_pairs: pairs must be FP32 or BF16")
+    if y.shape[0] != m * topk or weights.shape != ids.shape or (shared is not None and tuple(shared.shape) != (m, h)):
+        raise ValueError("moe_combine_pairs: y [M * k, H], ids / weights [M, k], shared [M, H]")
+    if gate_w is not None and shared is not None and (x is None or tuple(x.shape) != (m, h) or gate_w.numel() != h):
+        raise ValueError("moe_combine_pairs: the gate takes x [M, H] and gate_w [H] (the layer's input rows)")
     # every converted operand is bound to a name until the launch is enqueued
     yc, ids32, wt = y.contiguous(), ids.to(torch.int32).contiguous(), weights.float().contiguous()
     sh = None if shared is None else shared.to(torch.bfloat16).contiguous()
@@ -110,3 +114,15 @@ def moe_combine_pairs(y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
                                                _lib.ptr(xx), _lib.ptr(gw), e_lo, e_n, m, topk, h, _lib.ptr(out), _lib.stream()),
                "moe_combine_pairs")
     return out
+
+
+def moe_combine(routed: torch.Tensor, shared: torch.Tensor, x: torch.Tensor, gate_w: torch.Tensor) -> torch.Tensor:
+    """bf16(routed + sigmoid(x . gate_w) * shared) for BF16 routed / shared [M, H] (hibana/kernels/flashnext_fused.py:
+    506-526): the combine kernel on one pair a row at weight 1, whose rounded sum is `routed` itself."""
+    if routed.dtype != torch.bfloat16 or routed.ndim != 2 or shared.shape != routed.shape or x.shape != routed.shape or gate_w.numel() != routed.shape[1]:
+        raise ValueError("moe_combine: routed, shared and x must be BF16 [M, H] of one shape, gate_w [H]")
+    m = routed.shape[0]
+    ids = torch.zeros((m, 1), dtype=torch.int32, device=routed.device)
+    ones = torch.ones((m, 1), dtype=torch.float32, device=routed.device)
+    return moe_combine_pairs(routed, ids, ones, shared, x, gate_w, 0, 1)
+

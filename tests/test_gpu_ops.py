@@ -83,6 +83,20 @@ def test_silu_mul_quant_groups_is_the_two_ops_in_one_launch(m, inter, pairs):
         ops.silu_mul_quant_groups(gu[:, :-2], pairs)
 
 
+def test_moe_combine_of_a_routed_sum_and_the_gated_shared_expert():
+    from hibana_amd.kernels import ops
+    g = torch.Generator().manual_seed(12)
+    routed, shared = torch.randn(9, 256, generator=g).bfloat16(), torch.randn(9, 256, generator=g).bfloat16()
+    x, gate = torch.randn(9, 256, generator=g).bfloat16(), torch.randn(256, generator=g) * 0.1  # the layer's input rows: the same width
+    got = ops.moe_combine(routed.cuda(), shared.cuda(), x.cuda(), gate.cuda()).cpu()
+    gv = torch.sigmoid((x.double() @ gate.double()))[:, None]
+    want = (routed.double() + gv * shared.double()).float().bfloat16()
+    # one BF16 unit at most, and rarely: the gate's dot product and exponential are FP32 on the device
+    # (where the two terms cancel, the gate's last bits show against the small sum: an absolute term beside the relative)
+    assert ((got.float() - want.float()).abs() <= want.float().abs() * 2.0 ** -7 + 1e-5 * (1 + shared.float().abs())).all()
+    assert (got.view(torch.int16) != want.view(torch.int16)).float().mean() < 0.02
+
+
 def test_relu2_in_place():
     from hibana_amd.model import nemotron_moe
     g = torch.Generator().manual_seed(9)
