@@ -371,6 +371,33 @@ def dense_decode(args) -> dict:
     return line
 
 
+def routing_only(args) -> dict:
+    """`--routing [ROWS]`: the routing launches alone at Flash-Next's router shape (512 experts, top 10), graph-replayed:
+    `route_topk` and the budgeted `route_budget` (keep 4, budget 64) at decode / verify row counts."""
+    import torch
+
+    from hibana_amd.kernels import ops
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    g = torch.Generator(device=dev).manual_seed(7)
+    rows_out = {}
+    for rows in ((args.routing,) if args.routing else (1, 16, 64, 320)):
+        feeds = [(torch.randn(rows, 512, device=dev, generator=g) * 1.2).bfloat16() for _ in range(8)]
+        floats = [f.float() for f in feeds]
+        entry = {}
+        for name, call in (("route_topk", lambda i: ops.route_topk(floats[i % 8], 10)), ("route_budget", lambda i: ops.route_budget(feeds[i % 8], 10, 4, 64))):
+            call(0)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                outs = [call(i) for i in range(args.steps)]
+            entry[name + "_us"] = round(median(replay_times(graph, args.steps)) * 1e3, 2)
+            del outs, graph
+        rows_out[str(rows)] = entry
+    return {"metric": "routing microseconds a call (512 experts, top 10; budgeted: keep 4, budget 64)", "by_rows": rows_out, "steps": args.steps}
+
+
 def replay_times(graph, steps: int, floor_s: float = 0.2, least: int = 5):
     """Per-step milliseconds of repeated replays of a graph of `steps` steps: at least `least` replays and at least
     `floor_s` seconds of them, each bracketed by synchronizations."""
@@ -484,6 +511,8 @@ def main() -> int:
     ap.add_argument("--rows", type=int, default=1, help="configs 0 and 1: activation rows M")
     ap.add_argument("--small-rows", type=int, default=0, help="config 4: only its block (with a shared expert) at this many rows (1 .. 16) through the "
                     "small-call kernels")
+    ap.add_argument("--routing", type=int, nargs="?", const=0, default=None, metavar="ROWS",
+                    help="only the routing launches (route_topk, route_budget) at ROWS rows (none given: 1 / 16 / 64 / 320)")
     ap.add_argument("--headline-only", action="store_true", help="config 3 without the other configurations' lines (profiling runs)")
     ap.add_argument("--e4m3", action="store_true", help="configs 2 and 3: the reference kernel's own arithmetic (activations rounded to E4M3 per "
                     "32-group, FP8 MFMA) instead of the weight-only form; no CPU leg")
@@ -501,6 +530,9 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
         return 2
+    if args.routing is not None:
+        print(json.dumps(routing_only(args)))
+        return 0
     if args.config == 4:
         print(json.dumps(latent_small_only(args) if args.small_rows else latent_prefill(args)))
         return 0

@@ -61,9 +61,12 @@ SIGNATURES = {
     "hb_w3_moe_layer_logits_e4m3": (_I, [_EX, _EX, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P]),
     "hb_moe_combine_pairs": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P]),
     "hb_silu_and_mul": (_I, [_P, _L, _I, _I, _P, _P]),
+    "hb_silu_mul": (_I, [_P, _L, _I, _I, _P, _P]),
     "hb_relu2": (_I, [_P, _L, _I, _L, _P]),
     "hb_silu_mul_quant_groups": (_I, [_P, _L, _I, _I, _I, _P, _P, _P]),
     "hb_route_softmax_topk": (_I, [_P, _I, _I, _I, _P, _I, _I, _P, _P, _P]),
+    "hb_route_budget_workspace_bytes": (_L, [_I]),
+    "hb_route_budget": (_I, [_P, _I, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P, _L, _P, _P, _P]),
     "hb_route_sigmoid_topk": (_I, [_P, _L, _P, _I, _I, _I, _I, _P, _I, _I, _P, _P, _P, _P]),
     "hb_nvfp4_tiled_bytes": (_Z, [_L, _I]),
     "hb_nvfp4_repack": (_I, [_P, _P, _I, _L, _I, _P, _P]),

@@ -839,7 +839,9 @@ extern "C" int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int
 
 // out[r, c] = bf16( bf16(silu(gate)) * up ) of BF16 rows holding `half` gate and `half` up columns: [gate | up]
 // (pairs == 0) or alternating blocks of `pairs` gate columns and their `pairs` up columns. The roundings are those of
-// the BF16 tensor expression silu(gate) * up (hibana/kernels/ops.py:86-92 of the reference). Two columns a thread.
+// the BF16 tensor expression silu(gate) * up (hibana/kernels/ops.py:86-92 of the reference); without CHAIN the FP32
+// product is rounded once. Two columns a thread.
+template <bool CHAIN>
 __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __restrict__ x, int64_t rows, int half, int pairs, uint16_t* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // column pair i % (half / 2) of row i / (half / 2)
   const int per_row = half >> 1;
@@ -851,18 +853,34 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __res
   const uint32_t g2 = *reinterpret_cast<const uint32_t*>(row + gate_at), u2 = *reinterpret_cast<const uint32_t*>(row + up_at);
   const float g0 = __uint_as_float(g2 << 16), g1 = __uint_as_float(g2 & 0xffff0000u);
   const float u0 = __uint_as_float(u2 << 16), u1 = __uint_as_float(u2 & 0xffff0000u);
-  const float s0 = round_bf16(g0 / (1.0f + expf(-g0))), s1 = round_bf16(g1 / (1.0f + expf(-g1)));
+  float s0 = g0 / (1.0f + expf(-g0)), s1 = g1 / (1.0f + expf(-g1));
+  if (CHAIN) s0 = round_bf16(s0), s1 = round_bf16(s1);
   *reinterpret_cast<uint32_t*>(out + r * half + c) = (uint32_t)f32_to_bf16_bits(s0 * u0) | ((uint32_t)f32_to_bf16_bits(s1 * u1) << 16);
 }
 
-extern "C" int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int pairs, void* out, void* stream) {
+static int silu_mul_launch(const void* gate_up, int64_t rows, int half, int pairs, bool chain, void* out, void* stream) {
   if (!gate_up || !out) return HB_ENULL;
   if (rows <= 0 || half <= 0 || half % 2 || pairs < 0 || (pairs && (pairs % 2 || half % pairs))) return HB_EINVAL;
   if (!aligned(gate_up, 4) || !aligned(out, 4)) return HB_EINVAL;
   const int64_t threads = rows * (half / 2);
-  hipLaunchKernelGGL(silu_and_mul_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, as_stream(stream),
-                     static_cast<const uint16_t*>(gate_up), rows, half, pairs, static_cast<uint16_t*>(out));
+  const dim3 grid((unsigned)((threads + 255) / 256));
+  if (chain) {
+    hipLaunchKernelGGL(silu_and_mul_kernel<true>, grid, dim3(256), 0, as_stream(stream), static_cast<const uint16_t*>(gate_up), rows, half, pairs,
+                       static_cast<uint16_t*>(out));
+  } else {
+    hipLaunchKernelGGL(silu_and_mul_kernel<false>, grid, dim3(256), 0, as_stream(stream), static_cast<const uint16_t*>(gate_up), rows, half, pairs,
+                       static_cast<uint16_t*>(out));
+  }
   return launch_status();
+}
+
+extern "C" int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int pairs, void* out, void* stream) {
+  return silu_mul_launch(gate_up, rows, half, pairs, true, out, stream);
+}
+
+// bf16(silu(gate) * up) from the FP32 product: one rounding (silu_mul, hibana/kernels/flashnext_fused.py:624-639).
+extern "C" int hb_silu_mul(const void* gate_up, int64_t rows, int half, int pairs, void* out, void* stream) {
+  return silu_mul_launch(gate_up, rows, half, pairs, false, out, stream);
 }
 
 // (q, scales) = the per-(row, 32-group) E4M3 rounding of silu(gate) * up in one launch: BF16 [rows, 2 half] with the

@@ -51,6 +51,22 @@ def silu_and_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:
     return out.reshape(*gate_up.shape[:-1], half)
 
 
+def silu_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:
+    """bf16(silu(gate) * up) of BF16 [M, 2 I] from the FP32 product, one rounding (hibana/kernels/flashnext_fused.py:
+    624-639); columns as in `silu_and_mul`."""
+    if gate_up.dtype != torch.bfloat16 or gate_up.ndim != 2 or gate_up.shape[1] % 4:
+        raise ValueError("silu_mul: BF16 [M, 2 I] with I even")
+    half = gate_up.shape[1] // 2
+    if pairs and (pairs % 2 or half % pairs):
+        raise ValueError("silu_mul: pairs must be even and divide I")
+    _lib.need_gpu(gate_up)
+    gu = gate_up.contiguous()
+    out = torch.empty((gu.shape[0], half), dtype=torch.bfloat16, device=gu.device)
+    if gu.shape[0]:
+        _lib.check(_lib.lib().hb_silu_mul(_lib.ptr(gu), gu.shape[0], half, pairs, _lib.ptr(out), _lib.stream()), "silu_mul")
+    return out
+
+
 def silu_mul_quant_groups(gate_up: torch.Tensor, pairs: int = 0, torch_chain: bool = False):
     """`w3.quant_groups(silu_mul(gate_up))` in one launch, bit for bit: BF16 [M, 2I] -> (E4M3 [M, I], FP32 scales
     [M, I/32]); `pairs`: gate and up interleaved in blocks of that many columns; `torch_chain`: the product as
@@ -85,6 +101,37 @@ def route_topk(logits: torch.Tensor, k: int, slots: torch.Tensor | None = None, 
     if m:
         _lib.check(_lib.lib().hb_route_softmax_topk(_lib.ptr(lg), m, e, k, _lib.ptr(sl), steps, int(repeat), _lib.ptr(ids), _lib.ptr(w),
                                                     _lib.stream()), "route_topk")
+    return ids, w
+
+
+ROUTE_CANDIDATES = 20  # a row takes its experts from its 20 largest logits
+
+
+def route_budget(logits: torch.Tensor, k: int, keep: int, budget: int, slots: torch.Tensor | None = None, steps: int = 1,
+                 repeat: bool = False, per_request: int = 0, min_cap: int = 0):
+    """Budgeted top-k (hibana/kernels/flashnext_fused.py:462-502): BF16 [R, E] logits -> (int32 ids [R, k], FP32 weights
+    [R, k]). The experts the call reads are chosen for the whole call under a cap: every real row's top `keep`, then the
+    experts with the most softmax probability within the real rows' top k until the set holds the cap (`budget`, or
+    with `per_request`, min(budget, max(min_cap, per_request x the real requests))); each real row takes its candidates
+    (its 20 largest logits, an exact tie to the lower expert) in the set, in rank order, up to k, its weights the
+    softmax over E renormalized over them. Slots left over (all of a padded row's: slots[r // steps] == 0) hold id E at
+    weight 0, or with `repeat` the row's top 1 (a padded row: row 0's)."""
+    if logits.dtype != torch.bfloat16 or logits.ndim != 2:
+        raise ValueError("route_budget: BF16 [R, E] logits")
+    r, e = logits.shape
+    if not (ROUTE_CANDIDATES <= e <= 1024 and 1 <= k <= ROUTE_CANDIDATES and 0 <= keep <= ROUTE_CANDIDATES) or budget < 0 or steps < 1 or r % steps:
+        raise ValueError("route_budget: 20 <= E <= 1024, k and keep at most 20, whole requests of `steps` rows")
+    if slots is not None and slots.numel() < r // steps:
+        raise ValueError("route_budget: a slot for every request")
+    _lib.need_gpu(logits, slots)
+    lg = logits.contiguous()
+    sl = None if slots is None else slots.to(torch.int32).contiguous()
+    ids = torch.empty((r, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((r, k), dtype=torch.float32, device=logits.device)
+    if r:
+        ws = torch.empty((_lib.lib().hb_route_budget_workspace_bytes(r),), dtype=torch.uint8, device=logits.device)
+        _lib.check(_lib.lib().hb_route_budget(_lib.ptr(lg), r, e, k, keep, budget, _lib.ptr(sl), steps, int(repeat), per_request, min_cap,
+                                              _lib.ptr(ws), ws.numel(), _lib.ptr(ids), _lib.ptr(w), _lib.stream()), "route_budget")
     return ids, w
 
 

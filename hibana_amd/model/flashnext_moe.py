@@ -10,8 +10,10 @@
 The block is assembled from tensors already on the device (a loader's job ends there). The routed experts are a
 `W3Experts`; the shared expert is either a one-expert `W3Experts` or the pair of linears the reference holds
 (`shared_gate_up` with rows [gate; up], `shared_down`), whose 3-bit copies are re-stored once, at construction, in the
-experts' row order (`shared_from_linears`). Budgeted expert selection (HIBANA_MOE_KEEP / HIBANA_MOE_BUDGET of the
-reference) is not built: every call routes top-k.
+experts' row order (`shared_from_linears`). Budgeted expert selection (HIBANA_MOE_KEEP / HIBANA_MOE_BUDGET /
+HIBANA_MOE_BUDGET_PER_REQUEST of the reference's configuration) is the constructor's `keep` / `budget` / `per_request`:
+decode and verify forwards then read at most a budget of distinct experts (`ops.route_budget`); slots left over name no
+expert, which the 3-bit kernels skip.
 """
 from __future__ import annotations
 
@@ -38,14 +40,25 @@ def shared_from_linears(gate_up: w3.W3Weight, down: w3.W3Weight) -> w3_moe.W3Exp
 
 
 class MoeLayer:
+    MIN_GUARANTEE = 2  # hibana/model/flashnext/moe.py:146-149
+    MIN_CAP = 16
+
     def __init__(self, router: torch.Tensor, shared_gate: torch.Tensor, experts: w3_moe.W3Experts, topk: int, shared: w3_moe.W3Experts | None = None,
-                 shared_gate_up=None, shared_down=None):
+                 shared_gate_up=None, shared_down=None, keep: int = 0, budget: int = 0, per_request: int = 0):
         """router BF16 [E, H]; shared_gate [1, H] or [H] (the shared expert's sigmoid gate); `experts` this rank's 3-bit
         experts (a range base .. base + experts - 1 of the E); the shared expert as `shared`, or as the two linears
-        `shared_gate_up` / `shared_down` with 3-bit copies attached (`.w3`)."""
+        `shared_gate_up` / `shared_down` with 3-bit copies attached (`.w3`). `keep` (below topk; topk or more, or 0, is
+        the served route): each token's own top experts in decode and verify forwards; with `budget`, the cap on the
+        distinct experts such a forward reads, `per_request` its share a request
+        (hibana/model/flashnext/moe.py:86-93)."""
+        if keep < 0 or budget < 0 or per_request < 0:
+            raise ValueError(f"keep {keep}, budget {budget}, per_request {per_request}: not negative")
         self.router = router.contiguous()
         self.experts, self.hidden = router.shape
         self.topk = topk
+        self.keep = keep if keep < topk else 0
+        self.budget = budget if self.keep else 0
+        self.per_request = per_request
         self.shared_gate = shared_gate.float().reshape(1, -1).contiguous()
         self.shared_gate_vec = self.shared_gate.reshape(-1)
         self.w3 = w3_moe.tile(experts)
@@ -76,11 +89,28 @@ class MoeLayer:
             return getattr(ctx, "seq_slots", None), int(getattr(ctx, "verify_steps", 1))
         return None, 1
 
+    def guarantee(self, rows: int, steps: int) -> int:
+        """Each token's guaranteed top experts under a budget: 2 cap / rows within [MIN_GUARANTEE, keep], the cap that of
+        the call's shape (hibana/model/flashnext/moe.py:151-158)."""
+        cap = min(self.budget, max(self.MIN_CAP, self.per_request * (rows // steps))) if self.per_request else self.budget
+        return max(min(self.MIN_GUARANTEE, self.keep), min(self.keep, 2 * cap // rows))
+
+    def selects(self, ctx) -> bool:
+        """Whether this forward takes the budgeted selection: decode and verify forwards of a layer with a `keep`."""
+        return bool(self.keep) and getattr(ctx, "mode", None) in ("decode", "verify")
+
     def route(self, x: torch.Tensor, ctx=None):
         """(ids int32 [M, k], weights FP32 [M, k]); padded rows of a decode / verify graph name no expert
-        (hibana/model/flashnext/moe.py:122-144; softmax -> top-k -> renormalize at every size)."""
+        (hibana/model/flashnext/moe.py:122-144; softmax -> top-k -> renormalize at every size). With a `keep`, decode
+        and verify forwards take each token's top `keep` alone (ids [M, keep]) or, under a budget, the selection of
+        `ops.route_budget`."""
         logits = torch.mm(x, self.router.T)
         slots, steps = self._padding(ctx)
+        if self.selects(ctx):
+            if not self.budget:
+                return ops.route_topk(logits, self.keep)
+            return ops.route_budget(logits, self.topk, self.guarantee(logits.shape[0], steps), self.budget, slots, steps, repeat=False,
+                                    per_request=self.per_request, min_cap=self.MIN_CAP)
         return ops.route_topk(logits, self.topk, slots, steps, repeat=False)
 
     def routed(self, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
@@ -90,7 +120,7 @@ class MoeLayer:
     def __call__(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
         x = x.contiguous()
         slots, _ = self._padding(ctx)
-        if slots is None:  # routing, plan, both streams and the combine as one chain
+        if slots is None and not self.selects(ctx):  # routing, plan, both streams and the combine as one chain
             logits = torch.mm(x, self.router.T).float()
             return w3_moe.moe_layer_logits(self.w3, x, logits, self.topk, shared=self.shared, gate_vec=self.shared_gate_vec)
         ids, weights = self.route(x, ctx)

@@ -232,6 +232,10 @@ int hb_moe_combine_pairs(const void* pairs, int pairs_bf16, const int32_t* ids, 
  * ref: ops.silu_and_mul, hibana/kernels/ops.py:86-92. */
 int hb_silu_and_mul(const void* gate_up, int64_t rows, int half, int pairs, void* out, void* stream);
 
+/* The same from the FP32 product, rounded once: out = bf16(silu(gate) * up) (shapes and `pairs` as hb_silu_and_mul).
+ * ref: silu_mul, hibana/kernels/flashnext_fused.py:624-639. */
+int hb_silu_mul(const void* gate_up, int64_t rows, int half, int pairs, void* out, void* stream);
+
 /* x = bf16(relu(x)^2) in place, BF16 [rows, n] with rows `stride` elements apart (n and stride even): the square in FP32
  * with one rounding. ref: relu2_, hibana/model/nemotron/moe.py:316-321 (the expert kernels do it in their epilogues). */
 int hb_relu2(void* x, int64_t rows, int n, int64_t stride, void* stream);
@@ -262,6 +266,27 @@ int hb_route_softmax_topk(const float* logits, int m, int e, int k, const int32_
 int hb_route_sigmoid_topk(const float* fused, int64_t stride, const float* bias, int m, int e, int k, int latent,
                           const int32_t* slots, int steps, int repeat, int32_t* ids, float* weights, void* lat,
                           void* stream);
+
+/* Budgeted top-k: the experts one decode / verify forward reads are chosen for all its rows, under a cap. logits BF16
+ * [r, e] contiguous (20 <= e <= 1024) -> ids int32 [r, k], weights FP32 [r, k] (k, keep <= HB_ROUTE_CANDIDATES).
+ *   the set: every real row's top `keep`, then the experts with the most softmax probability within the real rows'
+ *   top k, summed over the rows (equal sums: the lower expert), until it holds the cap (more only when the guaranteed
+ *   experts alone exceed it); the cap is `budget`, or with per_request > 0,
+ *   min(budget, max(min_cap, per_request x the real requests)), a request being `steps` consecutive rows;
+ *   a real row takes its candidates (its HB_ROUTE_CANDIDATES largest logits, largest first, an exact tie to the lower
+ *   expert, -0 equal to +0) that are in the set, in rank order, up to k, at the FP32 softmax over e renormalized over
+ *   the ones taken.
+ * Slots left over (all of a padded row's; row t is real iff slots == NULL or slots[t / steps] != 0; r % steps == 0)
+ * hold id e at weight 0, or with repeat != 0 the row's first candidate (a padded row: row 0's) at weight 0.
+ * Two launches, the same bits on every run; nothing is allocated: `workspace` (4-byte aligned, at least
+ * hb_route_budget_workspace_bytes(r)) holds the rows' candidates between the launches.
+ * ref: route_budget, hibana/kernels/flashnext_fused.py:322-502 (the rule row by row:
+ * tests/unit/test_moe_selection.py:19-58); caller MoeLayer.route, hibana/model/flashnext/moe.py:122-135. */
+#define HB_ROUTE_CANDIDATES 20
+int64_t hb_route_budget_workspace_bytes(int r);
+int hb_route_budget(const void* logits, int r, int e, int k, int keep, int budget, const int32_t* slots, int steps,
+                    int repeat, int per_request, int min_cap, void* workspace, int64_t workspace_bytes, int32_t* ids,
+                    float* weights, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
  * NVFP4 format: E2M1 codes two per byte (element 2i in the low nibble), one E4M3 scale per 16 weights, one FP32

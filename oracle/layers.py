@@ -19,6 +19,13 @@ points of the reference kept.
                          descending, renormalized
   route_sigmoid_topk     hibana/model/nemotron/moe.py:1-12, tests/nemotron_reference.py:550-565: top-k of
                          sigmoid + bias (ties to the lower id), weights from the plain sigmoid, renormalized, scaled
+  route_budget_ref       hibana/kernels/flashnext_fused.py:322-502 (the rank / score / select / pick launches) with the
+                         rule as tests/unit/test_moe_selection.py:19-58 writes it out row by row: candidates = the 20
+                         largest logits (ties to the lower expert, -0 == +0), core = real rows' top keep, score = sum
+                         in row order of the FP32 softmax within the real rows' top k, the set = core + best-scoring
+                         others (score > 0, equal scores to the lower expert) up to the cap, rows take their
+                         candidates in the set in rank order
+  silu_mul               hibana/kernels/flashnext_fused.py:624-639: bf16(silu(gate) * up) from the FP32 product
   latent_moe_ref         tests/nemotron_reference.py:568-593 (ReLU^2 latent experts, BF16 linears, FP32 accumulate)
   silu_and_mul           hibana/kernels/ops.py:86-92
   quant_e4m3_groups      hibana/kernels/w3_moe.py:187-190 (the torch mirror of the activation rounding, the definition
@@ -36,7 +43,10 @@ one == two dense products; all weights zero == zero; a permutation of slots with
 per-pair Python loops on tiny shapes written from the formula in w3_moe.py:205-213, torch.topk/softmax for the
 routing, and sortedness/CSR invariants for the plan. quant_e4m3_groups: a brute-force nearest-value search over the
 256-entry E4M3 table (ties to the even code) on random and hand-made groups, the group maximum landing on +-448 * s, and
-groups that are already E4M3 multiples of their scale coming back unchanged.
+groups that are already E4M3 multiples of their scale coming back unchanged. route_budget_ref: a hand-worked call
+whose set and rows follow from the rule by inspection, a cap no smaller than the rows' top-k union == a stable
+descending sort's top k with the renormalized softmax of torch, padded requests == the call on the real rows alone, and
+the invariants the reference's own unit test states (tests/unit/test_moe_selection.py:66-106).
 """
 from __future__ import annotations
 
@@ -217,6 +227,54 @@ def route_sigmoid_topk(logits: torch.Tensor, bias: torch.Tensor, k: int, scaling
     w = s.gather(1, ids)
     w = w / (w.sum(-1, keepdim=True) + 1e-20) * scaling
     return ids.to(torch.int32), w.contiguous()
+
+
+ROUTE_CANDIDATES = 20
+
+
+def route_budget_ref(logits: torch.Tensor, k: int, keep: int, budget: int, slots=None, steps: int = 1, repeat: bool = False,
+                     per_request: int = 0, min_cap: int = 0, given=None):
+    """-> (ids int32 [R, k], weights FP32 [R, k], the set, its guaranteed part, the FP32 scores [E]). `given`: the rows
+    take their experts from this set instead of the selected one (the second half of the rule alone)."""
+    lg = logits.float().cpu().numpy().astype(np.float32)
+    r, e = lg.shape
+    real = [slots is None or int(slots[t // steps]) != 0 for t in range(r)]
+    cap = budget
+    if per_request > 0:
+        cap = min(budget, max(min_cap, per_request * sum(1 for t in range(0, r, steps) if real[t])))
+    ex = np.exp(lg - lg.max(-1, keepdims=True), dtype=np.float32)
+    p = ex / ex.sum(-1, keepdims=True, dtype=np.float32)
+    # a stable ascending sort of the negated logits: the largest first, equal logits (both zeros among them) in id order
+    cand = [np.argsort(-(row + np.float32(0.0)), kind="stable")[:ROUTE_CANDIDATES].tolist() for row in lg]
+    core = {x for c, live in zip(cand, real) if live for x in c[:keep]}
+    score = np.zeros(e, dtype=np.float32)
+    for t, c in enumerate(cand):
+        if real[t]:
+            for x in c[:k]:
+                score[x] = np.float32(score[x] + p[t, x])
+    rest = sorted((x for x in range(e) if x not in core and score[x] > 0), key=lambda x: (-float(score[x]), x))
+    chosen = core | set(rest[:max(0, cap - len(core))]) if given is None else set(given)
+    ids = np.full((r, k), e, dtype=np.int32)
+    w = np.zeros((r, k), dtype=np.float32)
+    for t, c in enumerate(cand):
+        row = [x for x in c if x in chosen][:k] if real[t] else []
+        if row:
+            taken = p[t, row]
+            ids[t, :len(row)] = row
+            w[t, :len(row)] = taken / taken.sum(dtype=np.float32)
+        if repeat:
+            ids[t, len(row):] = c[0] if real[t] else cand[0][0]
+    return torch.from_numpy(ids), torch.from_numpy(w), chosen, core, score
+
+
+def silu_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:
+    half = gate_up.shape[-1] // 2
+    if pairs:
+        blocks = gate_up.unflatten(-1, (half // pairs, 2, pairs))
+        g, u = blocks[..., 0, :].flatten(-2).float(), blocks[..., 1, :].flatten(-2).float()
+    else:
+        g, u = gate_up[..., :half].float(), gate_up[..., half:].float()
+    return (g * torch.sigmoid(g) * u).to(torch.bfloat16)
 
 
 def latent_experts_ref(lat: torch.Tensor, ids: np.ndarray, weights: torch.Tensor, get_expert):

@@ -59,6 +59,13 @@ def test_validation_without_a_gpu():
     assert lib.hb_nvfp4_gemm_workspace_bytes(64, 100, 5120) == 0
     assert lib.hb_nvfp4_gemm_ws(None, 64, None, 1.0, 128, 128, 0, None, None, 0, None) == _lib.HB_ENULL
     assert lib.hb_relu2(None, 1, 2, 2, None) == _lib.HB_ENULL and lib.hb_relu2(256, 1, 3, 4, None) == _lib.HB_EINVAL
+    assert lib.hb_silu_mul(None, 1, 2, 0, None, None) == _lib.HB_ENULL and lib.hb_silu_mul(256, 1, 3, 0, 256, None) == _lib.HB_EINVAL
+    # budgeted routing: 20 candidates a row, whole requests, a workspace for the candidates
+    assert lib.hb_route_budget_workspace_bytes(12) == 12 * 20 * 8 and lib.hb_route_budget_workspace_bytes(0) == 0
+    assert lib.hb_route_budget(None, 12, 512, 10, 4, 64, None, 1, 0, 0, 0, 256, 1920, 256, 256, None) == _lib.HB_ENULL
+    for r, e, k, keep, steps in [(12, 19, 10, 4, 1), (12, 1025, 10, 4, 1), (12, 512, 21, 4, 1), (12, 512, 10, 21, 1), (12, 512, 10, 4, 5)]:
+        assert lib.hb_route_budget(256, r, e, k, keep, 64, None, steps, 0, 0, 0, 256, 1920, 256, 256, None) == _lib.HB_EINVAL
+    assert lib.hb_route_budget(256, 12, 512, 10, 4, 64, None, 1, 0, 0, 0, 256, 1919, 256, 256, None) == _lib.HB_EWORKSPACE
     # the small latent block: shapes and pointers are checked before anything is launched
     nv = _lib.HbNvfp4Experts(256, 256, 256, 256, 8, 0, 256, 128, 256, 0)
     lw = _lib.HbLatentWeights(256, 256, 256, C.pointer(nv), 256, 256, 1.0, 1.0, 8, 256, 512, 640)
@@ -130,6 +137,46 @@ def test_host_logic_mirrors_the_reference_interface(monkeypatch):
         w3.quant_groups(torch.zeros(1, 32))  # not BF16
     with pytest.raises(RuntimeError):
         w3.quant_groups(torch.zeros(1, 32, dtype=torch.bfloat16))  # no CPU path
+
+
+def test_budgeted_selection_settings_and_which_forwards_take_it(monkeypatch):
+    """`MoeLayer`'s keep / budget / per_request as the reference resolves them, the guarantee by the call's shape (the
+    values of tests/unit/test_moe_selection.py:150-171 of the reference), and the routing call each forward makes."""
+    from types import SimpleNamespace
+
+    from hibana_amd.model import flashnext_moe
+    from hibana_amd.model.flashnext_moe import MoeLayer
+
+    def layer(keep=4, budget=64, per_request=12, topk=10):
+        it = MoeLayer.__new__(MoeLayer)
+        it.router = torch.zeros(512, 32, dtype=torch.bfloat16)
+        it.topk = topk
+        it.keep = keep if keep < topk else 0
+        it.budget = budget if it.keep else 0
+        it.per_request = per_request
+        return it
+
+    assert [layer(keep=k).keep for k in (0, 1, 4, 9, 10, 12)] == [0, 1, 4, 9, 0, 0]
+    assert (layer(keep=0).budget, layer(keep=10).budget, layer(keep=4).budget) == (0, 0, 64)
+    shapes = [(1, 1), (1, 5), (1, 8), (4, 5), (1, 9), (2, 9), (8, 5), (16, 4), (64, 4), (128, 1)]  # requests x rows a request
+    assert [layer().guarantee(r * s, s) for r, s in shapes] == [4, 4, 4, 4, 3, 2, 3, 2, 2, 2]
+    assert layer(keep=1).guarantee(256, 4) == 1 and layer(per_request=0).guarantee(5, 5) == 4
+    calls = []
+    stub = SimpleNamespace(
+        route_budget=lambda logits, k, keep, budget, slots=None, steps=1, repeat=False, per_request=0, min_cap=0:
+            calls.append(("budget", k, keep, budget, slots, steps, repeat, per_request, min_cap)) or "budget",
+        route_topk=lambda logits, k, slots=None, steps=1, repeat=False: calls.append(("topk", k, slots, steps)) or f"top{k}")
+    monkeypatch.setattr(flashnext_moe, "ops", stub)
+    x = torch.zeros(20, 32, dtype=torch.bfloat16)
+    verify_slots, decode_slots = torch.tensor([3, 1, 4, 0], dtype=torch.int32), torch.tensor([7] * 13 + [0] * 7, dtype=torch.int32)
+    assert layer().route(x, SimpleNamespace(mode="verify", seq_slots=verify_slots, verify_steps=5)) == "budget"
+    assert layer().route(x, SimpleNamespace(mode="decode", slots=decode_slots)) == "budget"
+    assert calls == [("budget", 10, 4, 64, verify_slots, 5, False, 12, 16), ("budget", 10, 4, 64, decode_slots, 1, False, 12, 16)]
+    del calls[:]
+    assert layer(budget=0).route(x, SimpleNamespace(mode="decode", slots=decode_slots)) == "top4"  # keep alone: each token's top 4
+    assert layer().route(x, SimpleNamespace(mode="prefill")) == "top10"
+    assert layer(keep=0, budget=0).route(x, SimpleNamespace(mode="decode", slots=decode_slots)) == "top10"
+    assert [c[:2] for c in calls] == [("topk", 4), ("topk", 10), ("topk", 10)] and calls[2][2] is decode_slots
 
 
 def test_bench_refuses_more_than_one_gpu():

@@ -211,3 +211,43 @@ def test_attach_model_takes_calibrated_copies(tmp_path):
     mdl, lins = model()
     report = w3.attach_model(mdl, log=lambda *_: None, codebook="uniform")
     assert report["matrices"] == 2 and mdl.w3_identity == "nearest:uniform" and all(lin.w3.tiled is not None for lin in lins)
+
+
+@pytest.mark.parametrize("m,mode,budget", [(6, "verify", 8), (5, "decode", 0), (1, "decode", 6)])
+def test_moe_layer_block_under_a_budget(m, mode, budget):
+    """Decode and verify forwards of a layer with a `keep`: the routing is `ops.route_budget`'s (or each token's top
+    `keep` alone), slots left over name no expert, and the block is the oracle's on those ids; prefill routes top-k."""
+    from hibana_amd.kernels import ops
+    from hibana_amd.model.flashnext_moe import MoeLayer
+    e, hidden, inter, topk, keep = 32, 256, 128, 4, 2
+    ex, per = random_experts(e, hidden, inter, True, 71)
+    shared, shared_per = random_experts(1, hidden, inter, True, 72)
+    get = oracle_expert_getter(per, True, inter)
+    g = torch.Generator().manual_seed(73 + m)
+    router = (torch.randn(e, hidden, generator=g) * 0.3).bfloat16()
+    gate_vec = torch.randn(1, hidden, generator=g) * 0.05
+    layer = MoeLayer(router.cuda(), gate_vec.cuda(), ex, topk, shared=shared, keep=keep, budget=budget, per_request=3)
+    x = torch.randn(m, hidden, generator=g).bfloat16()
+    steps = 2 if mode == "verify" else 1
+    slots = torch.ones(m // steps, dtype=torch.int32)
+    if m > 1:
+        slots[-1] = 0
+    ctx = SimpleNamespace(mode=mode, slots=slots.cuda(), seq_slots=slots.cuda(), verify_steps=steps)
+    ids, weights = layer.route(x.cuda(), ctx)
+    logits = torch.mm(x.cuda(), router.cuda().T)
+    if budget:
+        want_ids, want_w = ops.route_budget(logits, topk, layer.guarantee(m, steps), budget, slots.cuda(), steps, per_request=3, min_cap=16)
+        ref = layers.route_budget_ref(logits.cpu(), topk, layer.guarantee(m, steps), budget, slots, steps, per_request=3, min_cap=16)
+        assert torch.equal(ids.cpu(), ref[0])
+        torch.testing.assert_close(weights.cpu(), ref[1], rtol=1e-5, atol=0)
+    else:
+        want_ids, want_w = ops.route_topk(logits, keep)
+        assert ids.shape == (m, keep)
+    assert torch.equal(ids, want_ids) and torch.equal(weights, want_w)
+    got = layer(x.cuda(), ctx)
+    sh = oracle_expert_getter(shared_per, True, inter)(0)
+    want = layers.moe_layer_ref(x, ids.cpu().numpy(), weights.cpu(), get, True, shared=sh, gate_vec=gate_vec.reshape(-1), e_n=e)
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    served = layer.route(x.cuda(), SimpleNamespace(mode="prefill"))[0]
+    assert served.shape == (m, topk) and (served < e).all()
