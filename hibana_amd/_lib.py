@@ -67,6 +67,8 @@ SIGNATURES = {
     "hb_route_softmax_topk": (_I, [_P, _I, _I, _I, _P, _I, _I, _P, _P, _P]),
     "hb_route_budget_workspace_bytes": (_L, [_I]),
     "hb_route_budget": (_I, [_P, _I, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P, _L, _P, _P, _P]),
+    "hb_route_budget_sigmoid_workspace_bytes": (_L, [_I, _I]),
+    "hb_route_budget_sigmoid": (_I, [_P, _L, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P, _L, _P, _P, _P, _P]),
     "hb_route_sigmoid_topk": (_I, [_P, _L, _P, _I, _I, _I, _I, _P, _I, _I, _P, _P, _P, _P]),
     "hb_nvfp4_tiled_bytes": (_Z, [_L, _I]),
     "hb_nvfp4_repack": (_I, [_P, _P, _I, _L, _I, _P, _P]),

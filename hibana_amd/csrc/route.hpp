@@ -48,6 +48,7 @@ struct RouteParams {
   int32_t* ids;
   float* weights;
   uint16_t* lat;         // sigmoid: BF16 [m, latent], the row's latent columns
+  float* raw;            // or null: [m, k], the weights before renormalization (a padded row: those of the row it repeats)
 };
 
 // THROUGH: the logits were written by other workgroups of the same launch and are read past the compute die's L2.
@@ -149,6 +150,7 @@ __device__ __forceinline__ int route_row(const RouteParams& p, int r, int lane, 
   if (lane < p.k && write) {
     store_through(&p.ids[(int64_t)r * p.k + lane], id);  // the plan may read it in this very launch, from another workgroup
     p.weights[(int64_t)r * p.k + lane] = w;
+    if (p.raw) p.raw[(int64_t)r * p.k + lane] = mine;
   }
   if (weight) *weight = w;
   return id;

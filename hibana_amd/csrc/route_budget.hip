@@ -1,11 +1,15 @@
 // Budgeted expert selection: a cap on the distinct experts one decode or verify forward reads, chosen for all its rows
 // (route_budget, hibana/kernels/flashnext_fused.py:322-502 of the reference; the rule row by row:
-// tests/unit/test_moe_selection.py:19-58). Two launches, no atomics on floating-point data, no host synchronization:
-//   1. rank: a wavefront a row finds the row's 20 largest BF16 logits (an exact tie to the lower expert; -0 equals +0)
-//      and their softmax probabilities over all experts;
-//   2. pick: one workgroup sums each expert's probability within the real rows' top k, takes every real row's top
-//      `keep` and then the best-scoring other experts up to the cap, and gives each real row its candidates in that
-//      set in rank order, up to k, at probabilities renormalized over them.
+// tests/unit/test_moe_selection.py:19-58; the latent MoE's form with its own ranking, hibana/model/nemotron/moe.py:
+// 124-313). Two launches, no atomics on floating-point data, no host synchronization:
+//   1. rank: a wavefront a row finds the row's candidates, best first, with the weight each would carry: the 20 largest
+//      BF16 logits (an exact tie to the lower expert; -0 equals +0) and their softmax probabilities over all experts,
+//      or the top k of sigmoid + bias with the plain sigmoids (the routing kernel itself, which also writes each
+//      candidate's share of the row's top k: its score contribution);
+//   2. pick: one workgroup sums each expert's contributions over the real rows' top k, takes every real row's top
+//      `keep` (its top `fallback` when those alone exceed the cap) and then the best-scoring other experts up to the
+//      cap, and gives each real row its candidates in that set in rank order, up to k, at weights renormalized over
+//      them.
 #include "route.hpp"
 #include "stream_common.hpp"
 
@@ -16,11 +20,15 @@ constexpr int BUDGET_THREADS = 1024, BUDGET_WAVES = BUDGET_THREADS / 64;
 constexpr int BUDGET_BATCH = 8;   // rows whose candidates a wavefront requests at once
 
 struct BudgetParams {
-  const uint16_t* logits;  // BF16 [r, e]
+  const uint16_t* logits;  // softmax form: BF16 [r, e]
   const int32_t* slots;    // row t is real iff slots[t / steps] != 0 (null: every row)
   int r, e, k, keep, budget, per_request, min_cap, steps, repeat;
-  int32_t* cand;           // [r, 20]: the row's candidates, largest logit first
-  float* prob;             // [r, 20]: their softmax probabilities
+  int cands;               // candidates a row (20, or k in the sigmoid form), at most 32
+  int fallback;            // or 0: the guarantee when the rows' top `keep` alone exceed the cap
+  float eps;               // added to the sum a row's weights are divided by
+  int32_t* cand;           // [r, cands]: the row's candidates, best first
+  float* prob;             // [r, cands]: the weight each carries before renormalization
+  const float* share;      // [r, cands]: what a candidate within the row's top k adds to its expert's score
   int32_t* ids;            // [r, k]
   float* weights;          // [r, k]
 };
@@ -84,14 +92,16 @@ __global__ __launch_bounds__(64) void route_rank_kernel(BudgetParams q) {
 // One workgroup. Scores: wavefront w adds the rows t = w (mod copies) into a copy of its own, in row order, and the
 // copies are added in wavefront order (the same bits on every run). The set: wavefront 0 holds every expert's key in
 // registers (column j * 64 + lane, as above) and finds the need-th largest by bisection on its bits, each step one
-// ballot a register. The rows: two a wavefront at a time, one in each half.
-template <int PER>
+// ballot a register. The rows: two a wavefront at a time, one in each half. IN_ORDER: a row's weights are divided by
+// the sum of the taken ones added in rank order, as the routing kernel adds a row's top k (a row that keeps all of its
+// top k gets that kernel's weights bit for bit); otherwise by a butterfly sum.
+template <int PER, bool IN_ORDER>
 __global__ __launch_bounds__(BUDGET_THREADS) void route_pick_kernel(BudgetParams q, int copies_n) {
   extern __shared__ float copies[];  // [copies_n][e]
   __shared__ uint32_t keys[BUDGET_THREADS];
-  __shared__ uint8_t core[BUDGET_THREADS], chosen[BUDGET_THREADS];
+  __shared__ uint8_t core[BUDGET_THREADS], core_fallback[BUDGET_THREADS], chosen[BUDGET_THREADS];
   __shared__ int real_requests;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, e = q.e, r = q.r;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, e = q.e, r = q.r, cands = q.cands;
   // the candidates of the rows this wavefront will write (half a wavefront a row), requested before anything else
   const int half = lane >> 5, hl = lane & 31;
   constexpr int PAIRS = BUDGET_BATCH / 2;
@@ -101,15 +111,16 @@ __global__ __launch_bounds__(BUDGET_THREADS) void route_pick_kernel(BudgetParams
 #pragma unroll
     for (int b = 0; b < PAIRS; b++) {
       const int t = t0 + 2 * BUDGET_WAVES * b + half;
-      const bool live = t < r && hl < BUDGET_CANDIDATES;
-      cd[b] = live ? q.cand[(int64_t)t * BUDGET_CANDIDATES + hl] : 0;
-      pv[b] = live ? q.prob[(int64_t)t * BUDGET_CANDIDATES + hl] : 0.f;
+      const bool live = t < r && hl < cands;
+      cd[b] = live ? q.cand[(int64_t)t * cands + hl] : 0;
+      pv[b] = live ? q.prob[(int64_t)t * cands + hl] : 0.f;
     }
   };
   request(2 * wave);
   const int first = q.repeat ? q.cand[0] : e;  // a padded row's slots under `repeat`: row 0's first candidate
   for (int i = tid; i < copies_n * e; i += BUDGET_THREADS) copies[i] = 0.f;
   core[tid] = 0;
+  core_fallback[tid] = 0;
   if (tid == 0) real_requests = 0;
   __syncthreads();
   if (q.per_request > 0 && q.slots) {  // padded requests do not count towards the cap (an integer sum: any order)
@@ -118,7 +129,7 @@ __global__ __launch_bounds__(BUDGET_THREADS) void route_pick_kernel(BudgetParams
     if (mine) atomicAdd(&real_requests, mine);
   }
   auto real_row = [&](int t) { return t < r && (!q.slots || q.slots[t / q.steps] != 0); };
-  // scores: an expert's probability within the real rows' top k; core: the real rows' top `keep`
+  // scores: what the real rows' top k add to their experts; core: the real rows' top `keep` (and top `fallback`)
   if (wave < copies_n) {
     float* mine = copies + wave * e;
     for (int t0 = wave; t0 < r; t0 += copies_n * BUDGET_BATCH) {
@@ -128,14 +139,15 @@ __global__ __launch_bounds__(BUDGET_THREADS) void route_pick_kernel(BudgetParams
 #pragma unroll
       for (int b = 0; b < BUDGET_BATCH; b++) {
         const int t = t0 + b * copies_n;
-        real[b] = real_row(t) && lane < BUDGET_CANDIDATES;
-        sc[b] = real[b] ? q.cand[(int64_t)t * BUDGET_CANDIDATES + lane] : 0;
-        sp[b] = real[b] ? q.prob[(int64_t)t * BUDGET_CANDIDATES + lane] : 0.f;
+        real[b] = real_row(t) && lane < cands;
+        sc[b] = real[b] ? q.cand[(int64_t)t * cands + lane] : 0;
+        sp[b] = real[b] ? q.share[(int64_t)t * cands + lane] : 0.f;
       }
 #pragma unroll
       for (int b = 0; b < BUDGET_BATCH; b++) {  // a row's candidates are distinct experts: no two lanes meet
         if (real[b] && lane < q.k) mine[sc[b]] += sp[b];
         if (real[b] && lane < q.keep) core[sc[b]] = 1;
+        if (real[b] && lane < q.fallback) core_fallback[sc[b]] = 1;
       }
     }
   }
@@ -144,20 +156,34 @@ __global__ __launch_bounds__(BUDGET_THREADS) void route_pick_kernel(BudgetParams
     float score = 0.f;
     if (tid < e)
       for (int w = 0; w < copies_n; w++) score += copies[w * e + tid];
-    keys[tid] = !core[tid] && tid < e && score > 0.f ? __float_as_uint(score) : 0u;  // positive floats order as their bits
+    keys[tid] = tid < e && score > 0.f ? __float_as_uint(score) : 0u;  // positive floats order as their bits
   }
   __syncthreads();
   if (wave == 0) {
-    uint32_t kk[PER];  // columns past e hold key 0 and no core flag
-    int in_core = 0, contenders = 0;
-#pragma unroll
-    for (int j = 0; j < PER; j++) {
-      kk[j] = keys[j * 64 + lane];
-      in_core += __popcll(__ballot(core[j * 64 + lane] != 0));
-      contenders += __popcll(__ballot(kk[j] != 0u));
-    }
     int cap = q.budget;
     if (q.per_request > 0) cap = min(cap, max(q.min_cap, q.per_request * (q.slots ? real_requests : r / q.steps)));
+    bool guaranteed[PER];  // columns past e hold no flag and key 0
+    int in_core = 0;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      guaranteed[j] = core[j * 64 + lane] != 0;
+      in_core += __popcll(__ballot(guaranteed[j]));
+    }
+    if (q.fallback > 0 && cap > 0 && in_core > cap) {  // the floors overflow the cap: each row's top `fallback` only
+      in_core = 0;
+#pragma unroll
+      for (int j = 0; j < PER; j++) {
+        guaranteed[j] = core_fallback[j * 64 + lane] != 0;
+        in_core += __popcll(__ballot(guaranteed[j]));
+      }
+    }
+    uint32_t kk[PER];
+    int contenders = 0;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      kk[j] = guaranteed[j] ? 0u : keys[j * 64 + lane];
+      contenders += __popcll(__ballot(kk[j] != 0u));
+    }
     const int need = cap - in_core;
     // the set takes the keys above `at` and, of those equal to it, the `quota` lowest experts
     uint32_t at = 0xffffffffu;
@@ -188,7 +214,7 @@ __global__ __launch_bounds__(BUDGET_THREADS) void route_pick_kernel(BudgetParams
       const bool equal = kk[j] == at && kk[j] != 0u;
       const uint64_t mask = __ballot(equal);
       const int before = seen + __popcll(mask & ((1ull << lane) - 1ull));
-      chosen[j * 64 + lane] = core[j * 64 + lane] != 0 || kk[j] > at || (equal && before < quota);
+      chosen[j * 64 + lane] = guaranteed[j] || kk[j] > at || (equal && before < quota);
       seen += __popcll(mask);
     }
   }
@@ -201,13 +227,26 @@ __global__ __launch_bounds__(BUDGET_THREADS) void route_pick_kernel(BudgetParams
       const int t = t0 + 2 * BUDGET_WAVES * b + half;
       if (t - half >= r) break;
       const bool real = real_row(t);
-      const bool pull = t < r && hl < BUDGET_CANDIDATES && chosen[cd[b]] != 0;
+      const bool pull = t < r && hl < cands && chosen[cd[b]] != 0;
       const uint32_t mask = (uint32_t)(__ballot(pull) >> (32 * half));
       const int slot = __popc(mask & ((1u << hl) - 1u));
       const bool mine = pull && slot < q.k && real;
       float total = mine ? pv[b] : 0.f;
+      if (IN_ORDER) {
+        const float part = total;
+        float lower = 0.f, upper = 0.f;
 #pragma unroll
-      for (int d = 16; d >= 1; d >>= 1) total += __shfl_xor(total, d);  // stays within the half
+        for (int i = 0; i < 32; i++)
+          if (i < cands) {
+            lower += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, part), i));
+            upper += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, part), i + 32));
+          }
+        total = half ? upper : lower;
+      } else {
+#pragma unroll
+        for (int d = 16; d >= 1; d >>= 1) total += __shfl_xor(total, d);  // stays within the half
+      }
+      total += q.eps;
       const int used = real ? min(__popc(mask), q.k) : 0;
       const int top_a = __builtin_amdgcn_readlane(cd[b], 0), top_b = __builtin_amdgcn_readlane(cd[b], 32);
       if (mine) {
@@ -219,6 +258,29 @@ __global__ __launch_bounds__(BUDGET_THREADS) void route_pick_kernel(BudgetParams
         q.weights[(int64_t)t * q.k + hl] = 0.f;
       }
     }
+  }
+}
+
+// The sigmoid form's rank launch: the routing kernel on k candidates, its ids as the candidates, its renormalized
+// weights as their shares, the plain sigmoids beside them; it also rounds the row's latent columns.
+template <int PER>
+__global__ __launch_bounds__(64) void route_rank_sigmoid_kernel(RouteParams p) {
+  route_row<true, PER>(p, blockIdx.x, threadIdx.x);
+}
+
+static void launch_pick(const BudgetParams& q, bool in_order, hipStream_t s) {
+  const int copies_n = q.e <= 512 ? BUDGET_WAVES : BUDGET_WAVES / 2;  // 32 KB of LDS either way
+  const size_t lds = (size_t)copies_n * q.e * sizeof(float);
+  if (q.e <= 512) {
+    if (in_order) {
+      HB_LAUNCH((route_pick_kernel<8, true>), dim3(1), dim3(BUDGET_THREADS), lds, s, q, copies_n);
+    } else {
+      HB_LAUNCH((route_pick_kernel<8, false>), dim3(1), dim3(BUDGET_THREADS), lds, s, q, copies_n);
+    }
+  } else if (in_order) {
+    HB_LAUNCH((route_pick_kernel<16, true>), dim3(1), dim3(BUDGET_THREADS), lds, s, q, copies_n);
+  } else {
+    HB_LAUNCH((route_pick_kernel<16, false>), dim3(1), dim3(BUDGET_THREADS), lds, s, q, copies_n);
   }
 }
 
@@ -241,8 +303,10 @@ extern "C" int hb_route_budget(const void* logits, int r, int e, int k, int keep
   q.logits = static_cast<const uint16_t*>(logits);
   q.slots = slots;
   q.r = r, q.e = e, q.k = k, q.keep = keep, q.budget = budget, q.per_request = per_request, q.min_cap = min_cap, q.steps = steps, q.repeat = repeat;
+  q.cands = BUDGET_CANDIDATES;
   q.cand = static_cast<int32_t*>(workspace);
   q.prob = reinterpret_cast<float*>(q.cand + (int64_t)r * BUDGET_CANDIDATES);
+  q.share = q.prob;  // a candidate's softmax probability is also what it adds to its expert's score
   q.ids = ids, q.weights = weights;
   hipStream_t s = as_stream(stream);
   if (e <= 512) {
@@ -250,11 +314,42 @@ extern "C" int hb_route_budget(const void* logits, int r, int e, int k, int keep
   } else {
     HB_LAUNCH((route_rank_kernel<16>), dim3((unsigned)r), dim3(64), 0, s, q);
   }
-  const int copies_n = e <= 512 ? BUDGET_WAVES : BUDGET_WAVES / 2;  // 32 KB of LDS either way
-  if (e <= 512) {
-    HB_LAUNCH(route_pick_kernel<8>, dim3(1), dim3(BUDGET_THREADS), (size_t)copies_n * e * sizeof(float), s, q, copies_n);
+  launch_pick(q, false, s);
+  return launch_status();
+}
+
+extern "C" int64_t hb_route_budget_sigmoid_workspace_bytes(int r, int k) { return r > 0 && k > 0 ? (int64_t)r * k * 12 : 0; }
+
+extern "C" int hb_route_budget_sigmoid(const float* fused, int64_t stride, const float* bias, int r, int e, int k, int latent, int keep, int budget,
+                                       const int32_t* slots, int steps, int repeat, int per_request, int fallback, void* workspace,
+                                       int64_t workspace_bytes, int32_t* ids, float* weights, void* lat, void* stream) {
+  if (!fused || !bias || !workspace || !ids || !weights || (latent > 0 && !lat)) return HB_ENULL;
+  if (r <= 0 || e <= 0 || e > BUDGET_THREADS || k <= 0 || k > 32 || k > e || latent < 0 || stride < (int64_t)e + latent || keep < 0 || keep > k ||
+      fallback < 0 || fallback > keep || budget < 0 || steps <= 0 || r % steps || per_request < 0)
+    return HB_EINVAL;
+  if (!aligned(fused, 4) || !aligned(bias, 4) || !aligned(workspace, 4) || !aligned(slots, 4) || !aligned(ids, 4) || !aligned(weights, 4) ||
+      !aligned(lat, 2))
+    return HB_EINVAL;
+  if (workspace_bytes < hb_route_budget_sigmoid_workspace_bytes(r, k)) return HB_EWORKSPACE;
+  BudgetParams q{};
+  q.slots = slots;
+  q.r = r, q.e = e, q.k = k, q.keep = keep, q.budget = budget, q.per_request = per_request, q.min_cap = 0, q.steps = steps, q.repeat = repeat;
+  q.cands = k, q.fallback = fallback, q.eps = 1e-20f;
+  q.cand = static_cast<int32_t*>(workspace);
+  q.prob = reinterpret_cast<float*>(q.cand + (int64_t)r * k);
+  float* share = q.prob + (int64_t)r * k;
+  q.share = share;
+  q.ids = ids, q.weights = weights;
+  RouteParams p{};  // every row ranks as a real one: which rows count is the pick launch's business
+  p.logits = fused, p.stride = stride, p.bias = bias;
+  p.steps = 1, p.e = e, p.k = k, p.per = (e + 63) / 64, p.latent = latent, p.pad_id = e, p.sigmoid = 1;
+  p.ids = q.cand, p.weights = share, p.raw = q.prob, p.lat = static_cast<uint16_t*>(lat);
+  hipStream_t s = as_stream(stream);
+  if (p.per <= 8) {
+    HB_LAUNCH((route_rank_sigmoid_kernel<8>), dim3((unsigned)r), dim3(64), 0, s, p);
   } else {
-    HB_LAUNCH(route_pick_kernel<16>, dim3(1), dim3(BUDGET_THREADS), (size_t)copies_n * e * sizeof(float), s, q, copies_n);
+    HB_LAUNCH((route_rank_sigmoid_kernel<16>), dim3((unsigned)r), dim3(64), 0, s, p);
   }
+  launch_pick(q, true, s);
   return launch_status();
 }

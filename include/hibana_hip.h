@@ -288,6 +288,24 @@ int hb_route_budget(const void* logits, int r, int e, int k, int keep, int budge
                     int repeat, int per_request, int min_cap, void* workspace, int64_t workspace_bytes, int32_t* ids,
                     float* weights, void* stream);
 
+/* The latent MoE's budgeted top-k: hb_route_budget's selection on hb_route_sigmoid_topk's ranking. fused FP32
+ * [r, stride] (e router logits, then `latent` columns), bias [e] -> ids int32 [r, k], weights FP32 [r, k], lat BF16
+ * [r, latent]; k <= 32, e <= 1024. A row's candidates are its top k by sigmoid + bias (equal scores to the lower
+ * expert); a candidate adds its renormalized weight s / (sum of the row's k sigmoids) to its expert's score; the set
+ * is every real row's top `keep`, then the best-scoring other experts up to the cap (`budget`, or with per_request > 0,
+ * min(budget, per_request x the real requests); a budget of 0: the guaranteed experts alone). `fallback` (0: none;
+ * at most keep): when the rows' top `keep` alone exceed a cap above 0, each real row is guaranteed only its top
+ * `fallback`. A real row takes its candidates in the set in rank order; its weights are the plain sigmoids over
+ * (their sum in rank order + 1e-20): a row that keeps all k gets hb_route_sigmoid_topk's weights bit for bit. Slots left
+ * over (all of a padded row's) hold the row's first candidate (a padded row: row 0's) at weight 0, or id e when
+ * repeat == 0. Two launches; `workspace` (4-byte aligned) of hb_route_budget_sigmoid_workspace_bytes(r, k).
+ * ref: route_budget, hibana/model/nemotron/moe.py:124-313; caller NemotronMoe.route / fallback, :453-474. */
+int64_t hb_route_budget_sigmoid_workspace_bytes(int r, int k);
+int hb_route_budget_sigmoid(const float* fused, int64_t stride, const float* bias, int r, int e, int k, int latent,
+                            int keep, int budget, const int32_t* slots, int steps, int repeat, int per_request,
+                            int fallback, void* workspace, int64_t workspace_bytes, int32_t* ids, float* weights,
+                            void* lat, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * NVFP4 format: E2M1 codes two per byte (element 2i in the low nibble), one E4M3 scale per 16 weights, one FP32
  * global scale. ref: hibana/weights/modelopt.py:57-81,150-156.

@@ -25,6 +25,9 @@ points of the reference kept.
                          in row order of the FP32 softmax within the real rows' top k, the set = core + best-scoring
                          others (score > 0, equal scores to the lower expert) up to the cap, rows take their
                          candidates in the set in rank order
+  route_budget_sigmoid_ref  hibana/model/nemotron/moe.py:124-313: the same selection (`budget_rule`) on the top k by
+                         sigmoid + bias, plain-sigmoid weights over (sum + 1e-20), shares renormalized over the
+                         row's k, a `fallback` guarantee when the rows' top keep exceed the cap
   silu_mul               hibana/kernels/flashnext_fused.py:624-639: bf16(silu(gate) * up) from the FP32 product
   latent_moe_ref         tests/nemotron_reference.py:568-593 (ReLU^2 latent experts, BF16 linears, FP32 accumulate)
   silu_and_mul           hibana/kernels/ops.py:86-92
@@ -47,6 +50,8 @@ groups that are already E4M3 multiples of their scale coming back unchanged. rou
 whose set and rows follow from the rule by inspection, a cap no smaller than the rows' top-k union == a stable
 descending sort's top k with the renormalized softmax of torch, padded requests == the call on the real rows alone, and
 the invariants the reference's own unit test states (tests/unit/test_moe_selection.py:66-106).
+route_budget_sigmoid_ref: a hand-worked call (bias choosing, plain sigmoids weighing, the fallback guarantee), a cap
+that holds every row's top k == route_sigmoid_topk, and the invariants of tests/gpu/test_bolt_kernels.py:188-216.
 """
 from __future__ import annotations
 
@@ -232,10 +237,46 @@ def route_sigmoid_topk(logits: torch.Tensor, bias: torch.Tensor, k: int, scaling
 ROUTE_CANDIDATES = 20
 
 
+def budget_rule(cand, prob, share, e: int, k: int, keep: int, cap: int, real, repeat: bool = False, fallback: int = 0, eps: float = 0.0,
+                given=None):
+    """The selection from the rows' candidate lists (best first): prob[t][c] the weight candidate c of row t carries
+    before renormalization, share[t][c] what it adds to its expert's score when within the row's top k. The set: the
+    real rows' top `keep` (their top `fallback` when those exceed a cap above 0), then the best-scoring other experts
+    (score > 0, equal scores to the lower expert) up to `cap`; a real row takes its candidates in the set, in rank
+    order, up to k, at prob / (their sum in rank order + eps). `given`: a set to take instead of the selected one.
+    -> (ids int32 [R, k], weights FP32 [R, k], the set, its guaranteed part, the FP32 scores [E])
+    (hibana/kernels/flashnext_fused.py:378-456; hibana/model/nemotron/moe.py:166-263)."""
+    r = len(cand)
+    core = {x for c, live in zip(cand, real) if live for x in c[:keep]}
+    if fallback > 0 and cap > 0 and len(core) > cap:
+        core = {x for c, live in zip(cand, real) if live for x in c[:fallback]}
+    score = np.zeros(e, dtype=np.float32)
+    for t, c in enumerate(cand):
+        if real[t]:
+            for j, x in enumerate(c[:k]):
+                score[x] = np.float32(score[x] + np.float32(share[t][j]))
+    rest = sorted((x for x in range(e) if x not in core and score[x] > 0), key=lambda x: (-float(score[x]), x))
+    chosen = core | set(rest[:max(0, cap - len(core))]) if given is None else set(given)
+    ids = np.full((r, k), e, dtype=np.int32)
+    w = np.zeros((r, k), dtype=np.float32)
+    for t, c in enumerate(cand):
+        row = [j for j, x in enumerate(c) if x in chosen][:k] if real[t] else []
+        if row:
+            total = np.float32(0.0)
+            for j in row:
+                total = np.float32(total + np.float32(prob[t][j]))
+            total = np.float32(total + np.float32(eps))
+            ids[t, :len(row)] = [c[j] for j in row]
+            w[t, :len(row)] = [np.float32(prob[t][j]) / total for j in row]
+        if repeat:
+            ids[t, len(row):] = c[0] if real[t] else cand[0][0]
+    return torch.from_numpy(ids), torch.from_numpy(w), chosen, core, score
+
+
 def route_budget_ref(logits: torch.Tensor, k: int, keep: int, budget: int, slots=None, steps: int = 1, repeat: bool = False,
                      per_request: int = 0, min_cap: int = 0, given=None):
-    """-> (ids int32 [R, k], weights FP32 [R, k], the set, its guaranteed part, the FP32 scores [E]). `given`: the rows
-    take their experts from this set instead of the selected one (the second half of the rule alone)."""
+    """Flash-Next's form: candidates = a row's 20 largest logits, weights and shares = the FP32 softmax over E; the
+    cap is `budget`, or with `per_request`, min(budget, max(min_cap, per_request x the real requests))."""
     lg = logits.float().cpu().numpy().astype(np.float32)
     r, e = lg.shape
     real = [slots is None or int(slots[t // steps]) != 0 for t in range(r)]
@@ -246,25 +287,34 @@ def route_budget_ref(logits: torch.Tensor, k: int, keep: int, budget: int, slots
     p = ex / ex.sum(-1, keepdims=True, dtype=np.float32)
     # a stable ascending sort of the negated logits: the largest first, equal logits (both zeros among them) in id order
     cand = [np.argsort(-(row + np.float32(0.0)), kind="stable")[:ROUTE_CANDIDATES].tolist() for row in lg]
-    core = {x for c, live in zip(cand, real) if live for x in c[:keep]}
-    score = np.zeros(e, dtype=np.float32)
-    for t, c in enumerate(cand):
-        if real[t]:
-            for x in c[:k]:
-                score[x] = np.float32(score[x] + p[t, x])
-    rest = sorted((x for x in range(e) if x not in core and score[x] > 0), key=lambda x: (-float(score[x]), x))
-    chosen = core | set(rest[:max(0, cap - len(core))]) if given is None else set(given)
-    ids = np.full((r, k), e, dtype=np.int32)
-    w = np.zeros((r, k), dtype=np.float32)
-    for t, c in enumerate(cand):
-        row = [x for x in c if x in chosen][:k] if real[t] else []
-        if row:
-            taken = p[t, row]
-            ids[t, :len(row)] = row
-            w[t, :len(row)] = taken / taken.sum(dtype=np.float32)
-        if repeat:
-            ids[t, len(row):] = c[0] if real[t] else cand[0][0]
-    return torch.from_numpy(ids), torch.from_numpy(w), chosen, core, score
+    prob = [p[t, c] for t, c in enumerate(cand)]
+    return budget_rule(cand, prob, prob, e, k, keep, cap, real, repeat, given=given)
+
+
+def route_budget_sigmoid_ref(fused: torch.Tensor, bias: torch.Tensor, k: int, latent: int, keep: int, budget: int, slots=None, steps: int = 1,
+                             per_request: int = 0, repeat: bool = True, fallback: int = 0, cand=None, given=None):
+    """The latent MoE's form (hibana/model/nemotron/moe.py:124-313): candidates = a row's top k by sigmoid + bias (equal
+    scores to the lower expert; `cand`: lists to take instead), weights = the plain sigmoids over (their sum + 1e-20),
+    shares = the sigmoids over the sum of the row's k; the cap is `budget`, or with `per_request`,
+    min(budget, per_request x the real requests)."""
+    e = fused.shape[1] - latent
+    r = fused.shape[0]
+    real = [slots is None or int(slots[t // steps]) != 0 for t in range(r)]
+    cap = budget
+    if per_request > 0:
+        cap = min(budget, per_request * sum(1 for t in range(0, r, steps) if real[t]))
+    s = torch.sigmoid(fused[:, :e].float().cpu())
+    if cand is None:
+        cand = torch.sort(s + bias.float().cpu(), dim=-1, descending=True, stable=True).indices[:, :k].tolist()
+    prob = [s[t, c].numpy() for t, c in enumerate(cand)]
+    share = []
+    for row in prob:
+        total = np.float32(0.0)
+        for v in row:
+            total = np.float32(total + v)
+        share.append(row / np.float32(total + np.float32(1e-20)))
+    out = budget_rule(cand, prob, share, e, k, keep, cap, real, repeat, fallback, 1e-20, given)
+    return out + (fused[:, e:].cpu().bfloat16(),)
 
 
 def silu_mul(gate_up: torch.Tensor, pairs: int = 0) -> torch.Tensor:

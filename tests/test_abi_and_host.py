@@ -66,6 +66,11 @@ def test_validation_without_a_gpu():
     for r, e, k, keep, steps in [(12, 19, 10, 4, 1), (12, 1025, 10, 4, 1), (12, 512, 21, 4, 1), (12, 512, 10, 21, 1), (12, 512, 10, 4, 5)]:
         assert lib.hb_route_budget(256, r, e, k, keep, 64, None, steps, 0, 0, 0, 256, 1920, 256, 256, None) == _lib.HB_EINVAL
     assert lib.hb_route_budget(256, 12, 512, 10, 4, 64, None, 1, 0, 0, 0, 256, 1919, 256, 256, None) == _lib.HB_EWORKSPACE
+    assert lib.hb_route_budget_sigmoid_workspace_bytes(12, 22) == 12 * 22 * 12
+    assert lib.hb_route_budget_sigmoid(None, 640, 256, 12, 512, 22, 128, 6, 64, None, 1, 1, 0, 0, 256, 3168, 256, 256, 256, None) == _lib.HB_ENULL
+    for e, k, keep, fallback, stride in [(512, 33, 6, 0, 640), (1025, 22, 6, 0, 1200), (512, 22, 23, 0, 640), (512, 22, 6, 7, 640), (512, 22, 6, 0, 639)]:
+        assert lib.hb_route_budget_sigmoid(256, stride, 256, 12, e, k, 128, keep, 64, None, 1, 1, 0, fallback, 256, 1 << 20, 256, 256, 256, None) == _lib.HB_EINVAL
+    assert lib.hb_route_budget_sigmoid(256, 640, 256, 12, 512, 22, 128, 6, 64, None, 1, 1, 0, 0, 256, 3167, 256, 256, 256, None) == _lib.HB_EWORKSPACE
     # the small latent block: shapes and pointers are checked before anything is launched
     nv = _lib.HbNvfp4Experts(256, 256, 256, 256, 8, 0, 256, 128, 256, 0)
     lw = _lib.HbLatentWeights(256, 256, 256, C.pointer(nv), 256, 256, 1.0, 1.0, 8, 256, 512, 640)
@@ -177,6 +182,32 @@ def test_budgeted_selection_settings_and_which_forwards_take_it(monkeypatch):
     assert layer().route(x, SimpleNamespace(mode="prefill")) == "top10"
     assert layer(keep=0, budget=0).route(x, SimpleNamespace(mode="decode", slots=decode_slots)) == "top10"
     assert [c[:2] for c in calls] == [("topk", 4), ("topk", 10), ("topk", 10)] and calls[2][2] is decode_slots
+
+
+def test_latent_block_budget_settings_and_fallback():
+    """`NemotronMoe`'s keep / budget / per_request and the guarantee it falls back to (cap / rows within
+    [SHARE_MIN, keep), hibana/model/nemotron/moe.py:464-474), worked out by hand from the rule."""
+    from types import SimpleNamespace
+
+    from hibana_amd.model.nemotron_moe import NemotronMoe
+
+    def block(keep, budget, per_request, topk=22):
+        it = NemotronMoe.__new__(NemotronMoe)
+        it.topk = topk
+        it.keep = keep if keep < topk else 0
+        it.budget = budget if it.keep else 0
+        it.per_request = per_request
+        return it
+
+    assert [block(k, 64, 0).keep for k in (0, 6, 21, 22, 30)] == [0, 6, 21, 0, 0] and block(22, 64, 0).budget == 0
+    b = block(12, 64, 12)
+    assert b.fallback(4, 1) == 0     # cap min(64, 48): 48 // 4 = 12, the floor itself
+    assert b.fallback(16, 1) == 8    # cap 64: 64 // 16 = 4, raised to SHARE_MIN
+    assert b.fallback(6, 1) == 10    # cap 64: 64 // 6 = 10
+    assert b.fallback(16, 8) == 8    # two requests: cap 24, 24 // 16 = 1, raised to SHARE_MIN
+    assert block(12, 0, 12).fallback(16, 1) == 0 and block(6, 64, 0).fallback(16, 1) == 0  # no cap; SHARE_MIN is the floor itself
+    assert b.selects(SimpleNamespace(mode="decode")) and b.selects(SimpleNamespace(mode="verify"))
+    assert not b.selects(SimpleNamespace(mode="prefill")) and not b.selects(None) and not block(0, 64, 12).selects(SimpleNamespace(mode="decode"))
 
 
 def test_bench_refuses_more_than_one_gpu():

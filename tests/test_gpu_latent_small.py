@@ -224,3 +224,44 @@ def test_small_block_on_an_expert_range(m):
         total += small.block(x, ws, ids, w, rank.small_weights()).float()
     mx, nr = errors(total.bfloat16(), want.bfloat16())
     assert mx < MAX_REL and nr < 2 * NORM_REL, (mx, nr)
+
+
+@pytest.mark.parametrize("m,mode,w3", [(6, "verify", False), (4, "decode", False), (6, "verify", True), (40, "verify", False)])
+def test_block_under_a_budget(m, mode, w3):
+    """Decode and verify forwards of a block with a `keep`: the router's launch leaves the routing to the budgeted
+    selection, the block plans from its ids (hibana/model/nemotron/moe.py:484-502); past sixteen rows the same routing
+    feeds the large-call path. The oracle follows the selection's own ids."""
+    from hibana_amd.kernels import nemotron_moe as small
+    from hibana_amd.model import nemotron_moe
+    e, hidden, latent, inter, topk, sh_inter = GEOMETRIES["many"] if not w3 else (16, 512, 256, 128, 4, 640)
+    block, ref = _block(e, hidden, latent, inter, topk, sh_inter, 90, w3=w3)
+    block.keep, block.budget, block.per_request = 2, 12, 5
+    steps = 1 if mode == "decode" else 2
+    slots = torch.ones(m // steps, dtype=torch.int32)
+    slots[-1] = 0
+    ctx = SimpleNamespace(mode=mode, slots=slots.cuda(), seq_slots=slots.cuda(), verify_steps=steps)
+    x = torch.randn(m, hidden, generator=torch.Generator().manual_seed(m)).bfloat16()
+    got = block(x.cuda(), ctx)
+    if m > block.SMALL_ROWS:
+        fused = torch.mm(x.cuda(), block.gate_fc1.T, out_dtype=torch.float32)
+    else:
+        fused = small.router(x.cuda(), block.small_weights(), None, topk, route=False)[0]
+    ids, w, lat = block.route(fused, slots.cuda(), steps, select=True)
+    want_ids, want_w, _ = nemotron_moe.route_budget(fused, block.bias, topk, latent, 2, 12, slots.cuda(), steps, per_request=5, repeat=not w3,
+                                                    fallback=block.fallback(m, steps))
+    assert torch.equal(ids, want_ids) and torch.equal(w, want_w)
+    real = m - steps
+    used = {int(v) for t in range(real) for v, wt in zip(ids[t].tolist(), w[t].tolist()) if wt > 0}
+    assert len(used) <= max(min(12, 5 * (m // steps - 1)), len({int(v) for v in ids[:real, :2].reshape(-1).tolist()}))
+    assert not w[real:].any()
+    if w3:
+        from hibana_amd.kernels import w3_moe
+        y = w3_moe.w3_moe(block.w3, lat, ids, w).cpu().double() @ ref.fc2.double().T
+        h = layers.nvfp4_dense_ref(x, ref.su[0], ref.su[1], relu2=True)
+        want = (y + layers.nvfp4_dense_ref(h, ref.sd[0], ref.sd[1]).double()).float().bfloat16()
+    else:
+        want = _oracle(ref, x, ids, w)
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < 2 * NORM_REL, (mx, nr)
+    plain = block(x.cuda(), SimpleNamespace(mode="prefill"))  # prefill routes every token's top k
+    assert not torch.equal(plain[:real], got[:real])

@@ -158,3 +158,117 @@ def test_silu_mul_rounds_once():
         # the FP32 sigmoid of the two sides may differ in its last place: a BF16 result may then sit one step apart
         assert (got != want).float().mean() < 0.005
         torch.testing.assert_close(got.float(), want.float(), rtol=2.0 ** -7, atol=1e-30)
+
+
+# ------------------------------------------------------------------ the latent MoE's form (sigmoid + bias ranking)
+
+def check_sigmoid(fused, bias, k, latent, keep, cap, slots=None, steps=1, per_request=0, repeat=True, fallback=0):
+    """The device ranks a row as its plain routing does (checked against the oracle on its own), so the candidates are
+    the device's own top k: a last-bit difference between the two sides' sigmoids cannot reorder them."""
+    from hibana_amd.model import nemotron_moe
+    e = fused.shape[1] - latent
+    dev = lambda t: None if t is None else t.cuda()  # noqa: E731
+    ids, w, lat = nemotron_moe.route_budget(dev(fused), dev(bias), k, latent, keep, cap, dev(slots), steps, per_request, repeat, fallback)
+    ids, w = ids.cpu(), w.cpu()
+    cand = nemotron_moe.route_topk(dev(fused), dev(bias), k, latent)[0].cpu().tolist()
+    real = [slots is None or int(slots[t // steps]) != 0 for t in range(fused.shape[0])]
+    _, _, want, core, score, want_lat = layers.route_budget_sigmoid_ref(fused, bias, k, latent, keep, cap, slots, steps, per_request, repeat, fallback, cand=cand)
+    if per_request:
+        cap = min(cap, per_request * sum(1 for t in range(0, len(real), steps) if real[t]))
+    got = {int(x) for t in range(len(real)) if real[t] for x, v in zip(ids[t].tolist(), w[t].tolist()) if v > 0}
+    assert core <= got and len(got) <= max(cap, len(core))
+    differ = (got - core) ^ (want - core)
+    if differ:
+        edge = [float(score[x]) for x in (got | want) - core]
+        assert all(abs(float(score[x]) - min(edge)) <= 1e-5 * max(1.0, max(edge)) for x in differ), differ
+    rids, rw, _, _, _, _ = layers.route_budget_sigmoid_ref(fused, bias, k, latent, keep, cap, slots, steps, 0, repeat, fallback, cand=cand, given=got)
+    assert torch.equal(ids, rids)
+    torch.testing.assert_close(w, rw, rtol=1e-5, atol=0)
+    assert torch.equal(lat.cpu(), want_lat)
+    return ids, w, got
+
+
+@pytest.mark.parametrize("m,keep,cap", [(8, 6, 20), (32, 4, 48), (8, 6, 0), (8, 9, 512), (16, 3, 30)])
+@pytest.mark.parametrize("repeat", [True, False])
+def test_sigmoid_form_at_the_top_9_of_432(m, keep, cap, repeat):
+    """The invariants of the reference's own test (tests/gpu/test_bolt_kernels.py:188-216) and, with every top 9 in the
+    set, the plain routing's ids and weights bit for bit."""
+    from hibana_amd.model import nemotron_moe
+    g = torch.Generator().manual_seed(19 + m)
+    experts, latent, k = 432, 1024, 9
+    fused = torch.randn(m, experts + latent, generator=g) * 2
+    bias = torch.randn(experts, generator=g) * 0.1
+    slots = torch.tensor([1] * (m // 8 - 1) + [0], dtype=torch.int32)  # the last request padded
+    ids, w, got = check_sigmoid(fused, bias, k, latent, min(keep, k), cap, slots, 8, repeat=repeat)
+    real = m - 8
+    order = nemotron_moe.route_topk(fused.cuda(), bias.cuda(), k, latent)[0].cpu()
+    s = torch.sigmoid(fused[:, :experts])
+    for t in range(real):
+        live = w[t] > 0
+        assert torch.equal(ids[t, :min(keep, k)], order[t, :min(keep, k)])
+        picked = ids[t][live].long()
+        torch.testing.assert_close(w[t][live], s[t, picked] / s[t, picked].sum(), rtol=2e-6, atol=1e-7)
+        assert (ids[t][~live] == (ids[t, 0] if repeat else experts)).all()
+    assert not w[real:].any() and (ids[real:] == (order[0, 0] if repeat else experts)).all()
+    if cap >= real * k:
+        plain = nemotron_moe.route_topk(fused.cuda(), bias.cuda(), k, latent, slots.cuda(), 8, repeat)
+        assert torch.equal(ids, plain[0].cpu()) and torch.equal(w, plain[1].cpu())
+
+
+@pytest.mark.parametrize("m,cap", [(4, 44), (16, 64), (16, 128), (1, 22), (64, 96)])
+def test_sigmoid_form_at_the_top_22_of_512(m, cap):
+    g = torch.Generator().manual_seed(1000 + m)
+    experts, latent, k = 512, 1024, 22
+    fused = torch.randn(m, experts + latent, generator=g) * 1.5
+    bias = torch.randn(experts, generator=g) * 0.1
+    keep = max(4, min(8, cap // m))
+    slots = torch.tensor([1] * max(1, m - 1) + [0] * (m > 1), dtype=torch.int32)  # the last row padded
+    check_sigmoid(fused, bias, k, latent, keep, cap, slots, 1)
+    check_sigmoid(fused, bias, k, latent, keep, cap, None, 1, per_request=12)
+    check_sigmoid(fused, bias, k, latent, keep, cap, slots, 1, repeat=False)
+
+
+def test_sigmoid_form_falls_back_when_the_floors_exceed_the_cap():
+    g = torch.Generator().manual_seed(5)
+    experts, latent, k = 512, 64, 22
+    fused = torch.randn(16, experts + latent, generator=g) * 1.5
+    bias = torch.zeros(experts)
+    full = check_sigmoid(fused, bias, k, latent, 12, 48)[2]           # sixteen rows' top 12: far more than 48 experts, all kept
+    assert len(full) > 48
+    capped = check_sigmoid(fused, bias, k, latent, 12, 48, fallback=2)[2]  # guaranteed only their top 2: the cap holds
+    assert len(capped) == 48
+    assert check_sigmoid(fused, bias, k, latent, 12, 0, fallback=2)[2] == check_sigmoid(fused, bias, k, latent, 12, 0)[2]  # no cap, no fallback
+    roomy = check_sigmoid(fused[:2], bias, k, latent, 12, 48, fallback=2)[2]  # two rows' top 12 fit: the floors stand
+    assert len(roomy) == 44  # their 44 candidates in all
+
+
+@pytest.mark.parametrize("experts,k", [(32, 32), (100, 8), (1000, 32), (1024, 6)])
+def test_sigmoid_form_at_other_expert_counts(experts, k):
+    g = torch.Generator().manual_seed(experts)
+    for m, keep, cap in [(1, 1, 4), (9, 2, 12), (33, 3, 40)]:
+        fused = torch.randn(m, experts + 8, generator=g) * 2
+        bias = torch.randn(experts, generator=g) * 0.1
+        check_sigmoid(fused, bias, k, 8, min(keep, k), cap)
+
+
+def test_sigmoid_form_graph_replay():
+    from hibana_amd.model import nemotron_moe
+    g = torch.Generator().manual_seed(2)
+    experts, latent, k = 512, 256, 22
+    feeds = [(torch.randn(16, experts + latent, generator=g) * 1.5, s) for s in paddings(4, 9) + [torch.arange(1, 5, dtype=torch.int32)]]
+    bias = (torch.randn(experts, generator=g) * 0.1).cuda()
+    fused, slots = feeds[0][0].cuda(), feeds[0][1].cuda()
+    call = lambda f, s: nemotron_moe.route_budget(f, bias, k, latent, 6, 40, s, 4, per_request=16, fallback=2)  # noqa: E731
+    call(fused, slots)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = call(fused, slots)
+    for f, s in feeds + feeds[:2]:
+        fused.copy_(f)
+        slots.copy_(s)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = call(f.cuda(), s.cuda())
+        assert all(torch.equal(a.view(torch.int32) if a.dtype == torch.float32 else a, b.view(torch.int32) if b.dtype == torch.float32 else b)
+                   for a, b in zip(out, eager))

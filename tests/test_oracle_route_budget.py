@@ -1,7 +1,8 @@
 """Pins of the oracle's budgeted expert selection (oracle/layers.py `route_budget_ref`, following
 hibana/kernels/flashnext_fused.py:322-502 and the rule of tests/unit/test_moe_selection.py:19-58): a hand-worked call,
 the reduction to a sorted top-k, padded requests, exact ties, the cap per request, and the invariants the reference's
-unit test states."""
+unit test states; the latent MoE's form (`route_budget_sigmoid_ref`, hibana/model/nemotron/moe.py:124-313) by a
+hand-worked call, the reduction to plain sigmoid routing and the invariants of tests/gpu/test_bolt_kernels.py:188-216."""
 import math
 
 import numpy as np
@@ -124,3 +125,67 @@ def test_silu_mul_rounds_the_fp32_product_once():
     assert (got.double() - exact).abs().max() <= (exact.abs() * 2.0 ** -8 + 1e-30).max()
     pairs = layers.silu_mul(torch.cat((gu[:, :32], gu[:, 64:96], gu[:, 32:64], gu[:, 96:]), 1), 32)
     assert torch.equal(pairs, got)
+
+
+def test_the_sigmoid_form_worked_by_hand():
+    """Eight experts, k = 3. Sigmoids 0.9 / 0.75 / 0.5 / 0.1 from logits ln 9 / ln 3 / 0 / -ln 9; a bias of 1 puts
+    expert 5 (sigmoid 0.1) first in both rows' choice, and its weight stays 0.1."""
+    hi, mid, low = math.log(9.0), math.log(3.0), -math.log(9.0)
+    fused = torch.full((2, 8), low)
+    fused[0, [0, 1, 2]] = torch.tensor([hi, mid, 0.0])
+    fused[1, [2, 1, 3]] = torch.tensor([hi, mid, 0.0])
+    bias = torch.zeros(8)
+    bias[5] = 1.0
+    run = lambda **kw: layers.route_budget_sigmoid_ref(fused, bias, 3, 0, **kw)  # noqa: E731
+    # the guaranteed expert 5 and the one expert both rows hold below it
+    ids, w, chosen, core, score, _ = run(keep=1, budget=2)
+    assert core == {5} and chosen == {1, 5}
+    assert np.allclose(score[[0, 1, 2]], [0.9 / 1.75, 1.5 / 1.75, 0.9 / 1.75], rtol=1e-6) and score[0] == score[2]
+    assert ids.tolist() == [[5, 1, 5], [5, 1, 5]]  # the slot left over repeats the row's first choice
+    assert np.allclose(w.numpy(), [[0.1 / 0.85, 0.75 / 0.85, 0.0]] * 2, rtol=1e-6)
+    # experts 0 and 2 score the same: the lower one takes the third place
+    ids, w, chosen, _, _, _ = run(keep=1, budget=3)
+    assert chosen == {0, 1, 5} and ids.tolist() == [[5, 0, 1], [5, 1, 5]]
+    assert np.allclose(w[0].numpy(), np.array([0.1, 0.9, 0.75]) / 1.75, rtol=1e-6)
+    assert run(keep=1, budget=3, repeat=False)[0].tolist() == [[5, 0, 1], [5, 1, 8]]
+    # the rows' top 2 are three experts, above a cap of 2: they all stay, unless a fallback of 1 guarantees only expert 5
+    assert run(keep=2, budget=2)[2] == {0, 2, 5}
+    ids, _, chosen, core, _, _ = run(keep=2, budget=2, fallback=1)
+    assert core == {5} and chosen == {1, 5} and ids.tolist() == [[5, 1, 5], [5, 1, 5]]
+    assert run(keep=2, budget=0, fallback=1)[2] == {0, 2, 5}  # no cap: nothing to fall back from
+
+
+def test_the_sigmoid_form_with_every_top_k_in_the_set_is_plain_routing():
+    g = torch.Generator().manual_seed(8)
+    e, k, latent = 432, 9, 16
+    fused = torch.randn(16, e + latent, generator=g) * 2
+    bias = torch.randn(e, generator=g) * 0.1
+    slots = torch.tensor([1, 0], dtype=torch.int32)
+    ids, w, _, _, _, lat = layers.route_budget_sigmoid_ref(fused, bias, k, latent, 6, 512, slots, 8, repeat=False)
+    want_ids, want_w = layers.route_sigmoid_topk(fused[:8, :e], bias, k)
+    assert torch.equal(ids[:8], want_ids)
+    torch.testing.assert_close(w[:8], want_w, rtol=1e-6, atol=0)
+    assert (ids[8:] == e).all() and not w[8:].any()
+    assert torch.equal(lat, fused[:, e:].bfloat16())
+
+
+def test_the_sigmoid_form_invariants():
+    g = torch.Generator().manual_seed(19)
+    e, k, latent = 432, 9, 0
+    for m, keep, cap in [(8, 6, 20), (32, 4, 48), (8, 6, 0)]:
+        fused = torch.randn(m, e, generator=g) * 2
+        bias = torch.randn(e, generator=g) * 0.1
+        slots = torch.tensor([1] * (m // 8 - 1) + [0], dtype=torch.int32)
+        real = m - 8
+        ids, w, chosen, core, _, _ = layers.route_budget_sigmoid_ref(fused, bias, k, latent, keep, cap, slots, 8)
+        s = torch.sigmoid(fused)
+        order = torch.sort(s + bias, dim=-1, descending=True, stable=True).indices[:, :k]
+        assert core == set(order[:real, :keep].reshape(-1).tolist()) and len(chosen) <= max(cap, len(core))
+        for t in range(real):
+            live = w[t] > 0
+            assert torch.equal(ids[t, :keep].long(), order[t, :keep])
+            picked = ids[t][live].long()
+            assert picked.tolist() == [x for x in order[t].tolist() if x in chosen]
+            torch.testing.assert_close(w[t][live], s[t, picked] / s[t, picked].sum(), rtol=1e-6, atol=1e-7)
+            assert (ids[t][~live] == ids[t, 0]).all()
+        assert not w[real:].any() and (ids[real:] == order[0, 0]).all()
