@@ -144,6 +144,7 @@ def latent_prefill(args) -> dict:
     del outs
     gemm_flops = tokens * topk * 2 * inter * latent  # one expert GEMM (fc1 or fc2), useful flops
     fc1_ms = mean(per_kernel["fc1"])
+    mfma_tflops = mfma_rate_tflops(dev)
     cpu, check = None, None
     if not args.no_cpu:
         cpu, check = latent_cpu_leg(block, ex, fc1.bfloat16().cpu(), fc2.cpu(), x, latent, inter)
@@ -159,7 +160,9 @@ def latent_prefill(args) -> dict:
                    "timed_as": "replays of one HIP graph of all steps; value and ms_per_step are the median replay"},
         "roofline": {"bound": "mfma", "kernel": "tile_kernel<TileNvfp4, fc1 relu2>", "achieved": gemm_flops / (fc1_ms * 1e-3) / 1e12,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "launch_flops": gemm_flops, "launch_ms": fc1_ms},
+                     "traffic": None, "launch_flops": gemm_flops, "launch_ms": fc1_ms, "peak_measured": mfma_tflops,
+                     "frac_of_measured": gemm_flops / (fc1_ms * 1e-3) / 1e12 / mfma_tflops,
+                     "peak_measured_how": "BF16 16x16x32 MFMAs on registers alone in this run (hb_debug_mfma_rate)"},
         "layer_chain": {"kernel_ms": {n: mean(v) for n, v in per_kernel.items()}},
         "decode_calls": small,
         "cpu_baseline": cpu,
@@ -438,6 +441,27 @@ def stream_read_gbs(dev, mib: int = 1024) -> float:
         if i >= 2:
             times.append(e0.elapsed_time(e1))
     return src.numel() / (median(times) * 1e-3) / 1e9
+
+
+def mfma_rate_tflops(dev, blocks: int = 2048, iters: int = 4096) -> float:
+    """What a kernel that only multiplies gets from this device's matrix cores: BF16 16x16x32 MFMAs on registers, eight
+    wavefronts a workgroup (hb_debug_mfma_rate), median of seven runs timed with events on the stream it runs on."""
+    import torch
+
+    from hibana_amd import _lib
+    sink = torch.zeros(blocks, dtype=torch.float32, device=dev)
+    times, flops = [], 0
+    for i in range(9):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        flops = _lib.lib().hb_debug_mfma_rate(blocks, iters, _lib.ptr(sink), _lib.stream())
+        e1.record()
+        torch.cuda.synchronize()
+        if flops <= 0:
+            raise RuntimeError(f"hb_debug_mfma_rate: {flops}")
+        if i >= 2:
+            times.append(e0.elapsed_time(e1))
+    return flops / (median(times) * 1e-3) / 1e12
 
 
 def traffic_ratio():

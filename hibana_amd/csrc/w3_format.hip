@@ -269,3 +269,35 @@ extern "C" int hb_debug_stream_read(const void* src, size_t bytes, void* sink, v
                      static_cast<uint32_t*>(sink));
   return launch_status();
 }
+
+// Measurement hook: the rate this device's matrix cores give a kernel that does nothing else, the yardstick an expert
+// GEMM is held against. Every wavefront runs `iters` rounds of eight independent v_mfma_f32_16x16x32_bf16 (16 384
+// FLOP each) on registers; eight wavefronts a workgroup, two a SIMD.
+__global__ __launch_bounds__(512) void mfma_rate_kernel(int iters, float* __restrict__ sink) {
+  const int lane = threadIdx.x & 63;
+  bf16x8_t a, b;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    a[j] = (__bf16)(0.001f * (float)(lane + j));
+    b[j] = (__bf16)(0.002f * (float)(lane ^ j));
+  }
+  f32x4_t acc[8];
+#pragma unroll
+  for (int c = 0; c < 8; c++) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < iters; i++) {
+#pragma unroll
+    for (int c = 0; c < 8; c++) acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[c], 0, 0, 0);
+  }
+  float fold = 0.f;
+#pragma unroll
+  for (int c = 0; c < 8; c++) fold += acc[c].x + acc[c].y + acc[c].z + acc[c].w;
+  if (fold == 12345.678f) sink[blockIdx.x] = fold;  // (practically never: the products stay, the store does not cost)
+}
+
+extern "C" int64_t hb_debug_mfma_rate(int blocks, int iters, void* sink, void* stream) {
+  if (!sink) return -HB_ENULL;
+  if (blocks <= 0 || blocks > 65536 || iters <= 0 || iters > (1 << 20) || !aligned(sink, 4)) return -HB_EINVAL;
+  hipLaunchKernelGGL(mfma_rate_kernel, dim3((unsigned)blocks), dim3(512), 0, as_stream(stream), iters, static_cast<float*>(sink));
+  if (launch_status() != HB_OK) return -HB_ELAUNCH;
+  return (int64_t)blocks * 8 * iters * 8 * 16384;  // the launch's FLOP
+}

@@ -66,6 +66,12 @@ int hb_debug_trace(void* buffer);
  * hold a weight stream's rate against. `sink`: at least bytes / 65536 + 1 uint32 (practically never written). */
 int hb_debug_stream_read(const void* src, size_t bytes, void* sink, void* stream);
 
+/* Measurement hook (no counterpart in the reference): `blocks` workgroups of eight wavefronts each run `iters` rounds of
+ * eight independent BF16 MFMAs (16x16x32) on registers - the rate this device's matrix cores give a kernel that does
+ * nothing else, to hold an expert GEMM's rate against. Returns the launch's FLOP (negative: an error code negated).
+ * `sink`: at least `blocks` floats (practically never written). */
+int64_t hb_debug_mfma_rate(int blocks, int iters, void* sink, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * W3 format: 3-bit (or 2-bit) codes into an 8-entry E4M3 codebook, one E4M3 scale per 32 weights along K, one FP32
  * multiplier per output row.
