@@ -1018,7 +1018,7 @@ extern "C" int hb_debug_events(void* const* events, int count) {
   return HB_OK;
 }
 
-extern "C" int hb_version(void) { return 1000; }
+extern "C" int hb_version(void) { return 1003; }  // minor: the entry points added since 1.0 (the small latent block, hb_nvfp4_gemm_ws, budgeted routing)
 
 extern "C" const char* hb_error_string(int code) {
   switch (code) {
