@@ -59,6 +59,7 @@ SIGNATURES = {
     "hb_w3_moe_layer_static": (_I, [_EX, _EX, _P, _P, _P, _P, _I, _I, _P, _P]),
     "hb_w3_moe_layer_e4m3": (_I, [_EX, _EX, _P, _P, _P, _P, _I, _I, _P, _P, _Z, _P]),
     "hb_w3_moe_layer_logits": (_I, [_EX, _EX, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P]),
+    "hb_w3_moe_layer_budget": (_I, [_EX, _EX, _P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P]),
     "hb_w3_moe_layer_logits_e4m3": (_I, [_EX, _EX, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P]),
     "hb_moe_combine_pairs": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P]),
     "hb_silu_and_mul": (_I, [_P, _L, _I, _I, _P, _P]),

@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "route.hpp"
+#include "route_budget.hpp"
 #include "stream_common.hpp"
 
 namespace hb {
@@ -397,6 +398,22 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int3
   plan_work<false>(ids, pairs, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, nullptr, 1, 0, 0, lds);
 }
 
+// Budgeted selection and the plan of its ids in one launch: the selection is one workgroup's work already, and so is
+// the plan of a decode or verify call; the ids go through to memory and are waited for before the plan reads them back
+// past the L2, as in the routing launch above. `PLAN`: false leaves the plan to launches of its own (a call of more
+// pairs than one workgroup plans).
+template <int PER, bool PLAN>
+__global__ __launch_bounds__(PLAN_THREADS) void moe_budget_plan_kernel(BudgetParams q, int copies_n, int e_lo, int e_n, int shared_rows,
+                                                                       int32_t* __restrict__ plan, int32_t* __restrict__ order, int slot_rows,
+                                                                       int slot_cap) {
+  extern __shared__ int lds[];
+  budget_pick<PER, false>(q, copies_n, reinterpret_cast<float*>(lds));
+  if (!PLAN) return;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's ids have reached memory
+  __syncthreads();                                    // ... and everyone's; the selection's use of the LDS is over
+  plan_work<false>(q.ids, q.r * q.k, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, nullptr, 1, 0, 0, lds);
+}
+
 // ---------------------------------------------------------------------------------------------------- combine
 //
 // out[r, c] = bf16( bf16(sum over the row's local slots, in selection order, of fma(w, y)) + g * shared ), one
@@ -751,6 +768,56 @@ int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* 
   rp.ids = ids;
   rp.weights = weights;
   return launch_route_plan(rp, m, e_lo, e_n, shared_rows, ws, stream, slot_rows, job);
+}
+
+int moe_launch_budget_plan(const BudgetRoute& b, int m, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
+                           const MoeWorkspace& ws, void* scratch, hipStream_t stream, int slot_rows) {
+  static_assert(BUDGET_THREADS == PLAN_THREADS, "the selection and the plan share a workgroup");
+  const int64_t pairs = (int64_t)m * topk;
+  const size_t plan_lds = ((size_t)(PLAN_WAVES + 1) * e_n + 3 * (PLAN_WAVES + 1)) * sizeof(int);
+  if (plan_lds > 64 * 1024 || e_n > PLAN_THREADS || pairs > 0x3fffffff) return HB_EINVAL;
+  if (!b.logits || !scratch) return HB_ENULL;
+  if (b.e < BUDGET_CANDIDATES || b.e > BUDGET_THREADS || topk > BUDGET_CANDIDATES || b.keep < 0 || b.keep > BUDGET_CANDIDATES || b.budget < 0 ||
+      b.steps <= 0 || m % b.steps || b.per_request < 0 || b.min_cap < 0 || !aligned(b.logits, 2) || !aligned(b.slots, 4) || !aligned(scratch, 4))
+    return HB_EINVAL;
+  BudgetParams q{};
+  q.logits = b.logits;
+  q.slots = b.slots;
+  q.r = m, q.e = b.e, q.k = topk, q.keep = b.keep, q.budget = b.budget, q.per_request = b.per_request, q.min_cap = b.min_cap, q.steps = b.steps,
+  q.repeat = b.repeat;
+  q.cands = BUDGET_CANDIDATES;
+  q.cand = static_cast<int32_t*>(scratch);
+  q.prob = reinterpret_cast<float*>(q.cand + (int64_t)m * BUDGET_CANDIDATES);
+  q.share = q.prob;
+  q.ids = ids, q.weights = weights;
+  const bool small = b.e <= 512;
+  if (small) {
+    HB_LAUNCH((route_rank_kernel<8>), dim3((unsigned)m), dim3(64), 0, stream, q);
+  } else {
+    HB_LAUNCH((route_rank_kernel<16>), dim3((unsigned)m), dim3(64), 0, stream, q);
+  }
+  const int copies_n = small ? BUDGET_WAVES : BUDGET_WAVES / 2;
+  const size_t pick_lds = (size_t)copies_n * b.e * sizeof(float);
+  const int slot_cap = (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows);
+  if (pairs < PLAN_WIDE_PAIRS) {
+    const size_t lds = std::max(pick_lds, plan_lds);
+    if (small) {
+      HB_LAUNCH((moe_budget_plan_kernel<8, true>), dim3(1), dim3(PLAN_THREADS), lds, stream, q, copies_n, e_lo, e_n, shared_rows, ws.plan, ws.order, slot_rows,
+                slot_cap);
+    } else {
+      HB_LAUNCH((moe_budget_plan_kernel<16, true>), dim3(1), dim3(PLAN_THREADS), lds, stream, q, copies_n, e_lo, e_n, shared_rows, ws.plan, ws.order, slot_rows,
+                slot_cap);
+    }
+    return HB_OK;
+  }
+  if (small) {
+    HB_LAUNCH((moe_budget_plan_kernel<8, false>), dim3(1), dim3(PLAN_THREADS), pick_lds, stream, q, copies_n, e_lo, e_n, shared_rows, ws.plan, ws.order,
+              slot_rows, slot_cap);
+  } else {
+    HB_LAUNCH((moe_budget_plan_kernel<16, false>), dim3(1), dim3(PLAN_THREADS), pick_lds, stream, q, copies_n, e_lo, e_n, shared_rows, ws.plan, ws.order,
+              slot_rows, slot_cap);
+  }
+  return moe_launch_plan(ids, pairs, e_lo, e_n, shared_rows, ws, stream, slot_rows, nullptr);
 }
 
 int latent_launch_router(const LatentRouter& r, hipStream_t stream) {

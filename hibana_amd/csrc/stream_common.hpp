@@ -508,6 +508,17 @@ void moe_launch_quant_rows(const uint16_t* x, int64_t m, int k, uint8_t* q, floa
 // Softmax top-k routing of `m` rows of `e` logits into ids / weights [m, topk], then the plan of those ids: one launch
 // for up to a few dozen rows, two beyond.
 int moe_check_route(int m, int e, int k);  // HB_EINVAL for a row the routing wavefront cannot hold
+
+// A routed call whose experts are chosen under a budget (route_budget.hpp): BF16 logits [m, e] and the rule's settings.
+struct BudgetRoute {
+  const uint16_t* logits;
+  int e, keep, budget, steps, repeat, per_request, min_cap;
+  const int32_t* slots;  // or null: every row is real
+};
+// Rank, then the selection and the plan of its ids in one workgroup's launch (the selection leaves ids / weights in the
+// caller's arrays). `scratch`: room for the rows' candidates between the two launches (160 bytes a row).
+int moe_launch_budget_plan(const BudgetRoute& b, int m, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
+                           const MoeWorkspace& ws, void* scratch, hipStream_t stream, int slot_rows = ROWS_PER_SLOT);
 int moe_launch_route_plan(const float* logits, int m, int e, int topk, int32_t* ids, float* weights, int e_lo, int e_n, int shared_rows,
                           const MoeWorkspace& ws, hipStream_t stream, int slot_rows = ROWS_PER_SLOT, const QuantJob* job = nullptr);
 

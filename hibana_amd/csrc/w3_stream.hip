@@ -961,6 +961,7 @@ struct Routing {  // set: the chain routes `logits` [m, e] itself into the calle
   int e;
   int32_t* ids;
   float* weights;
+  const BudgetRoute* budget = nullptr;  // ... under a budget, from BF16 logits (`logits` is then unused)
 };
 
 int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void* x, const int32_t* ids, int m, int topk,
@@ -982,11 +983,17 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
                               : QuantJob{static_cast<const uint16_t*>(x), (int64_t)m * ex->hidden / 8, ws.xq, ws.xs, 0, 0};
   const QuantJob* job = e4m3 || split ? &xjob : nullptr;
   // one token from its logits, a slot a selection, and fc2 + combine as one launch after it: fc1 routes for itself
-  const bool route_in_fc1 = route && m == 1 && combine && !e4m3 && !split && !dense && topk <= 63 && slots == topk + shared_rows &&
+  const bool route_in_fc1 = route && !route->budget && m == 1 && combine && !e4m3 && !split && !dense && topk <= 63 && slots == topk + shared_rows &&
                             slots + (combine->gate_vec && combine->shared ? ONE_GATE_WAVES : 0) <= ONE_MAX_WAVES && g_tune.moe_one == 0 &&
                             moe_check_route(m, route->e, topk) == HB_OK;
   if (route_in_fc1) {
     // (nothing to launch here)
+  } else if (route && route->budget) {
+    if (e4m3) return HB_EINVAL;  // weight-only
+    if (job) moe_launch_quant_groups(*job, stream);  // the selection's launch carries no rounding job: the two-plane form of x in a launch of its own
+    // the rows' candidates rest where the pair outputs will go: the selection has read them before fc2 writes
+    if (int e = moe_launch_budget_plan(*route->budget, m, topk, route->ids, route->weights, ex->base, ex->experts, shared_rows, ws, ws.y, stream, slot_rows))
+      return e;
   } else if (route) {
     if (int e = moe_launch_route_plan(route->logits, m, route->e, topk, route->ids, route->weights, ex->base, ex->experts, shared_rows, ws, stream,
                                       slot_rows, job))
@@ -1256,6 +1263,16 @@ extern "C" int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_e
   if (!logits) return HB_ENULL;
   if (!aligned(logits, 4)) return HB_EINVAL;
   const Routing route{logits, experts_total, ids, weights};
+  return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, &route);
+}
+
+extern "C" int hb_w3_moe_layer_budget(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,
+                                      const void* logits, int experts_total, int m, int topk, int keep, int budget, const int32_t* slots, int steps,
+                                      int per_request, int min_cap, int32_t* ids, float* weights, void* out, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+  if (!logits) return HB_ENULL;
+  const BudgetRoute b{static_cast<const uint16_t*>(logits), experts_total, keep, budget, steps, 0, per_request, min_cap, slots};
+  const Routing route{nullptr, experts_total, ids, weights, &b};
   return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, workspace, workspace_bytes, stream, &route);
 }
 

@@ -215,6 +215,40 @@ def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, 
     return (out, ids, wt) if return_routing else out
 
 
+def moe_layer_budget(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, topk: int, keep: int, budget: int,
+                     slots: torch.Tensor | None = None, steps: int = 1, per_request: int = 0, min_cap: int = 0, shared: W3Experts | None = None,
+                     gate_vec: torch.Tensor | None = None, return_routing: bool = False):
+    """`moe_layer` from the router's BF16 logits [M, E_total] under a budget: `ops.route_budget`'s selection (slots left
+    over name no expert) runs in the same chain, its second launch also planning the call
+    (hibana/model/flashnext/moe.py:122-135,177-192). The bits of `route_budget` followed by `moe_layer`. With
+    `return_routing`, also the ids and weights it used."""
+    if x.dtype != torch.bfloat16 or x.ndim != 2 or x.shape[1] != experts.shape13[1]:
+        raise ValueError("moe_layer_budget: x must be BF16 [M, hidden]")
+    if logits.ndim != 2 or logits.shape[0] != x.shape[0] or logits.dtype != torch.bfloat16:
+        raise ValueError("moe_layer_budget: logits must be BF16 [M, experts]")
+    m, e_total = logits.shape
+    if not (20 <= e_total <= 1024 and 1 <= topk <= 20 and 0 <= keep <= 20) or budget < 0 or steps < 1 or m % steps:
+        raise ValueError("moe_layer_budget: 20 <= E <= 1024, topk and keep at most 20, whole requests of `steps` rows")
+    if slots is not None and slots.numel() < m // steps:
+        raise ValueError("moe_layer_budget: a slot for every request")
+    _lib.need_gpu(x, logits, slots)
+    out = torch.empty((m, experts.shape2[0]), dtype=torch.bfloat16, device=x.device)
+    ids = torch.empty((m, topk), dtype=torch.int32, device=x.device)
+    wt = torch.empty((m, topk), dtype=torch.float32, device=x.device)
+    if m:
+        st = _struct(experts)
+        sh = _struct(shared) if shared is not None else None
+        need = _lib.lib().hb_w3_moe_workspace_bytes(m, topk, C.byref(st), int(shared is not None))
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+        gv = None if gate_vec is None else gate_vec.float().contiguous()
+        sl = None if slots is None else slots.to(torch.int32).contiguous()
+        xc, lg = x.contiguous(), logits.contiguous()
+        _lib.check(_lib.lib().hb_w3_moe_layer_budget(C.byref(st), C.byref(sh) if sh is not None else None, _lib.ptr(gv), _lib.ptr(xc), _lib.ptr(lg),
+                                                     e_total, m, topk, keep, budget, _lib.ptr(sl), steps, per_request, min_cap, _lib.ptr(ids),
+                                                     _lib.ptr(wt), _lib.ptr(out), _lib.ptr(ws), need, _lib.stream()), "moe_layer_budget")
+    return (out, ids, wt) if return_routing else out
+
+
 # ------------------------------------------------------------------ offline: 3-bit experts from NVFP4 experts
 
 @torch.no_grad()

@@ -123,5 +123,10 @@ class MoeLayer:
         if slots is None and not self.selects(ctx):  # routing, plan, both streams and the combine as one chain
             logits = torch.mm(x, self.router.T).float()
             return w3_moe.moe_layer_logits(self.w3, x, logits, self.topk, shared=self.shared, gate_vec=self.shared_gate_vec)
+        if self.selects(ctx) and self.budget:  # the selection's launches and the experts' as one chain
+            logits = torch.mm(x, self.router.T)
+            _, steps = self._padding(ctx)
+            return w3_moe.moe_layer_budget(self.w3, x, logits, self.topk, self.guarantee(x.shape[0], steps), self.budget, slots, steps,
+                                           per_request=self.per_request, min_cap=self.MIN_CAP, shared=self.shared, gate_vec=self.shared_gate_vec)
         ids, weights = self.route(x, ctx)
         return w3_moe.moe_layer(self.w3, x, ids, weights, shared=self.shared, gate_vec=self.shared_gate_vec)

@@ -224,6 +224,19 @@ int hb_w3_moe_layer_logits_e4m3(const hb_w3_experts* routed, const hb_w3_experts
                                 const void* x, const float* logits, int experts_total, int m, int topk, int32_t* ids,
                                 float* weights, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same layer from the router's BF16 logits [m, experts_total] under a budget: the experts are chosen by
+ * hb_route_budget's rule (keep, budget, slots / steps, per_request, min_cap as there; slots left over name no expert:
+ * id experts_total at weight 0, which the experts skip), written to ids / weights (caller's buffers), then the chain of
+ * hb_w3_moe_layer. Two launches ahead of the experts': the rows' candidates, then one workgroup that selects and also
+ * plans (up to 8191 pairs; beyond, the plan's own launches follow). Weight-only arithmetic. topk and keep at most
+ * HB_ROUTE_CANDIDATES, 20 <= experts_total <= 1024, m a multiple of steps. The same ids, weights and output as
+ * hb_route_budget followed by hb_w3_moe_layer, bit for bit.
+ * ref: MoeLayer.__call__ with the budgeted branch of its route step, hibana/model/flashnext/moe.py:122-135,177-192. */
+int hb_w3_moe_layer_budget(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec,
+                           const void* x, const void* logits, int experts_total, int m, int topk, int keep, int budget,
+                           const int32_t* slots, int steps, int per_request, int min_cap, int32_t* ids, float* weights,
+                           void* out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* out = bf16( bf16(sum over the row's local slots of w * pairs) + g * shared ) from unsummed pair outputs (FP32 or,
  * pairs_bf16 != 0, BF16) [m * topk, h]; shared BF16 [m, h] or NULL; gate_vec float32 [h] or NULL (then g = 1; x
  * unused). ref: moe_combine_pairs, hibana/kernels/flashnext_fused.py:530-571; with shared == NULL it is

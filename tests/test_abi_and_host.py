@@ -66,6 +66,7 @@ def test_validation_without_a_gpu():
     for r, e, k, keep, steps in [(12, 19, 10, 4, 1), (12, 1025, 10, 4, 1), (12, 512, 21, 4, 1), (12, 512, 10, 21, 1), (12, 512, 10, 4, 5)]:
         assert lib.hb_route_budget(256, r, e, k, keep, 64, None, steps, 0, 0, 0, 256, 1920, 256, 256, None) == _lib.HB_EINVAL
     assert lib.hb_route_budget(256, 12, 512, 10, 4, 64, None, 1, 0, 0, 0, 256, 1919, 256, 256, None) == _lib.HB_EWORKSPACE
+    assert lib.hb_w3_moe_layer_budget(None, None, None, 256, 256, 512, 4, 10, 4, 64, None, 1, 0, 0, 256, 256, 256, 256, 1 << 20, None) == _lib.HB_ENULL
     assert lib.hb_route_budget_sigmoid_workspace_bytes(12, 22) == 12 * 22 * 12
     assert lib.hb_route_budget_sigmoid(None, 640, 256, 12, 512, 22, 128, 6, 64, None, 1, 1, 0, 0, 256, 3168, 256, 256, 256, None) == _lib.HB_ENULL
     for e, k, keep, fallback, stride in [(512, 33, 6, 0, 640), (1025, 22, 6, 0, 1200), (512, 22, 23, 0, 640), (512, 22, 6, 7, 640), (512, 22, 6, 0, 639)]:

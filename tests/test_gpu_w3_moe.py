@@ -181,6 +181,45 @@ def test_layer_from_logits_is_route_then_layer(gated, m):
     assert torch.equal(w3_moe.moe_layer_logits(ex, x, logits, TOPK), w3_moe.moe_layer(ex, x, ids, wts))
 
 
+@pytest.mark.parametrize("m,steps", [(1, 1), (5, 5), (12, 3), (32, 8), (200, 1)])
+def test_layer_under_a_budget_is_route_budget_then_layer(m, steps):
+    """`moe_layer_budget`: the selection's second launch also plans the call; ids, weights and output are the bits of
+    `ops.route_budget` followed by `moe_layer`, with padded requests, a cap per request, and a call of more pairs
+    than one workgroup plans (the plan's own launches then follow)."""
+    from hibana_amd.kernels import ops, w3_moe
+    e = 32  # the selection takes a row's candidates from its 20 largest logits
+    ex, _ = random_experts(e, H, I, True, 31)
+    shared_ex, _ = random_experts(1, H, I, True, 78)
+    g = torch.Generator().manual_seed(50 + m)
+    x = torch.randn(m, H, generator=g).bfloat16().cuda()
+    logits = (torch.randn(m, e, generator=g) * 1.5).bfloat16().cuda()
+    slots = torch.ones(m // steps, dtype=torch.int32)
+    if m // steps > 1:
+        slots[-1] = 0
+    topk = 10 if m < 200 else 20  # 200 x 20 pairs... below the wide plan; the wide case follows
+    for keep, budget, per_request in [(2, 12, 0), (3, 24, 4), (0, 8, 0)]:
+        ids, wts = ops.route_budget(logits, topk, keep, budget, slots.cuda(), steps, per_request=per_request, min_cap=6)
+        want = w3_moe.moe_layer(ex, x, ids, wts, shared=shared_ex)
+        got, got_ids, got_w = w3_moe.moe_layer_budget(ex, x, logits, topk, keep, budget, slots.cuda(), steps, per_request=per_request, min_cap=6,
+                                                      shared=shared_ex, return_routing=True)
+        assert torch.equal(got_ids, ids) and torch.equal(got_w, wts) and torch.equal(got, want)
+    got = w3_moe.moe_layer_budget(ex, x, logits, topk, 2, 12)  # no slots, no shared expert
+    ids, wts = ops.route_budget(logits, topk, 2, 12)
+    assert torch.equal(got, w3_moe.moe_layer(ex, x, ids, wts))
+
+
+def test_layer_under_a_budget_with_more_pairs_than_one_workgroup_plans():
+    from hibana_amd.kernels import ops, w3_moe
+    e, m, topk = 32, 900, 10  # 9000 pairs: the plan is shared among workgroups
+    ex, _ = random_experts(e, H, I, True, 31)
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(m, H, generator=g).bfloat16().cuda()
+    logits = (torch.randn(m, e, generator=g) * 1.5).bfloat16().cuda()
+    ids, wts = ops.route_budget(logits, topk, 2, 24)
+    got, got_ids, got_w = w3_moe.moe_layer_budget(ex, x, logits, topk, 2, 24, return_routing=True)
+    assert torch.equal(got_ids, ids) and torch.equal(got_w, wts) and torch.equal(got, w3_moe.moe_layer(ex, x, ids, wts))
+
+
 def _one_token_both_ways(call):
     """`call()` with one token's fc2 and combine as one launch (the library's choice) and as two."""
     from hibana_amd import _lib
