@@ -423,29 +423,39 @@ constexpr int COMBINE_SPAN = 512;  // columns per workgroup (two per thread)
 
 // A row's weighted sum of its pairs at columns c, c + 1, in selection order (FP32 fma chain). The pairs of B slots are
 // read together (so the loads are all in flight at once) and a dropped slot contributes fma(0, 0, v).
-template <int B>
+template <int B, bool BF16>
 __device__ __forceinline__ void combine_pairs_batches(const CombineParams& p, int r, int c, float& v0, float& v1) {
   for (int s0 = 0; s0 < p.topk; s0 += B) {
-    float y0[B], y1[B], w[B];
+    // every load of the batch is asked for before any is used: ids and weights (the same for the whole workgroup),
+    // then the pairs - also a dropped slot's, whose values are then set aside
+    int e[B];
+    float w[B], y0[B], y1[B];
+    uint32_t half[B];
+    float2 full[B];
 #pragma unroll
     for (int j = 0; j < B; j++) {
       const int s = min(s0 + j, p.topk - 1);
-      const int e = p.ids[r * p.topk + s] - p.e_lo;
-      const bool keep = s0 + j < p.topk && e >= 0 && e < p.e_n;
+      e[j] = p.ids[r * p.topk + s];
+      w[j] = p.weights[r * p.topk + s];
+    }
+#pragma unroll
+    for (int j = 0; j < B; j++) {
+      const int s = min(s0 + j, p.topk - 1);
       const int64_t at = ((int64_t)r * p.topk + s) * p.h + c;
-      float a, b;
-      if (p.pairs_bf16) {
-        const uint32_t two = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.pairs) + at);
-        a = __uint_as_float(two << 16);
-        b = __uint_as_float(two & 0xffff0000u);
+      if (BF16) {
+        half[j] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.pairs) + at);
       } else {
-        const float2 two = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.pairs) + at);
-        a = two.x;
-        b = two.y;
+        full[j] = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.pairs) + at);
       }
+    }
+#pragma unroll
+    for (int j = 0; j < B; j++) {
+      const int local = e[j] - p.e_lo;
+      const bool keep = s0 + j < p.topk && local >= 0 && local < p.e_n;
+      const float a = BF16 ? __uint_as_float(half[j] << 16) : full[j].x, b = BF16 ? __uint_as_float(half[j] & 0xffff0000u) : full[j].y;
       y0[j] = keep ? a : 0.f;
       y1[j] = keep ? b : 0.f;
-      w[j] = keep ? p.weights[r * p.topk + s] : 0.f;
+      w[j] = keep ? w[j] : 0.f;
     }
 #pragma unroll
     for (int j = 0; j < B; j++) {
@@ -469,19 +479,24 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
   const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
   if (c >= p.h) return;
   float v0 = 0.f, v1 = 0.f;
-  combine_pairs_batches<B>(p, r, c, v0, v1);
-  if (p.shared) {
+  float2 shared_f32 = {0.f, 0.f};
+  uint32_t shared_bf16 = 0;
+  if (p.shared) {  // asked for ahead of the pairs
     const int64_t at = (int64_t)r * p.shared_stride + c;
-    float s0, s1;
     if (p.shared_f32) {
-      const float2 two = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.shared) + at);
-      s0 = two.x;
-      s1 = two.y;
+      shared_f32 = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.shared) + at);
     } else {
-      const uint32_t two = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.shared) + at);
-      s0 = __uint_as_float(two << 16);
-      s1 = __uint_as_float(two & 0xffff0000u);
+      shared_bf16 = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.shared) + at);
     }
+  }
+  if (p.pairs_bf16) {
+    combine_pairs_batches<B, true>(p, r, c, v0, v1);
+  } else {
+    combine_pairs_batches<B, false>(p, r, c, v0, v1);
+  }
+  if (p.shared) {
+    const float s0 = p.shared_f32 ? shared_f32.x : __uint_as_float(shared_bf16 << 16);
+    const float s1 = p.shared_f32 ? shared_f32.y : __uint_as_float(shared_bf16 & 0xffff0000u);
     v0 = combine_shared(v0, g, s0);
     v1 = combine_shared(v1, g, s1);
   }

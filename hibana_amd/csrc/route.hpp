@@ -9,9 +9,10 @@ namespace hb {
 // Top-k routing, one wavefront per row: softmax over all experts, top-k, renormalized
 // (hibana/kernels/flashnext_fused.py:278-319 of the reference), or sigmoid scores chosen by score + bias with the plain
 // scores as weights (hibana/model/nemotron/moe.py:57-121). Lane l holds experts l * per .. l * per + per - 1 in
-// registers as order-preserving 32-bit keys, so a selection round is a register scan, one wave-wide integer maximum
-// (DPP within rows of 16, four scalar reads across them) and a ballot: among equal scores the lowest lane, then the
-// lowest register, wins - the lowest expert id.
+// registers as order-preserving 32-bit keys, so a selection round is one wave-wide integer maximum (DPP within rows of
+// 16, four scalar reads across them) and a ballot: among equal scores the lowest lane, then the lowest register,
+// wins - the lowest expert id. Up to eight registers a lane are sorted once and a round looks at their heads; with
+// sixteen a round scans them.
 constexpr int ROUTE_PER_LANE = 16;
 
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
@@ -58,6 +59,7 @@ template <bool SIGMOID, int PER, bool THROUGH = false>
 __device__ __forceinline__ int route_row(const RouteParams& p, int r, int lane, bool write = true, float* weight = nullptr) {
   const int e = p.e, per = p.per, first = lane * per;
   auto logit = [](const float* at) -> float { if constexpr (THROUGH) return load_through(at); else return *at; };
+  const bool padded = p.slots && p.slots[r / p.steps] == 0;  // asked for first: the answer picks the row the logits are read from
   if (SIGMOID && p.lat && write) {  // the row's latent columns, rounded: four a lane and sixteen loads in flight where the row allows
     const float* src = p.logits + (int64_t)r * p.stride + e;
     uint16_t* dst = p.lat + (int64_t)r * p.latent;
@@ -78,24 +80,27 @@ __device__ __forceinline__ int route_row(const RouteParams& p, int r, int lane, 
       for (int c = lane; c < p.latent; c += 64) dst[c] = bf16_of(logit(src + c));
     }
   }
-  const bool padded = p.slots && p.slots[r / p.steps] == 0;
   const float* row = p.logits + (int64_t)(padded ? 0 : r) * p.stride;  // a padded row repeats row 0's first choice
   float val[PER];   // the weight an expert would get before renormalization
   uint32_t key[PER];
+  float lg[PER];    // the lane's logits: every load is asked for before the first is used
+#pragma unroll
+  for (int j = 0; j < PER; j++) lg[j] = logit(row + min(first + j, e - 1));
   if (SIGMOID) {
+    float bs[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) bs[j] = p.bias[min(first + j, e - 1)];
 #pragma unroll
     for (int j = 0; j < PER; j++) {
-      const int i = first + j;
-      const bool real = j < per && i < e;
-      val[j] = real ? 1.0f / (1.0f + expf(-logit(row + i))) : 0.f;
-      key[j] = real ? score_key(val[j] + p.bias[i]) : 0u;
+      const bool real = j < per && first + j < e;
+      val[j] = real ? 1.0f / (1.0f + expf(-lg[j])) : 0.f;
+      key[j] = real ? score_key(val[j] + bs[j]) : 0u;
     }
   } else {
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < PER; j++) {
-      const int i = first + j;
-      val[j] = j < per && i < e ? logit(row + i) : -INFINITY;
+      val[j] = j < per && first + j < e ? lg[j] : -INFINITY;
       mx = fmaxf(mx, val[j]);
     }
 #pragma unroll
@@ -115,30 +120,79 @@ __device__ __forceinline__ int route_row(const RouteParams& p, int r, int lane, 
   }
   float total = 0.f, mine = 0.f;
   int mine_id = 0;
-  for (int s = 0; s < p.k; s++) {
-    uint32_t best = 0;
-    int at = 0;
-    float bv = 0.f;
+  if constexpr (PER == 8) {
+    // The lane's registers in descending order once (adjacent exchanges on a strictly larger right neighbour only, so
+    // equal keys keep ascending index), their indices as nibbles of one register: a round is then the wave-wide
+    // maximum of the heads and the winner's list moving up by one.
+    uint32_t at[PER];
 #pragma unroll
-    for (int j = 0; j < PER; j++)
-      if (key[j] > best) {  // ascending index within the lane: the first of equals stays
-        best = key[j];
-        at = j;
-        bv = val[j];
+    for (int j = 0; j < PER; j++) at[j] = j;
+#pragma unroll
+    for (int pass = 0; pass < PER; pass++) {
+#pragma unroll
+      for (int j = pass & 1; j + 1 < PER; j += 2) {
+        const bool swap = key[j + 1] > key[j];
+        const uint32_t ka = key[j], kb = key[j + 1], ia = at[j], ib = at[j + 1];
+        key[j] = swap ? kb : ka;
+        key[j + 1] = swap ? ka : kb;
+        at[j] = swap ? ib : ia;
+        at[j + 1] = swap ? ia : ib;
       }
-    const uint32_t top = wave_max_u32(best);
-    const int winner = __builtin_ctzll(__ballot(best == top));
-    const int wj = __builtin_amdgcn_readlane(at, winner);
-    const float wv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv), winner));
-    total += wv;
-    if (lane == s) {
-      mine = wv;
-      mine_id = winner * per + wj;
     }
-    if (lane == winner) {
+    uint32_t order = 0;
+#pragma unroll
+    for (int j = 0; j < PER; j++) order |= at[j] << (4 * j);
+    uint32_t mine_key = 0;
+    for (int s = 0; s < p.k; s++) {
+      const uint32_t top = wave_max_u32(key[0]);
+      const int winner = __builtin_ctzll(__ballot(key[0] == top));
+      const int wj = __builtin_amdgcn_readlane((int)order, winner) & 15;
+      if (lane == s) {
+        mine_key = top;
+        mine_id = winner * per + wj;
+      }
+      if (lane == winner) {
+#pragma unroll
+        for (int j = 0; j + 1 < PER; j++) key[j] = key[j + 1];
+        key[PER - 1] = 0u;
+        order >>= 4;
+      }
+    }
+    if (lane < p.k) {
+      if (SIGMOID) {  // the key is score + bias: the plain score is made again from the logit
+        mine = 1.0f / (1.0f + expf(-logit(row + mine_id)));
+      } else {        // the key is the probability's own bits
+        const uint32_t u = mine_key ^ 0x80000000u;
+        mine = __builtin_bit_cast(float, u ^ (uint32_t)(((int32_t)u >> 31) & 0x7fffffff));
+      }
+    }
+    for (int s = 0; s < p.k; s++) total += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), s));  // in rank order
+  } else {
+    for (int s = 0; s < p.k; s++) {
+      uint32_t best = 0;
+      int at = 0;
+      float bv = 0.f;
 #pragma unroll
       for (int j = 0; j < PER; j++)
-        if (j == wj) key[j] = 0u;
+        if (key[j] > best) {  // ascending index within the lane: the first of equals stays
+          best = key[j];
+          at = j;
+          bv = val[j];
+        }
+      const uint32_t top = wave_max_u32(best);
+      const int winner = __builtin_ctzll(__ballot(best == top));
+      const int wj = __builtin_amdgcn_readlane(at, winner);
+      const float wv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv), winner));
+      total += wv;
+      if (lane == s) {
+        mine = wv;
+        mine_id = winner * per + wj;
+      }
+      if (lane == winner) {
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+          if (j == wj) key[j] = 0u;
+      }
     }
   }
   int id = mine_id;

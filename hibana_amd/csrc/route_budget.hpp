@@ -52,22 +52,32 @@ template <int PER>
 __global__ __launch_bounds__(64) void route_rank_kernel(BudgetParams q) {
   const int t = blockIdx.x, lane = threadIdx.x, e = q.e;
   const uint16_t* row = q.logits + (int64_t)t * e;
-  uint32_t key[PER];
+  uint32_t key[PER], raw[PER];
   float val[PER];
+#pragma unroll
+  for (int j = 0; j < PER; j++) raw[j] = row[min(j * 64 + lane, e - 1)];  // all of the lane's loads before any use
 #pragma unroll
   for (int j = 0; j < PER; j++) {
     const int col = j * 64 + lane;
-    const uint32_t h = col < e ? row[col] : 0u;
+    const uint32_t h = raw[j];
     key[j] = col < e ? (bf16_order(h) << 16) | (uint32_t)(0xffff - col) : 0u;
     val[j] = col < e ? __uint_as_float(h << 16) : -INFINITY;
   }
-  float mx = -INFINITY, sum = 0.f, mine = 0.f;
+  // the lane's keys in descending order once: a round is the wave-wide maximum of the heads, and the winner's list
+  // moves up by one
+#pragma unroll
+  for (int pass = 0; pass < PER; pass++) {
+#pragma unroll
+    for (int j = pass & 1; j + 1 < PER; j += 2) {
+      const uint32_t hi = max(key[j], key[j + 1]), lo = min(key[j], key[j + 1]);
+      key[j] = hi;
+      key[j + 1] = lo;
+    }
+  }
+  float mx = -INFINITY, sum = 0.f, mine_v = 0.f;
   int mine_id = 0;
   for (int c = 0; c < BUDGET_CANDIDATES; c++) {
-    uint32_t best = 0;
-#pragma unroll
-    for (int j = 0; j < PER; j++) best = max(best, key[j]);
-    const uint32_t top = wave_max_u32(best);
+    const uint32_t top = wave_max_u32(key[0]);
     const int col = 0xffff - (int)(top & 0xffffu);
     const float v = bf16_order_value(top >> 16);
     if (c == 0) {  // the row's maximum: the softmax denominator over all experts
@@ -77,15 +87,16 @@ __global__ __launch_bounds__(64) void route_rank_kernel(BudgetParams q) {
       sum = wave_sum(sum);
     }
     if (lane == c) {
-      mine = expf(v - mx) / sum;
+      mine_v = v;
       mine_id = col;
     }
     if (lane == (col & 63)) {
 #pragma unroll
-      for (int j = 0; j < PER; j++)
-        if (j == (col >> 6)) key[j] = 0u;
+      for (int j = 0; j + 1 < PER; j++) key[j] = key[j + 1];
+      key[PER - 1] = 0u;
     }
   }
+  const float mine = expf(mine_v - mx) / sum;
   if (lane < BUDGET_CANDIDATES) {
     q.cand[(int64_t)t * BUDGET_CANDIDATES + lane] = mine_id;
     q.prob[(int64_t)t * BUDGET_CANDIDATES + lane] = mine;

@@ -565,7 +565,18 @@ int latent_launch_out(const uint16_t* fc2, const uint16_t* routed, const uint16_
 // partial sums in `red` (LDS); after a barrier any thread reads g from them.
 __device__ __forceinline__ void combine_gate_partial(const uint16_t* x, const float* gate_vec, int hx, int64_t r, int t, float* red) {
   float dot = 0.f;
-  for (int i = t; i < hx; i += 256) dot += bf16_bits_to_f32(x[r * hx + i]) * gate_vec[i];
+  for (int i0 = t; i0 < hx; i0 += 8 * 256) {  // eight of the thread's terms asked for together, added in the order of i
+    float xv[8], gv[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int i = min(i0 + 256 * j, hx - 1);
+      xv[j] = bf16_bits_to_f32(x[r * hx + i]);
+      gv[j] = gate_vec[i];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (i0 + 256 * j < hx) dot += xv[j] * gv[j];
+  }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) dot += __shfl_xor(dot, d);
   if ((t & 63) == 0) red[t >> 6] = dot;
