@@ -589,11 +589,13 @@ def main() -> int:
     # the dominant kernel: the weight stream - one launch for fc1 and fc2 (every distinct expert's and the shared expert's
     # two matrices, read once), or, at one token and in the E4M3 mode, fc1's launch
     fused = "fc1 + fc2" in kernel_ms
-    dominant = "fc1 + fc2" if fused else "fc1"
+    routed_in_fc1 = "route + fc1" in kernel_ms  # one token: fc1's wavefronts route the row themselves
+    dominant = "fc1 + fc2" if fused else "route + fc1" if routed_in_fc1 else "fc1"
     launch_bytes = mean([(d + 1) * (EXPERT_BYTES if fused else FC1_BYTES) for d in distinct])
     launch_ms = kernel_ms[dominant]
     achieved = launch_bytes / (launch_ms * 1e-3) / 1e9
-    kernel_name = ("w3_fc12_kernel<fc1 gated + fc2>" if fused else "w3_stream_kernel<fc1 gated, E4M3>" if args.e4m3 else "w3_stream_kernel<fc1 gated>")
+    kernel_name = ("w3_fc12_kernel<fc1 gated + fc2>" if fused else "w3_fc1_route_one_kernel<route + fc1 gated>" if routed_in_fc1
+                   else "w3_stream_kernel<fc1 gated, E4M3>" if args.e4m3 else "w3_stream_kernel<fc1 gated>")
     read_gbs = stream_read_gbs(dev)
 
     m1 = None

@@ -96,7 +96,10 @@ __device__ __forceinline__ void compute_half_chunk(const Chunk& ch, const u32x4_
 
 // ------------------------------------------------------------------------------------------------ the weight ring
 // (ring.hpp) for W3 blocks: three 16-byte loads a lane of codes, one 4-byte load a lane of scales.
-struct W3Ring {
+// AUX: the loads' cache policy - 2 (non-temporal) for a call that streams far more than the caches hold, 0 for one
+// token's few megabytes, which come in faster as ordinary loads.
+template <int AUX>
+struct W3RingOf {
   typedef hb::Chunk Chunk;
   static constexpr int BLOCK_BYTES = W3_BLOCK_BYTES, LOADS = 4;
   // the lane's byte offsets in a block for the 16-byte and the 4-byte loads, and where it reads them back
@@ -108,10 +111,10 @@ struct W3Ring {
   }
   static __device__ __forceinline__ void request(const RingSource& src, int chunk, lds_ptr_t slot) {
     const uint32_t at = (uint32_t)chunk * W3_BLOCK_BYTES;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 0, 2);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024, 2);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 2048, 2);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 4, src.scales, at, W3_SCALE_OFFSET, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 0, AUX);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024, AUX);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 2048, AUX);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 4, src.scales, at, W3_SCALE_OFFSET, AUX);
     __builtin_amdgcn_sched_barrier(0);  // asked for here, not wherever the scheduler would sink it below the arithmetic
   }
   template <int BEHIND, int SLOT>  // BEHIND: requests that may stay outstanding
@@ -129,6 +132,8 @@ struct W3Ring {
         : "memory");
   }
 };
+typedef W3RingOf<2> W3Ring;
+typedef W3RingOf<0> W3RingCached;
 constexpr int RING_BYTES = ring_bytes<W3Ring>();  // LDS per wavefront; its first 4 KB double as the K-split exchange
 
 // ------------------------------------------------------------------------------------------- slots of one to four rows
@@ -532,7 +537,7 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
 // scales (p.oq, p.oq_scale), the activation rounding done in its epilogue.
 // SPLIT: slots of at most four rows read the two-plane form of the activations (p.a2) and run on the FP8 matrix cores.
 // One workgroup's work: slot `sl` (with rows), the run `bx` of p.nbw 64-row blocks; `rings`: the launch's dynamic LDS.
-template <int EPI, bool A8, bool SPLIT>
+template <int EPI, bool A8, bool SPLIT, class Ring = W3Ring>
 __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Slot& sl, int bx, uint8_t* rings) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: kept in scalars
   const WaveShare share = wave_share(p, wave);
@@ -548,13 +553,13 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Sl
       if (active) {
         scale = sl.rs[nb * 64 + lane];
         if (EPI == EPI_FC2) pairs.ask(p, sl, 0);
-        stream_block<EPI, FewActs8, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+        stream_block<EPI, FewActs8, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
       }
       finish_few<EPI, QUANT>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs);
     } else {
       RowScales rs{};
       if (active) {
-        stream_block<EPI, FullActs8, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+        stream_block<EPI, FullActs8, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
         rs = row_scales<true>(sl, nb, lane & 15);
       }
       finish_block<EPI, true, RING_BYTES / 4, QUANT>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
@@ -568,7 +573,7 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Sl
       if (EPI == EPI_FC2) pairs.ask(p, sl, 0);
       xs.ask<EPI>(p, sl, 0);
       FewSplitActs acts;
-      stream_block<EPI, FewSplitActs, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3, acts);
+      stream_block<EPI, FewSplitActs, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3, acts);
       acts.fold(acc0, acc1, acc2, acc3);
     }
     finish_few<EPI, false, true>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs, xs);
@@ -578,13 +583,13 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Sl
     if (active) {
       scale = sl.rs[nb * 64 + lane];  // row 16 q + r16 of the block: asked for ahead of the chunks, there when the epilogue wants it
       if (EPI == EPI_FC2) pairs.ask(p, sl, 0);
-      stream_block<EPI, FewActs, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);  // at least one chunk: ks <= chunks
+      stream_block<EPI, FewActs, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);  // at least one chunk: ks <= chunks
     }
     finish_few<EPI>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs);
   } else {
     RowScales rs{};
     if (active) {
-      stream_block<EPI, FullActs, W3Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      stream_block<EPI, FullActs, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
       rs = row_scales<true>(sl, nb, lane & 15);
     }
     finish_block<EPI, true, RING_BYTES / 4>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
@@ -636,7 +641,7 @@ __global__ __launch_bounds__(1024) void w3_fc1_route_one_kernel(StreamParams p, 
     if (!__builtin_amdgcn_readlane((int)here, slot)) return;  // uniform over the workgroup
     expert = __builtin_amdgcn_readlane(local, slot);
   }
-  stream_workgroup<EPI, false, false>(p, make_slot(p, slot, expert, slot, 1), blockIdx.x, rings);
+  stream_workgroup<EPI, false, false, W3RingCached>(p, make_slot(p, slot, expert, slot, 1), blockIdx.x, rings);
 }
 
 // fc1 and fc2 of a routed call in ONE launch, so that fc2's workgroups fill the compute units that fc1's last, partly
@@ -747,7 +752,7 @@ __global__ __launch_bounds__(1024) void w3_fc2_combine_one_kernel(StreamParams p
         for (int t = 0; t < 4; t++) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         FewPairs pairs;
         pairs.ask(p, sl, row0);
-        stream_block<EPI_FC2, FewActs, W3Ring>(p, sl, row0, nb, 0, p.chunks, lane, reinterpret_cast<uint8_t*>(mine), acc[0], acc[1], acc[2], acc[3]);
+        stream_block<EPI_FC2, FewActs, W3RingCached>(p, sl, row0, nb, 0, p.chunks, lane, reinterpret_cast<uint8_t*>(mine), acc[0], acc[1], acc[2], acc[3]);
 #pragma unroll
         for (int t = 0; t < 4; t++) {
           mine[(t * 4 + 0) * 64 + lane] = acc[t].x;
