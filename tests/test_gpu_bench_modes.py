@@ -32,6 +32,22 @@ def test_decode_modes(flags, kernel):
     assert 0 < roof["frac"] < 1 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-9
 
 
+def test_headline_modes():
+    line = run("--no-cpu", "--headline-only", "--layers", "2", "--steps", "24", "--warmup", "4", "--copy-mib", "64")
+    assert "w3_fc12_kernel" in line["roofline"]["kernel"] and line["cpu_baseline"] is None and line["m1"]["value"] > 0
+    assert line["config"]["workload"].startswith("BASELINE config 3") and line["vs_baseline"] is None and line["dtype"] == "bf16"
+    line = run("--e4m3", "--headline-only", "--layers", "2", "--steps", "24", "--warmup", "4")
+    assert "E4M3" in line["metric"] and line["value"] > 0
+
+
+def test_prefill_layer_and_its_small_calls():
+    line = run("--config", "4", "--no-cpu", "--steps", "10", "--warmup", "2")
+    assert line["roofline"]["bound"] == "mfma" and line["roofline"]["peak"] == 2500.0 and 0 < line["roofline"]["frac"] < 1
+    assert "tile_kernel<TileNvfp4" in line["roofline"]["kernel"] and line["unit"] == "tokens/s"
+    line = run("--config", "4", "--small-rows", "4", "--steps", "8", "--warmup", "2")
+    assert line["rows"] == 4 and line["us_per_call"] > 0
+
+
 def test_routing_mode():
     line = run("--routing", "16", "--steps", "12")
     assert line["by_rows"]["16"]["route_topk_us"] > 0 and line["by_rows"]["16"]["route_budget_us"] > 0
