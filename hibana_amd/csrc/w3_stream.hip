@@ -1057,7 +1057,21 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
     if (combine) moe_launch_combine(*combine, stream);
     return launch_status();
   }
-  const Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
+  Launch l1{g_tune.moe_fc1_ksplit, g_tune.moe_fc1_nbw}, l2{g_tune.moe_fc2_ksplit, g_tune.moe_fc2_nbw};
+  // Decode batches of a few rows to a couple of dozen leave the device partly empty under the general rule (K split 4,
+  // one block a workgroup; fc2: four blocks). Measured on the fused launch at hidden 2048 / intermediate 512: up to
+  // about 48 busy slots fc1 with K split 2 on two blocks and fc2 with K split 4 is 3 - 5 % faster a step, from 64 to
+  // 128 busy slots both with K split 2 on two blocks 3 %; beyond that the general rule wins.
+  const bool unset = !l1.ks && !l1.nbw && !l2.ks && !l2.nbw;
+  if (unset && !e4m3 && m > 1 && g_tune.moe_fused != 2 && p.chunks >= 8 && f2.chunks >= 4) {
+    if (est <= 48) {
+      l1 = Launch{2, 2};
+      l2 = Launch{4, 1};
+    } else if (est >= 64 && est <= 128) {
+      l1 = Launch{2, 2};
+      l2 = Launch{2, 2};
+    }
+  }
   if (e4m3) {  // x and h go through the activation rounding: x_q -> fc1 -> h_q -> fc2
     p.aq = ws.xq;
     p.aq_scale = ws.xs;

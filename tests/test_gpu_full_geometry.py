@@ -52,7 +52,7 @@ def _from_bits(a: np.ndarray) -> torch.Tensor:
     return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
 
 
-@pytest.mark.parametrize("m", [1, 32])
+@pytest.mark.parametrize("m", [1, 4, 8, 16, 32])  # 8 and 16: the launches' shapes for partly filled devices
 def test_w3_moe_layer_at_the_benchmark_geometry(w3_layer, m):
     from hibana_amd import synthetic
     from hibana_amd.kernels import ops, w3_moe
@@ -70,7 +70,7 @@ def test_w3_moe_layer_at_the_benchmark_geometry(w3_layer, m):
     ref_ids = torch.topk(torch.softmax(logits.float().cpu(), -1), TOPK).indices
     assert (ids.cpu().long().sort(-1).values == ref_ids.sort(-1).values).float().mean() > 0.99
     distinct = int(torch.unique(ids).numel())
-    assert distinct == TOPK if m == 1 else distinct > 64
+    assert distinct == TOPK if m == 1 else distinct > min(64, 4 * m)
     idn, wn = ids.cpu().numpy(), weights.cpu().numpy()
     want, ran = c_port.moe_layer(h_routed, _bits(x), idn, wn, h_shared)
     assert ran == distinct
