@@ -443,6 +443,41 @@ def stream_read_gbs(dev, mib: int = 1024) -> float:
     return src.numel() / (median(times) * 1e-3) / 1e9
 
 
+def ring_skeleton_gbs(dev, experts: int = 137, regions: int = 6) -> float:
+    """What the W3 stream's request structure gets without its arithmetic (hb_debug_ring_skeleton): `experts` x 16
+    blocks of 53 248 bytes - fc1 of a verify step - at expert-sized runs scattered over a region four times as large,
+    four wavefronts a block, each four chunks through the two-slot LDS ring, activations beside them, the K split's
+    exchange and a store; a region a launch out of `regions` (nothing stays in the caches); twelve launches one after the
+    other between two events, the median repetition's time a launch."""
+    import torch
+
+    from hibana_amd import _lib
+    place_bytes, groups = 53248, experts * 16
+    region = 4 * groups * place_bytes
+    src = torch.empty(regions * region, dtype=torch.uint8, device=dev).random_()
+    order = torch.randperm(4 * experts, generator=torch.Generator().manual_seed(7))[:experts]
+    table = (order[:, None] * 16 + torch.arange(16)[None, :]).reshape(-1).to(torch.int32).to(dev)
+    acts = torch.zeros(32 * 4096, dtype=torch.uint8, device=dev)
+    out = torch.empty(groups * 256, dtype=torch.float32, device=dev)
+    sink = torch.zeros(groups, dtype=torch.int32, device=dev)
+    def launch(i: int):
+        at = src[(i % regions) * region:(i % regions + 1) * region]
+        _lib.check(_lib.lib().hb_debug_ring_skeleton(_lib.ptr(at), at.numel(), _lib.ptr(table), groups, _lib.ptr(acts), _lib.ptr(out), _lib.ptr(sink),
+                                                     _lib.stream()), "ring skeleton")
+
+    times = []
+    for rep in range(6):  # the launches of a repetition follow one another on the stream, as a graph's kernels do
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(2 * regions):
+            launch(i)
+        e1.record()
+        torch.cuda.synchronize()
+        if rep:
+            times.append(e0.elapsed_time(e1) / (2 * regions))
+    return groups * place_bytes / (median(times) * 1e-3) / 1e9
+
+
 def mfma_rate_tflops(dev, blocks: int = 2048, iters: int = 4096) -> float:
     """What a kernel that only multiplies gets from this device's matrix cores: BF16 16x16x32 MFMAs on registers, eight
     wavefronts a workgroup (hb_debug_mfma_rate), median of seven runs timed with events on the stream it runs on."""
@@ -597,6 +632,7 @@ def main() -> int:
     kernel_name = ("w3_fc12_kernel<fc1 gated + fc2>" if fused else "w3_fc1_route_one_kernel<route + fc1 gated>" if routed_in_fc1
                    else "w3_stream_kernel<fc1 gated, E4M3>" if args.e4m3 else "w3_stream_kernel<fc1 gated>")
     read_gbs = stream_read_gbs(dev)
+    skeleton_gbs = None if decode else ring_skeleton_gbs(dev, experts=round(mean(distinct)) + 1)
 
     m1 = None
     if not decode:  # the other half of the metric, in the same run: the layer at one token
@@ -642,7 +678,11 @@ def main() -> int:
                      # rocprofv3 --pmc on this workload (the summary under profiles/ states it), applied to this run's bytes
                      "traffic": None if ratio is None else ratio * launch_bytes, "launch_bytes": launch_bytes, "launch_ms": launch_ms,
                      "peak_measured": read_gbs, "frac_of_measured": achieved / read_gbs,
-                     "peak_measured_how": "plain streaming read of 1 GiB in this run (hb_debug_stream_read)"},
+                     "peak_measured_how": "plain streaming read of 1 GiB in this run (hb_debug_stream_read)",
+                     # fc1's traffic of this step without the arithmetic: blocks of 53 KB at expert-sized runs, four chunks
+                     # a wavefront through the two-slot LDS ring, activations beside them, the exchange and a store
+                     "skeleton": skeleton_gbs, "frac_of_skeleton": None if skeleton_gbs is None else achieved / skeleton_gbs,
+                     "skeleton_how": "the stream's requests without its arithmetic in this run (hb_debug_ring_skeleton)"},
         "layer_chain": {"algorithmic_bytes_per_step": step_bytes, "achieved_GBs": chain_gbs, "frac_of_hbm_peak": chain_gbs / HBM_PEAK_GBS,
                         "kernel_ms": kernel_ms},
         "m1": m1,

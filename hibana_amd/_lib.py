@@ -42,6 +42,7 @@ SIGNATURES = {
     "hb_debug_events": (_I, [_P, _I]),
     "hb_debug_trace": (_I, [_P]),
     "hb_debug_stream_read": (_I, [_P, _Z, _P, _P]),
+    "hb_debug_ring_skeleton": (_I, [_P, _Z, _P, _I, _P, _P, _P, _P]),
     "hb_debug_mfma_rate": (_L, [_I, _I, _P, _P]),
     "hb_w3_tiled_bytes": (_Z, [_L, _I]),
     "hb_w3_repack": (_I, [_P, _P, _L, _I, _I, _P, _P]),

@@ -270,6 +270,78 @@ extern "C" int hb_debug_stream_read(const void* src, size_t bytes, void* sink, v
   return launch_status();
 }
 
+// Measurement hook: the weight stream's traffic without its arithmetic - what its request structure alone gets from
+// this device. A workgroup of four wavefronts reads one 64-row block of sixteen 3328-byte chunks (53 248 bytes, at
+// place table[group] of `src`: a dependent read first, as the stream reads its plan entry), each wavefront four of
+// the chunks through a two-slot LDS ring (LDS-direct loads, read back with ds_read_b128, the next chunk but one asked
+// for after each read-back), with sixteen bytes of activations a lane and chunk beside them; then the K split's
+// exchange (sixteen floats a lane to LDS, a barrier, four partial sums back) and one store a lane. LDS a workgroup as
+// the stream's (four workgroups a compute unit).
+constexpr int SKELETON_CHUNK = W3_BLOCK_BYTES, SKELETON_PIECE = 4 * SKELETON_CHUNK, SKELETON_LDS = 40000;
+__global__ __launch_bounds__(256) void ring_skeleton_kernel(const uint8_t* __restrict__ src, const int32_t* __restrict__ table, int places,
+                                                            const u32x4_t* __restrict__ acts, float* __restrict__ out, uint32_t* __restrict__ sink) {
+  extern __shared__ __align__(16) uint8_t rings[];
+  typedef __attribute__((address_space(3))) uint8_t* lds_t;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t mine = (int64_t)blockIdx.x * 4 + wv;
+  const int64_t wave = (int64_t)min(max(table[blockIdx.x], 0), places - 1) * 4 + wv;
+  const lds_t slot0 = (lds_t)(rings + wv * 2 * SKELETON_CHUNK), slot1 = slot0 + SKELETON_CHUNK;
+  const __amdgpu_buffer_rsrc_t row = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(src + wave * SKELETON_PIECE), 0, SKELETON_PIECE, 0x00020000);
+  auto ask = [&](lds_t slot, int c) {
+    const uint32_t at = (uint32_t)c * SKELETON_CHUNK;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(row, slot, 16, 16u * lane, at, 0, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(row, slot, 16, 16u * lane, at, 1024, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(row, slot, 16, 16u * lane, at, 2048, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(row, slot, 4, 4u * lane, at, 3072, 2);
+  };
+  const u32x4_t* arow = acts + ((wave * 7) & 31) * 256 + (wv * 4) * 16 + (lane >> 2);  // one of 32 rows of 4 KB, this wavefront's K quarter
+  u32x4_t held[2];
+  ask(slot0, 0);
+  held[0] = arow[0];
+  ask(slot1, 1);
+  held[1] = arow[16];
+  uint32_t fold = 0;
+  const uint32_t base = (uint32_t)(uintptr_t)slot0 + 16u * lane;
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    u32x4_t a, b, d;
+    if (c < 3) {  // the next chunk's four loads and activation load may stay outstanding
+      asm volatile("s_waitcnt vmcnt(5)\n\tds_read_b128 %0, %3 offset:%4\n\tds_read_b128 %1, %3 offset:%5\n\tds_read_b128 %2, %3 offset:%6\n\ts_waitcnt lgkmcnt(0)"
+                   : "=&v"(a), "=&v"(b), "=&v"(d)
+                   : "v"(base), "n"((c & 1) * SKELETON_CHUNK), "n"((c & 1) * SKELETON_CHUNK + 1024), "n"((c & 1) * SKELETON_CHUNK + 2048)
+                   : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)\n\tds_read_b128 %0, %3 offset:%4\n\tds_read_b128 %1, %3 offset:%5\n\tds_read_b128 %2, %3 offset:%6\n\ts_waitcnt lgkmcnt(0)"
+                   : "=&v"(a), "=&v"(b), "=&v"(d)
+                   : "v"(base), "n"((c & 1) * SKELETON_CHUNK), "n"((c & 1) * SKELETON_CHUNK + 1024), "n"((c & 1) * SKELETON_CHUNK + 2048)
+                   : "memory");
+    }
+    if (c + 2 < 4) ask((c & 1) ? slot1 : slot0, c + 2);
+    fold ^= a.x ^ b.y ^ d.z ^ held[c & 1].x ^ held[c & 1].w;
+    if (c + 2 < 4) held[c & 1] = arow[16 * (c + 2)];
+  }
+  float* part = reinterpret_cast<float*>(rings) + wv * (2 * SKELETON_CHUNK / 4);
+#pragma unroll
+  for (int j = 0; j < 16; j++) part[j * 64 + lane] = __uint_as_float((fold + j) & 0x3fffffffu);
+  __syncthreads();
+  float v = 0.f;
+#pragma unroll
+  for (int k = 0; k < 4; k++) v += reinterpret_cast<const float*>(rings)[k * (2 * SKELETON_CHUNK / 4) + wv * 64 + lane];
+  out[mine * 64 + lane] = v;
+  if (fold == 0x9e3779b9u) sink[blockIdx.x] = fold;  // (practically never)
+}
+
+extern "C" int hb_debug_ring_skeleton(const void* src, size_t src_bytes, const int32_t* table, int groups, const void* acts, float* out, void* sink,
+                                      void* stream) {
+  if (!src || !table || !acts || !out || !sink) return HB_ENULL;
+  const int64_t places = (int64_t)(src_bytes / (4 * SKELETON_PIECE));
+  if (groups <= 0 || places <= 0 || places > 0x7fffffff || !aligned(src, 16) || !aligned(table, 4) || !aligned(acts, 16) || !aligned(out, 4) || !aligned(sink, 4))
+    return HB_EINVAL;
+  hipLaunchKernelGGL(ring_skeleton_kernel, dim3((unsigned)groups), dim3(256), SKELETON_LDS, as_stream(stream), static_cast<const uint8_t*>(src), table,
+                     (int)places, static_cast<const u32x4_t*>(acts), out, static_cast<uint32_t*>(sink));
+  return launch_status();
+}
+
 // Measurement hook: the rate this device's matrix cores give a kernel that does nothing else, the yardstick an expert
 // GEMM is held against. Every wavefront runs `iters` rounds of eight independent v_mfma_f32_16x16x32_bf16 (16 384
 // FLOP each) on registers; eight wavefronts a workgroup, two a SIMD.

@@ -66,6 +66,15 @@ int hb_debug_trace(void* buffer);
  * hold a weight stream's rate against. `sink`: at least bytes / 65536 + 1 uint32 (practically never written). */
 int hb_debug_stream_read(const void* src, size_t bytes, void* sink, void* stream);
 
+/* Measurement hook (no counterpart in the reference): the W3 weight stream's traffic without its arithmetic - what its
+ * request structure alone gets from this device, the ceiling to hold the stream's rate against. `groups` workgroups of
+ * four wavefronts each read one block of 53 248 bytes (sixteen 3328-byte chunks, four a wavefront through a two-slot
+ * LDS ring of LDS-direct loads) at place table[group] of `src` (places of 53 248 bytes, src_bytes / 53 248 of them; a
+ * table value outside is clamped), with a dependent read of the table first, sixteen bytes of `acts` (32 rows of 4 KB) a
+ * lane and chunk, the K split's exchange through LDS and one store a lane to `out` (groups x 256 floats). `sink`: at
+ * least `groups` uint32 (practically never written). */
+int hb_debug_ring_skeleton(const void* src, size_t src_bytes, const int32_t* table, int groups, const void* acts, float* out, void* sink, void* stream);
+
 /* Measurement hook (no counterpart in the reference): `blocks` workgroups of eight wavefronts each run `iters` rounds of
  * eight independent BF16 MFMAs (16x16x32) on registers - the rate this device's matrix cores give a kernel that does
  * nothing else, to hold an expert GEMM's rate against. Returns the launch's FLOP (negative: an error code negated).

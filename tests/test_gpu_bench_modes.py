@@ -35,6 +35,8 @@ def test_decode_modes(flags, kernel):
 def test_headline_modes():
     line = run("--no-cpu", "--headline-only", "--layers", "2", "--steps", "24", "--warmup", "4", "--copy-mib", "64")
     assert "w3_fc12_kernel" in line["roofline"]["kernel"] and line["cpu_baseline"] is None and line["m1"]["value"] > 0
+    roof = line["roofline"]  # the two yardsticks of the same run: a plain read, and the stream's requests without its arithmetic
+    assert roof["achieved"] < roof["skeleton"] < roof["peak_measured"] < roof["peak"]
     assert line["config"]["workload"].startswith("BASELINE config 3") and line["vs_baseline"] is None and line["dtype"] == "bf16"
     line = run("--e4m3", "--headline-only", "--layers", "2", "--steps", "24", "--warmup", "4")
     assert "E4M3" in line["metric"] and line["value"] > 0
