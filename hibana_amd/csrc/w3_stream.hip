@@ -291,76 +291,66 @@ struct FewActs8 {  // E4M3 activations: eight codes a lane and chunk, and the sc
 };
 
 // The four-row body on the two-plane form of the activations (split_row): E4M3 activations times the codebook's E4M3
-// bytes as v_perm_b32 delivers them, on v_mfma_f32_16x16x32_fp8_fp8 - no conversion of the weights at all. The sixteen
-// MFMA rows carry (32-group parity g) x (plane hi / lo) x (slot row i): A row 8 g + 4 hl + i holds plane hl of slot
-// row i over the k of groups g and g + 2 only. The MFMAs of groups 0 and 1 chain into one accumulator, those of groups
-// 2 and 3 into a second one; lane (q, r16) then holds, for its four slot rows, group q / 2 (second accumulator: 2 + q / 2),
-// plane q % 2, and folds that group's scale. Both planes are in the same units, so everything a lane and its three
-// neighbours in q hold for a slot row adds up: the second accumulator is added to the first after the last chunk and
-// the exchange of finish_few does the rest; the row's activation scale multiplies the result there.
+// bytes as v_perm_b32 delivers them, on v_mfma_f32_16x16x128_f8f6f4 - no conversion of the weights at all, and one
+// MFMA a plane for all of a 16-row tile's 128 k. The MFMA's k index (q, byte b of a lane's 32) is k = 32 (b / 8) + 8 q
+// + b % 8 of the chunk on both sides: the weights' eight selector dwords in their order, and for the activations the
+// lane's eight bytes of its own 32-group in dwords 2 g, 2 g + 1 with zeros in the other six - A row 4 g + t is slot row
+// t over group g only, so register i of lane (q, r16) of the result is group q's sum for slot row i and weight row r16,
+// as in the BF16 form. Both planes are in the same units and add in the MFMA's accumulator; the row's activation scale
+// multiplies the result in finish_few.
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+
 struct FewSplitActs {
   typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
   static constexpr int LOADS = 2;
-  u32x2_t held[2][2];   // [chunk parity][the lane's lower / upper group]: eight E4M3 bytes each
-  f32x4_t more[4];      // the second accumulator of each 16-row tile
-  bool upper;           // this lane's A row belongs to groups 1 and 3
-  uint32_t s8;          // where the lane's OUTPUT rows find their group's scale in a tile's scale dword
-  const uint8_t* at;    // the lane's bytes of its lower group in the wavefront's first chunk
+  u32x2_t held[2][2];   // [chunk parity][plane]: the lane's eight E4M3 bytes of its own group
+  int grp;
+  uint32_t q8;
+  const uint8_t* at;    // the lane's bytes of the upper plane in the wavefront's first chunk
   __device__ __forceinline__ void load(int slot, int i) {
     held[slot][0] = *reinterpret_cast<const u32x2_t*>(at + (int64_t)i * 256);
-    held[slot][1] = *reinterpret_cast<const u32x2_t*>(at + (int64_t)i * 256 + 64);
+    held[slot][1] = *reinterpret_cast<const u32x2_t*>(at + (int64_t)i * 256 + 128);
   }
   template <int EPI>
   __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int row0, int c0, int n, int lane) {
     const int q = lane >> 4, r16 = lane & 15;
-    upper = r16 >= 8;
-    s8 = 8 * (q >> 1);
-    at = p.a2 + activation_row_index<EPI>(p, sl, row0 + (r16 & 3)) * (2 * p.a_stride) + (int64_t)c0 * 256 + ((r16 >> 2) & 1) * 128 + (upper ? 32 : 0) + 8 * q;
-#pragma unroll
-    for (int t = 0; t < 4; t++) more[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    grp = r16 >> 2;
+    q8 = 8 * q;
+    at = p.a2 + activation_row_index<EPI>(p, sl, row0 + (r16 & 3)) * (2 * p.a_stride) + (int64_t)c0 * 256 + 32 * grp + 8 * q;
     load(0, 0);
     if (n > 1) load(1, 1);
   }
-  __device__ __forceinline__ void tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const long (&a)[4], f32x4_t& acc, f32x4_t& acc2,
-                                       uint32_t lut_lo, uint32_t lut_hi) const {
+  static __device__ __forceinline__ void tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const i32x8_t& upper, const i32x8_t& lower, f32x4_t& acc,
+                                              uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
     uint32_t sel[8];
     w3_selectors(q0, q1, q2, sel);
-    long b[4];
+    i32x8_t b;
 #pragma unroll
-    for (int j = 0; j < 4; j++) b[j] = fp8x8(__builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j]), __builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j + 1]));
-    f32x4_t lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
-    lo = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[0], b[0], lo, 0, 0, 0);
-    hi = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[2], b[2], hi, 0, 0, 0);
-    lo = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[1], b[1], lo, 0, 0, 0);
-    hi = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[3], b[3], hi, 0, 0, 0);
-    const uint32_t mine = scales >> s8;
-    const float s_lo = __builtin_amdgcn_cvt_f32_fp8(mine, 0), s_hi = __builtin_amdgcn_cvt_f32_fp8(mine, 2);
-    acc.x = fmaf(lo.x, s_lo, acc.x);
-    acc.y = fmaf(lo.y, s_lo, acc.y);
-    acc.z = fmaf(lo.z, s_lo, acc.z);
-    acc.w = fmaf(lo.w, s_lo, acc.w);
-    acc2.x = fmaf(hi.x, s_hi, acc2.x);
-    acc2.y = fmaf(hi.y, s_hi, acc2.y);
-    acc2.z = fmaf(hi.z, s_hi, acc2.z);
-    acc2.w = fmaf(hi.w, s_hi, acc2.w);
+    for (int j = 0; j < 8; j++) b[j] = (int)__builtin_amdgcn_perm(lut_hi, lut_lo, sel[j]);
+    f32x4_t part = {0.f, 0.f, 0.f, 0.f};
+    part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(upper, b, part, 0, 0, 0, 0, 0, 0);
+    part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(lower, b, part, 0, 0, 0, 0, 0, 0);
+    const float s = __builtin_amdgcn_cvt_f32_fp8(scales >> q8, 0);  // the scale of this lane's group
+    acc.x = fmaf(part.x, s, acc.x);
+    acc.y = fmaf(part.y, s, acc.y);
+    acc.z = fmaf(part.z, s, acc.z);
+    acc.w = fmaf(part.w, s, acc.w);
   }
   template <int ODD, bool MORE2, bool MORE1>
   __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
-    const long mine_lo = fp8x8(held[ODD][0].x, held[ODD][0].y), mine_hi = fp8x8(held[ODD][1].x, held[ODD][1].y);
-    // MFMA j (group j): the lane's bytes when its A row belongs to that group's parity, zero otherwise
-    const long a[4] = {upper ? 0L : mine_lo, upper ? mine_lo : 0L, upper ? 0L : mine_hi, upper ? mine_hi : 0L};
-    tile(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, a, acc0, more[0], sl.lut_lo, sl.lut_hi);
-    tile(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, a, acc1, more[1], sl.lut_lo, sl.lut_hi);
-    tile(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, a, acc2, more[2], sl.lut_lo, sl.lut_hi);
-    tile(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, a, acc3, more[3], sl.lut_lo, sl.lut_hi);
+    i32x8_t upper, lower;  // the lane's bytes in its group's two dwords, zero in the others
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      upper[2 * j] = grp == j ? (int)held[ODD][0].x : 0;
+      upper[2 * j + 1] = grp == j ? (int)held[ODD][0].y : 0;
+      lower[2 * j] = grp == j ? (int)held[ODD][1].x : 0;
+      lower[2 * j + 1] = grp == j ? (int)held[ODD][1].y : 0;
+    }
+    tile(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, upper, lower, acc0, sl.lut_lo, sl.lut_hi, q8);
+    tile(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, upper, lower, acc1, sl.lut_lo, sl.lut_hi, q8);
+    tile(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, upper, lower, acc2, sl.lut_lo, sl.lut_hi, q8);
+    tile(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, upper, lower, acc3, sl.lut_lo, sl.lut_hi, q8);
     if (MORE2) load(ODD, i + 2);
-  }
-  // after the last chunk: the two accumulators of a tile hold parts of the same sums
-  __device__ __forceinline__ void fold(f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3) const {
-    acc0 += more[0];
-    acc1 += more[1];
-    acc2 += more[2];
-    acc3 += more[3];
   }
 };
 
@@ -572,9 +562,7 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Sl
       scale = sl.rs[nb * 64 + lane];
       if (EPI == EPI_FC2) pairs.ask(p, sl, 0);
       xs.ask<EPI>(p, sl, 0);
-      FewSplitActs acts;
-      stream_block<EPI, FewSplitActs, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3, acts);
-      acts.fold(acc0, acc1, acc2, acc3);
+      stream_block<EPI, FewSplitActs, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
     }
     finish_few<EPI, false, true>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs, xs);
   } else if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
