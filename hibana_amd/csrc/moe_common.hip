@@ -1100,7 +1100,7 @@ extern "C" int hb_debug_events(void* const* events, int count) {
   return HB_OK;
 }
 
-extern "C" int hb_version(void) { return 1003; }  // minor: the entry points added since 1.0 (the small latent block, hb_nvfp4_gemm_ws, budgeted routing)
+extern "C" int hb_version(void) { return 1004; }  // minor: the entry points added since 1.0 (the small latent block, hb_nvfp4_gemm_ws, budgeted routing, the layer under a budget, the ring skeleton hook)
 
 extern "C" const char* hb_error_string(int code) {
   switch (code) {
