@@ -313,7 +313,7 @@ def dense_decode(args) -> dict:
             xr = torch.randn(rows, k, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
             yr = torch.empty(rows, n, dtype=torch.bfloat16, device=dev)
             need = lib.hb_nvfp4_gemm_workspace_bytes(rows, n, k)
-            ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+            ws = torch.zeros(max(need, 16), dtype=torch.uint8, device=dev)  # a workspace starts with its head zero
 
             def run(i: int):
                 _lib.check(lib.hb_nvfp4_gemm_ws(_lib.ptr(xr), rows, _lib.ptr(mats[i % args.layers]), 1.0 / 448.0, n, k, 0, _lib.ptr(yr), _lib.ptr(ws), need,
@@ -462,8 +462,8 @@ def ring_skeleton_gbs(dev, experts: int = 137, regions: int = 6) -> float:
     sink = torch.zeros(groups, dtype=torch.int32, device=dev)
     def launch(i: int):
         at = src[(i % regions) * region:(i % regions + 1) * region]
-        _lib.check(_lib.lib().hb_debug_ring_skeleton(_lib.ptr(at), at.numel(), _lib.ptr(table), groups, _lib.ptr(acts), _lib.ptr(out), _lib.ptr(sink),
-                                                     _lib.stream()), "ring skeleton")
+        _lib.check(_lib.lib().hb_debug_ring_skeleton(_lib.ptr(at), at.numel(), _lib.ptr(table), groups, _lib.ptr(acts), acts.numel(), _lib.ptr(out),
+                                                     out.numel() * 4, _lib.ptr(sink), sink.numel() * 4, _lib.stream()), "ring skeleton")
 
     times = []
     for rep in range(6):  # the launches of a repetition follow one another on the stream, as a graph's kernels do

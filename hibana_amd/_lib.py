@@ -40,9 +40,12 @@ SIGNATURES = {
     "hb_error_string": (C.c_char_p, [_I]),
     "hb_tune": (_I, [C.c_char_p, _I]),
     "hb_debug_events": (_I, [_P, _I]),
-    "hb_debug_trace": (_I, [_P]),
+    "hb_debug_trace": (_I, [_P, _L]),
     "hb_debug_stream_read": (_I, [_P, _Z, _P, _P]),
-    "hb_debug_ring_skeleton": (_I, [_P, _Z, _P, _I, _P, _P, _P, _P]),
+    "hb_debug_ring_skeleton": (_I, [_P, _Z, _P, _I, _P, _Z, _P, _Z, _P, _Z, _P]),
+    "hb_debug_workspace_layout": (_I, [_I, _I, _EX, _I, C.POINTER(C.c_int64)]),
+    "hb_workspace_reset": (_I, [_P, _Z, _P]),
+    "hb_workspace_status": (_I, [_P, C.POINTER(C.c_int32), _I, _P]),
     "hb_debug_mfma_rate": (_L, [_I, _I, _P, _P]),
     "hb_w3_tiled_bytes": (_Z, [_L, _I]),
     "hb_w3_repack": (_I, [_P, _P, _L, _I, _I, _P, _P]),
@@ -118,6 +121,39 @@ def ptr(t: torch.Tensor | None) -> int | None:
 
 def stream() -> int:
     return torch.cuda.current_stream().cuda_stream
+
+
+WORKSPACE_ZERO_BYTES = 1 << 20
+_workspaces: dict[tuple[int, int, str], torch.Tensor] = {}
+
+
+def workspace(device: torch.device, need: int, kind: str = "moe") -> torch.Tensor:
+    """A workspace of at least `need` bytes for a call on the current stream of `device`: one buffer a (device, stream,
+    kind of call), kept between calls and grown when a call needs more, handed over with its head zero as the library
+    asks (its arrival counters and fault word; every call leaves them zero again). Calls on one stream follow one
+    another, so they can share it; calls on different streams get different buffers and share nothing. `kind` keeps
+    apart calls that are in progress together on one stream (a latent block's workspace lives across several calls,
+    among them a routed one)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (index, torch.cuda.current_stream(device).cuda_stream, kind)
+    have = _workspaces.get(key)
+    if have is None or have.numel() < need:
+        have = torch.empty(max(need, 4096), dtype=torch.uint8, device=device)
+        have[:WORKSPACE_ZERO_BYTES].zero_()  # a fill kernel on the current stream (capturable); the rest needs no start value
+        _workspaces[key] = have
+    return have
+
+
+def workspace_status(ws: torch.Tensor | None) -> int:
+    """The fault word of a workspace (None: the library's own scratch) once the current stream's work is done: 0, or
+    HB_FAULT_* bits."""
+    word = C.c_int32(-1)
+    check(lib().hb_workspace_status(ptr(ws), C.byref(word), 1, stream()), "workspace_status")
+    return word.value
+
+
+def workspace_reset(ws: torch.Tensor | None) -> None:
+    check(lib().hb_workspace_reset(ptr(ws), 0 if ws is None else ws.numel(), stream()), "workspace_reset")
 
 
 def need_gpu(*tensors: torch.Tensor) -> None:

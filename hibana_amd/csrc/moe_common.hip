@@ -156,6 +156,95 @@ __device__ __forceinline__ void plan_few_pairs(const int32_t* ids, int pairs, in
   }
 }
 
+// What every form of the plan writes behind the experts' slots: the shared expert's slots and rows, "no rows" in the
+// entries the launches' grids reach beyond the last slot (a workgroup learns that it has nothing to do from its own
+// entry, without a second dependent read of the count), the slots' arrival counters at zero, the header.
+__device__ __forceinline__ void plan_tail(int32_t* __restrict__ plan, int32_t* __restrict__ order, int pairs, int shared_rows, int slot_rows, int slot_cap,
+                                          int slots, int distinct, int kept) {
+  const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
+  for (int s = threadIdx.x; s < shared_slots; s += blockDim.x) {
+    int32_t* entry = plan + PLAN_HEADER + 4 * s;
+    entry[0] = -1;
+    entry[1] = kept + s * slot_rows;
+    entry[2] = min(slot_rows, shared_rows - s * slot_rows);
+    entry[3] = 0;
+  }
+  for (int r = threadIdx.x; r < shared_rows; r += blockDim.x) order[kept + r] = pairs + r;
+  for (int s = slots + threadIdx.x; s < slot_cap; s += blockDim.x) {
+    int32_t* entry = plan + PLAN_HEADER + 4 * s;
+    entry[0] = entry[1] = entry[2] = entry[3] = 0;
+  }
+  for (int s = threadIdx.x; s < slot_cap; s += blockDim.x) plan_done(plan, slot_cap)[s * DONE_PITCH] = 0;
+  if (threadIdx.x == 0) {
+    plan[0] = slots;
+    plan[1] = distinct;
+    plan[2] = kept;
+  }
+}
+
+// The plan of a call of at most PLAN_ROWS_MAX rows in which no row names an expert twice (the library's own routing
+// of a decode or verify call), by one workgroup of PLAN_THREADS: an expert's rows are one bit each of a 64-bit word in
+// LDS (integer ORs: their order does not matter), its pair count is the word's population, and a pair's place among
+// its expert's is the population below its row's bit - ascending pair index, as the general form places them. One
+// trip to memory for the ids (every thread's loads asked for together), one scan, no per-tile matching. Writes
+// exactly what plan_work writes.
+constexpr int PLAN_ROWS_MAX = 64;
+constexpr int PLAN_ROWS_PER_THREAD = 4;  // 64 rows of at most 64 selections over 1024 threads
+__device__ __forceinline__ void plan_by_rows(const int32_t* ids, int rows, int topk, int e_lo, int e_n, int shared_rows, int32_t* __restrict__ plan,
+                                             int32_t* __restrict__ order, int slot_rows, int slot_cap, int* lds) {
+  uint32_t* occ_lo = reinterpret_cast<uint32_t*>(lds);  // [e_n] rows 0 .. 31 that name expert e
+  uint32_t* occ_hi = occ_lo + e_n;                      // [e_n] rows 32 .. 63
+  int* start = lds + 2 * e_n;                           // [e_n] first sorted position of expert e
+  int* scratch = start + e_n;                           // [3 * (PLAN_WAVES + 1)]
+  const int pairs = rows * topk;
+  int mine[PLAN_ROWS_PER_THREAD], row_of[PLAN_ROWS_PER_THREAD];
+#pragma unroll
+  for (int j = 0; j < PLAN_ROWS_PER_THREAD; j++) {  // asked for before anything else is done
+    const int q = threadIdx.x + j * PLAN_THREADS;
+    mine[j] = q < pairs ? load_through(&ids[q]) - e_lo : -1;
+  }
+  for (int e = threadIdx.x; e < 2 * e_n; e += PLAN_THREADS) occ_lo[e] = 0u;
+#pragma unroll
+  for (int j = 0; j < PLAN_ROWS_PER_THREAD; j++) row_of[j] = (threadIdx.x + j * PLAN_THREADS) / topk;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < PLAN_ROWS_PER_THREAD; j++) {
+    if (mine[j] < 0 || mine[j] >= e_n) mine[j] = -1;
+    if (mine[j] >= 0) atomicOr(row_of[j] < 32 ? &occ_lo[mine[j]] : &occ_hi[mine[j]], 1u << (row_of[j] & 31));
+  }
+  __syncthreads();
+  const int e = threadIdx.x;  // one thread an expert: the launch keeps e_n <= PLAN_THREADS
+  const int count = e < e_n ? __popc(occ_lo[e]) + __popc(occ_hi[e]) : 0;
+  const int my_slots = (count + slot_rows - 1) / slot_rows;
+  const bool heavy = 4 * count > slot_rows;
+  Scan3 tot;  // as in plan_work: rows; heavy slots with the distinct experts in the upper half; light slots
+  const Scan3 at = block_exclusive_scan3(Scan3{count, (heavy ? my_slots : 0) | (count > 0 ? 1 << 16 : 0), heavy ? 0 : my_slots}, scratch, &tot);
+  const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
+  const int kept = tot.a, distinct = tot.b >> 16, heavy_slots = tot.b & 0xffff;
+  const int slots = shared_slots + heavy_slots + tot.c;
+  if (e < e_n) {
+    start[e] = at.a;
+    const int my_slot = shared_slots + (heavy ? (at.b & 0xffff) : heavy_slots + at.c);
+    for (int s = 0; s < my_slots; s++) {
+      int32_t* entry = plan + PLAN_HEADER + 4 * (my_slot + s);
+      entry[0] = e;
+      entry[1] = at.a + s * slot_rows;
+      entry[2] = min(slot_rows, count - s * slot_rows);
+      entry[3] = 0;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < PLAN_ROWS_PER_THREAD; j++) {
+    if (mine[j] < 0) continue;
+    const int r = row_of[j];
+    const uint32_t lo = occ_lo[mine[j]], hi = occ_hi[mine[j]];
+    const int below = r < 32 ? __popc(lo & ((1u << r) - 1u)) : __popc(lo) + __popc(hi & ((1u << (r - 32)) - 1u));
+    order[start[mine[j]] + below] = threadIdx.x + j * PLAN_THREADS;
+  }
+  plan_tail(plan, order, pairs, shared_rows, slot_rows, slot_cap, slots, distinct, kept);
+}
+
 // The plan itself, by one workgroup of PLAN_THREADS (`group` of `groups` when many pairs are shared): `lds` is the
 // launch's dynamic LDS.
 template <bool WIDE>  // false: one workgroup (phase 0) and nothing of the shared form compiled in
@@ -268,26 +357,7 @@ __device__ __forceinline__ void plan_work(const int32_t* ids, int pairs, int e_l
     }
   }
   __syncthreads();
-  for (int s = threadIdx.x; s < shared_slots; s += PLAN_THREADS) {
-    int32_t* entry = plan + PLAN_HEADER + 4 * s;
-    entry[0] = -1;
-    entry[1] = kept + s * slot_rows;
-    entry[2] = min(slot_rows, shared_rows - s * slot_rows);
-    entry[3] = 0;
-  }
-  for (int r = threadIdx.x; r < shared_rows; r += PLAN_THREADS) order[kept + r] = pairs + r;
-  // entries the launches' grids reach beyond the last slot say "no rows": a workgroup learns that it has nothing to do
-  // from its own entry, without a second dependent read of the count
-  for (int s = slots + threadIdx.x; s < slot_cap; s += PLAN_THREADS) {
-    int32_t* entry = plan + PLAN_HEADER + 4 * s;
-    entry[0] = entry[1] = entry[2] = entry[3] = 0;
-  }
-  for (int s = threadIdx.x; s < slot_cap; s += PLAN_THREADS) plan_done(plan, slot_cap)[s * DONE_PITCH] = 0;
-  if (threadIdx.x == 0) {
-    plan[0] = slots;
-    plan[1] = distinct;
-    plan[2] = kept;
-  }
+  plan_tail(plan, order, pairs, shared_rows, slot_rows, slot_cap, slots, distinct, kept);
   if (phase == 2) return;
   }
   // stable placement: each wavefront walks its segment 64 pairs at a time; a lane's position is its expert's running
@@ -361,20 +431,18 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int32_t* i
 
 // Routing and plan of a verify-sized call in ONE launch: `route_groups` workgroups route ROUTE_GROUP_ROWS rows each (a
 // row a wavefront, spread over the device, as the routing launch does), and the one that finishes last plans - it
-// learns that it is the last from a ticket counter of the library (`route_tickets`, zero when the library is loaded and
-// put back to zero by every last arriver, as the split-K counters of the reference's dense kernel are,
-// hibana/kernels/csrc/w3_gemm.cu:230-240). A workgroup's ids are written through to memory and waited for before its
-// ticket is drawn, and the plan reads ids past its own L2 (store_through / load_through): no cache write-back, no
-// invalidate. Launches in flight together draw from different counters
-// (`ticket`: the host hands them out round-robin, ROUTE_TICKETS of them). Workgroups past the routing ones round the
-// job's activations, as in moe_plan_kernel.
-constexpr int ROUTE_TICKETS = 1024;
+// learns that it is the last from an arrival counter in the call's own workspace (plan[PLAN_TICKET]: zero when the
+// caller hands the workspace over, put back to zero by every last arriver, as the split-K counters of the reference's
+// dense kernel are, hibana/kernels/csrc/w3_gemm.cu:230-240), so calls in flight together, each on a workspace of its
+// own, share nothing. A workgroup's ids are written through to memory and waited for before its ticket is drawn, and
+// the plan reads ids past its own L2 (store_through / load_through): no cache write-back, no invalidate. Nobody
+// waits: a workgroup that is not the last leaves. `by_rows`: the rows name no expert twice and are at most
+// PLAN_ROWS_MAX (plan_by_rows). Workgroups past the routing ones round the job's activations, as in moe_plan_kernel.
 constexpr int ROUTE_GROUP_ROWS = 1;
-static __device__ unsigned int route_tickets[ROUTE_TICKETS];
 
 __global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int32_t* ids, int pairs, int e_lo, int e_n, int shared_rows,
                                                                       int32_t* __restrict__ plan, int32_t* __restrict__ order, RouteParams route,
-                                                                      int route_rows, int route_groups, int ticket, int slot_rows, int slot_cap,
+                                                                      int route_rows, int route_groups, int by_rows, int slot_rows, int slot_cap,
                                                                       QuantJob job) {
   extern __shared__ int lds[];
   __shared__ int last;
@@ -389,13 +457,18 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int3
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    const unsigned drawn = atomicAdd(&route_tickets[ticket], 1u);
+    unsigned* ticket = reinterpret_cast<unsigned*>(plan + PLAN_TICKET);
+    const unsigned drawn = atomicAdd(ticket, 1u);
     last = drawn == (unsigned)route_groups - 1u;
-    if (last) route_tickets[ticket] = 0u;  // every other workgroup of this launch has drawn: the counter is free again
+    if (last) store_through(plan + PLAN_TICKET, 0);  // every other workgroup of this launch has drawn: the counter is zero for the next call
   }
   __syncthreads();
   if (!last) return;  // the last arriver: every row's ids are in memory, and the plan reads them from there (load_through)
-  plan_work<false>(ids, pairs, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, nullptr, 1, 0, 0, lds);
+  if (by_rows) {
+    plan_by_rows(ids, route_rows, route.k, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, lds);
+  } else {
+    plan_work<false>(ids, pairs, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, nullptr, 1, 0, 0, lds);
+  }
 }
 
 // Budgeted selection and the plan of its ids in one launch: the selection is one workgroup's work already, and so is
@@ -708,8 +781,7 @@ void moe_launch_quant_groups(const QuantJob& job, hipStream_t stream) {
   HB_LAUNCH(quant_groups_kernel, dim3(groups), dim3(256), 0, stream, job);
 }
 
-static std::atomic<unsigned> g_route_ticket_next{0};
-static std::atomic<int> g_route_plan_fused{0};  // hb_tune("route_plan", 2): routing and plan as two launches
+static std::atomic<int> g_route_plan_fused{0};  // hb_tune("route_plan", 2): routing and plan as two launches; 1: the general plan also where plan_by_rows serves
 int moe_tune(const char* key, int value) {
   if (strcmp(key, "route_plan") || value < 0 || value > 2) return HB_EINVAL;
   g_route_plan_fused.store(value, std::memory_order_relaxed);
@@ -750,9 +822,10 @@ static int launch_route_plan(const RouteParams& rp, int m, int e_lo, int e_n, in
   if (m > ROUTE_FUSED_ROWS && pairs < PLAN_WIDE_PAIRS && g_route_plan_fused.load(std::memory_order_relaxed) != 2) {
     // a verify-sized call: the routing spread over the device, the plan by the workgroup that finishes last
     const int groups = (m + ROUTE_GROUP_ROWS - 1) / ROUTE_GROUP_ROWS;
-    const int ticket = (int)(g_route_ticket_next.fetch_add(1u, std::memory_order_relaxed) % ROUTE_TICKETS);
+    // rows that name no expert twice: every row is real (a padded row repeats one id over its slots)
+    const int by_rows = !rp.slots && m <= PLAN_ROWS_MAX && rp.k <= 64 && g_route_plan_fused.load(std::memory_order_relaxed) != 1;
     HB_LAUNCH(moe_route_plan_kernel, dim3((unsigned)groups + plan_groups(job) - 1u), dim3(PLAN_THREADS), plan_lds, stream, rp.ids, (int)pairs, e_lo, e_n,
-              shared_rows, ws.plan, ws.order, rp, m, groups, ticket, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows),
+              shared_rows, ws.plan, ws.order, rp, m, groups, by_rows, slot_rows, (int)moe_max_slots(pairs, e_n, shared_rows, slot_rows),
               job ? *job : QuantJob{});
     return HB_OK;
   }
@@ -1084,10 +1157,20 @@ extern "C" int hb_route_sigmoid_topk(const float* fused, int64_t stride, const f
   return launch_status();
 }
 
-static std::atomic<int64_t*> g_trace{nullptr};
-int64_t* hb::moe_trace_buffer() { return g_trace.load(std::memory_order_relaxed); }
-extern "C" int hb_debug_trace(void* buffer) {
-  g_trace.store(static_cast<int64_t*>(buffer), std::memory_order_relaxed);
+static std::mutex g_trace_lock;
+static int64_t* g_trace = nullptr;
+static int64_t g_trace_records = 0;
+int64_t* hb::moe_trace_buffer(int64_t* records) {
+  std::lock_guard<std::mutex> hold(g_trace_lock);
+  *records = g_trace_records;
+  return g_trace;
+}
+#ifndef HB_NO_DEBUG_HOOKS
+extern "C" int hb_debug_trace(void* buffer, int64_t records) {
+  if (records < 0 || !aligned(buffer, 8)) return HB_EINVAL;
+  std::lock_guard<std::mutex> hold(g_trace_lock);
+  g_trace = records > 0 ? static_cast<int64_t*>(buffer) : nullptr;
+  g_trace_records = g_trace ? records : 0;
   return HB_OK;
 }
 
@@ -1099,8 +1182,9 @@ extern "C" int hb_debug_events(void* const* events, int count) {
   g_events_armed.store(count > 0, std::memory_order_relaxed);
   return HB_OK;
 }
+#endif
 
-extern "C" int hb_version(void) { return 1004; }  // minor: the entry points added since 1.0 (the small latent block, hb_nvfp4_gemm_ws, budgeted routing, the layer under a budget, the ring skeleton hook)
+extern "C" int hb_version(void) { return 1005; }  // minor: the entry points added since 1.0 (the small latent block, hb_nvfp4_gemm_ws, budgeted routing, the layer under a budget, the ring skeleton hook, hb_workspace_reset / hb_workspace_status with the counters in the caller's workspace)
 
 extern "C" const char* hb_error_string(int code) {
   switch (code) {

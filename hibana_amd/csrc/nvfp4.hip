@@ -501,13 +501,14 @@ static int nvfp4_gemm(const void* x, int m, const void* tiled, float global_scal
   // is shared among workgroups
   int ks = workspace && m > TILE_SPLIT_ROWS ? tile_split(m, p.n_blocks, p.chunks) : 1;
   if (g_nvfp4_tile_ks && workspace) ks = std::min(g_nvfp4_tile_ks.load(), p.chunks);
-  if (tile_partial_bytes(m, p.n_blocks, ks) > workspace_bytes) ks = 1;
+  if (tile_partial_bytes(m, p.n_blocks, ks) > workspace_bytes || tile_ticket_bytes(m, p.n_blocks) > HB_WORKSPACE_ZERO_BYTES) ks = 1;
   if (tile_takes(m, k) && tile_writes(y, false) && (g_nvfp4_tile == 1 || (g_nvfp4_tile == 0 && (ks > 1 || tile_serves_dense(m, p.n_blocks))))) {
     const int64_t tile_slots = (m + TILE_ROWS - 1) / TILE_ROWS;
     if (ks > 1) {
       p.tile_ks = ks;
       p.tile_mt = tile_partial_mt(m);
-      p.partial = static_cast<float*>(workspace);
+      p.tile_tickets = static_cast<uint32_t*>(workspace) + PLAN_HEADER;
+      p.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + tile_ticket_bytes(m, p.n_blocks));
     }
     if (int e = relu2 ? launch_tile<TileNvfp4, EPI_DENSE_RELU2>(p, tile_slots, m, stream) : launch_tile<TileNvfp4, EPI_DENSE>(p, tile_slots, m, stream)) return e;
     return launch_status();

@@ -14,7 +14,12 @@ constexpr bool epi_dense(int epi) { return epi == EPI_DENSE || epi == EPI_DENSE_
 constexpr bool epi_gathers(int epi) { return epi == EPI_FC1_GATED || epi == EPI_FC1_RELU2; }  // activation rows found through `order`
 constexpr int ROWS_PER_SLOT = 16;
 constexpr int MOE_WIDE_ROWS = 1024;  // rows from which a routed sum keeps its pair outputs in BF16 (the reference's WIDE_ROWS)
-constexpr int PLAN_HEADER = 16;  // plan[0] = slots, plan[1] = distinct experts, plan[2] = routed pairs kept
+constexpr int PLAN_HEADER = 16;  // plan[0] = slots, plan[1] = distinct experts, plan[2] = routed pairs kept, then the two words below
+// Two words of a workspace's head that no launch initializes: the caller hands the workspace over zero-filled once, and
+// every call leaves them as the next one needs them.
+constexpr int PLAN_TICKET = 3;  // the arrival counter of a launch whose last workgroup plans: zero between calls (the last arriver puts it back)
+constexpr int PLAN_FAULT = 4;   // sticky: a kernel whose bounded wait gave up ors its HB_FAULT_* bit in; only hb_workspace_reset clears it
+constexpr int WAIT_SPINS = 1 << 20;  // polls (about a second) before a wait gives up
 
 struct StreamParams {
   const uint8_t* w;       // tile layout, expert 0
@@ -49,10 +54,13 @@ struct StreamParams {
   int no_few;             // W3 stream: slots of at most four rows take the sixteen-row body too
   float* partial;         // tile kernel with K shared among workgroups: their partial tiles (see tile_kernel.hpp)
   int tile_ks, tile_mt;   // ... the workgroups a tile (1: none), the 16-row tiles a partial region holds
-  int tile_ticket;        // ... and the first of the launch's arrival counters
+  uint32_t* tile_tickets; // ... and the tiles' arrival counters (one a tile, in the caller's workspace: zero between calls)
   int64_t* trace;         // measurement hook (hb_debug_trace): a record a workgroup, else null
+  int64_t trace_records;  // ... and the records it holds
   int32_t* done;          // fc1 and fc2 in one launch: the slots' arrival counters (plan_done), else null
   int done_need;          // ... and the fc1 workgroups a slot has
+  int wait_spins;         // ... and the polls after which a wait for them gives up
+  int32_t* fault;         // ... which it records here (the workspace's PLAN_FAULT word)
 };
 
 // Device-scope accesses that do not rest in the compute die's own L2: a store that is written through to memory, a
@@ -75,12 +83,17 @@ __device__ __forceinline__ void store_through(uint16_t* at, uint16_t v) { __hip_
 constexpr int DONE_PITCH = 32;
 __host__ __device__ inline int32_t* plan_done(int32_t* plan, int64_t slot_cap) { return plan + (PLAN_HEADER + 4 * slot_cap + 31) / 32 * 32; }
 
-// Waits (every lane of the wavefront together) until the counter has reached `need`. The spin is bounded: a count that
-// never comes - it cannot, short of a fault elsewhere - ends the wait after about a second and the results are wrong,
-// but every wavefront still leaves.
-__device__ __forceinline__ void await_count(const int32_t* at, int need) {
-  for (int spins = 0; load_through(at) < need && spins < (1 << 20); spins++) __builtin_amdgcn_s_sleep(8);
+// Waits (every lane of the wavefront together) until the counter has reached `need`; false if it has not after `spins`
+// polls. The wait is bounded so that every wavefront leaves whatever happens elsewhere; a caller that gets false must
+// not use what the count guards (it records the fault and skips its work).
+__device__ __forceinline__ bool await_count(const int32_t* at, int need, int spins) {
+  bool there = load_through(at) >= need;
+  for (int n = 0; !there && n < spins; n++) {
+    __builtin_amdgcn_s_sleep(8);
+    there = load_through(at) >= need;
+  }
   asm volatile("" ::: "memory");  // what the count guards is read after it
+  return there;
 }
 
 // The epilogue's roundings use the hardware FP32 -> BF16 conversion (round to nearest even).
@@ -591,7 +604,7 @@ __device__ __forceinline__ float combine_shared(float routed, float g, float sha
 // Measurement hook: the caller's next (start, stop) event pair, if any is armed. A kernel launched through HB_LAUNCH
 // then carries the pair: the runtime stamps the two events with that kernel's own begin and end.
 bool moe_next_events(hipEvent_t* start, hipEvent_t* stop);
-int64_t* moe_trace_buffer();  // hb_debug_trace's buffer, or null
+int64_t* moe_trace_buffer(int64_t* records);  // hb_debug_trace's buffer and its capacity in records, or null
 
 #define HB_LAUNCH(kernel, grid, block, lds, stream, ...)                                            \
   do {                                                                                              \

@@ -58,10 +58,9 @@ __device__ __forceinline__ void stage_tile(const StreamParams& p, const uint32_t
 // (stores written through to memory and waited for: a release at device scope, which writes back the whole L2, costs
 // each workgroup tens of microseconds here), counts itself on the tile's arrival counter, and the one that arrives
 // last (an acquire, then ordinary loads) adds all the partial tiles in the order of z - the same sum whichever it is -
-// and runs the epilogue. The counters are the
-// library's (tile_tickets: zero between launches, put back by every last arriver; a launch takes a range of them).
-constexpr int TILE_TICKETS = 1 << 16;
-static __device__ unsigned int tile_tickets[TILE_TICKETS];
+// and runs the epilogue. The counters (p.tile_tickets, one a tile) lie at the head of the caller's workspace, ahead of
+// the partial tiles: zero when the caller hands the workspace over, put back to zero by every last arriver, so calls in
+// flight together on workspaces of their own share nothing.
 
 __device__ __forceinline__ void store_through16(f32x4_t* at, const f32x4_t& v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(at), "v"(v) : "memory");
@@ -163,7 +162,7 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
     __syncthreads();
     int* last = reinterpret_cast<int*>(rowtab);  // the row table has served
     if (threadIdx.x == 0) {
-      unsigned int* ticket = &tile_tickets[(p.tile_ticket + tile) & (TILE_TICKETS - 1)];
+      unsigned int* ticket = p.tile_tickets + tile;
       const unsigned drawn = atomicAdd(ticket, 1u);
       *last = drawn == (unsigned)p.tile_ks - 1u;
       if (*last) *ticket = 0u;
@@ -267,8 +266,6 @@ inline bool tile_writes(const void* out, bool f32) { return aligned(out, f32 ? 1
 
 // `slots`: the grid's second dimension (routed: the plan's upper bound; dense: ceil(m / TILE_ROWS)); `a_rows`: rows of
 // the activation matrix.
-static std::atomic<unsigned> g_tile_ticket_next{0};
-
 // Workgroups a tile for a dense call of m rows (K shared among them), given room for their partial tiles: about four
 // hundred workgroups in all (measured at 25600 x 5120: the best count from 24 to 128 rows), each with at least four
 // chunks. 1: the call has two hundred tiles or more and fills the device alone.
@@ -279,9 +276,12 @@ inline int tile_split(int m, int n_blocks, int chunks) {
 }
 constexpr int TILE_SPLIT_ROWS = 20;  // up to here two passes of the weight stream are the faster
 inline int tile_partial_mt(int m) { return (std::min(m, TILE_ROWS) + 15) / 16; }
+inline int64_t tile_count(int m, int n_blocks) { return (int64_t)((n_blocks + 3) / 4) * ((m + TILE_ROWS - 1) / TILE_ROWS); }
+// The workspace of a call whose tiles share K: the tiles' arrival counters (a multiple of 256 bytes), then the partial tiles.
+// (behind the PLAN_HEADER words every workspace begins with, so that the fault word means the same in all of them)
+inline size_t tile_ticket_bytes(int m, int n_blocks) { return ((size_t)(PLAN_HEADER + tile_count(m, n_blocks)) * sizeof(uint32_t) + 255) & ~(size_t)255; }
 inline size_t tile_partial_bytes(int m, int n_blocks, int ks) {
-  const int64_t tiles = (int64_t)((n_blocks + 3) / 4) * ((m + TILE_ROWS - 1) / TILE_ROWS);
-  return ks > 1 ? (size_t)tiles * ks * 4 * tile_partial_mt(m) * 4 * 64 * sizeof(f32x4_t) : 0;
+  return ks > 1 ? tile_ticket_bytes(m, n_blocks) + (size_t)tile_count(m, n_blocks) * ks * 4 * tile_partial_mt(m) * 4 * 64 * sizeof(f32x4_t) : 0;
 }
 
 template <class Fmt, int EPI>
@@ -291,8 +291,7 @@ static int launch_tile(StreamParams& p, int64_t slots, int64_t a_rows, hipStream
   const unsigned groups = (unsigned)((p.n_blocks + 3) / 4);
   const int ks = p.tile_ks > 1 ? p.tile_ks : 1;
   if (ks > 1) {
-    if (!p.partial || ks > p.chunks || (int64_t)groups * slots > TILE_TICKETS) return HB_EINVAL;
-    p.tile_ticket = (int)(g_tile_ticket_next.fetch_add(groups * (unsigned)slots, std::memory_order_relaxed) & (TILE_TICKETS - 1));
+    if (!p.partial || !p.tile_tickets || ks > p.chunks) return HB_EINVAL;
   }
   const dim3 grid(groups, (unsigned)slots, (unsigned)ks);
   HB_LAUNCH((tile_kernel<Fmt, EPI>), grid, dim3(256), 2 * TILE_BUF + TILE_ROWS * sizeof(int32_t), stream, p);

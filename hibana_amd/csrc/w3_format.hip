@@ -261,6 +261,7 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t* __restr
   if (fold == 0x9e3779b9u) sink[blockIdx.x] = fold;  // (practically never: the loads stay, the store does not cost)
 }
 
+#ifndef HB_NO_DEBUG_HOOKS
 extern "C" int hb_debug_stream_read(const void* src, size_t bytes, void* sink, void* stream) {
   if (!src || !sink) return HB_ENULL;
   if (bytes == 0 || bytes % 16384 || !aligned(src, 16) || !aligned(sink, 4)) return HB_EINVAL;
@@ -269,6 +270,7 @@ extern "C" int hb_debug_stream_read(const void* src, size_t bytes, void* sink, v
                      static_cast<uint32_t*>(sink));
   return launch_status();
 }
+#endif
 
 // Measurement hook: the weight stream's traffic without its arithmetic - what its request structure alone gets from
 // this device. A workgroup of four wavefronts reads one 64-row block of sixteen 3328-byte chunks (53 248 bytes, at
@@ -331,16 +333,20 @@ __global__ __launch_bounds__(256) void ring_skeleton_kernel(const uint8_t* __res
   if (fold == 0x9e3779b9u) sink[blockIdx.x] = fold;  // (practically never)
 }
 
-extern "C" int hb_debug_ring_skeleton(const void* src, size_t src_bytes, const int32_t* table, int groups, const void* acts, float* out, void* sink,
-                                      void* stream) {
+#ifndef HB_NO_DEBUG_HOOKS
+extern "C" int hb_debug_ring_skeleton(const void* src, size_t src_bytes, const int32_t* table, int groups, const void* acts, size_t acts_bytes, float* out,
+                                      size_t out_bytes, void* sink, size_t sink_bytes, void* stream) {
   if (!src || !table || !acts || !out || !sink) return HB_ENULL;
   const int64_t places = (int64_t)(src_bytes / (4 * SKELETON_PIECE));
   if (groups <= 0 || places <= 0 || places > 0x7fffffff || !aligned(src, 16) || !aligned(table, 4) || !aligned(acts, 16) || !aligned(out, 4) || !aligned(sink, 4))
     return HB_EINVAL;
+  // what the kernel touches: 32 activation rows of 4 KB, 256 floats of output and one sink word a workgroup
+  if (acts_bytes < 32 * 4096 || out_bytes < (size_t)groups * 256 * sizeof(float) || sink_bytes < (size_t)groups * sizeof(uint32_t)) return HB_EINVAL;
   hipLaunchKernelGGL(ring_skeleton_kernel, dim3((unsigned)groups), dim3(256), SKELETON_LDS, as_stream(stream), static_cast<const uint8_t*>(src), table,
                      (int)places, static_cast<const u32x4_t*>(acts), out, static_cast<uint32_t*>(sink));
   return launch_status();
 }
+#endif
 
 // Measurement hook: the rate this device's matrix cores give a kernel that does nothing else, the yardstick an expert
 // GEMM is held against. Every wavefront runs `iters` rounds of eight independent v_mfma_f32_16x16x32_bf16 (16 384
@@ -366,10 +372,12 @@ __global__ __launch_bounds__(512) void mfma_rate_kernel(int iters, float* __rest
   if (fold == 12345.678f) sink[blockIdx.x] = fold;  // (practically never: the products stay, the store does not cost)
 }
 
+#ifndef HB_NO_DEBUG_HOOKS
 extern "C" int64_t hb_debug_mfma_rate(int blocks, int iters, void* sink, void* stream) {
-  if (!sink) return -HB_ENULL;
-  if (blocks <= 0 || blocks > 65536 || iters <= 0 || iters > (1 << 20) || !aligned(sink, 4)) return -HB_EINVAL;
+  if (!sink) return HB_ENULL;  // the HB_E* codes are negative themselves
+  if (blocks <= 0 || blocks > 65536 || iters <= 0 || iters > (1 << 20) || !aligned(sink, 4)) return HB_EINVAL;
   hipLaunchKernelGGL(mfma_rate_kernel, dim3((unsigned)blocks), dim3(512), 0, as_stream(stream), iters, static_cast<float*>(sink));
-  if (launch_status() != HB_OK) return -HB_ELAUNCH;
+  if (launch_status() != HB_OK) return HB_ELAUNCH;
   return (int64_t)blocks * 8 * iters * 8 * 16384;  // the launch's FLOP
 }
+#endif

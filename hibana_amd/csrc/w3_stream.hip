@@ -637,10 +637,16 @@ __global__ __launch_bounds__(1024) void w3_fc1_route_one_kernel(StreamParams p, 
 // first every fc1 workgroup (slot-major, the slot table's order), then every fc2 workgroup. A slot's fc2 needs all of
 // the slot's h, that is all `groups1` fc1 workgroups of the slot: each of those, once its h is in memory (write-through
 // stores, waited for), adds one to the slot's arrival counter (plan_done: zero from the plan), and the slot's fc2
-// workgroups ask for their first weight blocks, then wait for the counter before they touch h (await_count, in the
-// bodies' start). fc2 workgroups cannot starve fc1: the hardware starts a grid's workgroups in index order, so when an
-// fc2 workgroup waits, every fc1 workgroup has started, and an fc1 workgroup waits for nothing; should that order ever
-// fail to hold, await_count's bound ends the wait. Same sums in the same order as the two launches: the same bits.
+// workgroups wait for the counter before they ask for anything (one wavefront polls with loads that bypass the L2, the
+// others stand at a barrier). What fc2 then reads of h it reads with ordinary loads: the lines were written through to
+// memory before the count, and this compute die's L2 cannot hold an older copy of them, because every launch starts
+// with its L2 invalidated and no workgroup of this launch reads a slot's h before the slot's count is complete (h rows
+// are whole 256-byte multiples on 256-byte boundaries, so no line of h is shared with anything read earlier).
+// fc2 workgroups cannot starve fc1: the hardware starts a grid's workgroups in index order, so when an fc2 workgroup
+// waits, every fc1 workgroup has started, and an fc1 workgroup waits for nothing. HIP does not promise that order;
+// should it ever fail to hold, await_count's bound ends the wait, the workgroup records HB_FAULT_WAIT in the
+// workspace's fault word (hb_workspace_status reads it) and leaves without storing anything. hb_tune("moe_fused", 2)
+// runs the two layers as two launches, which wait for nothing. Same sums in the same order either way: the same bits.
 //
 // Order of the grid: slot-major, fc2 of a slot `lag` slots behind its fc1 - fc1(0) .. fc1(lag - 1), then fc1(s), fc2(s -
 // lag) for s = lag .., then the last `lag` slots' fc2. With `lag` about the slots whose workgroups fill the device once,
@@ -687,13 +693,23 @@ __global__ __launch_bounds__(1024) void w3_fc12_kernel(StreamParams p1, StreamPa
     const Slot sl = slot_of<EPI_FC2>(p2, slot);
     if (sl.rows <= 0) return;
     rows = sl.rows;
-    // one wavefront polls for the workgroup; the others wait at the barrier
-    if (threadIdx.x < 64) await_count(p2.done + slot * DONE_PITCH, p2.done_need);
+    // one wavefront polls for the workgroup; the others wait at the barrier and learn the outcome through LDS
+    int* outcome = reinterpret_cast<int*>(rings);
+    if (threadIdx.x < 64) {
+      const bool there = await_count(p2.done + slot * DONE_PITCH, p2.done_need, p2.wait_spins);
+      if (threadIdx.x == 0) {
+        *outcome = there;
+        if (!there) atomicOr(p2.fault, HB_FAULT_WAIT);  // the caller reads it with hb_workspace_status
+      }
+    }
     __syncthreads();
+    const bool there = *outcome != 0;
+    __syncthreads();  // read by everyone before the rings take the memory
+    if (!there) return;  // h is not known to be complete: this workgroup's outputs stay as they were
     if (p1.trace) t1 = (int64_t)wall_clock64();
     stream_workgroup<EPI_FC2, false, false>(p2, sl, id, rings);
   }
-  if (p1.trace && threadIdx.x == 0) {  // measurement hook: start, end of the wait, end (100 MHz ticks), rows
+  if (p1.trace && threadIdx.x == 0 && (int64_t)blockIdx.x < p1.trace_records) {  // measurement hook: start, end of the wait, end (100 MHz ticks), rows
     int64_t* rec = p1.trace + 4 * (int64_t)blockIdx.x;
     rec[0] = t0;
     rec[1] = t1;
@@ -806,7 +822,7 @@ struct TileW3 {
 
 // ---------------------------------------------------------------------------------------------------- host side
 struct Tuning {  // hb_tune's knobs: relaxed atomics, so a knob set from one thread while another launches is a plain race-free read
-  std::atomic<int> w3_tile{0}, w3_few{0}, w3_ksplit{0}, w3_nbw{0}, moe_fc1_ksplit{0}, moe_fc1_nbw{0}, moe_fc2_ksplit{0}, moe_fc2_nbw{0}, moe_one{0}, moe_split{0}, moe_fused{0}, moe_lag{0};
+  std::atomic<int> w3_tile{0}, w3_few{0}, w3_ksplit{0}, w3_nbw{0}, moe_fc1_ksplit{0}, moe_fc1_nbw{0}, moe_fc2_ksplit{0}, moe_fc2_nbw{0}, moe_one{0}, moe_split{0}, moe_fused{0}, moe_lag{0}, fault_inject{0};
 };
 static Tuning g_tune;
 
@@ -850,6 +866,7 @@ static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Lau
 
 using namespace hb;
 
+#ifndef HB_NO_DEBUG_HOOKS
 extern "C" int hb_tune(const char* key, int value) {
   if (!key) return HB_ENULL;
   struct {
@@ -857,7 +874,7 @@ extern "C" int hb_tune(const char* key, int value) {
     std::atomic<int>* slot;
   } table[] = {{"w3_tile", &g_tune.w3_tile}, {"w3_few", &g_tune.w3_few}, {"w3_ksplit", &g_tune.w3_ksplit},           {"w3_nbw", &g_tune.w3_nbw},
                {"moe_fc1_ksplit", &g_tune.moe_fc1_ksplit}, {"moe_fc1_nbw", &g_tune.moe_fc1_nbw},
-               {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}, {"moe_one", &g_tune.moe_one}, {"moe_split", &g_tune.moe_split}, {"moe_fused", &g_tune.moe_fused}, {"moe_lag", &g_tune.moe_lag}};
+               {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}, {"moe_one", &g_tune.moe_one}, {"moe_split", &g_tune.moe_split}, {"moe_fused", &g_tune.moe_fused}, {"moe_lag", &g_tune.moe_lag}, {"fault_inject", &g_tune.fault_inject}};
   for (auto& t : table)
     if (!strcmp(t.name, key)) {
       if (value < 0 || value > 16) return HB_EINVAL;
@@ -867,6 +884,7 @@ extern "C" int hb_tune(const char* key, int value) {
   if (moe_tune(key, value) == HB_OK) return HB_OK;
   return nvfp4_tune(key, value);
 }
+#endif
 
 extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, void* y, void* stream) {
   if (!x || !tiled || !row_scale || !y) return HB_ENULL;
@@ -1080,8 +1098,14 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
       const int64_t total = slots * (groups1 + groups2);
       if (total <= 0x7fffffff) {
         q1.done = q2.done = plan_done(ws.plan, slots);
-        q1.trace = moe_trace_buffer();
+        q1.trace = moe_trace_buffer(&q1.trace_records);
         q1.done_need = q2.done_need = groups1;
+        q2.wait_spins = WAIT_SPINS;
+        q2.fault = ws.plan + PLAN_FAULT;
+        if (g_tune.fault_inject == 1) {  // a test of the give-up path: a count one above what can arrive, and a wait of a few polls
+          q2.done_need = groups1 + 1;
+          q2.wait_spins = 8;
+        }
         const int waves = q1.ks * q1.nbw;
         // about the slots whose workgroups fill the device once (four workgroups of four wavefronts a compute unit)
         const int lag_tuned = g_tune.moe_lag.load();
@@ -1145,6 +1169,22 @@ extern "C" size_t hb_w3_moe_workspace_bytes(int m, int topk, const hb_w3_experts
   if (!routed || m <= 0 || topk <= 0 || check_experts(routed) != HB_OK) return 0;
   return moe_carve(nullptr, m, topk, routed->experts, routed->inter, routed->hidden_out, shared, routed->hidden).bytes;
 }
+
+#ifndef HB_NO_DEBUG_HOOKS
+extern "C" int hb_debug_workspace_layout(int m, int topk, const hb_w3_experts* routed, int shared, int64_t* offsets) {
+  if (!routed || !offsets) return HB_ENULL;
+  if (m <= 0 || topk <= 0 || check_experts(routed) != HB_OK) return HB_EINVAL;
+  char* base = reinterpret_cast<char*>(uintptr_t(1) << 20);  // any address: only differences are returned
+  const MoeWorkspace ws = moe_carve(base, m, topk, routed->experts, routed->inter, routed->hidden_out, shared, routed->hidden);
+  offsets[0] = reinterpret_cast<char*>(ws.plan) - base;
+  offsets[1] = reinterpret_cast<char*>(ws.order) - base;
+  offsets[2] = reinterpret_cast<char*>(ws.h) - base;
+  offsets[3] = reinterpret_cast<char*>(ws.y) - base;
+  offsets[4] = reinterpret_cast<char*>(plan_done(ws.plan, moe_max_slots((int64_t)m * topk, routed->experts, shared ? m : 0))) - base;
+  offsets[5] = moe_max_slots((int64_t)m * topk, routed->experts, shared ? m : 0);
+  return HB_OK;
+}
+#endif
 
 extern "C" int hb_w3_moe(const hb_w3_experts* routed, const void* x, const int32_t* ids, const float* weights, int m, int topk, int mode,
                          void* out, void* workspace, size_t workspace_bytes, void* stream) {
@@ -1262,6 +1302,35 @@ extern "C" int hb_w3_moe_layer_static(const hb_w3_experts* routed, const hb_w3_e
   void* ptr = scratch_of_current_device();
   if (!ptr) return HB_ELAUNCH;
   return moe_layer(routed, shared, gate_vec, x, ids, weights, m, topk, out, ptr, HB_STATIC_SCRATCH_BYTES, stream, nullptr);
+}
+
+// ------------------------------------------------------------------------------------- a workspace's head words
+__global__ __launch_bounds__(256) void workspace_zero_kernel(uint32_t* at, size_t words) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < words; i += (size_t)gridDim.x * 256) at[i] = 0u;
+}
+
+extern "C" int hb_workspace_reset(void* workspace, size_t workspace_bytes, void* stream) {
+  if (!workspace) {  // the library's own scratch (hb_w3_moe_layer_static)
+    workspace = scratch_of_current_device();
+    workspace_bytes = HB_STATIC_SCRATCH_BYTES;
+    if (!workspace) return HB_ELAUNCH;
+  }
+  if (!aligned(workspace, 16) || workspace_bytes < 4) return HB_EINVAL;
+  const size_t words = std::min<size_t>(workspace_bytes, HB_WORKSPACE_ZERO_BYTES) / 4;
+  hipLaunchKernelGGL(workspace_zero_kernel, dim3((unsigned)std::min<size_t>((words + 255) / 256, 1024)), dim3(256), 0, as_stream(stream),
+                     static_cast<uint32_t*>(workspace), words);
+  return launch_status();
+}
+
+extern "C" int hb_workspace_status(const void* workspace, int32_t* status, int wait, void* stream) {
+  if (!status) return HB_ENULL;
+  if (!workspace) workspace = scratch_of_current_device();
+  if (!workspace) return HB_ELAUNCH;
+  if (!aligned(workspace, 16)) return HB_EINVAL;
+  if (hipMemcpyAsync(status, static_cast<const int32_t*>(workspace) + PLAN_FAULT, sizeof(int32_t), hipMemcpyDeviceToHost, as_stream(stream)) != hipSuccess)
+    return HB_ELAUNCH;
+  if (wait && hipStreamSynchronize(as_stream(stream)) != hipSuccess) return HB_ELAUNCH;
+  return HB_OK;
 }
 
 extern "C" int hb_w3_moe_layer_logits(const hb_w3_experts* routed, const hb_w3_experts* shared, const float* gate_vec, const void* x,

@@ -81,7 +81,7 @@ class B12xExperts:
             return out
         st = self._struct()
         need = _lib.lib().hb_nvfp4_moe_workspace_bytes(m, topk, C.byref(st))
-        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+        ws = _lib.workspace(x.device, need)
         ids32 = ids.to(torch.int32).contiguous()
         wt = weights.float().contiguous()
         xc = x.contiguous()

@@ -93,7 +93,7 @@ def router(x: torch.Tensor, weights: SmallWeights, bias: torch.Tensor | None, k:
     need = _lib.lib().hb_latent_workspace_bytes(C.byref(st), m, k)
     if need == 0:
         raise ValueError("router: the block's shapes are not ones the kernels take")
-    buffer = torch.empty(need, dtype=torch.uint8, device=dev)
+    buffer = _lib.workspace(dev, need, "latent")  # the stream's own: a Workspace serves until the next `router` on this stream
     fused = torch.empty((m, weights.experts_total + weights.latent), dtype=torch.float32, device=dev)
     ids = torch.empty((m, k), dtype=torch.int32, device=dev)
     wts = torch.empty((m, k), dtype=torch.float32, device=dev)

@@ -31,7 +31,7 @@ def nvfp4_linear(x: torch.Tensor, lin, prequantized=None, relu2: bool = False) -
     if m:
         xc = x.contiguous()  # held until the launch is enqueued: a temporary's block could be handed out again before that
         need = _lib.lib().hb_nvfp4_gemm_workspace_bytes(m, lin.out_features, lin.in_features)  # a few dozen rows: K shared among workgroups
-        ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+        ws = _lib.workspace(x.device, need, "gemm") if need else None
         _lib.check(_lib.lib().hb_nvfp4_gemm_ws(_lib.ptr(xc), m, _lib.ptr(lin.tiled), lin.global_scale, lin.out_features, lin.in_features, int(relu2),
                                                _lib.ptr(y), _lib.ptr(ws), need, _lib.stream()), "nvfp4_linear")
     return y

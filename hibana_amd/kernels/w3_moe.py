@@ -150,7 +150,7 @@ def w3_moe(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: torc
         return out
     st = _struct(experts)
     need = _lib.lib().hb_w3_moe_workspace_bytes(m, k, C.byref(st), 0)
-    ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    ws = _lib.workspace(x.device, need)
     ids32 = ids.to(torch.int32).contiguous()
     wt = weights.float().contiguous()
     mode |= MOE_E4M3 if e4m3 else 0
@@ -174,7 +174,7 @@ def moe_layer(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: t
     st = _struct(experts)
     sh = _struct(shared) if shared is not None else None
     need = _lib.lib().hb_w3_moe_workspace_bytes(m, k, C.byref(st), int(shared is not None))
-    ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    ws = _lib.workspace(x.device, need)
     ids32 = ids.to(torch.int32).contiguous()
     wt = weights.float().contiguous()
     gv = None if gate_vec is None else gate_vec.float().contiguous()
@@ -205,7 +205,7 @@ def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, 
         st = _struct(experts)
         sh = _struct(shared) if shared is not None else None
         need = _lib.lib().hb_w3_moe_workspace_bytes(m, topk, C.byref(st), int(shared is not None))
-        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+        ws = _lib.workspace(x.device, need)
         gv = None if gate_vec is None else gate_vec.float().contiguous()
         entry = _lib.lib().hb_w3_moe_layer_logits_e4m3 if e4m3 else _lib.lib().hb_w3_moe_layer_logits
         xc, lg = x.contiguous(), logits.contiguous()
@@ -239,7 +239,7 @@ def moe_layer_budget(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, 
         st = _struct(experts)
         sh = _struct(shared) if shared is not None else None
         need = _lib.lib().hb_w3_moe_workspace_bytes(m, topk, C.byref(st), int(shared is not None))
-        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+        ws = _lib.workspace(x.device, need)
         gv = None if gate_vec is None else gate_vec.float().contiguous()
         sl = None if slots is None else slots.to(torch.int32).contiguous()
         xc, lg = x.contiguous(), logits.contiguous()

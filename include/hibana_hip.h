@@ -7,6 +7,15 @@
  * kernels use no floating-point atomics, so results are bitwise repeatable and the calls are graph-capturable.
  * Return value: HB_OK (0) or a negative HB_E* code; hb_error_string() names it.
  *
+ * Workspaces. A workspace begins with a few words that no launch initializes: arrival counters (of the launch whose
+ * last workgroup plans a routed call; of the tiles whose K several workgroups share) and a fault word. The caller
+ * hands a workspace over with its first min(bytes, HB_WORKSPACE_ZERO_BYTES) bytes ZERO, once, before its first use
+ * (hipMemsetAsync, or hb_workspace_reset); every call that completes leaves the counters zero again, so one workspace
+ * serves any number of calls one after the other. The library keeps no counters of its own: calls that are in flight
+ * together (different streams, or graphs replayed side by side) must each have a workspace of their own and then share
+ * nothing; two calls in flight on ONE workspace race on everything in it. A call that was aborted midway (a reset
+ * device, a killed launch) may leave a counter standing: hb_workspace_reset puts the workspace back in service.
+ *
  * Citations "ref:" give the interface of the reference (sharar-project/hibana, paths relative to its tree) that the
  * entry point replaces.
  */
@@ -35,6 +44,32 @@ enum {
 int hb_version(void);
 const char* hb_error_string(int code);
 
+/* The bytes at a workspace's head that must be zero before its first use (or all of it, if it is smaller). */
+#define HB_WORKSPACE_ZERO_BYTES (1u << 20)
+
+/* Bits of a workspace's fault word. HB_FAULT_WAIT: a workgroup of a launch that runs a routed call's fc1 and fc2
+ * together waited for its slot's fc1 workgroups longer than the bound allows (about a second) - it has stored nothing,
+ * so rows of the call's output are stale. The launch relies on the hardware starting a grid's workgroups in index
+ * order; the bound and this bit are what happens should that ever fail. */
+enum { HB_FAULT_WAIT = 1 };
+
+/* Zero a workspace's head (its first min(bytes, HB_WORKSPACE_ZERO_BYTES) bytes: the arrival counters and the fault
+ * word) with a small kernel on `stream` - capturable, no hipMemset. For a new workspace, and to put one back in
+ * service after a fault or an aborted call. workspace == NULL: the library's own scratch (hb_w3_moe_layer_static).
+ * No counterpart in the reference (its kernels' split-K counters live in a torch tensor it zeroes at allocation,
+ * hibana/kernels/csrc/w3_gemm.cu:230-240). */
+int hb_workspace_reset(void* workspace, size_t workspace_bytes, void* stream);
+
+/* Copy a workspace's fault word (0: no fault; HB_FAULT_* bits otherwise; sticky until hb_workspace_reset) to *status
+ * (HOST memory) behind the work already enqueued on `stream`. wait != 0: synchronize the stream before returning, so
+ * *status is valid on return; wait == 0: only enqueue the copy (*status is valid once the caller has synchronized;
+ * pinned host memory keeps the copy asynchronous). workspace == NULL: the library's own scratch. The word means
+ * something in the workspaces of the routed calls (hb_w3_moe*, hb_nvfp4_moe, hb_latent_*); other workspaces hold zero
+ * there. No counterpart in the reference. */
+int hb_workspace_status(const void* workspace, int32_t* status, int wait, void* stream);
+
+#ifndef HB_NO_DEBUG_HOOKS  /* a build with -DHB_NO_DEBUG_HOOKS exports none of hb_tune / hb_debug_*: a serving process cannot race on them */
+
 /* Tuning knobs for experiments and tests; value 0 restores the built-in choice. "w3_ksplit" / "w3_nbw",
  * "moe_fc1_ksplit" / "moe_fc1_nbw", "moe_fc2_ksplit" / "moe_fc2_nbw", "nvfp4_ksplit" / "nvfp4_nbw": K splits and 64-row
  * blocks per workgroup (their product at most 16); "w3_tile" / "nvfp4_tile": 1 forces the MFMA tile kernel, 2 the weight
@@ -56,10 +91,12 @@ int hb_tune(const char* key, int value);
  * of the plan's three. count = 0 switches the hook off. Not for captured graphs. */
 int hb_debug_events(void* const* events, int count);
 
-/* Measurement hook (no counterpart in the reference): `buffer` (device, int64, four values a workgroup of the launch
- * that runs a routed call's fc1 and fc2 together; NULL switches it off) receives, per workgroup that had rows, its start,
- * the end of its wait for fc1 (fc2 workgroups; else 0) and its end, in ticks of the 100 MHz device clock, and its rows. */
-int hb_debug_trace(void* buffer);
+/* Measurement hook (no counterpart in the reference): `buffer` (device, int64, four values a record, `records` of them;
+ * NULL or 0 switches it off) receives, per workgroup of the launch that runs a routed call's fc1 and fc2 together (the
+ * workgroup's index in the launch's grid is the record's; workgroups past `records` write nothing), if it had rows: its
+ * start, the end of its wait for fc1 (fc2 workgroups; else 0) and its end, in ticks of the 100 MHz device clock, and its
+ * rows (bit 16: an fc1 workgroup). The hook stays armed until it is switched off: the buffer must outlive that. */
+int hb_debug_trace(void* buffer, int64_t records);
 
 /* Measurement hook (no counterpart in the reference): one plain streaming read of `bytes` (a multiple of 16 KB) from
  * `src`, 128-bit loads, sixteen in flight a lane - the read rate this device gives a kernel that does nothing else, to
@@ -72,14 +109,17 @@ int hb_debug_stream_read(const void* src, size_t bytes, void* sink, void* stream
  * LDS ring of LDS-direct loads) at place table[group] of `src` (places of 53 248 bytes, src_bytes / 53 248 of them; a
  * table value outside is clamped), with a dependent read of the table first, sixteen bytes of `acts` (32 rows of 4 KB) a
  * lane and chunk, the K split's exchange through LDS and one store a lane to `out` (groups x 256 floats). `sink`: at
- * least `groups` uint32 (practically never written). */
-int hb_debug_ring_skeleton(const void* src, size_t src_bytes, const int32_t* table, int groups, const void* acts, float* out, void* sink, void* stream);
+ * least `groups` uint32 (practically never written). The three sizes are checked against what the kernel touches
+ * (acts 131 072 bytes, out groups x 1024, sink groups x 4): HB_EINVAL for a buffer too small. */
+int hb_debug_ring_skeleton(const void* src, size_t src_bytes, const int32_t* table, int groups, const void* acts, size_t acts_bytes, float* out,
+                           size_t out_bytes, void* sink, size_t sink_bytes, void* stream);
 
 /* Measurement hook (no counterpart in the reference): `blocks` workgroups of eight wavefronts each run `iters` rounds of
  * eight independent BF16 MFMAs (16x16x32) on registers - the rate this device's matrix cores give a kernel that does
- * nothing else, to hold an expert GEMM's rate against. Returns the launch's FLOP (negative: an error code negated).
+ * nothing else, to hold an expert GEMM's rate against. Returns the launch's FLOP, or an HB_E* code (they are negative).
  * `sink`: at least `blocks` floats (practically never written). */
 int64_t hb_debug_mfma_rate(int blocks, int iters, void* sink, void* stream);
+#endif /* HB_NO_DEBUG_HOOKS */
 
 /* ------------------------------------------------------------------------------------------------------------------
  * W3 format: 3-bit (or 2-bit) codes into an 8-entry E4M3 codebook, one E4M3 scale per 32 weights along K, one FP32
@@ -172,6 +212,15 @@ enum { HB_MOE_SUM = 0, HB_MOE_PAIRS_F32 = 1, HB_MOE_PAIRS_BF16 = 2, HB_MOE_E4M3 
  * along). */
 size_t hb_w3_moe_workspace_bytes(int m, int topk, const hb_w3_experts* routed, int shared);
 
+#ifndef HB_NO_DEBUG_HOOKS
+/* Test hook (no counterpart in the reference): where a routed W3 call of this shape keeps its plan in its workspace, so
+ * that a test can read the plan back - offsets (HOST, six values): byte offsets of the slot table (int32: slots, distinct
+ * experts, kept pairs, ticket, fault word, ..., then from word 16 four words a slot: local expert id or -1 for the
+ * shared expert, first sorted position, rows, 0), of the sorted pair list (int32 [pairs + shared rows]), of h, of the
+ * pair outputs and of the slots' arrival counters; last, the slot table's capacity in slots. */
+int hb_debug_workspace_layout(int m, int topk, const hb_w3_experts* routed, int shared, int64_t* offsets);
+#endif
+
 /* Routed sum: out[r] = bf16( fma-chain over the row's slots, in selection order, of weights[r, s] * y[r, s] ),
  * y = fc2_e( act( bf16(fc1_e x_r) ) ) in FP32, h rounded to BF16. ids int32 [m, topk]; an id outside
  * [base, base + experts) adds nothing. mode HB_MOE_SUM: out BF16 [m, hidden_out]; HB_MOE_PAIRS_F32 / _BF16: out is
@@ -197,10 +246,11 @@ int hb_w3_moe_layer(const hb_w3_experts* routed, const hb_w3_experts* shared, co
  * sorted pair list, h and the pair outputs in a device array of HB_STATIC_SCRATCH_BYTES that the library itself holds
  * (one copy on every GPU it runs on, until the process ends). A call whose hb_w3_moe_workspace_bytes(m, topk, routed,
  * shared != NULL) exceeds that returns HB_ESCRATCH and enqueues nothing (the benchmark's verify step - 32 tokens, top-10,
- * 512 experts of 2048 x 512 and a shared one - takes 3.7 MB). It calls no allocator. Nothing in the array has to start
- * at zero (every launch of the chain writes what it later reads), so nothing is cleared. All calls on one GPU share
- * the array: two calls that overlap on one GPU (different streams, or replays of graphs holding them) race; on one
- * stream they are ordered like any other work.
+ * 512 experts of 2048 x 512 and a shared one - takes 3.7 MB). It calls no allocator. The array is zero when the library
+ * is loaded and every call leaves its head words zero, as with any workspace; everything else a launch of the chain
+ * writes before it is read, so nothing is cleared. All calls on one GPU share the array: two calls that overlap on one
+ * GPU (different streams, or replays of graphs holding them) race; on one stream they are ordered like any other work.
+ * hb_workspace_status(NULL, ...) reads its fault word, hb_workspace_reset(NULL, 0, stream) puts it back in service.
  * No counterpart in the reference (its op allocates its scratch from torch's caching allocator on every call,
  * hibana/kernels/csrc/w3_gemm.cu:1234-1247); for the callers above. */
 #define HB_STATIC_SCRATCH_BYTES (8u << 20)
@@ -362,8 +412,8 @@ int hb_nvfp4_gemm(const void* x, int m, const void* tiled, float global_scale, i
  * stream's sixteen rows a pass over the matrix and too few to fill the device with 128-row tiles, share K among the
  * workgroups of a tile; their partial tiles meet in `workspace` and whichever workgroup of a tile finishes last adds them
  * in one fixed order: the result does not depend on the schedule. hb_nvfp4_gemm_workspace_bytes: what a call of this
- * shape uses (0: none, the call is hb_nvfp4_gemm's). No counterpart in the reference (cuBLASLt / FlashInfer own their
- * workspaces there). */
+ * shape uses (0: none, the call is hb_nvfp4_gemm's); the tiles' arrival counters lie at its head (zero before the first
+ * use, see "Workspaces" above). No counterpart in the reference (cuBLASLt / FlashInfer own their workspaces there). */
 size_t hb_nvfp4_gemm_workspace_bytes(int m, int n, int k);
 int hb_nvfp4_gemm_ws(const void* x, int m, const void* tiled, float global_scale, int n, int k, int relu2, void* y,
                      void* workspace, size_t workspace_bytes, void* stream);

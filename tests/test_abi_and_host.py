@@ -55,7 +55,8 @@ def test_validation_without_a_gpu():
     assert lib.hb_nvfp4_gemm(256, 1, 260, 1.0, 128, 128, 0, 256, None) == _lib.HB_EINVAL  # tile layout on 4
     # the dense product with a workspace: sizes only (no launch without a GPU)
     assert lib.hb_nvfp4_gemm_workspace_bytes(8, 25600, 5120) == 0 and lib.hb_nvfp4_gemm_workspace_bytes(2048, 25600, 5120) == 0
-    assert lib.hb_nvfp4_gemm_workspace_bytes(64, 25600, 5120) == 100 * 4 * 4 * 4 * 4 * 64 * 16  # 100 tiles x 4 shares of K x 4 wavefronts x 4 row tiles x 4 x 64 lanes x 16 B
+    # the header words and 100 arrival counters (a multiple of 256 bytes), then 100 tiles x 4 shares of K x 4 wavefronts x 4 row tiles x 4 x 64 lanes x 16 B
+    assert lib.hb_nvfp4_gemm_workspace_bytes(64, 25600, 5120) == 512 + 100 * 4 * 4 * 4 * 4 * 64 * 16
     assert lib.hb_nvfp4_gemm_workspace_bytes(64, 100, 5120) == 0
     assert lib.hb_nvfp4_gemm_ws(None, 64, None, 1.0, 128, 128, 0, None, None, 0, None) == _lib.HB_ENULL
     assert lib.hb_relu2(None, 1, 2, 2, None) == _lib.HB_ENULL and lib.hb_relu2(256, 1, 3, 4, None) == _lib.HB_EINVAL

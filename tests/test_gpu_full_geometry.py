@@ -147,7 +147,8 @@ def test_nvfp4_dense_at_the_benchmark_geometry(nvfp4_dense, m, kernel):
 
 def test_nvfp4_dense_partial_tiles_do_not_depend_on_what_the_workspace_held(nvfp4_dense):
     """64 rows at config 1's size share K among four workgroups a tile: whichever finishes last must find the others'
-    partial tiles in memory. The workspace is filled with NaN before every call; every call gives the first one's bits,
+    partial tiles in memory. The workspace is filled with NaN before every call (and its head put back to zero, as the
+    library asks of a new workspace); every call gives the first one's bits,
     which are the stream's result to the summation order."""
     from hibana_amd import _lib
     from hibana_amd.kernels import ops
@@ -162,6 +163,7 @@ def test_nvfp4_dense_partial_tiles_do_not_depend_on_what_the_workspace_held(nvfp
     first = None
     for _ in range(12):
         ws.fill_(float("nan"))
+        _lib.check(lib.hb_workspace_reset(_lib.ptr(ws), need, _lib.stream()), "reset")  # the head (the tiles' arrival counters) starts at zero
         _lib.check(lib.hb_nvfp4_gemm_ws(_lib.ptr(x), m, _lib.ptr(lin.tiled), lin.global_scale, n, k, 0, _lib.ptr(y), _lib.ptr(ws), need, _lib.stream()), "gemm")
         if first is None:
             first = y.clone()

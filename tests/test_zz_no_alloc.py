@@ -18,7 +18,7 @@ def _both(ex, sh, gate, x, ids, weights):
     st, ss = w3_moe._struct(ex), w3_moe._struct(sh)
     need = lib.hb_w3_moe_workspace_bytes(m, k, C.byref(st), 1)
     assert 0 < need <= 8 << 20
-    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
     want = torch.zeros((m, ex.shape2[0]), dtype=torch.bfloat16, device="cuda")
     got = torch.zeros_like(want)
     _lib.check(lib.hb_w3_moe_layer(C.byref(st), C.byref(ss), _lib.ptr(gate), _lib.ptr(x), _lib.ptr(ids), _lib.ptr(weights), m, k, _lib.ptr(want),
