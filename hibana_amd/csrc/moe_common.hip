@@ -50,6 +50,45 @@ struct Scan3 {
   int a, b, c;
 };
 
+// Inclusive prefix sum over the wavefront's lanes without LDS: shifts within rows of sixteen lanes, then the rows' last
+// lanes broadcast to the rows after them (DPP).
+__device__ __forceinline__ int wave_inclusive_sum(int x) {
+  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, false);  // row_shr:1
+  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, false);  // row_shr:2
+  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, false);  // row_shr:4
+  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, false);  // row_shr:8
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+  return x;
+}
+
+// Exclusive scan over the workgroup of two words a thread whose four 16-bit halves are sums of their own (none reaches
+// 65536, so no carry crosses a half): one DPP scan a word in each wavefront, the wavefronts' totals through LDS, one
+// barrier. `total` receives the two sums. scratch: 2 * PLAN_WAVES ints, not in use by anyone before the call's barrier.
+struct Scan2 {
+  int lo, hi;
+};
+__device__ __forceinline__ Scan2 block_exclusive_scan2(Scan2 v, int* scratch, Scan2* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int lo = wave_inclusive_sum(v.lo), hi = wave_inclusive_sum(v.hi);
+  if (lane == 63) {
+    scratch[wave] = lo;
+    scratch[PLAN_WAVES + wave] = hi;
+  }
+  __syncthreads();
+  int before_lo = 0, before_hi = 0, all_lo = 0, all_hi = 0;
+  for (int w = 0; w < waves; w++) {  // the same address in every lane: broadcast reads
+    const int a = scratch[w], b = scratch[PLAN_WAVES + w];
+    before_lo += w < wave ? a : 0;
+    before_hi += w < wave ? b : 0;
+    all_lo += a;
+    all_hi += b;
+  }
+  total->lo = all_lo;
+  total->hi = all_hi;
+  return Scan2{before_lo + lo - v.lo, before_hi + hi - v.hi};
+}
+
 // Exclusive scan of three integers per thread over the workgroup at once; `total` receives the three sums.
 __device__ __forceinline__ Scan3 block_exclusive_scan3(Scan3 v, int* scratch /* 3 * (PLAN_WAVES + 1) ints */, Scan3* total) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -160,7 +199,7 @@ __device__ __forceinline__ void plan_few_pairs(const int32_t* ids, int pairs, in
 // entries the launches' grids reach beyond the last slot (a workgroup learns that it has nothing to do from its own
 // entry, without a second dependent read of the count), the slots' arrival counters at zero, the header.
 __device__ __forceinline__ void plan_tail(int32_t* __restrict__ plan, int32_t* __restrict__ order, int pairs, int shared_rows, int slot_rows, int slot_cap,
-                                          int slots, int distinct, int kept) {
+                                          int slots, int distinct, int kept, bool counters = true) {
   const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
   for (int s = threadIdx.x; s < shared_slots; s += blockDim.x) {
     int32_t* entry = plan + PLAN_HEADER + 4 * s;
@@ -174,7 +213,8 @@ __device__ __forceinline__ void plan_tail(int32_t* __restrict__ plan, int32_t* _
     int32_t* entry = plan + PLAN_HEADER + 4 * s;
     entry[0] = entry[1] = entry[2] = entry[3] = 0;
   }
-  for (int s = threadIdx.x; s < slot_cap; s += blockDim.x) plan_done(plan, slot_cap)[s * DONE_PITCH] = 0;
+  if (counters)
+    for (int s = threadIdx.x; s < slot_cap; s += blockDim.x) plan_done(plan, slot_cap)[s * DONE_PITCH] = 0;
   if (threadIdx.x == 0) {
     plan[0] = slots;
     plan[1] = distinct;
@@ -191,11 +231,11 @@ __device__ __forceinline__ void plan_tail(int32_t* __restrict__ plan, int32_t* _
 constexpr int PLAN_ROWS_MAX = 64;
 constexpr int PLAN_ROWS_PER_THREAD = 4;  // 64 rows of at most 64 selections over 1024 threads
 __device__ __forceinline__ void plan_by_rows(const int32_t* ids, int rows, int topk, int e_lo, int e_n, int shared_rows, int32_t* __restrict__ plan,
-                                             int32_t* __restrict__ order, int slot_rows, int slot_cap, int* lds) {
+                                             int32_t* __restrict__ order, int slot_rows, int slot_cap, int* lds, bool cleared = false) {
   uint32_t* occ_lo = reinterpret_cast<uint32_t*>(lds);  // [e_n] rows 0 .. 31 that name expert e
   uint32_t* occ_hi = occ_lo + e_n;                      // [e_n] rows 32 .. 63
   int* start = lds + 2 * e_n;                           // [e_n] first sorted position of expert e
-  int* scratch = start + e_n;                           // [3 * (PLAN_WAVES + 1)]
+  int* scratch = start + e_n;                           // [2 * PLAN_WAVES]
   const int pairs = rows * topk;
   int mine[PLAN_ROWS_PER_THREAD], row_of[PLAN_ROWS_PER_THREAD];
 #pragma unroll
@@ -214,21 +254,23 @@ __device__ __forceinline__ void plan_by_rows(const int32_t* ids, int rows, int t
   }
   __syncthreads();
   const int e = threadIdx.x;  // one thread an expert: the launch keeps e_n <= PLAN_THREADS
-  const int count = e < e_n ? __popc(occ_lo[e]) + __popc(occ_hi[e]) : 0;
+  const int count = e < e_n ? __popc(occ_lo[e]) + __popc(occ_hi[e]) : 0;  // at most 64
   const int my_slots = (count + slot_rows - 1) / slot_rows;
   const bool heavy = 4 * count > slot_rows;
-  Scan3 tot;  // as in plan_work: rows; heavy slots with the distinct experts in the upper half; light slots
-  const Scan3 at = block_exclusive_scan3(Scan3{count, (heavy ? my_slots : 0) | (count > 0 ? 1 << 16 : 0), heavy ? 0 : my_slots}, scratch, &tot);
+  // four sums in two words: rows (at most 4096) and light slots; heavy slots and distinct experts (at most 1024 each)
+  Scan2 tot;
+  const Scan2 at = block_exclusive_scan2(Scan2{count | (heavy ? 0 : my_slots) << 16, (heavy ? my_slots : 0) | (count > 0 ? 1 << 16 : 0)}, scratch, &tot);
   const int shared_slots = (shared_rows + slot_rows - 1) / slot_rows;
-  const int kept = tot.a, distinct = tot.b >> 16, heavy_slots = tot.b & 0xffff;
-  const int slots = shared_slots + heavy_slots + tot.c;
+  const int kept = tot.lo & 0xffff, distinct = tot.hi >> 16, heavy_slots = tot.hi & 0xffff;
+  const int slots = shared_slots + heavy_slots + (tot.lo >> 16);
   if (e < e_n) {
-    start[e] = at.a;
-    const int my_slot = shared_slots + (heavy ? (at.b & 0xffff) : heavy_slots + at.c);
+    const int my_start = at.lo & 0xffff;
+    start[e] = my_start;
+    const int my_slot = shared_slots + (heavy ? (at.hi & 0xffff) : heavy_slots + (at.lo >> 16));
     for (int s = 0; s < my_slots; s++) {
       int32_t* entry = plan + PLAN_HEADER + 4 * (my_slot + s);
       entry[0] = e;
-      entry[1] = at.a + s * slot_rows;
+      entry[1] = my_start + s * slot_rows;
       entry[2] = min(slot_rows, count - s * slot_rows);
       entry[3] = 0;
     }
@@ -242,7 +284,8 @@ __device__ __forceinline__ void plan_by_rows(const int32_t* ids, int rows, int t
     const int below = r < 32 ? __popc(lo & ((1u << r) - 1u)) : __popc(lo) + __popc(hi & ((1u << (r - 32)) - 1u));
     order[start[mine[j]] + below] = threadIdx.x + j * PLAN_THREADS;
   }
-  plan_tail(plan, order, pairs, shared_rows, slot_rows, slot_cap, slots, distinct, kept);
+  // `cleared`: the launch's other workgroups have already put "no rows" into every entry and zeroed the arrival counters
+  plan_tail(plan, order, pairs, shared_rows, slot_rows, cleared ? slots : slot_cap, slots, distinct, kept, !cleared);
 }
 
 // The plan itself, by one workgroup of PLAN_THREADS (`group` of `groups` when many pairs are shared): `lds` is the
@@ -454,6 +497,16 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int3
   if (wave < ROUTE_GROUP_ROWS && r < route_rows) {
     route_any(route, r, threadIdx.x & 63);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this row's ids (write-through stores) have reached memory before the ticket is drawn
+  } else if (by_rows && wave >= ROUTE_GROUP_ROWS) {
+    // Meanwhile the wavefronts that route nothing put "no rows" into every entry of the slot table and zero the slots'
+    // arrival counters, a word a thread over the launch's routing workgroups - with stores that go through to memory
+    // and are waited for, so the words are there, and in no L2 as modified lines, before anyone's ticket: the planner's
+    // own stores to the entries it fills come after its ticket and are the only modified copies.
+    constexpr int IDLE = PLAN_THREADS - 64 * ROUTE_GROUP_ROWS;
+    int32_t* done = plan_done(plan, slot_cap);
+    for (int i = blockIdx.x * IDLE + (int)threadIdx.x - 64 * ROUTE_GROUP_ROWS; i < 5 * slot_cap; i += route_groups * IDLE)
+      store_through(i < 4 * slot_cap ? plan + PLAN_HEADER + i : done + (i - 4 * slot_cap) * DONE_PITCH, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -465,7 +518,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_route_plan_kernel(const int3
   __syncthreads();
   if (!last) return;  // the last arriver: every row's ids are in memory, and the plan reads them from there (load_through)
   if (by_rows) {
-    plan_by_rows(ids, route_rows, route.k, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, lds);
+    plan_by_rows(ids, route_rows, route.k, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, lds, true);
   } else {
     plan_work<false>(ids, pairs, e_lo, e_n, shared_rows, plan, order, slot_rows, slot_cap, nullptr, 1, 0, 0, lds);
   }
