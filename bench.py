@@ -346,6 +346,13 @@ def dense_decode(args) -> dict:
     elapsed = median(times) * 1e-3 * args.steps
     del outs
     achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+    if args.copy_mib:  # a plain device copy of known size, for scaling the counters of a rocprofv3 --pmc run
+        src = torch.empty(args.copy_mib << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    ratio = traffic_ratio(f"traffic_ratio_config{args.config}_m1", "decode_configs_0_1_hbm_traffic.md") if m == 1 else None
     by_rows = None
     if args.config == 1:  # the same projection at the configuration's other row counts: microseconds a call, graph-replayed
         by_rows = {}
@@ -366,7 +373,9 @@ def dense_decode(args) -> dict:
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": what, "matrices_cycled": args.layers, "timed_as": "replays of one HIP graph of all steps; median replay"},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": None, "launch_bytes": nbytes, "launch_ms": kernel_ms},
+                     # HBM bytes a launch: scaled FETCH_SIZE + WRITE_SIZE over the algorithmic bytes, measured with
+                     # rocprofv3 --pmc on this workload (the summary under profiles/ states it), applied to this run's bytes
+                     "traffic": None if ratio is None else ratio * nbytes, "launch_bytes": nbytes, "launch_ms": kernel_ms},
         "cpu_baseline": None,
     }
     if by_rows:
@@ -499,14 +508,14 @@ def mfma_rate_tflops(dev, blocks: int = 2048, iters: int = 4096) -> float:
     return flops / (median(times) * 1e-3) / 1e12
 
 
-def traffic_ratio():
-    """HBM bytes a launch / algorithmic bytes of the fc1 + fc2 launch, from the committed counter summary (two rocprofv3
-    --pmc runs scaled by a plain copy of known size); None when the summary does not state it."""
+def traffic_ratio(name: str = "traffic_ratio_fc1_fc2", summary: str = "w3_moe_layer_config3_hbm_traffic.md"):
+    """HBM bytes a launch / algorithmic bytes of a kernel (by default the fc1 + fc2 launch), from the committed counter
+    summary (two rocprofv3 --pmc runs scaled by a plain copy of known size); None when the summary does not state it."""
     import os
     import re
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "w3_moe_layer_config3_hbm_traffic.md")
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", summary)
     try:
-        found = re.search(r"^traffic_ratio_fc1_fc2\s*=\s*([0-9.]+)", open(path).read(), re.M)
+        found = re.search(r"^" + name + r"\s*=\s*([0-9.]+)", open(path).read(), re.M)
     except OSError:
         return None
     return float(found.group(1)) if found else None
@@ -694,7 +703,8 @@ def main() -> int:
         del layers, x, logits, one_logits
         torch.cuda.empty_cache()
         others = {}
-        for name, mode, overrides in (("config1", dense_decode, {"config": 1, "rows": 1}), ("config4", latent_prefill, {"config": 4})):
+        for name, mode, overrides in (("config0", dense_decode, {"config": 0, "rows": 1}), ("config1", dense_decode, {"config": 1, "rows": 1}),
+                                      ("config4", latent_prefill, {"config": 4})):
             sub = argparse.Namespace(**{**vars(args), **overrides})
             try:
                 others[name] = mode(sub)

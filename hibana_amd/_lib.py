@@ -47,16 +47,16 @@ SIGNATURES = {
     "hb_workspace_reset": (_I, [_P, _Z, _P]),
     "hb_workspace_status": (_I, [_P, C.POINTER(C.c_int32), _I, _P]),
     "hb_debug_mfma_rate": (_L, [_I, _I, _P, _P]),
-    "hb_w3_tiled_bytes": (_Z, [_L, _I]),
-    "hb_w3_repack": (_I, [_P, _P, _L, _I, _I, _P, _P]),
+    "hb_w3_tiled_bytes": (_Z, [_L, _I, _I]),
+    "hb_w3_repack": (_I, [_P, _P, _L, _I, _I, _I, _P, _P]),
     "hb_w3_pack_codes": (_I, [_P, _P, _L, _I, _I, _P, _P, _P]),
-    "hb_w3_unpack": (_I, [_P, _L, _I, _P, _P, _P]),
+    "hb_w3_unpack": (_I, [_P, _L, _I, _I, _P, _P, _P]),
     "hb_w3_unpack_planes": (_I, [_P, _P, _L, _I, _I, _P, _P, _P]),
-    "hb_w3_dequant": (_I, [_P, _P, _L, _L, _I, _P, _P]),
-    "hb_w3_gemm": (_I, [_P, _I, _P, _P, _L, _I, _I, _P, _P]),
+    "hb_w3_dequant": (_I, [_P, _P, _L, _L, _I, _I, _P, _P]),
+    "hb_w3_gemm": (_I, [_P, _I, _P, _P, _L, _I, _I, _I, _P, _P]),
     "hb_w3_quant_groups": (_I, [_P, _L, _I, _P, _P, _P]),
     "hb_w3_quant_rows": (_I, [_P, _L, _I, _P, _P, _P]),
-    "hb_w3_gemm_e4m3": (_I, [_P, _P, _I, _P, _P, _L, _I, _I, _P, _P]),
+    "hb_w3_gemm_e4m3": (_I, [_P, _P, _I, _P, _P, _L, _I, _I, _I, _P, _P]),
     "hb_w3_moe_workspace_bytes": (_Z, [_I, _I, _EX, _I]),
     "hb_w3_moe": (_I, [_EX, _P, _P, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "hb_w3_moe_layer": (_I, [_EX, _EX, _P, _P, _P, _P, _I, _I, _P, _P, _Z, _P]),

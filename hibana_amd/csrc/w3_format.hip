@@ -5,9 +5,10 @@
 
 namespace hb {
 
-// One thread per (block, lane): builds the lane's twelve code dwords from the reference planes.
+// One thread per (block, lane): builds the lane's code dwords (twelve of a three-bit tile, eight of a two-bit one) from
+// the reference planes; two-bit codes into three-bit tiles leave the third bit zero.
 __global__ __launch_bounds__(256) void w3_repack_codes_kernel(const uint32_t* __restrict__ planes, int64_t blocks, int chunks,
-                                                              int bits, uint8_t* __restrict__ tiled) {
+                                                              int bits, int tile_bits, uint8_t* __restrict__ tiled) {
   const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (id >= blocks * 64) return;
   const int64_t blk = id >> 6;
@@ -27,19 +28,24 @@ __global__ __launch_bounds__(256) void w3_repack_codes_kernel(const uint32_t* __
           int pos, dw, dpos;
           w3_ref_bit_slot(n, k, b, bits, chunks, &word, &pos);
           const uint32_t bit = (planes[word] >> pos) & 1u;
-          w3_bit_slot(nt, j, i, b, &dw, &dpos);
+          if (tile_bits == 2) {
+            w2_bit_slot(nt, j, i, b, &dw, &dpos);
+          } else {
+            w3_bit_slot(nt, j, i, b, &dw, &dpos);
+          }
           d[dw] |= bit << dpos;
         }
       }
   }
-  uint8_t* base = tiled + blk * W3_BLOCK_BYTES;
+  uint8_t* base = tiled + blk * w3_block_bytes(tile_bits);
 #pragma unroll
-  for (int i = 0; i < 12; i++) *reinterpret_cast<uint32_t*>(base + w3_dword_offset(lane, i)) = d[i];
+  for (int i = 0; i < 12; i++)
+    if (i < 4 * tile_bits) *reinterpret_cast<uint32_t*>(base + w3_dword_offset(lane, i)) = d[i];
 }
 
 // One thread per scale byte of the tile layout.
 __global__ __launch_bounds__(256) void w3_repack_scales_kernel(const uint8_t* __restrict__ scales, int64_t blocks, int chunks,
-                                                               uint8_t* __restrict__ tiled) {
+                                                               int tile_bits, uint8_t* __restrict__ tiled) {
   const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (id >= blocks * 256) return;
   const int64_t blk = id >> 8;
@@ -47,7 +53,7 @@ __global__ __launch_bounds__(256) void w3_repack_scales_kernel(const uint8_t* __
   const int64_t nb = blk / chunks;
   const int c = (int)(blk % chunks);
   const int64_t n = nb * 64 + nt * 16 + r;
-  tiled[blk * W3_BLOCK_BYTES + w3_scale_offset(nt, r, j)] = scales[w3_ref_scale_slot(n, 4 * c + j, chunks)];
+  tiled[blk * w3_block_bytes(tile_bits) + w3_scale_base(tile_bits) + 16 * r + 4 * nt + j] = scales[w3_ref_scale_slot(n, 4 * c + j, chunks)];
 }
 
 // One thread per plane word of the reference layout.
@@ -86,7 +92,19 @@ __global__ __launch_bounds__(256) void w3_pack_scales_kernel(const uint8_t* __re
 }
 
 // One thread per (block, tile, lane): the lane's 32 codes of one 16-row tile.
-__global__ __launch_bounds__(256) void w3_unpack_kernel(const uint8_t* __restrict__ tiled, int64_t blocks, int chunks,
+// The eight selectors of tile nt of a lane, from either tile layout.
+__device__ __forceinline__ void tile_selectors(const uint8_t* base, int lane, int nt, int bits, uint32_t sel[8]) {
+  if (bits == 2) {
+    w2_selectors(*reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 2 * nt)),
+                 *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 2 * nt + 1)), sel);
+  } else {
+    w3_selectors(*reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt)),
+                 *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 1)),
+                 *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 2)), sel);
+  }
+}
+
+__global__ __launch_bounds__(256) void w3_unpack_kernel(const uint8_t* __restrict__ tiled, int64_t blocks, int chunks, int bits,
                                                         uint8_t* __restrict__ codes, uint8_t* __restrict__ scale_bytes) {
   const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (id >= blocks * 256) return;
@@ -95,14 +113,11 @@ __global__ __launch_bounds__(256) void w3_unpack_kernel(const uint8_t* __restric
   const int64_t nb = blk / chunks;
   const int c = (int)(blk % chunks);
   const int k = chunks * 128;
-  const uint8_t* base = tiled + blk * W3_BLOCK_BYTES;
+  const uint8_t* base = tiled + blk * w3_block_bytes(bits);
   const int64_t n = nb * 64 + nt * 16 + r;
   if (codes) {
-    const uint32_t q0 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt));
-    const uint32_t q1 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 1));
-    const uint32_t q2 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 2));
     uint32_t sel[8];
-    w3_selectors(q0, q1, q2, sel);
+    tile_selectors(base, lane, nt, bits, sel);
     for (int j = 0; j < 4; j++) {
       uint8_t* out = codes + n * k + c * 128 + j * 32 + q * 8;
       *reinterpret_cast<uint32_t*>(out) = sel[2 * j];
@@ -110,7 +125,7 @@ __global__ __launch_bounds__(256) void w3_unpack_kernel(const uint8_t* __restric
     }
   }
   if (scale_bytes && q == 0) {
-    for (int j = 0; j < 4; j++) scale_bytes[n * (k >> 5) + 4 * c + j] = base[w3_scale_offset(nt, r, j)];
+    for (int j = 0; j < 4; j++) scale_bytes[n * (k >> 5) + 4 * c + j] = base[w3_scale_base(bits) + 16 * r + 4 * nt + j];
   }
 }
 
@@ -142,7 +157,7 @@ __global__ __launch_bounds__(256) void w3_unpack_planes_kernel(const uint32_t* _
 // One thread per (block, tile, lane): 32 dequantized weights. Two FP32 products, each rounded:
 // effective = float(scale byte) * row_scale[row]; weight = level * effective.
 __global__ __launch_bounds__(256) void w3_dequant_kernel(const uint8_t* __restrict__ tiled, const float* __restrict__ row_scale,
-                                                         uint64_t lut, int64_t blocks, int chunks, float* __restrict__ out) {
+                                                         uint64_t lut, int64_t blocks, int chunks, int bits, float* __restrict__ out) {
   const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (id >= blocks * 256) return;
   const int64_t blk = id >> 8;
@@ -150,19 +165,16 @@ __global__ __launch_bounds__(256) void w3_dequant_kernel(const uint8_t* __restri
   const int64_t nb = blk / chunks;
   const int c = (int)(blk % chunks);
   const int k = chunks * 128;
-  const uint8_t* base = tiled + blk * W3_BLOCK_BYTES;
+  const uint8_t* base = tiled + blk * w3_block_bytes(bits);
   const int64_t n = nb * 64 + nt * 16 + r;
   float level[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) level[i] = e4m3_to_f32((uint32_t)(lut >> (8 * i)) & 0xffu);
-  const uint32_t q0 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt));
-  const uint32_t q1 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 1));
-  const uint32_t q2 = *reinterpret_cast<const uint32_t*>(base + w3_dword_offset(lane, 3 * nt + 2));
   uint32_t sel[8];
-  w3_selectors(q0, q1, q2, sel);
+  tile_selectors(base, lane, nt, bits, sel);
   const float row = row_scale[n];
   for (int j = 0; j < 4; j++) {
-    const float eff = __fmul_rn(e4m3_to_f32(base[w3_scale_offset(nt, r, j)]), row);
+    const float eff = __fmul_rn(e4m3_to_f32(base[w3_scale_base(bits) + 16 * r + 4 * nt + j]), row);
     float* o = out + n * k + c * 128 + j * 32 + q * 8;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
@@ -181,9 +193,9 @@ static inline unsigned grid_for(int64_t threads) { return (unsigned)((threads + 
 
 using namespace hb;
 
-extern "C" size_t hb_w3_tiled_bytes(int64_t rows, int k) {
-  if (rows <= 0 || k <= 0 || rows % W3_BLOCK_ROWS || k % W3_CHUNK) return 0;
-  return (size_t)(rows / W3_BLOCK_ROWS) * (size_t)(k / W3_CHUNK) * W3_BLOCK_BYTES;
+extern "C" size_t hb_w3_tiled_bytes(int64_t rows, int k, int bits) {
+  if (rows <= 0 || k <= 0 || rows % W3_BLOCK_ROWS || k % W3_CHUNK || (bits != 2 && bits != 3)) return 0;
+  return (size_t)(rows / W3_BLOCK_ROWS) * (size_t)(k / W3_CHUNK) * w3_block_bytes(bits);
 }
 
 static int check_shape(int64_t rows, int k, int bits) {
@@ -192,14 +204,15 @@ static int check_shape(int64_t rows, int k, int bits) {
   return HB_OK;
 }
 
-extern "C" int hb_w3_repack(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, void* tiled, void* stream) {
+extern "C" int hb_w3_repack(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, int tile_bits, void* tiled, void* stream) {
   if (!planes || !scales || !tiled) return HB_ENULL;
   if (int e = check_shape(rows, k, bits)) return e;
+  if (tile_bits != 3 && tile_bits != bits) return HB_EINVAL;  // codes are widened, never narrowed
   const int chunks = k / W3_CHUNK;
   const int64_t blocks = rows / W3_BLOCK_ROWS * chunks;
-  hipLaunchKernelGGL(w3_repack_codes_kernel, dim3(grid_for(blocks * 64)), dim3(256), 0, as_stream(stream), planes, blocks, chunks, bits,
+  hipLaunchKernelGGL(w3_repack_codes_kernel, dim3(grid_for(blocks * 64)), dim3(256), 0, as_stream(stream), planes, blocks, chunks, bits, tile_bits,
                      static_cast<uint8_t*>(tiled));
-  hipLaunchKernelGGL(w3_repack_scales_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), scales, blocks, chunks,
+  hipLaunchKernelGGL(w3_repack_scales_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), scales, blocks, chunks, tile_bits,
                      static_cast<uint8_t*>(tiled));
   return launch_status();
 }
@@ -214,13 +227,13 @@ extern "C" int hb_w3_pack_codes(const uint8_t* codes, const uint8_t* scale_bytes
   return launch_status();
 }
 
-extern "C" int hb_w3_unpack(const void* tiled, int64_t rows, int k, uint8_t* codes, uint8_t* scale_bytes, void* stream) {
+extern "C" int hb_w3_unpack(const void* tiled, int64_t rows, int k, int bits, uint8_t* codes, uint8_t* scale_bytes, void* stream) {
   if (!tiled) return HB_ENULL;
-  if (int e = check_shape(rows, k, 3)) return e;
+  if (int e = check_shape(rows, k, bits)) return e;
   const int chunks = k / W3_CHUNK;
   const int64_t blocks = rows / W3_BLOCK_ROWS * chunks;
   hipLaunchKernelGGL(w3_unpack_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), static_cast<const uint8_t*>(tiled),
-                     blocks, chunks, codes, scale_bytes);
+                     blocks, chunks, bits, codes, scale_bytes);
   return launch_status();
 }
 
@@ -233,13 +246,13 @@ extern "C" int hb_w3_unpack_planes(const uint32_t* planes, const uint8_t* scales
   return launch_status();
 }
 
-extern "C" int hb_w3_dequant(const void* tiled, const float* row_scale, int64_t lut, int64_t rows, int k, float* out, void* stream) {
+extern "C" int hb_w3_dequant(const void* tiled, const float* row_scale, int64_t lut, int64_t rows, int k, int bits, float* out, void* stream) {
   if (!tiled || !row_scale || !out) return HB_ENULL;
-  if (int e = check_shape(rows, k, 3)) return e;
+  if (int e = check_shape(rows, k, bits)) return e;
   const int chunks = k / W3_CHUNK;
   const int64_t blocks = rows / W3_BLOCK_ROWS * chunks;
   hipLaunchKernelGGL(w3_dequant_kernel, dim3(grid_for(blocks * 256)), dim3(256), 0, as_stream(stream), static_cast<const uint8_t*>(tiled),
-                     row_scale, (uint64_t)lut, blocks, chunks, out);
+                     row_scale, (uint64_t)lut, blocks, chunks, bits, out);
   return launch_status();
 }
 

@@ -17,6 +17,15 @@
 //                     64 nb + 16 nt + r, 32-group 4 c + j.
 //
 // The same density as the reference layout (3 bits + 1/4 bit per weight); the FP32 row scales stay a separate array.
+//
+// Two-bit matrices (four-level codebooks: the reference's two-plane variant, hibana/kernels/w3.py:12-19,89-91) have a
+// tile layout of their own at their own density (2 + 1/4 bits a weight): blocks of 2304 bytes,
+//   bytes    0..2047  codes: two 128-bit loads per lane; the lane's eight dwords hold tile nt in Q0 = D[2 nt],
+//                     Q1 = D[2 nt + 1], four 2-bit codes a byte: selector s = 2 j + i / 4 (byte i % 4 = weight (j, i)) is
+//                         s0 = Q0 & 0x03030303, s1 = (Q0 >> 2) & 0x03030303, s2 = (Q0 >> 4) & .., s3 = (Q0 >> 6) & ..,
+//                         s4 .. s7 the same of Q1;
+//   bytes 2048..2303  scales, as above.
+// The kernels that take either layout are told the `bits` of the tiles (3 or 2).
 #pragma once
 
 #include <stdint.h>
@@ -27,6 +36,30 @@ constexpr int W3_BLOCK_ROWS = 64;
 constexpr int W3_CHUNK = 128;
 constexpr int W3_BLOCK_BYTES = 3328;
 constexpr int W3_SCALE_OFFSET = 3072;
+
+constexpr int W2_BLOCK_BYTES = 2304;
+constexpr int W2_SCALE_OFFSET = 2048;
+__host__ __device__ constexpr int w3_block_bytes(int bits) { return bits == 2 ? W2_BLOCK_BYTES : W3_BLOCK_BYTES; }
+__host__ __device__ constexpr int w3_scale_base(int bits) { return bits == 2 ? W2_SCALE_OFFSET : W3_SCALE_OFFSET; }
+
+// Two-bit tiles: where bit b (0..1) of weight (tile nt, group j, element i) of a lane sits among the lane's eight dwords.
+__host__ __device__ inline void w2_bit_slot(int nt, int j, int i, int b, int* dword, int* pos) {
+  const int s = 2 * j + (i >> 2), byte = i & 3;
+  *dword = 2 * nt + (s >> 2);
+  *pos = 8 * byte + 2 * (s & 3) + b;
+}
+
+// The eight selectors of one two-bit tile from its two dwords.
+__host__ __device__ inline void w2_selectors(uint32_t q0, uint32_t q1, uint32_t sel[8]) {
+  sel[0] = q0 & 0x03030303u;
+  sel[1] = (q0 >> 2) & 0x03030303u;
+  sel[2] = (q0 >> 4) & 0x03030303u;
+  sel[3] = (q0 >> 6) & 0x03030303u;
+  sel[4] = q1 & 0x03030303u;
+  sel[5] = (q1 >> 2) & 0x03030303u;
+  sel[6] = (q1 >> 4) & 0x03030303u;
+  sel[7] = (q1 >> 6) & 0x03030303u;
+}
 
 // Where the three bits of weight (tile nt, group j, element i) of a lane sit among the lane's twelve dwords.
 // Returns for bit b (0..2) the dword index and the bit position.

@@ -34,6 +34,30 @@ struct Chunk {  // the weight side of one 64-row x 128-k block
   u32x4_t w0, w1, w2, sc;
 };
 
+struct Chunk2 {  // the same of a two-bit matrix: eight code dwords a lane
+  u32x4_t w0, w1, sc;
+};
+
+// The eight selectors of 16-row tile NT of a chunk, and the dword of its four scale bytes.
+template <int NT>
+__device__ __forceinline__ void chunk_selectors(const Chunk& ch, uint32_t sel[8]) {
+  if (NT == 0) w3_selectors(ch.w0.x, ch.w0.y, ch.w0.z, sel);
+  if (NT == 1) w3_selectors(ch.w0.w, ch.w1.x, ch.w1.y, sel);
+  if (NT == 2) w3_selectors(ch.w1.z, ch.w1.w, ch.w2.x, sel);
+  if (NT == 3) w3_selectors(ch.w2.y, ch.w2.z, ch.w2.w, sel);
+}
+template <int NT>
+__device__ __forceinline__ void chunk_selectors(const Chunk2& ch, uint32_t sel[8]) {
+  if (NT == 0) w2_selectors(ch.w0.x, ch.w0.y, sel);
+  if (NT == 1) w2_selectors(ch.w0.z, ch.w0.w, sel);
+  if (NT == 2) w2_selectors(ch.w1.x, ch.w1.y, sel);
+  if (NT == 3) w2_selectors(ch.w1.z, ch.w1.w, sel);
+}
+template <int NT, class C>
+__device__ __forceinline__ uint32_t chunk_scales(const C& ch) {
+  return NT == 0 ? ch.sc.x : NT == 1 ? ch.sc.y : NT == 2 ? ch.sc.z : ch.sc.w;
+}
+
 struct Rows {  // the activation side: four MFMA A fragments (one per 32-group), read from L2
   u32x4_t a0, a1, a2, a3;
 };
@@ -67,11 +91,11 @@ __device__ __forceinline__ bf16x8_t expand8(uint32_t sel_lo, uint32_t sel_hi, ui
 // Half of a 16-row tile of a chunk, sixteen activation rows: 32-groups 0 and 1 (HALF 0: their selectors come from the
 // tile's first two code dwords) or 2 and 3 (HALF 1). One MFMA is one group, so the group's scale is folded into the FP32
 // accumulator after it, in group order.
-template <int HALF>
-__device__ __forceinline__ void compute_half_tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const u32x4_t& a_lo, const u32x4_t& a_hi,
-                                                  f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi) {
+template <int HALF, int NT, class C>
+__device__ __forceinline__ void compute_half_tile(const C& ch, const u32x4_t& a_lo, const u32x4_t& a_hi, f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi) {
+  const uint32_t scales = chunk_scales<NT>(ch);
   uint32_t sel[8];
-  w3_selectors(q0, q1, q2, sel);  // the four the half does not use fold away
+  chunk_selectors<NT>(ch, sel);  // the four the half does not use fold away
   const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
   const f32x4_t p0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a_lo), expand8(sel[4 * HALF], sel[4 * HALF + 1], lut_lo, lut_hi), zero, 0, 0, 0);
   const f32x4_t p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a_hi), expand8(sel[4 * HALF + 2], sel[4 * HALF + 3], lut_lo, lut_hi), zero, 0, 0, 0);
@@ -85,21 +109,24 @@ __device__ __forceinline__ void compute_half_tile(uint32_t q0, uint32_t q1, uint
 
 // The four tiles of a chunk over one half of its groups: once a half is done its two activation fragments are free for
 // the next chunk's.
-template <int HALF>
-__device__ __forceinline__ void compute_half_chunk(const Chunk& ch, const u32x4_t& a_lo, const u32x4_t& a_hi, f32x4_t& acc0, f32x4_t& acc1,
+template <int HALF, class C>
+__device__ __forceinline__ void compute_half_chunk(const C& ch, const u32x4_t& a_lo, const u32x4_t& a_hi, f32x4_t& acc0, f32x4_t& acc1,
                                                    f32x4_t& acc2, f32x4_t& acc3, uint32_t lut_lo, uint32_t lut_hi) {
-  compute_half_tile<HALF>(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, a_lo, a_hi, acc0, lut_lo, lut_hi);
-  compute_half_tile<HALF>(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, a_lo, a_hi, acc1, lut_lo, lut_hi);
-  compute_half_tile<HALF>(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, a_lo, a_hi, acc2, lut_lo, lut_hi);
-  compute_half_tile<HALF>(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, a_lo, a_hi, acc3, lut_lo, lut_hi);
+  compute_half_tile<HALF, 0>(ch, a_lo, a_hi, acc0, lut_lo, lut_hi);
+  compute_half_tile<HALF, 1>(ch, a_lo, a_hi, acc1, lut_lo, lut_hi);
+  compute_half_tile<HALF, 2>(ch, a_lo, a_hi, acc2, lut_lo, lut_hi);
+  compute_half_tile<HALF, 3>(ch, a_lo, a_hi, acc3, lut_lo, lut_hi);
 }
 
 // ------------------------------------------------------------------------------------------------ the weight ring
 // (ring.hpp) for W3 blocks: three 16-byte loads a lane of codes, one 4-byte load a lane of scales.
 // AUX: the loads' cache policy - 2 (non-temporal) for a call that streams far more than the caches hold, 0 for one
 // token's few megabytes, which come in faster as ordinary loads.
+template <int AUX, int BITS = 3>
+struct W3RingOf;
+
 template <int AUX>
-struct W3RingOf {
+struct W3RingOf<AUX, 3> {
   typedef hb::Chunk Chunk;
   static constexpr int BLOCK_BYTES = W3_BLOCK_BYTES, LOADS = 4;
   // the lane's byte offsets in a block for the 16-byte and the 4-byte loads, and where it reads them back
@@ -132,8 +159,41 @@ struct W3RingOf {
         : "memory");
   }
 };
+// Two-bit blocks: two 16-byte loads a lane of codes, one 4-byte load a lane of scales; the two slots lie in the same
+// LDS a wavefront as a three-bit ring's (the launches size it for either).
+template <int AUX>
+struct W3RingOf<AUX, 2> {
+  typedef hb::Chunk2 Chunk;
+  static constexpr int BLOCK_BYTES = W2_BLOCK_BYTES, LOADS = 3;
+  static __device__ __forceinline__ void lanes(RingSource& src, int lane, int r16, uint32_t slot0, uint32_t& codes, uint32_t& scales) {
+    src.codes = 16u * lane;
+    src.scales = 4u * lane;
+    codes = slot0 + 16u * lane;
+    scales = slot0 + 16u * r16;
+  }
+  static __device__ __forceinline__ void request(const RingSource& src, int chunk, lds_ptr_t slot) {
+    const uint32_t at = (uint32_t)chunk * W2_BLOCK_BYTES;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 0, AUX);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024, AUX);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 4, src.scales, at, W2_SCALE_OFFSET, AUX);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  template <int BEHIND, int SLOT>
+  static __device__ __forceinline__ void take(Chunk& ch, uint32_t codes, uint32_t scales) {
+    asm volatile(
+        "s_waitcnt vmcnt(%5)\n\t"
+        "ds_read_b128 %0, %3 offset:%6\n\t"
+        "ds_read_b128 %1, %3 offset:%7\n\t"
+        "ds_read_b128 %2, %4 offset:%8\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(ch.w0), "=&v"(ch.w1), "=&v"(ch.sc)
+        : "v"(codes), "v"(scales), "n"(BEHIND), "n"(SLOT * W2_BLOCK_BYTES), "n"(SLOT * W2_BLOCK_BYTES + 1024), "n"(SLOT * W2_BLOCK_BYTES + W2_SCALE_OFFSET)
+        : "memory");
+  }
+};
 typedef W3RingOf<2> W3Ring;
 typedef W3RingOf<0> W3RingCached;
+typedef W3RingOf<2, 2> W2Ring;
 constexpr int RING_BYTES = ring_bytes<W3Ring>();  // LDS per wavefront; its first 4 KB double as the K-split exchange
 
 // ------------------------------------------------------------------------------------------- slots of one to four rows
@@ -166,10 +226,11 @@ __device__ __forceinline__ void store_pair(const StreamParams& p, int64_t pair, 
   }
 }
 
-__device__ __forceinline__ void compute_tile_few(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const Rows& ch, f32x4_t& acc,
-                                                 uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
+template <int NT, class C>
+__device__ __forceinline__ void compute_tile_few(const C& w, const Rows& ch, f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
+  const uint32_t scales = chunk_scales<NT>(w);
   uint32_t sel[8];
-  w3_selectors(q0, q1, q2, sel);
+  chunk_selectors<NT>(w, sel);
   f32x4_t part = {0.f, 0.f, 0.f, 0.f};
   part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a0), expand8(sel[0], sel[1], lut_lo, lut_hi), part, 0, 0, 0);
   part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ch.a1), expand8(sel[2], sel[3], lut_lo, lut_hi), part, 0, 0, 0);
@@ -188,10 +249,12 @@ __device__ __forceinline__ void compute_tile_few(uint32_t q0, uint32_t q1, uint3
 // activation codes of the chunk; xs: the activation scales of the slot's four rows at this lane's group.
 __device__ __forceinline__ long fp8x8(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
 
-__device__ __forceinline__ void compute_tile_few8(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const long a[4], const f32x4_t& xs,
-                                                  f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
+template <int NT, class C>
+__device__ __forceinline__ void compute_tile_few8(const C& w, const long a[4], const f32x4_t& xs, f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi,
+                                                  uint32_t q8) {
+  const uint32_t scales = chunk_scales<NT>(w);
   uint32_t sel[8];
-  w3_selectors(q0, q1, q2, sel);
+  chunk_selectors<NT>(w, sel);
   f32x4_t part = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int j = 0; j < 4; j++) {
@@ -205,20 +268,22 @@ __device__ __forceinline__ void compute_tile_few8(uint32_t q0, uint32_t q1, uint
   acc.w = fmaf(part.w, xs.w * s, acc.w);
 }
 
-__device__ __forceinline__ void compute_few8(const Chunk& ch, long a, const f32x4_t& xs, int grp, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
+template <class C>
+__device__ __forceinline__ void compute_few8(const C& ch, long a, const f32x4_t& xs, int grp, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
                                              f32x4_t& acc3, uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
   long rows[4];  // MFMA j's A operand: the lane's codes in its own group, zero in the others
 #pragma unroll
   for (int j = 0; j < 4; j++) rows[j] = grp == j ? a : 0L;
-  compute_tile_few8(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, rows, xs, acc0, lut_lo, lut_hi, q8);
-  compute_tile_few8(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, rows, xs, acc1, lut_lo, lut_hi, q8);
-  compute_tile_few8(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, rows, xs, acc2, lut_lo, lut_hi, q8);
-  compute_tile_few8(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, rows, xs, acc3, lut_lo, lut_hi, q8);
+  compute_tile_few8<0>(ch, rows, xs, acc0, lut_lo, lut_hi, q8);
+  compute_tile_few8<1>(ch, rows, xs, acc1, lut_lo, lut_hi, q8);
+  compute_tile_few8<2>(ch, rows, xs, acc2, lut_lo, lut_hi, q8);
+  compute_tile_few8<3>(ch, rows, xs, acc3, lut_lo, lut_hi, q8);
 }
 
 // `a`: the lane's sixteen activation bytes of the chunk (row r16 % 4 of the slot, the k range of group r16 / 4 that this
 // lane owns in the MFMA A operand); grp: that group.
-__device__ __forceinline__ void compute_few(const Chunk& ch, const u32x4_t& a, int grp, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
+template <class C>
+__device__ __forceinline__ void compute_few(const C& ch, const u32x4_t& a, int grp, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2,
                                             f32x4_t& acc3, uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
   const u32x4_t none = {0u, 0u, 0u, 0u};
   Rows rows;  // MFMA j's A operand: the lane's bytes in its own group, zero in the others
@@ -226,10 +291,10 @@ __device__ __forceinline__ void compute_few(const Chunk& ch, const u32x4_t& a, i
   rows.a1 = grp == 1 ? a : none;
   rows.a2 = grp == 2 ? a : none;
   rows.a3 = grp == 3 ? a : none;
-  compute_tile_few(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, rows, acc0, lut_lo, lut_hi, q8);
-  compute_tile_few(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, rows, acc1, lut_lo, lut_hi, q8);
-  compute_tile_few(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, rows, acc2, lut_lo, lut_hi, q8);
-  compute_tile_few(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, rows, acc3, lut_lo, lut_hi, q8);
+  compute_tile_few<0>(ch, rows, acc0, lut_lo, lut_hi, q8);
+  compute_tile_few<1>(ch, rows, acc1, lut_lo, lut_hi, q8);
+  compute_tile_few<2>(ch, rows, acc2, lut_lo, lut_hi, q8);
+  compute_tile_few<3>(ch, rows, acc3, lut_lo, lut_hi, q8);
 }
 
 // The two bodies of the stream differ in the activations: what registers they keep, when they ask for them, how a
@@ -251,8 +316,8 @@ struct FewActs {
     held[0] = load(0);
     if (n > 1) held[1] = load(1);
   }
-  template <int ODD, bool MORE2, bool MORE1>
-  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+  template <int ODD, bool MORE2, bool MORE1, class C>
+  __device__ __forceinline__ void step(const C& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
     compute_few(ch, held[ODD], grp, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi, q8);
     if (MORE2) held[ODD] = load(i + 2);
   }
@@ -283,8 +348,8 @@ struct FewActs8 {  // E4M3 activations: eight codes a lane and chunk, and the sc
     load(0, 0);
     if (n > 1) load(1, 1);
   }
-  template <int ODD, bool MORE2, bool MORE1>
-  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+  template <int ODD, bool MORE2, bool MORE1, class C>
+  __device__ __forceinline__ void step(const C& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
     compute_few8(ch, held[ODD], scale[ODD], grp, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi, q8);
     if (MORE2) load(ODD, i + 2);
   }
@@ -320,10 +385,12 @@ struct FewSplitActs {
     load(0, 0);
     if (n > 1) load(1, 1);
   }
-  static __device__ __forceinline__ void tile(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t scales, const i32x8_t& upper, const i32x8_t& lower, f32x4_t& acc,
-                                              uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
+  template <int NT, class C>
+  static __device__ __forceinline__ void tile(const C& w, const i32x8_t& upper, const i32x8_t& lower, f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi,
+                                              uint32_t q8) {
+    const uint32_t scales = chunk_scales<NT>(w);
     uint32_t sel[8];
-    w3_selectors(q0, q1, q2, sel);
+    chunk_selectors<NT>(w, sel);
     i32x8_t b;
 #pragma unroll
     for (int j = 0; j < 8; j++) b[j] = (int)__builtin_amdgcn_perm(lut_hi, lut_lo, sel[j]);
@@ -336,8 +403,8 @@ struct FewSplitActs {
     acc.z = fmaf(part.z, s, acc.z);
     acc.w = fmaf(part.w, s, acc.w);
   }
-  template <int ODD, bool MORE2, bool MORE1>
-  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+  template <int ODD, bool MORE2, bool MORE1, class C>
+  __device__ __forceinline__ void step(const C& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
     i32x8_t upper, lower;  // the lane's bytes in its group's two dwords, zero in the others
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -346,10 +413,10 @@ struct FewSplitActs {
       lower[2 * j] = grp == j ? (int)held[ODD][1].x : 0;
       lower[2 * j + 1] = grp == j ? (int)held[ODD][1].y : 0;
     }
-    tile(ch.w0.x, ch.w0.y, ch.w0.z, ch.sc.x, upper, lower, acc0, sl.lut_lo, sl.lut_hi, q8);
-    tile(ch.w0.w, ch.w1.x, ch.w1.y, ch.sc.y, upper, lower, acc1, sl.lut_lo, sl.lut_hi, q8);
-    tile(ch.w1.z, ch.w1.w, ch.w2.x, ch.sc.z, upper, lower, acc2, sl.lut_lo, sl.lut_hi, q8);
-    tile(ch.w2.y, ch.w2.z, ch.w2.w, ch.sc.w, upper, lower, acc3, sl.lut_lo, sl.lut_hi, q8);
+    tile<0>(ch, upper, lower, acc0, sl.lut_lo, sl.lut_hi, q8);
+    tile<1>(ch, upper, lower, acc1, sl.lut_lo, sl.lut_hi, q8);
+    tile<2>(ch, upper, lower, acc2, sl.lut_lo, sl.lut_hi, q8);
+    tile<3>(ch, upper, lower, acc3, sl.lut_lo, sl.lut_hi, q8);
     if (MORE2) load(ODD, i + 2);
   }
 };
@@ -374,8 +441,8 @@ struct FullActs {  // up to sixteen rows: lane (q, r16) feeds row r16, k 8 q .. 
     at = activation_row<EPI>(p, sl, lane & 15) + (int64_t)c0 * 128 + 8 * (lane >> 4);
     load_rows(held, at);
   }
-  template <int ODD, bool MORE2, bool MORE1>
-  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+  template <int ODD, bool MORE2, bool MORE1, class C>
+  __device__ __forceinline__ void step(const C& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
     const uint16_t* next = at + (int64_t)(i + 1) * 128;
     compute_half_chunk<0>(ch, held.a0, held.a1, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
     if (MORE1) {
@@ -426,33 +493,36 @@ struct FullActs8 {
     load_half(1, 0);
   }
   // groups 2 HALF and 2 HALF + 1 of the four tiles
-  template <int HALF>
-  __device__ __forceinline__ void half_chunk(const Chunk& ch, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, uint32_t lut_lo,
-                                             uint32_t lut_hi) const {
-    const uint32_t q0[4] = {ch.w0.x, ch.w0.w, ch.w1.z, ch.w2.y}, q1[4] = {ch.w0.y, ch.w1.x, ch.w1.w, ch.w2.z};
-    const uint32_t q2[4] = {ch.w0.z, ch.w1.y, ch.w2.x, ch.w2.w}, sc[4] = {ch.sc.x, ch.sc.y, ch.sc.z, ch.sc.w};
-    f32x4_t* acc[4] = {&acc0, &acc1, &acc2, &acc3};
+  // groups 2 HALF and 2 HALF + 1 of tile NT
+  template <int HALF, int NT, class C>
+  __device__ __forceinline__ void half_tile(const C& ch, f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi) const {
+    const uint32_t sc = chunk_scales<NT>(ch);
+    uint32_t sel[8];
+    chunk_selectors<NT>(ch, sel);  // the four the half does not use fold away
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-      uint32_t sel[8];
-      w3_selectors(q0[t], q1[t], q2[t], sel);  // the four the half does not use fold away
-#pragma unroll
-      for (int jj = 0; jj < 2; jj++) {
-        const int j = 2 * HALF + jj;
-        const long b = fp8x8(__builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j]), __builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j + 1]));
-        const f32x4_t part = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[j], b, f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-        const float ws = j == 0 ? __builtin_amdgcn_cvt_f32_fp8(sc[t], 0) : j == 1 ? __builtin_amdgcn_cvt_f32_fp8(sc[t], 1)
-                       : j == 2 ? __builtin_amdgcn_cvt_f32_fp8(sc[t], 2) : __builtin_amdgcn_cvt_f32_fp8(sc[t], 3);
-        const f32x2_t* xs = HALF ? xs_hi : xs_lo;
-        acc[t]->x = fmaf(part.x, (jj ? xs[0].y : xs[0].x) * ws, acc[t]->x);
-        acc[t]->y = fmaf(part.y, (jj ? xs[1].y : xs[1].x) * ws, acc[t]->y);
-        acc[t]->z = fmaf(part.z, (jj ? xs[2].y : xs[2].x) * ws, acc[t]->z);
-        acc[t]->w = fmaf(part.w, (jj ? xs[3].y : xs[3].x) * ws, acc[t]->w);
-      }
+    for (int jj = 0; jj < 2; jj++) {
+      const int j = 2 * HALF + jj;
+      const long b = fp8x8(__builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j]), __builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j + 1]));
+      const f32x4_t part = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[j], b, f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+      const float ws = j == 0 ? __builtin_amdgcn_cvt_f32_fp8(sc, 0) : j == 1 ? __builtin_amdgcn_cvt_f32_fp8(sc, 1)
+                     : j == 2 ? __builtin_amdgcn_cvt_f32_fp8(sc, 2) : __builtin_amdgcn_cvt_f32_fp8(sc, 3);
+      const f32x2_t* xs = HALF ? xs_hi : xs_lo;
+      acc.x = fmaf(part.x, (jj ? xs[0].y : xs[0].x) * ws, acc.x);
+      acc.y = fmaf(part.y, (jj ? xs[1].y : xs[1].x) * ws, acc.y);
+      acc.z = fmaf(part.z, (jj ? xs[2].y : xs[2].x) * ws, acc.z);
+      acc.w = fmaf(part.w, (jj ? xs[3].y : xs[3].x) * ws, acc.w);
     }
   }
-  template <int ODD, bool MORE2, bool MORE1>
-  __device__ __forceinline__ void step(const Chunk& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+  template <int HALF, class C>
+  __device__ __forceinline__ void half_chunk(const C& ch, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, uint32_t lut_lo,
+                                             uint32_t lut_hi) const {
+    half_tile<HALF, 0>(ch, acc0, lut_lo, lut_hi);
+    half_tile<HALF, 1>(ch, acc1, lut_lo, lut_hi);
+    half_tile<HALF, 2>(ch, acc2, lut_lo, lut_hi);
+    half_tile<HALF, 3>(ch, acc3, lut_lo, lut_hi);
+  }
+  template <int ODD, bool MORE2, bool MORE1, class C>
+  __device__ __forceinline__ void step(const C& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
     half_chunk<0>(ch, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
     if (MORE1) load_half(0, i + 1);
     half_chunk<1>(ch, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi);
@@ -584,12 +654,12 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Sl
   }
 }
 
-template <int EPI, bool A8, bool SPLIT = false>
+template <int EPI, bool A8, bool SPLIT = false, int BITS = 3>  // BITS: the tile layout's (two-bit matrices have their own)
 __global__ __launch_bounds__(1024) void w3_stream_kernel(StreamParams p) {
   extern __shared__ __align__(16) uint8_t rings[];
   const Slot sl = slot_of<EPI>(p, blockIdx.y);
   if (sl.rows <= 0) return;  // a slot the plan did not fill: the whole workgroup leaves
-  stream_workgroup<EPI, A8, SPLIT>(p, sl, blockIdx.x, rings);
+  stream_workgroup<EPI, A8, SPLIT, W3RingOf<2, BITS>>(p, sl, blockIdx.x, rings);
 }
 
 // One token from its router logits: fc1 with the routing inside it, so that the call has no launch for routing and plan.
@@ -847,11 +917,22 @@ static int shape_stream(StreamParams& p, int64_t busy_slots, Launch want) {
 }
 
 template <int EPI>
-static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Launch want, hipStream_t stream) {
+static int launch_stream(StreamParams& p, int64_t slots, int64_t busy_slots, Launch want, hipStream_t stream, int bits = 3) {
   if (int e = shape_stream(p, busy_slots, want)) return e;
   const dim3 grid((unsigned)((p.n_blocks + p.nbw - 1) / p.nbw), (unsigned)slots);
   const int waves = p.ks * p.nbw;
   const size_t lds = (size_t)waves * RING_BYTES;
+  if (bits == 2) {  // dense calls only: the reference's two-plane matrices are dense linears (its draft head)
+    if constexpr (epi_dense(EPI)) {
+      if (p.aq) {
+        HB_LAUNCH((w3_stream_kernel<EPI, true, false, 2>), grid, dim3(64 * waves), lds, stream, p);
+      } else {
+        HB_LAUNCH((w3_stream_kernel<EPI, false, false, 2>), grid, dim3(64 * waves), lds, stream, p);
+      }
+      return HB_OK;
+    }
+    return HB_EINVAL;
+  }
   if (p.aq) {
     HB_LAUNCH((w3_stream_kernel<EPI, true>), grid, dim3(64 * waves), lds, stream, p);
   } else if (p.a2 && !p.no_few) {
@@ -886,9 +967,9 @@ extern "C" int hb_tune(const char* key, int value) {
 }
 #endif
 
-extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, void* y, void* stream) {
+extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, int bits, void* y, void* stream) {
   if (!x || !tiled || !row_scale || !y) return HB_ENULL;
-  if (m <= 0 || n <= 0 || k <= 0 || n % W3_BLOCK_ROWS || k % W3_CHUNK) return HB_EINVAL;
+  if (m <= 0 || n <= 0 || k <= 0 || n % W3_BLOCK_ROWS || k % W3_CHUNK || (bits != 2 && bits != 3)) return HB_EINVAL;
   if (!aligned(x, 16) || !aligned(tiled, 16) || !aligned(row_scale, 4) || !aligned(y, 2)) return HB_EINVAL;
   StreamParams p{};
   p.w = static_cast<const uint8_t*>(tiled);
@@ -902,13 +983,14 @@ extern "C" int hb_w3_gemm(const void* x, int m, const void* tiled, const float* 
   p.m = m;
   p.out = y;
   p.out_stride = n;
-  if (tile_takes(m, k) && tile_writes(y, false) && (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && tile_serves_dense(m, p.n_blocks)))) {
+  // (the MFMA tile kernel reads three-bit tiles; a two-bit matrix is served by the stream at every size)
+  if (bits == 3 && tile_takes(m, k) && tile_writes(y, false) && (g_tune.w3_tile == 1 || (g_tune.w3_tile == 0 && tile_serves_dense(m, p.n_blocks)))) {
     if (int e = launch_tile<TileW3, EPI_DENSE>(p, (m + TILE_ROWS - 1) / TILE_ROWS, m, as_stream(stream))) return e;
     return launch_status();
   }
   const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
   if (slots > 65535) return HB_EINVAL;
-  if (int e = launch_stream<EPI_DENSE>(p, slots, slots, Launch{g_tune.w3_ksplit, g_tune.w3_nbw}, as_stream(stream))) return e;
+  if (int e = launch_stream<EPI_DENSE>(p, slots, slots, Launch{g_tune.w3_ksplit, g_tune.w3_nbw}, as_stream(stream), bits)) return e;
   return launch_status();
 }
 
@@ -929,9 +1011,9 @@ extern "C" int hb_w3_quant_rows(const void* x, int64_t m, int k, void* q, float*
 }
 
 extern "C" int hb_w3_gemm_e4m3(const void* xq, const float* x_scale, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k,
-                               void* y, void* stream) {
+                               int bits, void* y, void* stream) {
   if (!xq || !x_scale || !tiled || !row_scale || !y) return HB_ENULL;
-  if (m <= 0 || n <= 0 || k <= 0 || n % W3_BLOCK_ROWS || k % W3_CHUNK || (int64_t)m * (k / 32) > 0xffffffffll) return HB_EINVAL;
+  if (m <= 0 || n <= 0 || k <= 0 || n % W3_BLOCK_ROWS || k % W3_CHUNK || (int64_t)m * (k / 32) > 0xffffffffll || (bits != 2 && bits != 3)) return HB_EINVAL;
   if (!aligned(xq, 8) || !aligned(x_scale, 8) || !aligned(tiled, 16) || !aligned(row_scale, 4) || !aligned(y, 2)) return HB_EINVAL;
   StreamParams p{};
   p.w = static_cast<const uint8_t*>(tiled);
@@ -948,7 +1030,7 @@ extern "C" int hb_w3_gemm_e4m3(const void* xq, const float* x_scale, int m, cons
   p.out_stride = n;
   const int64_t slots = (m + ROWS_PER_SLOT - 1) / ROWS_PER_SLOT;
   if (slots > 65535) return HB_EINVAL;
-  if (int e = launch_stream<EPI_DENSE>(p, slots, slots, Launch{g_tune.w3_ksplit, g_tune.w3_nbw}, as_stream(stream))) return e;
+  if (int e = launch_stream<EPI_DENSE>(p, slots, slots, Launch{g_tune.w3_ksplit, g_tune.w3_nbw}, as_stream(stream), bits)) return e;
   return launch_status();
 }
 
@@ -1016,7 +1098,7 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   const int64_t est = pairs < 2 * ex->experts ? (pairs + 1) / 2 + (shared_rows + 15) / 16 : slots;  // rough number of busy slots
   StreamParams p{};
   p.w = static_cast<const uint8_t*>(ex->fc1);
-  p.expert_bytes = (int64_t)hb_w3_tiled_bytes(n1, ex->hidden);
+  p.expert_bytes = (int64_t)hb_w3_tiled_bytes(n1, ex->hidden, 3);
   p.rows = ex->fc1_rows;
   p.expert_rows = n1;
   p.lut_lo = (uint32_t)((uint64_t)ex->fc1_lut & 0xffffffffu);
@@ -1039,7 +1121,7 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   p.out_stride = ex->inter;
   StreamParams f2 = p;
   f2.w = static_cast<const uint8_t*>(ex->fc2);
-  f2.expert_bytes = (int64_t)hb_w3_tiled_bytes(ex->hidden_out, ex->inter);
+  f2.expert_bytes = (int64_t)hb_w3_tiled_bytes(ex->hidden_out, ex->inter, 3);
   f2.rows = ex->fc2_rows;
   f2.expert_rows = ex->hidden_out;
   f2.lut_lo = (uint32_t)((uint64_t)ex->fc2_lut & 0xffffffffu);

@@ -62,6 +62,7 @@ class W3Weight:
     codebook: tuple[float, ...]
     lut: int  # the codebook as eight E4M3 bytes, entry i in byte i
     tiled: torch.Tensor | None = None  # uint8, the kernels' block layout (built by tile())
+    tile_bits: int = 0  # the bits of `tiled`'s tiles: the codebook's own (a two-bit matrix keeps its density), or 3 when widened
 
     @property
     def bytes(self) -> int:
@@ -94,20 +95,25 @@ def _codebook(codebook) -> tuple[float, ...]:
     return levels
 
 
-def tile(w3: W3Weight, release: bool = False) -> W3Weight:
-    """Build the kernels' block layout from the fragment-order tensors (once). `release` drops the latter."""
-    if w3.tiled is None:
+def tile(w3: W3Weight, release: bool = False, widen: bool = False) -> W3Weight:
+    """Build the kernels' block layout from the fragment-order tensors (once). `release` drops the latter. A two-bit
+    matrix gets two-bit tiles (2.25 bits a weight, what `w3_linear` streams); `widen`: three-bit tiles whatever the
+    codebook (the routed experts' kernels read only those)."""
+    want = 3 if widen else w3.bits
+    if w3.tiled is not None and w3.tile_bits == 0:
+        w3.tile_bits = 3  # a tiled copy handed in as it was loaded: three-bit tiles
+    if w3.tiled is None or w3.tile_bits != want:
         if w3.planes is None:
-            raise ValueError("W3Weight holds neither planes nor a tiled copy")
+            raise ValueError("W3Weight holds neither planes nor a tiled copy of the tiles asked for")
         _lib.need_gpu(w3.planes, w3.scales)
         n, k = w3.out_features, w3.in_features
-        size = _lib.lib().hb_w3_tiled_bytes(n, k)
+        size = _lib.lib().hb_w3_tiled_bytes(n, k, want)
         if size == 0:
             raise ValueError("W3 kernels need N a multiple of 64 and K a multiple of 128")
         tiled = torch.empty(size, dtype=torch.uint8, device=w3.planes.device)
         planes, scales = w3.planes.contiguous(), w3.scales.contiguous()
-        _lib.check(_lib.lib().hb_w3_repack(_lib.ptr(planes), _lib.ptr(scales), n, k, w3.bits, _lib.ptr(tiled), _lib.stream()), "w3 repack")
-        w3.tiled = tiled
+        _lib.check(_lib.lib().hb_w3_repack(_lib.ptr(planes), _lib.ptr(scales), n, k, w3.bits, want, _lib.ptr(tiled), _lib.stream()), "w3 repack")
+        w3.tiled, w3.tile_bits = tiled, want
     if release:
         w3.planes = w3.scales = None
     return w3
@@ -231,7 +237,7 @@ def _unpack(w3: W3Weight, want_codes: bool, want_scales: bool):
     codes8 = torch.empty((n, k), dtype=torch.uint8, device=dev) if want_codes else None
     raw = torch.empty((n, k // GROUP), dtype=torch.uint8, device=dev) if want_scales else None
     if w3.tiled is not None:
-        _lib.check(_lib.lib().hb_w3_unpack(_lib.ptr(w3.tiled), n, k, _lib.ptr(codes8), _lib.ptr(raw), _lib.stream()), "w3 unpack")
+        _lib.check(_lib.lib().hb_w3_unpack(_lib.ptr(w3.tiled), n, k, w3.tile_bits or 3, _lib.ptr(codes8), _lib.ptr(raw), _lib.stream()), "w3 unpack")
     else:
         planes, scales = w3.planes.contiguous(), w3.scales.contiguous()
         _lib.check(_lib.lib().hb_w3_unpack_planes(_lib.ptr(planes), _lib.ptr(scales), n, k, w3.bits,
@@ -259,7 +265,7 @@ def dequantize(w3: W3Weight) -> torch.Tensor:
     tile(w3)
     n, k = w3.out_features, w3.in_features
     out = torch.empty((n, k), dtype=torch.float32, device=w3.tiled.device)
-    _lib.check(_lib.lib().hb_w3_dequant(_lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut, n, k, _lib.ptr(out), _lib.stream()), "w3 dequantize")
+    _lib.check(_lib.lib().hb_w3_dequant(_lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut, n, k, w3.tile_bits, _lib.ptr(out), _lib.stream()), "w3 dequantize")
     return out
 
 
@@ -346,9 +352,9 @@ def w3_linear(x: torch.Tensor, w3: W3Weight, x_scale: torch.Tensor | None = None
             raise ValueError("w3_linear: x_scale must have 1, M or M * K/32 elements")
         scale = x_scale.float().reshape(-1, groups if x_scale.numel() == m * groups else 1).expand(m, groups).contiguous()
         _lib.check(_lib.lib().hb_w3_gemm_e4m3(_lib.ptr(x), _lib.ptr(scale), m, _lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut,
-                                              w3.out_features, k, _lib.ptr(y), _lib.stream()), "w3_linear")
+                                              w3.out_features, k, w3.tile_bits, _lib.ptr(y), _lib.stream()), "w3_linear")
         return y
-    _lib.check(_lib.lib().hb_w3_gemm(_lib.ptr(x), m, _lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut, w3.out_features, k,
+    _lib.check(_lib.lib().hb_w3_gemm(_lib.ptr(x), m, _lib.ptr(w3.tiled), _lib.ptr(w3.row_scale), w3.lut, w3.out_features, k, w3.tile_bits,
                                      _lib.ptr(y), _lib.stream()), "w3_linear")
     return y
 

@@ -104,7 +104,7 @@ def tile(experts: W3Experts, release: bool = False) -> W3Experts:
     """Build the kernels' block layout of both stacks (once); `release` drops the fragment-order tensors."""
     for fc1 in (True, False):
         if (experts.tiled13 if fc1 else experts.tiled2) is None:
-            stacked = w3.tile(experts.stacked(fc1))
+            stacked = w3.tile(experts.stacked(fc1), widen=True)  # the experts' kernels read three-bit tiles
             if fc1:
                 experts.tiled13 = stacked.tiled
             else:

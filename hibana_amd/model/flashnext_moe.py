@@ -5,6 +5,8 @@
     ids, w  = top-k of softmax(logits), renormalized          (padded rows of a graph: id E, weight 0)
     routed  = sum_k w_k * down_e(silu(gate_e x) * up_e x)      3-bit experts
     shared  = shared_down(silu(shared_gate x) * shared_up x)   3-bit, rides in the experts' launches as one more expert
+                                                               (calls the reference serves from the NVFP4 linears - more
+                                                               than w3.MAX_ROWS rows, or HIBANA_W3_DECODE off - run on them)
     out     = bf16(bf16(routed) + sigmoid(x . shared_gate_vec) * shared)
 
 The block is assembled from tensors already on the device (a loader's job ends there). The routed experts are a
@@ -66,8 +68,10 @@ class MoeLayer:
             raise ValueError(f"3-bit experts {experts.base}..{experts.base + experts.experts - 1}: the model has {self.experts}")
         if shared is None and shared_gate_up is not None:
             if getattr(shared_gate_up, "w3", None) is None or getattr(shared_down, "w3", None) is None:
-                raise ValueError("the shared expert's linears need their 3-bit copies (w3.attach)")
-            shared = shared_from_linears(shared_gate_up.w3, shared_down.w3)
+                if getattr(shared_gate_up, "weight", None) is None:
+                    raise ValueError("the shared expert's linears need their 3-bit copies (w3.attach) or NVFP4 weights to run on")
+            else:
+                shared = shared_from_linears(shared_gate_up.w3, shared_down.w3)
         self.shared = None if shared is None else w3_moe.tile(shared)
         self.shared_gate_up, self.shared_down = shared_gate_up, shared_down
 
@@ -117,8 +121,25 @@ class MoeLayer:
         """The routed experts' weighted sum (this rank's part) for x [M, H] -> BF16 [M, H]."""
         return w3_moe.w3_moe(self.w3, x, ids, weights)
 
+    def shared_on_linears(self, m: int) -> bool:
+        """Whether a call of `m` rows runs the shared expert on its own linears: the reference does, and takes their 3-bit
+        copies only where `ops.w3_decode` holds - at most w3.MAX_ROWS rows with HIBANA_W3_DECODE on
+        (hibana/model/flashnext/moe.py:181-189, hibana/kernels/ops.py:50-53). Linears that hold nothing but a 3-bit
+        copy (no NVFP4 weights to run) always ride in the experts' launches."""
+        lin = self.shared_gate_up
+        if lin is None or self.shared_down is None or getattr(lin, "weight", None) is None or getattr(lin, "in_features", None) is None:
+            return False
+        return not (ops.w3_decode(lin, m) and ops.w3_decode(self.shared_down, m))
+
     def __call__(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
         x = x.contiguous()
+        if self.shared_on_linears(x.shape[0]):
+            # the reference's own chain: the experts' unsummed pair outputs (BF16 from WIDE_ROWS rows), the shared expert
+            # on its linears (silu(gate) * up in between), the combine over both
+            ids, weights = self.route(x, ctx)
+            pairs = w3_moe.w3_moe(self.w3, x, ids, weights, pairs=True, pairs_bf16=x.shape[0] >= w3_moe.WIDE_ROWS)
+            shared = ops.nvfp4_linear(ops.silu_and_mul(ops.nvfp4_linear(x, self.shared_gate_up)), self.shared_down)
+            return ops.moe_combine_pairs(pairs, ids, weights, shared, x, self.shared_gate_vec, self.w3.base, self.w3.experts)
         slots, _ = self._padding(ctx)
         if slots is None and not self.selects(ctx):  # routing, plan, both streams and the combine as one chain
             logits = torch.mm(x, self.router.T).float()

@@ -132,40 +132,45 @@ int64_t hb_debug_mfma_rate(int blocks, int iters, void* sink, void* stream);
  * `rows` may stack several matrices (experts) of the same K as long as each has a multiple of 64 rows.
  * ---------------------------------------------------------------------------------------------------------------- */
 
-/* Bytes of the tile layout of a [rows, k] matrix; 0 if rows % 64 or k % 128. */
-size_t hb_w3_tiled_bytes(int64_t rows, int k);
+/* Bytes of the tile layout of a [rows, k] matrix of `bits`-bit tiles (3: blocks of 3328 bytes; 2: of 2304); 0 if
+ * rows % 64, k % 128 or bits is neither. */
+size_t hb_w3_tiled_bytes(int64_t rows, int k, int bits);
 
-/* Reference layout -> tile layout (load-time repack). bits = 3 or 2 (2-bit codes are widened to 3 bits).
- * ref: the layout contract of w3_gemm's operands, hibana/kernels/csrc/w3_gemm.cu:1299-1315; hook point
- * hibana/weights/w3_checkpoint.py:115-139 (CalibratedWeights._load). */
-int hb_w3_repack(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, void* tiled, void* stream);
+/* Reference layout -> tile layout (load-time repack). bits = 3 or 2: the planes' (the reference streams two planes for a
+ * four-level codebook, hibana/kernels/w3.py:12-19,89-91); tile_bits: the tiles' - bits itself (a two-bit matrix keeps
+ * its 2.25 bits a weight; hb_w3_gemm serves it), or 3 for two-bit codes widened into three-bit tiles (what the routed
+ * experts' kernels read).
+ * ref: the layout contract of w3_gemm's operands, hibana/kernels/csrc/w3_gemm.cu:1299-1315 (kernel template P, :113);
+ * hook point hibana/weights/w3_checkpoint.py:115-139 (CalibratedWeights._load). */
+int hb_w3_repack(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, int tile_bits, void* tiled, void* stream);
 
 /* codes uint8 [rows, k] + E4M3 scale bytes uint8 [rows, k/32] -> reference layout (planes, scales).
  * ref: w3._pack_codes_rows, hibana/kernels/w3.py:175-195. */
 int hb_w3_pack_codes(const uint8_t* codes, const uint8_t* scale_bytes, int64_t rows, int k, int bits, uint32_t* planes,
                      uint8_t* scales, void* stream);
 
-/* Tile layout -> codes uint8 [rows, k] and E4M3 scale bytes uint8 [rows, k/32] (either output may be NULL).
+/* Tile layout (of `bits`-bit tiles) -> codes uint8 [rows, k] and E4M3 scale bytes uint8 [rows, k/32] (either output may be NULL).
  * ref: w3.codes / the byte part of w3.group_scales, hibana/kernels/w3.py:217-236. */
-int hb_w3_unpack(const void* tiled, int64_t rows, int k, uint8_t* codes, uint8_t* scale_bytes, void* stream);
+int hb_w3_unpack(const void* tiled, int64_t rows, int k, int bits, uint8_t* codes, uint8_t* scale_bytes, void* stream);
 
 /* Reference layout -> codes / scale bytes, same outputs as hb_w3_unpack (the unpack of a checkpoint tensor as stored).
  * ref: hibana/kernels/w3.py:217-236. */
 int hb_w3_unpack_planes(const uint32_t* planes, const uint8_t* scales, int64_t rows, int k, int bits, uint8_t* codes,
                         uint8_t* scale_bytes, void* stream);
 
-/* Tile layout -> float32 [rows, k]: level[code] * (float(e4m3 scale) * row_scale[row]), both products rounded to
+/* Tile layout (of `bits`-bit tiles) -> float32 [rows, k]: level[code] * (float(e4m3 scale) * row_scale[row]), both products rounded to
  * FP32 in this order (bit-exact with the reference's unpack). `lut` = the codebook as 8 E4M3 bytes, entry i in byte i.
  * ref: w3.dequantize, hibana/kernels/w3.py:239-242; lut: w3.lut_of, :105-107. */
-int hb_w3_dequant(const void* tiled, const float* row_scale, int64_t lut, int64_t rows, int k, float* out, void* stream);
+int hb_w3_dequant(const void* tiled, const float* row_scale, int64_t lut, int64_t rows, int k, int bits, float* out, void* stream);
 
 /* y[m, n] = bf16( row_scale[n] * sum_g scale[n, g] * sum_{k in g} x[m, k] * level[code[n, k]] ), FP32 accumulation,
  * x BF16 [m, k] row-major with row stride k, y BF16 [m, n]. Any m >= 1 (the reference stops at 128 rows).
- * n % 64 == 0, k % 128 == 0.
+ * n % 64 == 0, k % 128 == 0. bits: the tiles' (3, or 2 for a matrix repacked at two bits: the weight stream then reads
+ * 2.25 bits a weight, as the reference's kernel does for its draft head's copy, hibana/proposers/draft_head.py:106).
  * ref: w3_gemm / w3_gemm_wide, hibana/kernels/csrc/w3_gemm.cu:1299-1331,1385-1413 (called by w3.w3_linear,
  * hibana/kernels/w3.py:340-365), in its weight-only form (BF16 activations are not re-quantized to E4M3). */
-int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, void* y,
-               void* stream);
+int hb_w3_gemm(const void* x, int m, const void* tiled, const float* row_scale, int64_t lut, int n, int k, int bits,
+               void* y, void* stream);
 
 /* The reference's activation rounding: x BF16 [m, k] (k % 32 == 0) -> q E4M3 bytes [m, k], scales float32 [m, k / 32]:
  * s = max(amax / 448, 1e-12) per (row, 32-group), q = e4m3(clamp(x / s, -448, 448)), IEEE FP32 divisions.
@@ -188,7 +193,7 @@ int hb_w3_quant_rows(const void* x, int64_t m, int k, void* q, float* scales, vo
  * ref: w3_gemm, hibana/kernels/csrc/w3_gemm.cu:105-108,209-210,1299-1331 (w3.w3_linear with E4M3 x, hibana/kernels/
  * w3.py:340-365). */
 int hb_w3_gemm_e4m3(const void* xq, const float* x_scale, int m, const void* tiled, const float* row_scale, int64_t lut,
-                    int n, int k, void* y, void* stream);
+                    int n, int k, int bits, void* y, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
  * Routed experts on W3 weights (gated SiLU when fc1 has 2*inter rows per expert in the reference's fc1_order, ReLU^2

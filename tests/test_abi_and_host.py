@@ -27,18 +27,30 @@ def test_library_exports_every_declared_symbol():
     assert sorted(_lib.SIGNATURES) == names  # the Python binding covers the header, nothing more, nothing less
 
 
+def test_a_build_without_debug_hooks_exports_none_of_them():
+    """-DHB_NO_DEBUG_HOOKS: hb_tune and every hb_debug_* are gone (a serving process cannot race on them), the rest of
+    the header is there; the default build has all of it. Host-only compiles: no device code is built here."""
+    from hibana_amd import build
+    hooks = {n for n in _declared() if n == "hb_tune" or n.startswith("hb_debug_")}
+    assert len(hooks) >= 7
+    assert build.host_symbols(no_debug_hooks=True) == set(_declared()) - hooks
+    assert build.host_symbols(no_debug_hooks=False) == set(_declared())
+
+
 def test_validation_without_a_gpu():
     lib = _lib.lib()
     assert lib.hb_version() >= 1000
     assert lib.hb_error_string(0) == b"ok" and b"workspace" in lib.hb_error_string(_lib.HB_EWORKSPACE)
-    assert lib.hb_w3_tiled_bytes(1024, 2048) == 1024 * 2048 * 3 // 8 + 1024 * 2048 // 32
-    assert lib.hb_w3_tiled_bytes(96, 2048) == 0 and lib.hb_w3_tiled_bytes(128, 100) == 0
+    assert lib.hb_w3_tiled_bytes(1024, 2048, 3) == 1024 * 2048 * 3 // 8 + 1024 * 2048 // 32
+    assert lib.hb_w3_tiled_bytes(1024, 2048, 2) == 1024 * 2048 * 2 // 8 + 1024 * 2048 // 32  # a two-bit matrix at its own density
+    assert lib.hb_w3_tiled_bytes(96, 2048, 3) == 0 and lib.hb_w3_tiled_bytes(128, 100, 3) == 0 and lib.hb_w3_tiled_bytes(128, 128, 4) == 0
     assert lib.hb_nvfp4_tiled_bytes(128, 256) == 128 * 256 // 2 + 128 * 256 // 16
     assert lib.hb_nvfp4_tiled_bytes(128, 64) == 0
     assert lib.hb_tune(b"no_such_knob", 1) == _lib.HB_EINVAL and lib.hb_tune(b"w3_ksplit", 17) == _lib.HB_EINVAL
     assert lib.hb_tune(b"w3_ksplit", 4) == 0 and lib.hb_tune(b"w3_ksplit", 0) == 0
-    assert lib.hb_w3_repack(None, None, 128, 128, 3, None, None) == _lib.HB_ENULL
-    assert lib.hb_w3_gemm(None, 1, None, None, 0, 128, 128, None, None) == _lib.HB_ENULL
+    assert lib.hb_w3_repack(None, None, 128, 128, 3, 3, None, None) == _lib.HB_ENULL
+    assert lib.hb_w3_repack(256, 256, 128, 128, 3, 2, 256, None) == _lib.HB_EINVAL  # codes are widened, never narrowed
+    assert lib.hb_w3_gemm(None, 1, None, None, 0, 128, 128, 3, None, None) == _lib.HB_ENULL
     assert lib.hb_nvfp4_gemm(None, 1, None, 1.0, 128, 128, 0, None, None) == _lib.HB_ENULL
     assert lib.hb_w3_moe_workspace_bytes(4, 2, None, 0) == 0
     ex = _lib.HbW3Experts(256, 256, 256, 256, 0, 0, 8, 0, 256, 128, 256, 1)  # (no call below reads through the pointers)
@@ -50,7 +62,8 @@ def test_validation_without_a_gpu():
     # pointers off the boundaries the kernels' vector accesses need are refused before anything is launched
     odd = _lib.HbW3Experts(264, 256, 256, 256, 0, 0, 8, 0, 256, 128, 256, 1)  # fc1 on an 8-byte boundary only
     assert lib.hb_w3_moe_workspace_bytes(32, 10, C.byref(odd), 1) == 0
-    assert lib.hb_w3_gemm(258, 1, 256, 256, 0, 128, 128, 256, None) == _lib.HB_EINVAL  # x on a 2-byte boundary
+    assert lib.hb_w3_gemm(258, 1, 256, 256, 0, 128, 128, 3, 256, None) == _lib.HB_EINVAL  # x on a 2-byte boundary
+    assert lib.hb_w3_gemm(256, 1, 256, 256, 0, 128, 128, 4, 256, None) == _lib.HB_EINVAL  # tiles of two or three bits
     assert lib.hb_w3_moe(C.byref(ex), 256, 256, 256, 1, 1, 0, 256, 264, 1 << 30, None) == _lib.HB_EINVAL  # workspace on 8
     assert lib.hb_nvfp4_gemm(256, 1, 260, 1.0, 128, 128, 0, 256, None) == _lib.HB_EINVAL  # tile layout on 4
     # the dense product with a workspace: sizes only (no launch without a GPU)

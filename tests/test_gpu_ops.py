@@ -175,6 +175,51 @@ def test_moe_layer_block(m, mode):
     assert torch.equal(layer(x.cuda(), None), layer(x.cuda(), SimpleNamespace(mode="prefill")))
 
 
+@pytest.mark.parametrize("m,decode", [(200, True), (40, False), (40, True)])
+def test_moe_layer_runs_the_shared_expert_where_the_reference_does(m, decode):
+    """The shared expert as the reference holds it - two NVFP4 linears with 3-bit copies attached: a call the reference
+    serves from the copies (at most w3.MAX_ROWS rows with HIBANA_W3_DECODE on, ops.w3_decode) runs them inside the
+    experts' launches; any other call (more rows, or the switch off) runs the NVFP4 linears and the combine over the
+    pair outputs (hibana/model/flashnext/moe.py:181-189). Each against the oracle on the weights that call uses."""
+    from hibana_amd.kernels import w3
+    from hibana_amd.model.flashnext_moe import MoeLayer
+    from hibana_amd.weights import modelopt
+    from oracle import nvfp4_format as onv
+    from tests.test_gpu_nvfp4_moe import _stack
+    e, hidden, inter, topk = 16, 256, 128, 4
+    ex, per = random_experts(e, hidden, inter, True, 91)
+    get = oracle_expert_getter(per, True, inter)
+    g = torch.Generator().manual_seed(92 + m)
+    router = (torch.randn(e, hidden, generator=g) * 0.3).bfloat16()
+    gate_vec = torch.randn(1, hidden, generator=g) * 0.05
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    lins, dense = [], []
+    for rows, k, seed, copy_seed in ((2 * inter, hidden, 93, 95), (hidden, inter, 94, 96)):  # gate_up rows [gate; up], down
+        (w, sc, g2) = _stack(1, rows, k, seed)
+        lin = modelopt.Nvfp4Linear(dev(w[0]), dev(onv.swizzle_block_scales(sc[0])).view(torch.float8_e4m3fn), torch.tensor(float(g2[0])).cuda(),
+                                   torch.tensor(1.0).cuda(), rows, k).tile()
+        copy, *_ = random_w3(rows, k, copy_seed)  # any 3-bit matrix: the two paths must be told apart
+        lin.w3 = to_device_w3(copy)
+        lins.append(lin)
+        dense.append((onv.unpack_fp4(w[0], sc[0]) * np.float32(g2[0]), ow3.dequantize(copy)))
+    layer = MoeLayer(router.cuda(), gate_vec.cuda(), ex, topk, shared_gate_up=lins[0], shared_down=lins[1])
+    x = torch.randn(m, hidden, generator=g).bfloat16()
+    w3.set_enabled(decode)
+    try:
+        on_linears = layer.shared_on_linears(m)
+        assert on_linears == (m > w3.MAX_ROWS or not decode)
+        got = layer(x.cuda(), None)
+        ids, weights = layer.route(x.cuda(), None)
+    finally:
+        w3.set_enabled(None)
+    which = 0 if on_linears else 1
+    gu, down = dense[0][which], dense[1][which]
+    shared_w13 = np.concatenate([gu[inter:], gu[:inter]])  # checkpoint order [up; gate]
+    want = layers.moe_layer_ref(x, ids.cpu().numpy(), weights.cpu(), get, True, shared=(shared_w13, down), gate_vec=gate_vec.reshape(-1), e_n=e)
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+
+
 def test_attach_model_takes_calibrated_copies(tmp_path):
     """attach_model with a W3 checkpoint: every projection gets the checkpoint's copy (tiled), the model's identity is
     the manifest's digest; a checkpoint that does not cover the model is refused; without one, nearest-level copies."""

@@ -30,13 +30,19 @@ def test_repack_unpack_and_dequantize_are_bit_exact(n, k, codebook):
     assert np.array_equal(w3.scale_bytes(dev).view(torch.uint8).cpu().numpy(), raw)
     # the kernels' block layout
     w3.tile(dev)
-    assert dev.tiled.numel() == n * k * 3 // 8 + n * k // 32
+    bits = 2 if codebook == "lloyd2" else 3  # a two-bit matrix keeps its density: 2.25 bits a weight
+    assert dev.tile_bits == bits and dev.tiled.numel() == n * k * bits // 8 + n * k // 32
     assert np.array_equal(w3.codes(dev).cpu().numpy(), q)
     assert np.array_equal(w3.scale_bytes(dev).view(torch.uint8).cpu().numpy(), raw)
     want = ow3.dequantize(packed)
     got = w3.dequantize(dev).cpu().numpy()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))  # FP32 bit patterns
     assert np.array_equal(w3.group_scales(dev).cpu().numpy().view(np.uint32), ow3.group_scales(packed).view(np.uint32))
+    if bits == 2:  # the same matrix widened into three-bit tiles (what the routed experts' kernels read): the same weights
+        wide = w3.tile(to_device_w3(packed), widen=True)
+        assert wide.tile_bits == 3 and wide.tiled.numel() == n * k * 3 // 8 + n * k // 32
+        assert np.array_equal(w3.codes(wide).cpu().numpy(), q)
+        assert np.array_equal(w3.dequantize(wide).cpu().numpy().view(np.uint32), want.view(np.uint32))
     w3.tile(dev, release=True)
     assert dev.planes is None and np.array_equal(w3.codes(dev).cpu().numpy(), q)
 

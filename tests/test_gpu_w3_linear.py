@@ -41,6 +41,40 @@ def test_w3_linear_matches_the_oracle(m, n, k, codebook):
     assert torch.equal(again, got)  # bitwise repeatable
 
 
+@pytest.mark.parametrize("m", [1, 4, 5, 16, 33, 128])
+@pytest.mark.parametrize("n,k", [(256, 384), (512, 2048), (128, 128), (3072, 1024)])  # the last: a draft head's shape (vocabulary rows x hidden)
+def test_two_bit_linear_matches_the_oracle(m, n, k, kernel_choice):
+    """A four-level codebook (the reference's two-plane variant, its draft head's copy: hibana/proposers/draft_head.py:106)
+    through the product at its own density - two-bit tiles, 2.25 bits a weight - on BF16 and on E4M3 activations, and the
+    same matrix widened into three-bit tiles gives the same bits."""
+    from hibana_amd.kernels import w3
+    packed, *_ = random_w3(n, k, 17, "lloyd2")
+    dev = to_device_w3(packed)
+    g = torch.Generator().manual_seed(300 + m)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    x[:, ::97] *= 30
+    dense = ow3.dequantize(packed)
+    want = layers.dense_ref(x, dense)
+    got = w3.w3_linear(x.cuda(), dev)
+    assert dev.tile_bits == 2 and dev.tiled.numel() == n * k // 4 + n * k // 32
+    mx, nr = errors(got, want)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    assert torch.equal(w3.w3_linear(x.cuda(), dev), got)
+    wide = w3.tile(to_device_w3(packed), widen=True)
+    assert wide.tile_bits == 3
+    if kernel_choice.startswith("stream"):  # the same sums from either layout (the MFMA tile kernel, which serves only three-bit tiles, adds in another order)
+        assert torch.equal(w3.w3_linear(x.cuda(), wide), got)
+    else:
+        mx, nr = errors(w3.w3_linear(x.cuda(), wide), want)
+        assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    q, s = w3.quant_groups(x.cuda())
+    want8 = layers.dense_a8_ref(x, dense)
+    got8 = w3.w3_linear(q, dev, s)
+    mx, nr = errors(got8, want8)
+    assert mx < MAX_REL and nr < NORM_REL, (mx, nr)
+    assert torch.equal(w3.w3_linear(q, wide, s), got8)
+
+
 def test_every_k_split_gives_close_results_and_the_unsplit_bits_repeat():
     from hibana_amd import _lib
     from hibana_amd.kernels import w3
