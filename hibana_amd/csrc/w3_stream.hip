@@ -194,6 +194,52 @@ struct W3RingOf<AUX, 2> {
 typedef W3RingOf<2> W3Ring;
 typedef W3RingOf<0> W3RingCached;
 typedef W3RingOf<2, 2> W2Ring;
+
+// A ring that brings in only what the 16-row tiles T0 .. T1 - 1 of a three-bit block need: tile t's three code dwords are
+// dwords 3 t .. 3 t + 2 of the lane's twelve, four to a 16-byte load, so the tiles' loads are 3 T0 / 4 .. (3 T1 - 1) / 4 (one
+// or two of the three for one tile or a pair of them), and the scales. The Chunk's other registers stay unset and unread.
+template <int AUX, int T0, int T1>
+struct W3RingPart {
+  typedef hb::Chunk Chunk;
+  static constexpr int L0 = 3 * T0 / 4, L1 = (3 * T1 - 1) / 4, CODE_LOADS = L1 - L0 + 1;
+  static constexpr int BLOCK_BYTES = W3_BLOCK_BYTES, LOADS = CODE_LOADS + 1;
+  static_assert(0 <= T0 && T0 < T1 && T1 <= 4 && CODE_LOADS >= 1 && CODE_LOADS <= 2, "a tile or a pair of tiles (the whole block: W3RingOf)");
+  static __device__ __forceinline__ void lanes(RingSource& src, int lane, int r16, uint32_t slot0, uint32_t& codes, uint32_t& scales) {
+    W3RingOf<AUX>::lanes(src, lane, r16, slot0, codes, scales);
+  }
+  static __device__ __forceinline__ void request(const RingSource& src, int chunk, lds_ptr_t slot) {
+    const uint32_t at = (uint32_t)chunk * W3_BLOCK_BYTES;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024 * L0, AUX);
+    if (CODE_LOADS == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 16, src.codes, at, 1024 * L1, AUX);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src.row, slot, 4, src.scales, at, W3_SCALE_OFFSET, AUX);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  static __device__ __forceinline__ u32x4_t& load_of(Chunk& ch, int l) { return l == 0 ? ch.w0 : l == 1 ? ch.w1 : ch.w2; }
+  template <int BEHIND, int SLOT>
+  static __device__ __forceinline__ void take(Chunk& ch, uint32_t codes, uint32_t scales) {
+    if (CODE_LOADS == 2) {
+      asm volatile(
+          "s_waitcnt vmcnt(%5)\n\t"
+          "ds_read_b128 %0, %3 offset:%6\n\t"
+          "ds_read_b128 %1, %3 offset:%7\n\t"
+          "ds_read_b128 %2, %4 offset:%8\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&v"(load_of(ch, L0)), "=&v"(load_of(ch, L1)), "=&v"(ch.sc)
+          : "v"(codes), "v"(scales), "n"(BEHIND), "n"(SLOT * W3_BLOCK_BYTES + 1024 * L0), "n"(SLOT * W3_BLOCK_BYTES + 1024 * L1),
+            "n"(SLOT * W3_BLOCK_BYTES + W3_SCALE_OFFSET)
+          : "memory");
+    } else {
+      asm volatile(
+          "s_waitcnt vmcnt(%4)\n\t"
+          "ds_read_b128 %0, %2 offset:%5\n\t"
+          "ds_read_b128 %1, %3 offset:%6\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&v"(load_of(ch, L0)), "=&v"(ch.sc)
+          : "v"(codes), "v"(scales), "n"(BEHIND), "n"(SLOT * W3_BLOCK_BYTES + 1024 * L0), "n"(SLOT * W3_BLOCK_BYTES + W3_SCALE_OFFSET)
+          : "memory");
+    }
+  }
+};
 constexpr int RING_BYTES = ring_bytes<W3Ring>();  // LDS per wavefront; its first 4 KB double as the K-split exchange
 
 // ------------------------------------------------------------------------------------------- slots of one to four rows
@@ -319,6 +365,26 @@ struct FewActs {
   template <int ODD, bool MORE2, bool MORE1, class C>
   __device__ __forceinline__ void step(const C& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
     compute_few(ch, held[ODD], grp, acc0, acc1, acc2, acc3, sl.lut_lo, sl.lut_hi, q8);
+    if (MORE2) held[ODD] = load(i + 2);
+  }
+};
+
+// FewActs over the 16-row tiles T0 .. T1 - 1 of the block only (the other accumulators stay zero).
+template <int T0, int T1>
+struct FewActsPart : FewActs {
+  template <int ODD, bool MORE2, bool MORE1, class C>
+  __device__ __forceinline__ void step(const C& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
+    const u32x4_t none = {0u, 0u, 0u, 0u};
+    const u32x4_t a = held[ODD];
+    Rows rows;  // as compute_few: the lane's bytes in its own group, zero in the others
+    rows.a0 = grp == 0 ? a : none;
+    rows.a1 = grp == 1 ? a : none;
+    rows.a2 = grp == 2 ? a : none;
+    rows.a3 = grp == 3 ? a : none;
+    if (T0 <= 0 && 0 < T1) compute_tile_few<0>(ch, rows, acc0, sl.lut_lo, sl.lut_hi, q8);
+    if (T0 <= 1 && 1 < T1) compute_tile_few<1>(ch, rows, acc1, sl.lut_lo, sl.lut_hi, q8);
+    if (T0 <= 2 && 2 < T1) compute_tile_few<2>(ch, rows, acc2, sl.lut_lo, sl.lut_hi, q8);
+    if (T0 <= 3 && 3 < T1) compute_tile_few<3>(ch, rows, acc3, sl.lut_lo, sl.lut_hi, q8);
     if (MORE2) held[ODD] = load(i + 2);
   }
 };
@@ -798,10 +864,25 @@ __global__ __launch_bounds__(1024) void w3_fc12_kernel(StreamParams p1, StreamPa
 constexpr int ONE_GATE_WAVES = 4;  // the gate's dot product is laid out over 256 threads
 constexpr int ONE_MAX_WAVES = 16;
 
+// One wavefront's product over all of K for the tiles T0 .. T1 - 1 of block row nb (the others' accumulators: zero).
+template <int T0, int T1>
+__device__ __forceinline__ void one_token_tiles(const StreamParams& p, const Slot& sl, int row0, int nb, int lane, uint8_t* ring, f32x4_t (&acc)[4]) {
+  if constexpr (T0 == 0 && T1 == 4) {
+    stream_block<EPI_FC2, FewActs, W3RingCached>(p, sl, row0, nb, 0, p.chunks, lane, ring, acc[0], acc[1], acc[2], acc[3]);
+  } else {
+    stream_block<EPI_FC2, FewActsPart<T0, T1>, W3RingPart<0, T0, T1>>(p, sl, row0, nb, 0, p.chunks, lane, ring, acc[0], acc[1], acc[2], acc[3]);
+  }
+}
+
+// PARTS: the workgroups a 64-row block (1, 2 or 4), each taking 4 / PARTS of its four 16-row tiles - the same sums a
+// column, over more compute units: a workgroup's wavefronts expand only their tiles' codes (a slot's whole K is four
+// chunks of 204 VALU instructions a wavefront otherwise, and a workgroup's ten or eleven wavefronts share four SIMDs)
+// and ask only for the 16-byte loads those tiles' dwords lie in (one or two of a chunk's three).
+template <int PARTS>
 __global__ __launch_bounds__(1024) void w3_fc2_combine_one_kernel(StreamParams p, CombineParams c, int slots) {
   extern __shared__ __align__(16) uint8_t rings[];  // a ring a streaming wavefront, then ys [topk + 1][64], then the gate's four partial sums
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int nb = blockIdx.x, q = lane >> 4, r16 = lane & 15;
+  const int nb = blockIdx.x / PARTS, part = blockIdx.x % PARTS, q = lane >> 4, r16 = lane & 15;
   float* ys = reinterpret_cast<float*>(rings + slots * RING_BYTES);
   float* red = ys + (p.topk + 1) * 64;
   // the chain's operands, a selection a lane, asked for now; a pair whose expert is not local has no slot: its place
@@ -826,7 +907,17 @@ __global__ __launch_bounds__(1024) void w3_fc2_combine_one_kernel(StreamParams p
         for (int t = 0; t < 4; t++) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         FewPairs pairs;
         pairs.ask(p, sl, row0);
-        stream_block<EPI_FC2, FewActs, W3RingCached>(p, sl, row0, nb, 0, p.chunks, lane, reinterpret_cast<uint8_t*>(mine), acc[0], acc[1], acc[2], acc[3]);
+        uint8_t* ring = reinterpret_cast<uint8_t*>(mine);
+        if (PARTS == 1) {
+          one_token_tiles<0, 4>(p, sl, row0, nb, lane, ring, acc);
+        } else if (PARTS == 2) {
+          if (part == 0) one_token_tiles<0, 2>(p, sl, row0, nb, lane, ring, acc); else one_token_tiles<2, 4>(p, sl, row0, nb, lane, ring, acc);
+        } else {
+          if (part == 0) one_token_tiles<0, 1>(p, sl, row0, nb, lane, ring, acc);
+          else if (part == 1) one_token_tiles<1, 2>(p, sl, row0, nb, lane, ring, acc);
+          else if (part == 2) one_token_tiles<2, 3>(p, sl, row0, nb, lane, ring, acc);
+          else one_token_tiles<3, 4>(p, sl, row0, nb, lane, ring, acc);
+        }
 #pragma unroll
         for (int t = 0; t < 4; t++) {
           mine[(t * 4 + 0) * 64 + lane] = acc[t].x;
@@ -848,6 +939,7 @@ __global__ __launch_bounds__(1024) void w3_fc2_combine_one_kernel(StreamParams p
   }
   __syncthreads();
   if (wave != 0) return;
+  if (PARTS > 1 && q / (4 / PARTS) != part) return;  // lane (q, r16) is column 16 q + r16: another workgroup's tile
   float v = 0.f;
   for (int s = 0; s < p.topk; s++) {
     const bool keep = __builtin_amdgcn_readlane((int)keep_mine, s) != 0;
@@ -892,7 +984,7 @@ struct TileW3 {
 
 // ---------------------------------------------------------------------------------------------------- host side
 struct Tuning {  // hb_tune's knobs: relaxed atomics, so a knob set from one thread while another launches is a plain race-free read
-  std::atomic<int> w3_tile{0}, w3_few{0}, w3_ksplit{0}, w3_nbw{0}, moe_fc1_ksplit{0}, moe_fc1_nbw{0}, moe_fc2_ksplit{0}, moe_fc2_nbw{0}, moe_one{0}, moe_split{0}, moe_fused{0}, moe_lag{0}, fault_inject{0};
+  std::atomic<int> w3_tile{0}, w3_few{0}, w3_ksplit{0}, w3_nbw{0}, moe_fc1_ksplit{0}, moe_fc1_nbw{0}, moe_fc2_ksplit{0}, moe_fc2_nbw{0}, moe_one{0}, moe_split{0}, moe_fused{0}, moe_lag{0}, fault_inject{0}, moe_one_parts{0};
 };
 static Tuning g_tune;
 
@@ -955,7 +1047,7 @@ extern "C" int hb_tune(const char* key, int value) {
     std::atomic<int>* slot;
   } table[] = {{"w3_tile", &g_tune.w3_tile}, {"w3_few", &g_tune.w3_few}, {"w3_ksplit", &g_tune.w3_ksplit},           {"w3_nbw", &g_tune.w3_nbw},
                {"moe_fc1_ksplit", &g_tune.moe_fc1_ksplit}, {"moe_fc1_nbw", &g_tune.moe_fc1_nbw},
-               {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}, {"moe_one", &g_tune.moe_one}, {"moe_split", &g_tune.moe_split}, {"moe_fused", &g_tune.moe_fused}, {"moe_lag", &g_tune.moe_lag}, {"fault_inject", &g_tune.fault_inject}};
+               {"moe_fc2_ksplit", &g_tune.moe_fc2_ksplit}, {"moe_fc2_nbw", &g_tune.moe_fc2_nbw}, {"moe_one", &g_tune.moe_one}, {"moe_split", &g_tune.moe_split}, {"moe_fused", &g_tune.moe_fused}, {"moe_lag", &g_tune.moe_lag}, {"fault_inject", &g_tune.fault_inject}, {"moe_one_parts", &g_tune.moe_one_parts}};
   for (auto& t : table)
     if (!strcmp(t.name, key)) {
       if (value < 0 || value > 16) return HB_EINVAL;
@@ -1236,8 +1328,16 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
     f2.ks = 1;
     f2.nbw = 1;
     set_split(f2);
-    HB_LAUNCH(w3_fc2_combine_one_kernel, dim3((unsigned)f2.n_blocks), dim3(64 * one_waves), (size_t)slots * RING_BYTES + (topk + 1) * 256 + 16, stream, f2,
-              *combine, (int)slots);
+    // the workgroups a 64-row block: as many as leave the launch within about the device's compute units
+    const int parts = g_tune.moe_one_parts ? g_tune.moe_one_parts.load() : f2.n_blocks <= 64 ? 4 : f2.n_blocks <= 128 ? 2 : 1;
+    const size_t lds = (size_t)slots * RING_BYTES + (topk + 1) * 256 + 16;
+    if (parts == 4) {
+      HB_LAUNCH(w3_fc2_combine_one_kernel<4>, dim3(4u * (unsigned)f2.n_blocks), dim3(64 * one_waves), lds, stream, f2, *combine, (int)slots);
+    } else if (parts == 2) {
+      HB_LAUNCH(w3_fc2_combine_one_kernel<2>, dim3(2u * (unsigned)f2.n_blocks), dim3(64 * one_waves), lds, stream, f2, *combine, (int)slots);
+    } else {
+      HB_LAUNCH(w3_fc2_combine_one_kernel<1>, dim3((unsigned)f2.n_blocks), dim3(64 * one_waves), lds, stream, f2, *combine, (int)slots);
+    }
     return launch_status();
   }
   if (int e = launch_stream<EPI_FC2>(f2, slots, est, l2, stream)) return e;
