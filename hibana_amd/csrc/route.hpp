@@ -84,8 +84,15 @@ __device__ __forceinline__ int route_row(const RouteParams& p, int r, int lane, 
   float val[PER];   // the weight an expert would get before renormalization
   uint32_t key[PER];
   float lg[PER];    // the lane's logits: every load is asked for before the first is used
+  if (!THROUGH && PER == 8 && per == 8 && e == 512 && !((p.stride | (int64_t)(reinterpret_cast<uintptr_t>(p.logits) >> 2)) & 3)) {
+    // the lane's eight logits are 32 consecutive bytes on a 16-byte boundary: two loads instead of eight
+    const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(row + first), hi = *reinterpret_cast<const f32x4_t*>(row + first + 4);
+    lg[0] = lo.x, lg[1] = lo.y, lg[2] = lo.z, lg[3] = lo.w;
+    if constexpr (PER >= 8) lg[4] = hi.x, lg[5] = hi.y, lg[6] = hi.z, lg[7] = hi.w;
+  } else {
 #pragma unroll
-  for (int j = 0; j < PER; j++) lg[j] = logit(row + min(first + j, e - 1));
+    for (int j = 0; j < PER; j++) lg[j] = logit(row + min(first + j, e - 1));
+  }
   if (SIGMOID) {
     float bs[PER];
 #pragma unroll
