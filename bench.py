@@ -15,7 +15,8 @@ events, against the vendor peak and against a plain streaming read measured in t
 
 The other BASELINE configs are `--config 2` (the same layer at M = 1), `--config 0` / `--config 1` (the w3 / NVFP4 dense
 decode projection, `--rows` for M) and `--config 4` (the NVFP4 latent-MoE layer on a 2048-token prefill chunk, MFMA
-roofline); they print the same kind of line without the CPU leg (config 2 keeps it).
+roofline); they print the same kind of line (configs 0, 2 and 4 with a CPU leg of their own). The default run carries
+configs 0, 1 and 4 as `other_configs` and config 2 as `m1`.
 """
 from __future__ import annotations
 
@@ -290,7 +291,7 @@ def dense_decode(args) -> dict:
         n = k = 5120
         nbytes = w3_bytes(n, k)
         args.layers = max(args.layers, -(-320_000_000 // nbytes))  # more than the 256 MB Infinity Cache holds, so that every step streams from HBM
-        mats = [w3.tile(synthetic.w3_matrix(n, k, 40 + i, dev, "uniform"), release=True) for i in range(args.layers)]
+        mats = [w3.tile(synthetic.w3_matrix(n, k, 40 + i, dev, "uniform"), release=bool(i) or args.no_cpu) for i in range(args.layers)]  # the CPU leg reads matrix 0 in the checkpoint layout
         x = torch.randn(m, k, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
 
         def step(i: int):
@@ -366,6 +367,29 @@ def dense_decode(args) -> dict:
                 outs = [run(i) for i in range(args.steps)]
             by_rows[str(rows)] = {"us_per_call": median(replay_times(g2, args.steps)) * 1e3, "kernel": name}
             del outs, g2
+    cpu, check = None, None
+    if args.config == 0 and not args.no_cpu:
+        # BASELINE config 0 is the reference's own CPU-runnable case: the C oracle's dense product (unpack the matrix from
+        # the checkpoint layout, FP32 matmul; OpenMP over the output rows) on this host's cores, whole calls for a few seconds
+        import numpy as np
+
+        from oracle import c_port
+        w0 = mats[0]
+        host = {"planes": w0.planes.view(torch.int32).cpu().numpy().view(np.uint32), "scales": w0.scales.cpu().numpy(), "row_scale": w0.row_scale.cpu().numpy(),
+                "out_features": n, "in_features": k, "codebook": w0.codebook}
+        xb = x.view(torch.int16).cpu().numpy().view(np.uint16)
+        want = c_port.linear(host, xb)
+        calls, spent = 0, 0.0
+        while spent < 8.0 and calls < 200:
+            t0 = time.perf_counter()
+            c_port.linear(host, xb)
+            spent += time.perf_counter() - t0
+            calls += 1
+        cpu = {"value": m * calls / spent, "unit": "tokens/s", "cores": c_port.threads(), "kind": "port",
+               "sample": f"{calls} whole calls of the {n} x {k} product at M = {m} on matrix 0: C/OpenMP oracle, unpack from the checkpoint layout + FP32 matmul"}
+        got = step(0).float().cpu()
+        ref = torch.from_numpy(want.view(np.int16).copy()).view(torch.bfloat16).float()
+        check = {"max_rel_vs_cpu_oracle": float((got - ref).abs().max() / ref.abs().max()), "norm_rel_vs_cpu_oracle": float((got - ref).norm() / ref.norm())}
     line = {
         "metric": "dense decode projection tokens/s, with achieved HBM GB/s", "value": m * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "ms_per_step_min": times[0], "ms_per_step_max": times[-1],
@@ -376,7 +400,8 @@ def dense_decode(args) -> dict:
                      # HBM bytes a launch: scaled FETCH_SIZE + WRITE_SIZE over the algorithmic bytes, measured with
                      # rocprofv3 --pmc on this workload (the summary under profiles/ states it), applied to this run's bytes
                      "traffic": None if ratio is None else ratio * nbytes, "launch_bytes": nbytes, "launch_ms": kernel_ms},
-        "cpu_baseline": None,
+        "cpu_baseline": cpu,
+        "parity": check,
     }
     if by_rows:
         line["by_rows"] = by_rows

@@ -32,6 +32,15 @@ def test_decode_modes(flags, kernel):
     assert 0 < roof["frac"] < 1 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-9
 
 
+def test_config_0_carries_the_cpu_leg_and_its_parity():
+    """The reference's own CPU-runnable case: the C oracle's dense product timed beside the GPU's, and the two results
+    held against each other (scale-relative 2e-2, norm-relative 4e-3)."""
+    line = run("--config", "0", "--steps", "12", "--warmup", "2")
+    cpu = line["cpu_baseline"]
+    assert cpu["kind"] == "port" and cpu["unit"] == "tokens/s" and cpu["value"] > 0 and cpu["cores"] >= 1 and "whole calls" in cpu["sample"]
+    assert line["parity"]["max_rel_vs_cpu_oracle"] < 2e-2 and line["parity"]["norm_rel_vs_cpu_oracle"] < 4e-3
+
+
 def test_headline_modes():
     line = run("--no-cpu", "--headline-only", "--layers", "2", "--steps", "24", "--warmup", "4", "--copy-mib", "64")
     assert "w3_fc12_kernel" in line["roofline"]["kernel"] and line["cpu_baseline"] is None and line["m1"]["value"] > 0
