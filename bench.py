@@ -291,13 +291,16 @@ def dense_decode(args) -> dict:
         n = k = 5120
         nbytes = w3_bytes(n, k)
         args.layers = max(args.layers, -(-320_000_000 // nbytes))  # more than the 256 MB Infinity Cache holds, so that every step streams from HBM
-        mats = [w3.tile(synthetic.w3_matrix(n, k, 40 + i, dev, "uniform"), release=bool(i) or args.no_cpu) for i in range(args.layers)]  # the CPU leg reads matrix 0 in the checkpoint layout
+        book = args.codebook  # "lloyd2": a two-bit matrix, streamed at 2.25 bits a weight
+        bits = 2 if book == "lloyd2" else 3
+        nbytes = n * k * bits // 8 + n * k // 32 + 4 * n
+        mats = [w3.tile(synthetic.w3_matrix(n, k, 40 + i, dev, book), release=bool(i) or args.no_cpu) for i in range(args.layers)]  # the CPU leg reads matrix 0 in the checkpoint layout
         x = torch.randn(m, k, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
 
         def step(i: int):
             return w3.w3_linear(x, mats[i % args.layers])
 
-        kernel, what = "w3_stream_kernel<dense>", f"BASELINE config 0: w3 dense linear {n} x {k}, M = {m}, uniform codebook"
+        kernel, what = "w3_stream_kernel<dense>", f"BASELINE config 0: w3 dense linear {n} x {k}, M = {m}, {book} codebook" + (" (two-bit tiles)" if bits == 2 else "")
     else:
         n, k = 25600, 5120
         size = lib.hb_nvfp4_tiled_bytes(n, k)
@@ -602,6 +605,8 @@ def main() -> int:
                     help="3: the headline w3 verify-batch layer (with the M = 1 layer as a sub-record); 2: the same layer at M = 1 alone; 0 / 1: the "
                          "w3 / NVFP4 dense decode projection; 4: the NVFP4 prefill layer")
     ap.add_argument("--rows", type=int, default=1, help="configs 0 and 1: activation rows M")
+    ap.add_argument("--codebook", default="uniform", choices=("uniform", "lloyd", "zero8", "lloyd2"),
+                    help="config 0: the matrix's codebook (lloyd2: four levels, the two-bit tile layout)")
     ap.add_argument("--small-rows", type=int, default=0, help="config 4: only its block (with a shared expert) at this many rows (1 .. 16) through the "
                     "small-call kernels")
     ap.add_argument("--routing", type=int, nargs="?", const=0, default=None, metavar="ROWS",

@@ -17,7 +17,7 @@ def w3_matrix(rows: int, k: int, seed: int, device="cuda", codebook="lloyd", row
     parts = []
     for r0 in range(0, rows, rows_per_piece):
         n = min(rows_per_piece, rows - r0)
-        q = torch.randint(0, 8, (n, k), generator=g, device=device, dtype=torch.uint8)
+        q = torch.randint(0, len(w3._codebook(codebook)), (n, k), generator=g, device=device, dtype=torch.uint8)  # codes of the book's levels (four: a two-bit matrix)
         s = (torch.randn(n, k // 128, generator=g, device=device).abs() * 0.02 + 1e-3).repeat_interleave(4, dim=1)
         row = (s.amax(dim=1) / torch.tensor(448.0, device=device)).clamp_min(1e-12)
         parts.append(w3.pack_codes(q, (s / row[:, None]).to(torch.float8_e4m3fn), row, codebook))
