@@ -99,6 +99,15 @@ __device__ __forceinline__ bool await_count(const int32_t* at, int need, int spi
 // The epilogue's roundings use the hardware FP32 -> BF16 conversion (round to nearest even).
 __device__ __forceinline__ uint16_t bf16_of(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 __device__ __forceinline__ float through_bf16(float f) { return (float)(__bf16)f; }
+// Two values rounded to BF16 by one packed conversion (v_cvt_pk_bf16_f32: `lo` in the low half), and the halves of such a
+// pair as FP32 again: the same roundings as bf16_of / through_bf16, half the conversions.
+typedef __attribute__((ext_vector_type(2))) float f32x2_pair_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_pair_t;
+__device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_pair_t{lo, hi}, bf16x2_pair_t));
+}
+__device__ __forceinline__ float pair_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float pair_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
 // silu with the fast exponential and division: the result is rounded to BF16 right after (8 significant bits).
 __device__ __forceinline__ float silu(float g) { return __fdividef(g, 1.0f + __expf(-g)); }

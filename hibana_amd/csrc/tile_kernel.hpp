@@ -195,15 +195,15 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
         if (EPI == EPI_FC1_GATED) {
 #pragma unroll
           for (int g = 0; g < 2; g++) {
-            uint16_t h[4];
+            float h[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
               const float su = Fmt::PER_ROW ? sl.rs[nb * 64 + 32 * g + 4 * q + r] : sl.scalar, sg = Fmt::PER_ROW ? sl.rs[nb * 64 + 32 * g + 16 + 4 * q + r] : sl.scalar;
-              const float up = through_bf16(acc[t][2 * g][r] * su), gate = through_bf16(acc[t][2 * g + 1][r] * sg);
-              h[r] = bf16_of(silu(gate) * up);
+              const uint32_t ug = bf16_pair(acc[t][2 * g][r] * su, acc[t][2 * g + 1][r] * sg);  // up and gate rounded to BF16 ...
+              h[r] = silu(pair_hi(ug)) * pair_lo(ug);                                          // ... and their product, rounded below
             }
             *reinterpret_cast<tile_u32x2_t*>(reinterpret_cast<uint16_t*>(p.out) + pos * p.out_stride + nb * 32 + 16 * g + 4 * q) =
-                tile_u32x2_t{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+                tile_u32x2_t{bf16_pair(h[0], h[1]), bf16_pair(h[2], h[3])};
           }
         } else {
           const int64_t at = (EPI == EPI_FC2 ? (int64_t)p.order[pos] : pos) * p.out_stride + nb * 64 + 4 * q;
@@ -212,16 +212,18 @@ __device__ __forceinline__ void tile_slot(const StreamParams& p, const Slot& sl,
             float y[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) y[r] = acc[t][nt][r] * (Fmt::PER_ROW ? sl.rs[nb * 64 + 16 * nt + 4 * q + r] : sl.scalar);
-            if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {
-#pragma unroll
-              for (int r = 0; r < 4; r++) {
-                const float h = fmaxf(through_bf16(y[r]), 0.f);
-                y[r] = h * h;
-              }
+            if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2) {  // bf16(relu(bf16(y))^2), two values a conversion
+              const uint32_t u01 = bf16_pair(y[0], y[1]), u23 = bf16_pair(y[2], y[3]);
+              // relu on the bits: a negative value (and -0) is a negative integer; a NaN stays one, as torch's relu leaves it
+              const float h0 = __int_as_float(max((int)(u01 << 16), 0)), h1 = __int_as_float(max((int)(u01 & 0xffff0000u), 0));
+              const float h2 = __int_as_float(max((int)(u23 << 16), 0)), h3 = __int_as_float(max((int)(u23 & 0xffff0000u), 0));
+              y[0] = h0 * h0;
+              y[1] = h1 * h1;
+              y[2] = h2 * h2;
+              y[3] = h3 * h3;
             }
             if (EPI == EPI_FC1_RELU2 || EPI == EPI_DENSE_RELU2 || EPI == EPI_DENSE || p.out_bf16) {
-              *reinterpret_cast<tile_u32x2_t*>(reinterpret_cast<uint16_t*>(p.out) + at + 16 * nt) =
-                  tile_u32x2_t{(uint32_t)bf16_of(y[0]) | ((uint32_t)bf16_of(y[1]) << 16), (uint32_t)bf16_of(y[2]) | ((uint32_t)bf16_of(y[3]) << 16)};
+              *reinterpret_cast<tile_u32x2_t*>(reinterpret_cast<uint16_t*>(p.out) + at + 16 * nt) = tile_u32x2_t{bf16_pair(y[0], y[1]), bf16_pair(y[2], y[3])};
             } else {
               *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(p.out) + at + 16 * nt) = f32x4_t{y[0], y[1], y[2], y[3]};
             }

@@ -421,48 +421,40 @@ struct FewActs8 {  // E4M3 activations: eight codes a lane and chunk, and the sc
   }
 };
 
-// The four-row body on the two-plane form of the activations (split_row): E4M3 activations times the codebook's E4M3
-// bytes as v_perm_b32 delivers them, on v_mfma_f32_16x16x128_f8f6f4 - no conversion of the weights at all, and one
-// MFMA a plane for all of a 16-row tile's 128 k. The MFMA's k index (q, byte b of a lane's 32) is k = 32 (b / 8) + 8 q
-// + b % 8 of the chunk on both sides: the weights' eight selector dwords in their order, and for the activations the
-// lane's eight bytes of its own 32-group in dwords 2 g, 2 g + 1 with zeros in the other six - A row 4 g + t is slot row
-// t over group g only, so register i of lane (q, r16) of the result is group q's sum for slot row i and weight row r16,
-// as in the BF16 form. Both planes are in the same units and add in the MFMA's accumulator; the row's activation scale
-// multiplies the result in finish_few.
-typedef __attribute__((ext_vector_type(8))) int i32x8_t;
-
-struct FewSplitActs {
-  typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
-  static constexpr int LOADS = 2;
-  u32x2_t held[2][2];   // [chunk parity][plane]: the lane's eight E4M3 bytes of its own group
+// Slots of at most TWO rows on the two-plane form of the activations (split_row: x = (hi + lo) * s, both E4M3), on
+// v_mfma_f32_16x16x32_fp8_fp8: both planes of both rows ride in the four A rows of a group - A row 4 g + 2 plane + t is
+// plane `plane` of slot row t over group g only - so the MFMA count is the BF16 body's (one a group and tile), the
+// weights are the codebook's E4M3 bytes as v_perm_b32 delivers them (no conversion: 132 VALU instructions a chunk
+// instead of 204) and an A operand is two registers. Both planes are in the same units and their sums add in
+// finish_few, where the row's activation scale multiplies the result. Register i of lane (q, r16) of a tile's result is group q's sum for
+// plane i / 2 of slot row i % 2 and weight row r16; finish_few adds the planes.
+struct FewPlaneActs {
+  static constexpr int LOADS = 1;
+  long held[2];       // the lane's eight E4M3 bytes (its row, plane and group) of the next even and the next odd chunk
   int grp;
   uint32_t q8;
-  const uint8_t* at;    // the lane's bytes of the upper plane in the wavefront's first chunk
-  __device__ __forceinline__ void load(int slot, int i) {
-    held[slot][0] = *reinterpret_cast<const u32x2_t*>(at + (int64_t)i * 256);
-    held[slot][1] = *reinterpret_cast<const u32x2_t*>(at + (int64_t)i * 256 + 128);
-  }
+  const uint8_t* at;  // ... of the wavefront's first chunk
+  __device__ __forceinline__ long load(int i) const { return *reinterpret_cast<const long*>(at + (int64_t)i * 256); }
   template <int EPI>
   __device__ __forceinline__ void start(const StreamParams& p, const Slot& sl, int row0, int c0, int n, int lane) {
     const int q = lane >> 4, r16 = lane & 15;
     grp = r16 >> 2;
     q8 = 8 * q;
-    at = p.a2 + activation_row_index<EPI>(p, sl, row0 + (r16 & 3)) * (2 * p.a_stride) + (int64_t)c0 * 256 + 32 * grp + 8 * q;
-    load(0, 0);
-    if (n > 1) load(1, 1);
+    at = p.a2 + activation_row_index<EPI>(p, sl, row0 + (r16 & 1)) * (2 * p.a_stride) + (int64_t)c0 * 256 + 64 * (r16 & 2) + 32 * grp + 8 * q;
+    held[0] = load(0);
+    if (n > 1) held[1] = load(1);
   }
   template <int NT, class C>
-  static __device__ __forceinline__ void tile(const C& w, const i32x8_t& upper, const i32x8_t& lower, f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi,
-                                              uint32_t q8) {
+  static __device__ __forceinline__ void tile(const C& w, const long a[4], f32x4_t& acc, uint32_t lut_lo, uint32_t lut_hi, uint32_t q8) {
     const uint32_t scales = chunk_scales<NT>(w);
     uint32_t sel[8];
     chunk_selectors<NT>(w, sel);
-    i32x8_t b;
-#pragma unroll
-    for (int j = 0; j < 8; j++) b[j] = (int)__builtin_amdgcn_perm(lut_hi, lut_lo, sel[j]);
     f32x4_t part = {0.f, 0.f, 0.f, 0.f};
-    part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(upper, b, part, 0, 0, 0, 0, 0, 0);
-    part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(lower, b, part, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const long b = fp8x8(__builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j]), __builtin_amdgcn_perm(lut_hi, lut_lo, sel[2 * j + 1]));
+      part = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[j], b, part, 0, 0, 0);
+    }
     const float s = __builtin_amdgcn_cvt_f32_fp8(scales >> q8, 0);  // the scale of this lane's group
     acc.x = fmaf(part.x, s, acc.x);
     acc.y = fmaf(part.y, s, acc.y);
@@ -471,21 +463,17 @@ struct FewSplitActs {
   }
   template <int ODD, bool MORE2, bool MORE1, class C>
   __device__ __forceinline__ void step(const C& ch, int i, f32x4_t& acc0, f32x4_t& acc1, f32x4_t& acc2, f32x4_t& acc3, const Slot& sl) {
-    i32x8_t upper, lower;  // the lane's bytes in its group's two dwords, zero in the others
+    long rows[4];  // MFMA j's A operand: the lane's bytes in its own group, zero in the others
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      upper[2 * j] = grp == j ? (int)held[ODD][0].x : 0;
-      upper[2 * j + 1] = grp == j ? (int)held[ODD][0].y : 0;
-      lower[2 * j] = grp == j ? (int)held[ODD][1].x : 0;
-      lower[2 * j + 1] = grp == j ? (int)held[ODD][1].y : 0;
-    }
-    tile<0>(ch, upper, lower, acc0, sl.lut_lo, sl.lut_hi, q8);
-    tile<1>(ch, upper, lower, acc1, sl.lut_lo, sl.lut_hi, q8);
-    tile<2>(ch, upper, lower, acc2, sl.lut_lo, sl.lut_hi, q8);
-    tile<3>(ch, upper, lower, acc3, sl.lut_lo, sl.lut_hi, q8);
-    if (MORE2) load(ODD, i + 2);
+    for (int j = 0; j < 4; j++) rows[j] = grp == j ? held[ODD] : 0L;
+    tile<0>(ch, rows, acc0, sl.lut_lo, sl.lut_hi, q8);
+    tile<1>(ch, rows, acc1, sl.lut_lo, sl.lut_hi, q8);
+    tile<2>(ch, rows, acc2, sl.lut_lo, sl.lut_hi, q8);
+    tile<3>(ch, rows, acc3, sl.lut_lo, sl.lut_hi, q8);
+    if (MORE2) held[ODD] = load(i + 2);
   }
 };
+constexpr int PLANE_ROWS = 2;
 
 // The activation scales of a slot's (up to) four rows, asked for ahead of the weights like the pair indices.
 struct FewScales {
@@ -603,7 +591,7 @@ struct FullActs8 {
 // multiplies by its tile's row scale (`scale`, asked for before the first chunk); a gated pair's gate comes from the
 // neighbouring tile's lane. Every wavefront of the workgroup must call it when K is split (one workgroup barrier).
 // QUANT (fc1 in the E4M3 activation mode): h leaves as codes and scales; a 32-group is two of the wavefront's DPP rows.
-template <int EPI, bool QUANT = false, bool SCALED = false>  // SCALED: the sums are of the two-plane activations and take their row's scale
+template <int EPI, bool QUANT = false, bool SCALED = false, bool PLANES = false>  // SCALED: the sums are of the two-plane activations and take their row's scale; PLANES: registers 2, 3 hold the lower plane of rows 0, 1
 __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl, int row0, float scale, int nb, bool active, int wave, int ks,
                                            int nbi, float* partial, const f32x4_t& acc0, const f32x4_t& acc1, const f32x4_t& acc2,
                                            const f32x4_t& acc3, const FewPairs& pairs = FewPairs{}, const FewScales& xs = FewScales{}) {
@@ -625,12 +613,13 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
   }
   if (!active) return;
   const float* first = partial + nbi * p.ks * STRIDE + r16;
-  const int rows = min(FEW_ROWS, sl.rows - row0);
+  const int rows = min(PLANES ? PLANE_ROWS : FEW_ROWS, sl.rows - row0);
   for (int r = ks; r < rows; r += p.ks) {
     const float* at = first + (q * 4 + r) * 64;
     float v = 0.f;
     for (int s = 0; s < p.ks; s++) {
       v += (at[0] + at[16]) + (at[32] + at[48]);
+      if (PLANES) v += (at[128] + at[144]) + (at[160] + at[176]);
       at += STRIDE;
     }
     const float y = SCALED ? v * scale * xs.of(r) : v * scale;
@@ -661,7 +650,7 @@ __device__ __forceinline__ void finish_few(const StreamParams& p, const Slot& sl
 // General kernel, any K: one workgroup per (run of p.nbw 64-row blocks, slot), K split p.ks ways across its wavefronts.
 // A8: E4M3 activations (p.aq, p.aq_scale), with the two bodies' FP8 forms; fc1 then writes h as E4M3 codes and
 // scales (p.oq, p.oq_scale), the activation rounding done in its epilogue.
-// SPLIT: slots of at most four rows read the two-plane form of the activations (p.a2) and run on the FP8 matrix cores.
+// SPLIT: slots of at most two rows read the two-plane form of the activations (p.a2) and run on the FP8 matrix cores.
 // One workgroup's work: slot `sl` (with rows), the run `bx` of p.nbw 64-row blocks; `rings`: the launch's dynamic LDS.
 template <int EPI, bool A8, bool SPLIT, class Ring = W3Ring>
 __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Slot& sl, int bx, uint8_t* rings) {
@@ -690,7 +679,7 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Sl
       }
       finish_block<EPI, true, RING_BYTES / 4, QUANT>(p, sl, rs, nb, active, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3);
     }
-  } else if (SPLIT && sl.rows <= FEW_ROWS) {  // uniform over the workgroup
+  } else if (SPLIT && sl.rows <= PLANE_ROWS) {  // uniform over the workgroup
     float scale = 0.f;
     FewPairs pairs{};
     FewScales xs{};
@@ -698,9 +687,9 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams& p, const Sl
       scale = sl.rs[nb * 64 + lane];
       if (EPI == EPI_FC2) pairs.ask(p, sl, 0);
       xs.ask<EPI>(p, sl, 0);
-      stream_block<EPI, FewSplitActs, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
+      stream_block<EPI, FewPlaneActs, Ring>(p, sl, 0, nb, share.c0, share.c1, lane, ring, acc0, acc1, acc2, acc3);
     }
-    finish_few<EPI, false, true>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs, xs);
+    finish_few<EPI, false, true, true>(p, sl, 0, scale, nb, active, wave, ks, nbi, reinterpret_cast<float*>(rings), acc0, acc1, acc2, acc3, pairs, xs);
   } else if (sl.rows <= FEW_ROWS && !p.no_few) {  // uniform over the workgroup
     float scale = 0.f;
     FewPairs pairs{};
@@ -1162,7 +1151,7 @@ int run_experts(const hb_w3_experts* ex, const hb_w3_experts* shared, const void
   const int64_t slots = moe_max_slots(pairs, ex->experts, shared_rows, slot_rows);
   if (slots > 65535) return HB_EINVAL;
   // E4M3 activations: x is rounded by further workgroups of the plan's launch, h in fc1's epilogue
-  // weight-only on the stream: x also in its two-plane form, for the slots of at most four rows (fc1 on the FP8 matrix cores)
+  // weight-only on the stream: x also in its two-plane form, for the slots of at most two rows (fc1 on the FP8 matrix cores)
   const bool split = !e4m3 && !dense && g_tune.moe_split == 1 && g_tune.w3_few != 2;
   const QuantJob xjob = split ? QuantJob{static_cast<const uint16_t*>(x), 0, ws.x2, ws.x2s, m, ex->hidden}
                               : QuantJob{static_cast<const uint16_t*>(x), (int64_t)m * ex->hidden / 8, ws.xq, ws.xs, 0, 0};

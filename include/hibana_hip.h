@@ -76,7 +76,7 @@ int hb_workspace_status(const void* workspace, int32_t* status, int wait, void* 
  * stream; "w3_few" / "nvfp4_few": 2 switches off the stream's body for slots of few rows (W3: at most four, NVFP4: at
  * most eight); "moe_one": 2 switches off the single launch that does one token's fc2 and combine; "moe_fused": 2 runs a
  * routed call's fc1 and fc2 as two launches; "moe_lag": the slots fc2 lags fc1 by in their common launch; "moe_split":
- * 1 gives fc1's few-row body a two-plane E4M3 form of x (FP8 matrix cores; 3e-4 of the norm); "route_plan": 2 keeps
+ * 1 gives fc1's slots of at most two rows a two-plane E4M3 form of x (FP8 matrix cores; 4e-4 of the norm); "route_plan": 2 keeps
  * routing and plan in separate launches; "nvfp4_tile_ks": the workgroups that share a tile's K in hb_nvfp4_gemm_ws.
  * Returns HB_EINVAL for an unknown key or a value out of range. The knobs are process-wide relaxed atomics: setting one
  * while another thread launches is a race-free read of either value, not a per-call setting. */
