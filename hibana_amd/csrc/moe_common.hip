@@ -550,14 +550,14 @@ constexpr int COMBINE_SPAN = 512;  // columns per workgroup (two per thread)
 // A row's weighted sum of its pairs at columns c, c + 1, in selection order (FP32 fma chain). The pairs of B slots are
 // read together (so the loads are all in flight at once) and a dropped slot contributes fma(0, 0, v).
 template <int B, bool BF16>
-__device__ __forceinline__ void combine_pairs_batches(const CombineParams& p, int r, int c, float& v0, float& v1) {
-  for (int s0 = 0; s0 < p.topk; s0 += B) {
-    // every load of the batch is asked for before any is used: ids and weights (the same for the whole workgroup),
-    // then the pairs - also a dropped slot's, whose values are then set aside
-    int e[B];
-    float w[B], y0[B], y1[B];
-    uint32_t half[B];
-    float2 full[B];
+struct CombineBatch {
+  int e[B];
+  float w[B];
+  uint32_t half[B];
+  float2 full[B];
+  // every load of the batch is asked for before any is used: ids and weights (the same for the whole workgroup), then
+  // the pairs - also a dropped slot's, whose values are then set aside (a pair's address does not depend on its id)
+  __device__ __forceinline__ void load(const CombineParams& p, int r, int c, int s0) {
 #pragma unroll
     for (int j = 0; j < B; j++) {
       const int s = min(s0 + j, p.topk - 1);
@@ -574,6 +574,9 @@ __device__ __forceinline__ void combine_pairs_batches(const CombineParams& p, in
         full[j] = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.pairs) + at);
       }
     }
+  }
+  __device__ __forceinline__ void add(const CombineParams& p, int s0, float& v0, float& v1) {
+    float y0[B], y1[B];
 #pragma unroll
     for (int j = 0; j < B; j++) {
       const int local = e[j] - p.e_lo;
@@ -589,44 +592,64 @@ __device__ __forceinline__ void combine_pairs_batches(const CombineParams& p, in
       v1 = fmaf(w[j], y1[j], v1);
     }
   }
+};
+
+struct CombineShared {  // the shared expert's two columns, FP32 or BF16
+  float2 f32 = {0.f, 0.f};
+  uint32_t bf16 = 0;
+  __device__ __forceinline__ void load(const CombineParams& p, int r, int c) {
+    const int64_t at = (int64_t)r * p.shared_stride + c;
+    if (p.shared_f32) {
+      f32 = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.shared) + at);
+    } else {
+      bf16 = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.shared) + at);
+    }
+  }
+};
+
+// One (row, 512-column span) a workgroup. The first batch of pairs and the shared expert's columns are asked for AHEAD
+// of the gate's dot product, whose barrier would otherwise stand between two trips to memory: the gate's own loads
+// follow them, and everything is on its way together.
+template <int B, bool BF16>
+__device__ __forceinline__ void combine_span(const CombineParams& p, float* red) {
+  const int r = blockIdx.x;
+  const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
+  const bool in = c < p.h;                                    // a thread past the row's end reads column 0 and stores nothing: it is needed at the barrier
+  const int cl = in ? c : 0;
+  CombineBatch<B, BF16> batch;
+  CombineShared sh;
+  batch.load(p, r, cl, 0);
+  if (p.shared) sh.load(p, r, cl);
+  float g = 1.0f;
+  if (p.gate_vec && p.shared) {  // uniform over the launch
+    combine_gate_partial(p.x, p.gate_vec, p.hx, r, threadIdx.x, red);
+    __syncthreads();
+    g = combine_gate_value(red);
+  }
+  float v0 = 0.f, v1 = 0.f;
+  batch.add(p, 0, v0, v1);
+  for (int s0 = B; s0 < p.topk; s0 += B) {
+    batch.load(p, r, cl, s0);
+    batch.add(p, s0, v0, v1);
+  }
+  if (p.shared) {
+    const float s0 = p.shared_f32 ? sh.f32.x : __uint_as_float(sh.bf16 << 16);
+    const float s1 = p.shared_f32 ? sh.f32.y : __uint_as_float(sh.bf16 & 0xffff0000u);
+    v0 = combine_shared(v0, g, s0);
+    v1 = combine_shared(v1, g, s1);
+  }
+  if (in) *reinterpret_cast<uint32_t*>(p.out + (int64_t)r * p.h + c) = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
 }
 // B: the slots read together - 8 or 12 where the call is long or top-k small, 24 for a short call of many slots
 // (one wait on memory instead of three); a kernel of its own each, so that the longer batches' registers are theirs alone.
 template <int B>
 __global__ __launch_bounds__(256) void moe_combine_kernel(CombineParams p) {
   __shared__ float red[4];
-  const int r = blockIdx.x;
-  float g = 1.0f;
-  if (p.gate_vec && p.shared) {
-    combine_gate_partial(p.x, p.gate_vec, p.hx, r, threadIdx.x, red);
-    __syncthreads();
-    g = combine_gate_value(red);
-  }
-  const int c = blockIdx.y * COMBINE_SPAN + 2 * threadIdx.x;  // h is even: a column pair is in or out together
-  if (c >= p.h) return;
-  float v0 = 0.f, v1 = 0.f;
-  float2 shared_f32 = {0.f, 0.f};
-  uint32_t shared_bf16 = 0;
-  if (p.shared) {  // asked for ahead of the pairs
-    const int64_t at = (int64_t)r * p.shared_stride + c;
-    if (p.shared_f32) {
-      shared_f32 = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.shared) + at);
-    } else {
-      shared_bf16 = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.shared) + at);
-    }
-  }
   if (p.pairs_bf16) {
-    combine_pairs_batches<B, true>(p, r, c, v0, v1);
+    combine_span<B, true>(p, red);
   } else {
-    combine_pairs_batches<B, false>(p, r, c, v0, v1);
+    combine_span<B, false>(p, red);
   }
-  if (p.shared) {
-    const float s0 = p.shared_f32 ? shared_f32.x : __uint_as_float(shared_bf16 << 16);
-    const float s1 = p.shared_f32 ? shared_f32.y : __uint_as_float(shared_bf16 & 0xffff0000u);
-    v0 = combine_shared(v0, g, s0);
-    v1 = combine_shared(v1, g, s1);
-  }
-  *reinterpret_cast<uint32_t*>(p.out + (int64_t)r * p.h + c) = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
 }
 
 // ------------------------------------------------------------------ the latent block's BF16 projections (M <= 16)
