@@ -188,8 +188,8 @@ def moe_layer(experts: W3Experts, x: torch.Tensor, ids: torch.Tensor, weights: t
 def moe_layer_logits(experts: W3Experts, x: torch.Tensor, logits: torch.Tensor, topk: int, shared: W3Experts | None = None,
                      gate_vec: torch.Tensor | None = None, return_routing: bool = False, e4m3: bool = False):
     """`moe_layer` from the router's FP32 logits [M, E_total]: softmax top-k routing (ops.route_topk's arithmetic) runs
-    in the same chain - inside the planning workgroup up to four rows; one token's fc2 and combine are one launch, so
-    a decode step is three -
+    in the same chain - several rows: one launch routes and plans, one does fc1 and fc2, one combines; one token: fc1's
+    wavefronts route the row themselves and fc2 and the combine are one launch, two in all -
     (hibana/model/flashnext/moe.py:122-144,177-192). With `return_routing`, also the ids and weights it used.
     `e4m3`: the experts' activations are rounded to E4M3 as in `moe_layer`."""
     if x.dtype != torch.bfloat16 or x.ndim != 2 or x.shape[1] != experts.shape13[1]:
