@@ -616,6 +616,8 @@ def main() -> int:
                     "32-group, FP8 MFMA) instead of the weight-only form; no CPU leg")
     ap.add_argument("--copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (a known-size "
                     "reference for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--tune", default="", metavar="KEY=VALUE[,KEY=VALUE]",
+                    help="measurement switches of the library (hb_tune) for a profiling run; the line says so in config.tune")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no sharding, no collectives); run with --gpus 1", file=sys.stderr)
@@ -628,15 +630,25 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
         return 2
+    tuned = {}
+    for item in filter(None, args.tune.split(",")):
+        from hibana_amd import _lib
+        key, _, value = item.partition("=")
+        _lib.check(_lib.lib().hb_tune(key.encode(), int(value)), f"hb_tune({key})")
+        tuned[key] = int(value)
+
+    def emit(line: dict) -> int:
+        if tuned:
+            line.setdefault("config", {})["tune"] = tuned  # not the library's built-in choices: a profiling line
+        print(json.dumps(line))
+        return 0
+
     if args.routing is not None:
-        print(json.dumps(routing_only(args)))
-        return 0
+        return emit(routing_only(args))
     if args.config == 4:
-        print(json.dumps(latent_small_only(args) if args.small_rows else latent_prefill(args)))
-        return 0
+        return emit(latent_small_only(args) if args.small_rows else latent_prefill(args))
     if args.config in (0, 1):
-        print(json.dumps(dense_decode(args)))
-        return 0
+        return emit(dense_decode(args))
     if args.e4m3:
         args.no_cpu = True  # the C oracle states the weight-only form
     decode = args.config == 2  # the layer at batch 1: logits from N(0, 1), ten experts and the shared one a step
@@ -742,8 +754,7 @@ def main() -> int:
                 others[name] = {"error": f"{type(err).__name__}: {err}"}
             torch.cuda.empty_cache()
         line["other_configs"] = others
-    print(json.dumps(line))
-    return 0
+    return emit(line)
 
 
 if __name__ == "__main__":
