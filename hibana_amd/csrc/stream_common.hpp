@@ -38,7 +38,7 @@ struct StreamParams {
   const uint8_t* aq;      // E4M3 activation mode: codes [rows, a_stride] ...
   const float* aq_scale;  // ... and their scales [rows, a_stride / 32]
   const uint8_t* a2;      // two-plane form of the BF16 activations (split_row below): [rows, a_stride / 128, 2, 128] E4M3 bytes ...
-  const float* a2_scale;  // ... and one FP32 scale a row; slots of at most four rows read these instead of `a`
+  const float* a2_scale;  // ... and one FP32 scale a row; slots of at most two rows read these instead of `a`
   const int32_t* plan;    // grouped calls: slot table
   const int32_t* order;   // grouped calls: sorted position -> pair index
   int m;                  // dense calls: rows
