@@ -928,7 +928,9 @@ __global__ __launch_bounds__(1024) void w3_fc2_combine_one_kernel(StreamParams p
   }
   __syncthreads();
   if (wave != 0) return;
-  if (PARTS > 1 && q / (4 / PARTS) != part) return;  // lane (q, r16) is column 16 q + r16: another workgroup's tile
+  // Every lane runs the chain and only the store is narrowed to this workgroup's tiles: the chain reads its operands
+  // from lanes 0 .. topk - 1, and what a lane outside the execution mask holds of a value computed earlier is not
+  // defined (the compiler may compute it after the branch that narrowed the mask).
   float v = 0.f;
   for (int s = 0; s < p.topk; s++) {
     const bool keep = __builtin_amdgcn_readlane((int)keep_mine, s) != 0;
@@ -936,7 +938,7 @@ __global__ __launch_bounds__(1024) void w3_fc2_combine_one_kernel(StreamParams p
     v = fmaf(keep ? w : 0.f, keep ? ys[s * 64 + lane] : 0.f, v);
   }
   if (c.shared) v = combine_shared(v, c.gate_vec ? combine_gate_value(red) : 1.0f, ys[p.topk * 64 + lane]);
-  c.out[nb * 64 + lane] = f32_to_bf16_bits(v);
+  if (PARTS == 1 || q / (4 / PARTS) == part) c.out[nb * 64 + lane] = f32_to_bf16_bits(v);  // lane (q, r16) is column 16 q + r16
 }
 
 // ------------------------------------------------------------------------------------ the prefill kernel's W3 format
